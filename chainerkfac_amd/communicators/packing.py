@@ -1,0 +1,136 @@
+"""Triangular pack / unpack of Kronecker factors and gradients into one flat
+float32 buffer: the single-GPU half of the reference communicator
+(chainerkfac/communicators/pure_nccl_communicator.py:110-148, :221-279).
+
+``arrays`` is a list (one entry per owning rank) of lists of
+``(array, triangular)`` pairs, exactly what ``chainerkfac.optimizers.kfac.extract``
+produces; arrays are float32 torch-ROCm tensors.  The collectives that sit
+between pack and unpack in the reference are not part of this package.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from .. import _lib
+from .. import device as _dev
+from . import _utility
+
+
+class _ArraysInfo(object):
+    """Descriptor of ``arrays`` in buffer order (reference ``_ArraysInfo``,
+    pure_nccl_communicator.py:221-279).  The tables live on the device inside a
+    plan of the C library and are uploaded once."""
+
+    def __init__(self, arrays):
+        flat, ranks, tris = [], [], []
+        for rank, local_arrays in enumerate(arrays):
+            for array, triangular in local_arrays:
+                if isinstance(array, torch.Tensor) and array.dtype not in (torch.float16, torch.float32):
+                    raise ValueError('dtype must be float16 or float32.')
+                _dev.require_gpu_tensor(array, 'array')
+                if triangular:
+                    if array.ndim != 2 or array.shape[0] != array.shape[1]:
+                        raise RuntimeError('triangular array must be a square matrix')
+                    tris.append(array.shape[0])
+                else:
+                    tris.append(0)
+                flat.append(array)
+                ranks.append(rank)
+        self.arrays = flat
+        self.n_arrays = len(flat)
+        self.rank = np.asarray(ranks, dtype=np.int32)
+        self.triangle_size = np.asarray(tris, dtype=np.int32)
+        sizes = np.asarray([a.numel() for a in flat], dtype=np.int64)
+        buf_sizes = np.where(self.triangle_size > 0,
+                             self.triangle_size.astype(np.int64) * (self.triangle_size + 1) // 2, sizes)
+        self.size_csum = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        self.buf_size_csum = np.concatenate([[0], np.cumsum(buf_sizes)]).astype(np.int64)
+        self.size_total = int(self.size_csum[-1])
+        self.buf_size_total = int(self.buf_size_csum[-1])
+        self.key = tuple((a.data_ptr(), a.numel(), t, r) for a, t, r in zip(flat, tris, ranks))
+        lib = _lib.load()
+        plan = ctypes.c_void_p()
+        _lib.check(lib.kfac_pack_plan_create(
+            self.n_arrays, _lib.ptr_array([a.data_ptr() for a in flat]),
+            _lib.i64_array(sizes), _lib.i32_array(tris), _lib.i32_array(ranks),
+            ctypes.byref(plan)))
+        self._plan = plan
+        assert lib.kfac_pack_plan_nelems(plan) == self.buf_size_total
+
+    @property
+    def plan(self):
+        return self._plan
+
+    def __del__(self):
+        plan = getattr(self, '_plan', None)
+        if plan is not None and _lib._lib is not None:
+            _lib._lib.kfac_pack_plan_destroy(plan)
+            self._plan = None
+
+    def show(self):
+        print('# ainfo: n_arrays: {}'.format(self.n_arrays))
+        print('# ainfo: size_total: {}'.format(self.size_total))
+        print('# ainfo: buf_size_total: {}'.format(self.buf_size_total))
+        for i in range(self.n_arrays):
+            print('# ainfo[{}], rank:{}, dptr:{}, size:{}, buf_size:{}, triangle_size:{}'.format(
+                i, self.rank[i], self.arrays[i].data_ptr(),
+                self.size_csum[i + 1] - self.size_csum[i],
+                self.buf_size_csum[i + 1] - self.buf_size_csum[i], self.triangle_size[i]))
+
+
+def _key_of(arrays):
+    return tuple((a.data_ptr(), a.numel(), bool(t), r)
+                 for r, local in enumerate(arrays) for a, t in local)
+
+
+class ArrayPacker(object):
+    """Holds the pack/unpack entry points of the reference communicator with
+    their signatures (``_pack_arrays_to_buffer`` / ``_unpack_arrays_from_buffer``,
+    pure_nccl_communicator.py:110-148).  Descriptors are cached per distinct
+    list of arrays, so steady-state calls upload nothing."""
+
+    def __init__(self, rank=0, max_cached=8):
+        self.rank = rank
+        self._cache = {}
+        self._max_cached = max_cached
+
+    def _info(self, arrays):
+        key = _key_of(arrays)
+        info = self._cache.get(key)
+        if info is None:
+            if len(self._cache) >= self._max_cached:
+                self._cache.pop(next(iter(self._cache)))
+            info = self._cache[key] = _ArraysInfo(arrays)
+        return info
+
+    def get_nelems(self, arrays):
+        return _utility.get_nelems(arrays)
+
+    @staticmethod
+    def _check_buf(gpu_buf, buf_dtype, need):
+        if buf_dtype is not None and np.dtype(buf_dtype) != np.float32:
+            raise ValueError('only a float32 buffer is supported, not {}'.format(buf_dtype))
+        _dev.require_gpu_tensor(gpu_buf, 'gpu_buf')
+        if gpu_buf.numel() < need:
+            raise ValueError('gpu_buf holds {} elements, {} needed'.format(gpu_buf.numel(), need))
+
+    def _pack_arrays_to_buffer(self, arrays, gpu_buf, buf_dtype=np.float32, target=-1,
+                               stream=None, debug=False):
+        info = self._info(arrays)
+        if debug and self.rank == 0:
+            info.show()
+        self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
+        _lib.check(_lib.load().kfac_pack_f32(
+            info.plan, gpu_buf.data_ptr(), gpu_buf.numel(), int(target),
+            _dev.stream_handle(stream)))
+
+    def _unpack_arrays_from_buffer(self, arrays, gpu_buf, buf_dtype=np.float32, target=-1,
+                                   divisor=1, stream=None, debug=False):
+        info = self._info(arrays)
+        if debug and self.rank == 0:
+            info.show()
+        self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
+        _lib.check(_lib.load().kfac_unpack_f32(
+            info.plan, gpu_buf.data_ptr(), gpu_buf.numel(), int(target), int(divisor),
+            _dev.stream_handle(stream)))

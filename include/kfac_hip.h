@@ -1,0 +1,215 @@
+/* kfac_hip.h -- C ABI of libkfac_hip.so: the K-FAC per-layer hot path of
+ * tyohei/chainerkfac as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every entry point is extern "C", returns 0 on success and a negative
+ *     KFAC_E* code on failure; kfac_last_error_string() describes the last
+ *     failure of the calling thread.  Nothing throws.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *     All work is enqueued on it; calls return without waiting for the GPU
+ *     unless stated otherwise.
+ *   - pointers named *_dev / x / gy / A / G / F / buf ... are device pointers
+ *     that the library borrows for the duration of the enqueued work.  Tables
+ *     (`ptrs`, `dims`, ...) are host arrays read before the call returns.
+ *   - all matrices are float32, C-contiguous, row-major; Kronecker factors are
+ *     full symmetric d x d arrays, as in the reference.
+ *   - the library is thread-compatible: one thread per plan / stream at a time.
+ *
+ * Each entry point cites the reference code it replaces (paths relative to the
+ * chainerkfac checkout).
+ */
+#ifndef KFAC_HIP_H_
+#define KFAC_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KFAC_ABI_VERSION 1
+
+#define KFAC_OK 0
+#define KFAC_EINVAL (-1)   /* bad argument (shape, null pointer, size)        */
+#define KFAC_EHIP (-2)     /* a HIP runtime call failed                        */
+#define KFAC_ENOMEM (-3)   /* caller workspace too small / allocation failed   */
+
+int kfac_abi_version(void);
+const char *kfac_last_error_string(void);
+
+/* ------------------------------------------------------------------------
+ * (4) Communicator buffer layout: triangular pack / unpack
+ * --------------------------------------------------------------------- */
+
+/* Packed length of a list of arrays: n(n+1)/2 for a triangular array of side
+ * n = triangle_size[i] (> 0), sizes[i] otherwise.
+ * Replaces communicators/_utility.py:72-83 (get_nelems).  Returns -1 on a
+ * triangular entry whose size is not triangle_size^2. */
+int64_t kfac_packed_nelems(int n_arrays, const int64_t *sizes,
+                           const int32_t *triangle_size);
+
+/* Descriptor of a list of arrays in buffer order; replaces _ArraysInfo
+ * (communicators/pure_nccl_communicator.py:221-279).  The tables are uploaded
+ * once; kfac_pack_plan_set_ptrs re-uploads only the pointers. */
+typedef struct kfac_pack_plan *kfac_pack_plan_t;
+
+int kfac_pack_plan_create(int n_arrays, const void *const *ptrs,
+                          const int64_t *sizes, const int32_t *triangle_size,
+                          const int32_t *rank_of, kfac_pack_plan_t *plan_out);
+int kfac_pack_plan_set_ptrs(kfac_pack_plan_t plan, const void *const *ptrs,
+                            void *stream);
+int64_t kfac_pack_plan_nelems(kfac_pack_plan_t plan);
+int kfac_pack_plan_destroy(kfac_pack_plan_t plan);
+
+/* buf[off_j + r(r+1)/2 + c] = M_j[r, c] for c <= r (triangular arrays), flat
+ * copy otherwise; arrays whose rank differs from target_rank are skipped when
+ * target_rank >= 0.  Replaces cupy_batched_pack_arrays and its launch
+ * (pure_nccl_communicator.py:300-377, :110-127). */
+int kfac_pack_f32(kfac_pack_plan_t plan, float *buf, int64_t buf_nelems,
+                  int target_rank, void *stream);
+
+/* M_j[r, c] = buf[off_j + tri(max(r,c), min(r,c))] / divisor for every r, c
+ * (both triangles), flat arrays copied and divided.  Replaces
+ * cupy_batched_unpack_arrays and its launch (pure_nccl_communicator.py:380-463,
+ * :129-148). */
+int kfac_unpack_f32(kfac_pack_plan_t plan, const float *buf, int64_t buf_nelems,
+                    int target_rank, int divisor, void *stream);
+
+/* ------------------------------------------------------------------------
+ * (1) Kronecker-factor construction:  C = beta*C + alpha * P^T P
+ *     beta = 1, alpha = scale/acc_iters gives the running accumulation of
+ *     optimizers/kfac.py:294-304; beta = 0 the plain covariance.
+ *     All of them need kfac_cov_workspace_bytes(d, rows) bytes of workspace.
+ * --------------------------------------------------------------------- */
+size_t kfac_cov_workspace_bytes(int d, int64_t rows);
+
+/* P = [x, 1] (ones column last iff append_ones), x is (n, d_in) row-major.
+ * With alpha = 1/n replaces FisherBlockLinear.compute_A
+ * (optimizers/fisher_blocks/connections/linear.py:14-27); with x = gy,
+ * append_ones = 0 and alpha = gy_scale^2/n replaces compute_G (:29-46); with
+ * the (n, 2C) batch-norm gradient matrix it is the last step of compute_F. */
+int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_ones,
+                        float alpha, float beta, float *C, void *ws,
+                        size_t ws_bytes, void *stream);
+
+/* P = im2col patches of the NCHW tensor x: rows (sample, y, x), columns
+ * (c, kh, kw) then the ones column; zero padding, floor output size.  The
+ * patch matrix is never materialised.  With alpha = 1/n replaces
+ * FisherBlockConvolution2D.compute_A (connections/convolution_2d.py:19-41). */
+int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, int kh,
+                        int kw, int sy, int sx, int ph, int pw, int append_ones,
+                        float alpha, float beta, float *C, void *ws,
+                        size_t ws_bytes, void *stream);
+
+/* P = gy viewed as (n*ho*wo, c) from the NCHW tensor gy, read in place.  With
+ * alpha = gy_scale^2/(n*ho*wo) replaces compute_G (convolution_2d.py:43-72). */
+int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, float alpha,
+                        float beta, float *C, void *ws, size_t ws_bytes,
+                        void *stream);
+
+/* Per-sample batch-norm gradient matrix U (n, 2C) = [sum_hw gy'*h | sum_hw gy']
+ * with h the batch-normalised x (biased variance, eps inside the root) and
+ * gy' = gy*gy_scale; hw = 1 for 2-D inputs.  Only the gamma half / beta half
+ * is written when has_beta / has_gamma is 0 (U is then (n, C)).  Replaces
+ * normalizations/batch_normalization.py:86-119; follow with
+ * kfac_cov_linear_f32(U, n, width, 0, 1/n, ...) for :121-131.
+ * Workspace: kfac_bn_workspace_bytes(n, c). */
+size_t kfac_bn_workspace_bytes(int n, int c);
+int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, int c,
+                            int hw, float eps, float gy_scale, int has_gamma,
+                            int has_beta, float *U, void *ws, size_t ws_bytes,
+                            void *stream);
+
+/* y_i = a*x_i + b*y_i over `count` arrays (host tables of device pointers).
+ * Moving average of optimizers/fisher_block.py:162-163 (a = decay on the new
+ * covariance, b = 1-decay) and the unfused accumulation of kfac.py:286-304. */
+int kfac_axpby_f32(const float *x, float *y, int64_t nelems, float a, float b,
+                   void *stream);
+
+/* ------------------------------------------------------------------------
+ * (2) Damping and the damped inverse
+ * --------------------------------------------------------------------- */
+
+/* One plan per list of factor dimensions; holds the tile schedule on the
+ * device.  The inverse of every matrix is potrf (blocked Cholesky) followed by
+ * potri (triangular inverse, then L^-T L^-1), all matrices advancing together
+ * one block column per launch. */
+typedef struct kfac_inverse_plan *kfac_inverse_plan_t;
+
+int kfac_inverse_plan_create(int count, const int32_t *dims,
+                             kfac_inverse_plan_t *plan_out);
+size_t kfac_inverse_plan_workspace_bytes(kfac_inverse_plan_t plan);
+int kfac_inverse_plan_destroy(kfac_inverse_plan_t plan);
+
+/* out_i = in_i^-1 for SPD in_i (dims given at plan creation); the full
+ * symmetric inverse is written.  in_i is read only.  info_dev[i] (device,
+ * int32) receives 0, or 1 + the index of the first non-positive pivot, which
+ * the reference GPU path silently ignores (dev_info is never read,
+ * optimizers/cholesky_inverse.py:42,94,100) and the NumPy path raises on.
+ * Replaces inverse(a, use_cholesky=True) (cholesky_inverse.py:16-102) and the
+ * per-factor loop of FisherBlock.update_invs (fisher_block.py:165-179). */
+int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
+                                 const float *const *in_ptrs,
+                                 float *const *out_ptrs, int32_t *info_dev,
+                                 void *ws, size_t ws_bytes, void *stream);
+
+/* Trace-norm pi and in-place damping of `count` (A, G) pairs:
+ *   pi = float32(sqrt((tr A * dim G) / (tr G * dim A)))   (1 if !use_pi)
+ *   diag(A) += pi*rW, diag(G) += rW/pi, the sums formed in float64 and
+ *   rounded to float32 on store.
+ * pi_out_dev (device, count floats, may be NULL) receives pi.
+ * Replaces compute_pi_tracenorm (fisher_block.py:23-42),
+ * FisherBlockConnection.get_diagvals (fisher_blocks/connection.py:66-77) and
+ * the fill_diagonal of update_invs (fisher_block.py:175). */
+typedef struct kfac_damp_plan *kfac_damp_plan_t;
+int kfac_damp_plan_create(int count, const int32_t *dimsA, const int32_t *dimsG,
+                          kfac_damp_plan_t *plan_out);
+int kfac_damp_plan_destroy(kfac_damp_plan_t plan);
+int kfac_pi_damp_batched_f32(kfac_damp_plan_t plan, float *const *A_ptrs,
+                             float *const *G_ptrs, const double *rW, int use_pi,
+                             float *pi_out_dev, void *stream);
+
+/* diag(M)[i] += (i < split ? v0 : v1), float64 sum rounded to float32.
+ * Batch-norm damping (normalizations/batch_normalization.py:133-157 with
+ * fisher_block.py:175). */
+int kfac_add_diag_f32(float *M, int d, int split, double v0, double v1,
+                      void *stream);
+
+/* ------------------------------------------------------------------------
+ * (3) Preconditioning
+ * --------------------------------------------------------------------- */
+
+/* kf = (Ginv . [gradW | gradb]) . Ainv, the left product first;
+ * kfW = kf[:, :dA-1] (or all of kf when gradb is NULL), kfb = kf[:, -1].
+ * gradW is (dG, dA - has_bias) row-major (the weight gradient reshaped to
+ * (c_out, -1)).  Workspace: kfac_precond_conn_workspace_bytes(dG, dA).
+ * Replaces compute_kfgrads (connections/linear.py:48-61,
+ * connections/convolution_2d.py:74-90) and the split of
+ * FisherBlockConnection.update_kfgrads (fisher_blocks/connection.py:51-61). */
+size_t kfac_precond_conn_workspace_bytes(int dG, int dA);
+int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ainv, int dA,
+                          const float *gradW, const float *gradb, float *kfW,
+                          float *kfb, void *ws, size_t ws_bytes, void *stream);
+
+/* kf = Finv . [g_gamma ; g_beta] split at n_gamma; if any element of kf is
+ * NaN every output is the raw gradient instead and *nan_flag_dev (device
+ * int32, may be NULL) is set to 1, else 0.  Either half may be absent
+ * (pointer NULL, size 0).  Workspace: d floats + 1 int.
+ * Replaces batch_normalization.py:159-191 and _check_nan (:21-33). */
+size_t kfac_precond_bn_workspace_bytes(int d);
+int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamma,
+                        int n_gamma, const float *g_beta, int n_beta,
+                        float *kf_gamma, float *kf_beta, int32_t *nan_flag_dev,
+                        void *ws, size_t ws_bytes, void *stream);
+
+/* v = momentum*v - lr*grad; param += v.  Replaces the 'kfac' elementwise
+ * kernel of KFACUpdateRule.update_core_gpu (optimizers/kfac.py:101-116). */
+int kfac_momentum_update_f32(float *param, float *v, const float *grad,
+                             int64_t nelems, float lr, float momentum,
+                             void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KFAC_HIP_H_ */
