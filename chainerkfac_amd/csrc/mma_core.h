@@ -1,0 +1,353 @@
+// FP32 MFMA tile engine shared by the covariance (SYRK), preconditioning (GEMM)
+// and inverse kernels.
+//
+// A workgroup of 256 threads (4 waves, 2 x 2) computes a (64*WM) x (64*WN)
+// tile of  D[i][j] = sum_k Aop(i, k) * Bop(j, k)  with v_mfma_f32_32x32x2_f32;
+// each wave owns WM x WN accumulator blocks of 32 x 32.  Operand panels
+// (rows x 32 k-values) are staged through LDS by "loaders" that know how an
+// operand is laid out in memory:
+//
+//   LoaderKC  k is the contiguous index:  (sample, row, l) tensors such as an
+//             NCHW activation viewed as rows = channel, k = (sample, pixel),
+//             and plain row-major matrices used as the k-contiguous operand.
+//   LoaderKS  row is the contiguous index: a row-major (k, row) matrix, e.g.
+//             the (batch, features) input of a Linear layer or the right-hand
+//             operand of an NN product; an optional extra row supplies the
+//             bias column (ones, or a second array).
+//   LoaderIM  implicit im2col: row = (c, kh, kw) [+ ones], k = (sample, y, x);
+//             the patch matrix is gathered straight from the NCHW tensor.
+//
+// LDS panel layouts: "RowK" (row-major, stride 33, used by KC/IM) and "KRow"
+// (k-major, stride rows+4, used by KS); both give conflict-free MFMA operand
+// reads.  The main loop keeps one LDS buffer and prefetches the next panel
+// into registers while the current one feeds the matrix cores.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace kfac {
+namespace mma {
+
+constexpr int KT = 32;        // k-values per LDS panel
+constexpr int THREADS = 256;  // 4 waves
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int ROWS>
+struct Panel {
+  static constexpr int kRowKStride = KT + 1;
+  static constexpr int kKRowStride = ROWS + 4;
+  static constexpr int kFloats =
+      (ROWS * kRowKStride > KT * kKRowStride) ? ROWS * kRowKStride : KT * kKRowStride;
+};
+
+// ---------------------------------------------------------------------------
+// LoaderKC: element (row, kg) at base + (kg / L) * sample_stride
+//                                     + row * row_stride + (kg % L)
+// rows >= rows_valid read as 0, except row == ones_row which reads as 1.
+// ---------------------------------------------------------------------------
+template <int ROWS>
+struct LoaderKC {
+  static constexpr bool kKRow = false;
+  static constexpr int NV = ROWS / 32;
+  struct Regs {
+    float4 v[NV];
+  };
+  const float *base;
+  long long sample_stride;
+  long long row_stride;
+  int L;           // k-values per sample
+  int rows_valid;
+  int ones_row;    // -1 if none
+  int vec;         // float4 loads allowed (strides, L multiples of 4, base aligned)
+
+  __device__ __forceinline__ void init(float *, int) const {}
+
+  __device__ __forceinline__ void load(Regs &r, int row0, long long k0,
+                                       long long k_end) const {
+    const int kq = (threadIdx.x & 7) * 4;
+    const int rr = threadIdx.x >> 3;
+    const long long kg = k0 + kq;
+    if (vec && kg + 3 < k_end) {
+      const long long s = kg / L;
+      const float *p = base + s * sample_stride + (kg - s * L);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int row = row0 + rr + 32 * i;
+        if (row < rows_valid)
+          r.v[i] = *reinterpret_cast<const float4 *>(p + (long long)row * row_stride);
+        else if (row == ones_row)
+          r.v[i] = make_float4(1.f, 1.f, 1.f, 1.f);
+        else
+          r.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else {
+      long long off[4];
+      bool ok[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const long long ke = kg + e;
+        ok[e] = ke < k_end;
+        const long long s = ok[e] ? ke / L : 0;
+        off[e] = ok[e] ? s * sample_stride + (ke - s * L) : 0;
+      }
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int row = row0 + rr + 32 * i;
+        float t[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (!ok[e])
+            t[e] = 0.f;
+          else if (row < rows_valid)
+            t[e] = base[off[e] + (long long)row * row_stride];
+          else
+            t[e] = (row == ones_row) ? 1.f : 0.f;
+        }
+        r.v[i] = make_float4(t[0], t[1], t[2], t[3]);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
+    const int kq = (threadIdx.x & 7) * 4;
+    const int rr = threadIdx.x >> 3;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      float *p = lds + (rr + 32 * i) * Panel<ROWS>::kRowKStride + kq;
+      p[0] = r.v[i].x;
+      p[1] = r.v[i].y;
+      p[2] = r.v[i].z;
+      p[3] = r.v[i].w;
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// LoaderKS: element (row, kg) at base + kg * ld + row for row < rows_valid;
+// row == rows_valid reads extra[kg] (or 1 when extra is null) if has_extra.
+// ---------------------------------------------------------------------------
+template <int ROWS>
+struct LoaderKS {
+  static constexpr bool kKRow = true;
+  static constexpr int RQ = ROWS / 4;          // row quads per k
+  static constexpr int KPP = THREADS / RQ;     // k-values per pass
+  static constexpr int NV = KT / KPP;
+  struct Regs {
+    float4 v[NV];
+  };
+  const float *base;
+  const float *extra;
+  long long ld;
+  int rows_valid;
+  int has_extra;
+  int vec;  // ld multiple of 4 and base 16-byte aligned
+
+  __device__ __forceinline__ void init(float *, int) const {}
+
+  __device__ __forceinline__ void load(Regs &r, int row0, long long k0,
+                                       long long k_end) const {
+    const int rq = (threadIdx.x % RQ) * 4;
+    const int kk = threadIdx.x / RQ;
+    const int row = row0 + rq;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const long long kg = k0 + kk + KPP * i;
+      if (kg >= k_end) {
+        r.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      } else if (vec && row + 3 < rows_valid) {
+        r.v[i] = *reinterpret_cast<const float4 *>(base + kg * ld + row);
+      } else {
+        float t[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int re = row + e;
+          if (re < rows_valid)
+            t[e] = base[kg * ld + re];
+          else if (re == rows_valid && has_extra)
+            t[e] = extra ? extra[kg] : 1.f;
+          else
+            t[e] = 0.f;
+        }
+        r.v[i] = make_float4(t[0], t[1], t[2], t[3]);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
+    const int rq = (threadIdx.x % RQ) * 4;
+    const int kk = threadIdx.x / RQ;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      *reinterpret_cast<float4 *>(lds + (kk + KPP * i) * Panel<ROWS>::kKRowStride + rq) = r.v[i];
+  }
+};
+
+// ---------------------------------------------------------------------------
+// LoaderIM: implicit im2col over an NCHW tensor.
+//   row = (c * kh + i) * kw + j  for row < d_patch, row == d_patch is the ones
+//   column when append_ones; kg = (sample * ho + oy) * wo + ox.
+// ---------------------------------------------------------------------------
+template <int ROWS>
+struct LoaderIM {
+  static constexpr bool kKRow = false;
+  static constexpr int NV = ROWS / 8;
+  struct Regs {
+    float v[NV];
+  };
+  const float *base;
+  int C, H, W, kh, kw, sy, sx, ph, pw, ho, wo;
+  int d_patch;
+  int append_ones;
+  int2 *table;  // LDS, ROWS entries: {offset inside a sample, (i << 16) | j} ; y = -1 zero row, -2 ones row
+
+  // Build the per-row table for panel rows [row0, row0 + ROWS).
+  __device__ __forceinline__ void init(float *lds_table, int row0) {
+    table = reinterpret_cast<int2 *>(lds_table);
+    for (int t = threadIdx.x; t < ROWS; t += THREADS) {
+      const int row = row0 + t;
+      int2 e;
+      if (row < d_patch) {
+        const int c = row / (kh * kw);
+        const int rem = row - c * (kh * kw);
+        const int i = rem / kw;
+        const int j = rem - i * kw;
+        e.x = (c * H + i) * W + j;
+        e.y = (i << 16) | j;
+      } else {
+        e.x = 0;
+        e.y = (row == d_patch && append_ones) ? -2 : -1;
+      }
+      table[t] = e;
+    }
+  }
+
+  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
+    const int k = threadIdx.x & 31;
+    const int rr = threadIdx.x >> 5;
+    const long long kg = k0 + k;
+    const bool kok = kg < k_end;
+    const int howo = ho * wo;
+    const long long s = kok ? kg / howo : 0;
+    const int rem = kok ? (int)(kg - s * howo) : 0;
+    const int oy = rem / wo;
+    const int ox = rem - oy * wo;
+    const int iy0 = oy * sy - ph;
+    const int ix0 = ox * sx - pw;
+    const long long idx0 = (s * C * H + iy0) * (long long)W + ix0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int2 e = table[rr + 8 * i];
+      float val = 0.f;
+      if (e.y >= 0) {
+        const int iy = iy0 + (e.y >> 16);
+        const int ix = ix0 + (e.y & 0xffff);
+        if (kok && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W)
+          val = base[idx0 + e.x];
+      } else if (e.y == -2) {
+        val = kok ? 1.f : 0.f;
+      }
+      r.v[i] = val;
+    }
+  }
+
+  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
+    const int k = threadIdx.x & 31;
+    const int rr = threadIdx.x >> 5;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      lds[(rr + 8 * i) * Panel<ROWS>::kRowKStride + k] = r.v[i];
+  }
+};
+
+// Operand fetch for one MFMA: lane l supplies element (row = l % 32, k = l / 32).
+template <int ROWS, bool KROW>
+__device__ __forceinline__ float fetch(const float *lds, int row, int k) {
+  if (KROW)
+    return lds[k * Panel<ROWS>::kKRowStride + row];
+  else
+    return lds[row * Panel<ROWS>::kRowKStride + k];
+}
+
+// Main loop.  acc[im][in] accumulates the 32x32 block at rows
+// (wave_m * WM + im) * 32 of the A panel and (wave_n * WN + in) * 32 of the B
+// panel.  When `same` (wave-uniform) the B operand is read from the A panel
+// and lb is not used.  ldsA / ldsB hold Panel<64*WM> / Panel<64*WN> floats.
+template <int WM, int WN, class LA, class LB>
+__device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, int rowB0,
+                                         long long kbeg, long long kend, bool same,
+                                         float *ldsA, float *ldsB,
+                                         floatx16 (&acc)[WM][WN]) {
+  constexpr int RA = 64 * WM, RB = 64 * WN;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane & 31, lk = lane >> 5;
+  typename LA::Regs ra;
+  typename LB::Regs rb;
+  if (kbeg < kend) {
+    la.load(ra, rowA0, kbeg, kend);
+    if (!same) lb.load(rb, rowB0, kbeg, kend);
+  }
+  const float *opB = same ? ldsA : ldsB;
+  for (long long k0 = kbeg; k0 < kend; k0 += KT) {
+    la.store(ra, ldsA);
+    if (!same) lb.store(rb, ldsB);
+    __syncthreads();
+    if (k0 + KT < kend) {
+      la.load(ra, rowA0, k0 + KT, kend);
+      if (!same) lb.load(rb, rowB0, k0 + KT, kend);
+    }
+#pragma unroll
+    for (int kk = 0; kk < KT / 2; ++kk) {
+      float a[WM], b[WN];
+#pragma unroll
+      for (int im = 0; im < WM; ++im)
+        a[im] = fetch<RA, LA::kKRow>(ldsA, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
+#pragma unroll
+      for (int in = 0; in < WN; ++in) {
+        if (same)
+          b[in] = fetch<RA, LA::kKRow>(opB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
+        else
+          b[in] = fetch<RB, LB::kKRow>(opB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
+      }
+#pragma unroll
+      for (int im = 0; im < WM; ++im)
+#pragma unroll
+        for (int in = 0; in < WN; ++in)
+          acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+}
+
+// Visit every accumulator element of this lane: f(row, col, value) with row /
+// col relative to the workgroup tile.
+template <int WM, int WN, class F>
+__device__ __forceinline__ void for_each_acc(floatx16 (&acc)[WM][WN], F f) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int im = 0; im < WM; ++im)
+#pragma unroll
+    for (int in = 0; in < WN; ++in)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = (wm * WM + im) * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int col = (wn * WN + in) * 32 + (lane & 31);
+        f(row, col, acc[im][in][v]);
+      }
+}
+
+template <int WM, int WN>
+__device__ __forceinline__ void zero_acc(floatx16 (&acc)[WM][WN]) {
+#pragma unroll
+  for (int im = 0; im < WM; ++im)
+#pragma unroll
+    for (int in = 0; in < WN; ++in)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[im][in][v] = 0.f;
+}
+
+}  // namespace mma
+}  // namespace kfac

@@ -1,10 +1,6 @@
 // Entry points not implemented yet: they fail loudly.
 #include "common.h"
 #define NOT_YET(name) return kfac::fail(KFAC_EINVAL, name " is not implemented yet")
-extern "C" size_t kfac_cov_workspace_bytes(int, int64_t) { return 0; }
-extern "C" int kfac_cov_linear_f32(const float *, int, int, int, float, float, float *, void *, size_t, void *) { NOT_YET("kfac_cov_linear_f32"); }
-extern "C" int kfac_cov_conv_a_f32(const float *, int, int, int, int, int, int, int, int, int, int, int, float, float, float *, void *, size_t, void *) { NOT_YET("kfac_cov_conv_a_f32"); }
-extern "C" int kfac_cov_conv_g_f32(const float *, int, int, int, float, float, float *, void *, size_t, void *) { NOT_YET("kfac_cov_conv_g_f32"); }
 extern "C" size_t kfac_bn_workspace_bytes(int, int) { return 0; }
 extern "C" int kfac_bn_grad_matrix_f32(const float *, const float *, int, int, int, float, float, int, int, float *, void *, size_t, void *) { NOT_YET("kfac_bn_grad_matrix_f32"); }
 extern "C" int kfac_inverse_plan_create(int, const int32_t *, kfac_inverse_plan_t *) { NOT_YET("kfac_inverse_plan_create"); }

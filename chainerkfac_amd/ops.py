@@ -1,0 +1,295 @@
+"""Thin tensor-level wrappers over the C ABI (one function per entry point).
+
+Inputs and outputs are float32 torch-ROCm tensors; all work is enqueued on
+torch's current stream (or the ``stream`` given).  These functions allocate
+outputs and workspace, check shapes and call libkfac_hip -- they do not
+compute anything themselves.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from . import device as _dev
+
+
+def _out(out, shape, like):
+    if out is None:
+        return torch.empty(shape, dtype=torch.float32, device=like.device)
+    _dev.require_gpu_tensor(out, 'out')
+    if tuple(out.shape) != tuple(shape):
+        raise ValueError('out has shape {}, expected {}'.format(tuple(out.shape), tuple(shape)))
+    return out
+
+
+def _cov_ws(d, rows, device):
+    lib = _lib.load()
+    nbytes = lib.kfac_cov_workspace_bytes(int(d), int(rows))
+    return _dev.workspace('cov', nbytes, device), nbytes
+
+
+def cov_linear(x, append_ones, alpha, beta=0.0, out=None, stream=None):
+    """out = beta*out + alpha * [x, 1]^T [x, 1] for x of shape (n, d_in)."""
+    _dev.require_gpu_tensor(x, 'x')
+    if x.ndim != 2:
+        raise ValueError('x must be 2-D')
+    n, d_in = x.shape
+    d = d_in + (1 if append_ones else 0)
+    if out is None and beta != 0.0:
+        raise ValueError('beta != 0 needs an existing out')
+    out = _out(out, (d, d), x)
+    ws, nbytes = _cov_ws(d, n, x.device)
+    _lib.check(_lib.load().kfac_cov_linear_f32(
+        x.data_ptr(), n, d_in, int(bool(append_ones)), alpha, beta, out.data_ptr(),
+        ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
+    return out
+
+
+def cov_conv_a(x, ksize, stride, pad, append_ones, alpha, beta=0.0, out=None, stream=None):
+    """out = beta*out + alpha * P^T P, P the im2col patch matrix of NCHW x
+    (columns (c, kh, kw) then ones)."""
+    _dev.require_gpu_tensor(x, 'x')
+    if x.ndim != 4:
+        raise ValueError('x must be NCHW')
+    kh, kw = (ksize, ksize) if isinstance(ksize, int) else ksize
+    sy, sx = (stride, stride) if isinstance(stride, int) else stride
+    ph, pw = (pad, pad) if isinstance(pad, int) else pad
+    n, c, h, w = x.shape
+    ho = (h + 2 * ph - kh) // sy + 1
+    wo = (w + 2 * pw - kw) // sx + 1
+    d = c * kh * kw + (1 if append_ones else 0)
+    if out is None and beta != 0.0:
+        raise ValueError('beta != 0 needs an existing out')
+    out = _out(out, (d, d), x)
+    ws, nbytes = _cov_ws(d, n * ho * wo, x.device)
+    _lib.check(_lib.load().kfac_cov_conv_a_f32(
+        x.data_ptr(), n, c, h, w, kh, kw, sy, sx, ph, pw, int(bool(append_ones)), alpha, beta,
+        out.data_ptr(), ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
+    return out
+
+
+def cov_conv_g(gy, alpha, beta=0.0, out=None, stream=None):
+    """out = beta*out + alpha * gy_mat^T gy_mat for NCHW gy viewed as (n*ho*wo, c)."""
+    _dev.require_gpu_tensor(gy, 'gy')
+    if gy.ndim != 4:
+        raise ValueError('gy must be NCHW')
+    n, c, ho, wo = gy.shape
+    if out is None and beta != 0.0:
+        raise ValueError('beta != 0 needs an existing out')
+    out = _out(out, (c, c), gy)
+    ws, nbytes = _cov_ws(c, n * ho * wo, gy.device)
+    _lib.check(_lib.load().kfac_cov_conv_g_f32(
+        gy.data_ptr(), n, c, ho * wo, alpha, beta, out.data_ptr(), ws.data_ptr(), ws.numel(),
+        _dev.stream_handle(stream)))
+    return out
+
+
+def bn_grad_matrix(x, gy, eps, gy_scale, has_gamma=True, has_beta=True, out=None, stream=None):
+    """(n, 2C) matrix [sum_hw gy'*h | sum_hw gy'] of a batch-norm layer."""
+    _dev.require_gpu_tensor(x, 'x')
+    _dev.require_gpu_tensor(gy, 'gy')
+    if x.ndim not in (2, 4):
+        raise RuntimeError('len(x.shape) must be 2 or 4, not {}.'.format(x.ndim))
+    if x.shape != gy.shape:
+        raise ValueError('x and gy shapes differ')
+    n, c = x.shape[0], x.shape[1]
+    hw = 1 if x.ndim == 2 else x.shape[2] * x.shape[3]
+    width = c * (int(bool(has_gamma)) + int(bool(has_beta)))
+    if width == 0:
+        raise RuntimeError('gamma and beta must not be None as the same time')
+    out = _out(out, (n, width), x)
+    lib = _lib.load()
+    nbytes = lib.kfac_bn_workspace_bytes(n, c)
+    ws = _dev.workspace('bn', nbytes, x.device)
+    _lib.check(lib.kfac_bn_grad_matrix_f32(
+        x.data_ptr(), gy.data_ptr(), n, c, hw, eps, gy_scale, int(bool(has_gamma)),
+        int(bool(has_beta)), out.data_ptr(), ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
+    return out
+
+
+def axpby(x, y, a, b, stream=None):
+    """y = a*x + b*y in place."""
+    _dev.require_gpu_tensor(x, 'x')
+    _dev.require_gpu_tensor(y, 'y')
+    if x.numel() != y.numel():
+        raise ValueError('size mismatch')
+    _lib.check(_lib.load().kfac_axpby_f32(x.data_ptr(), y.data_ptr(), x.numel(), a, b,
+                                          _dev.stream_handle(stream)))
+    return y
+
+
+def add_diag(M, v0, v1=None, split=None, stream=None):
+    """diag(M)[i] += v0 for i < split else v1 (float64 sum, float32 store)."""
+    _dev.require_gpu_tensor(M, 'M')
+    d = M.shape[0]
+    if M.ndim != 2 or M.shape[1] != d:
+        raise ValueError('M must be square')
+    if split is None:
+        split, v1 = d, v0
+    _lib.check(_lib.load().kfac_add_diag_f32(M.data_ptr(), d, int(split), float(v0), float(v1),
+                                             _dev.stream_handle(stream)))
+    return M
+
+
+class InversePlan(object):
+    """Schedule for inverting a fixed list of SPD matrix sizes together."""
+
+    def __init__(self, dims):
+        self.dims = tuple(int(d) for d in dims)
+        lib = _lib.load()
+        plan = ctypes.c_void_p()
+        _lib.check(lib.kfac_inverse_plan_create(len(self.dims), _lib.i32_array(self.dims),
+                                                ctypes.byref(plan)))
+        self._plan = plan
+        self.workspace_bytes = lib.kfac_inverse_plan_workspace_bytes(plan)
+
+    def __del__(self):
+        plan = getattr(self, '_plan', None)
+        if plan is not None and _lib._lib is not None:
+            _lib._lib.kfac_inverse_plan_destroy(plan)
+            self._plan = None
+
+    def run(self, mats, outs=None, info=None, stream=None):
+        if len(mats) != len(self.dims):
+            raise ValueError('expected {} matrices'.format(len(self.dims)))
+        for m, d in zip(mats, self.dims):
+            _dev.require_gpu_tensor(m, 'matrix')
+            if tuple(m.shape) != (d, d):
+                raise ValueError('matrix shape {} != ({}, {})'.format(tuple(m.shape), d, d))
+        if not mats:
+            return [], info
+        dev = mats[0].device
+        if outs is None:
+            outs = [torch.empty_like(m) for m in mats]
+        for o, d in zip(outs, self.dims):
+            _dev.require_gpu_tensor(o, 'out')
+            if tuple(o.shape) != (d, d):
+                raise ValueError('out shape mismatch')
+        if info is None:
+            info = torch.empty(len(mats), dtype=torch.int32, device=dev)
+        ws = _dev.workspace('inverse', self.workspace_bytes, dev)
+        _lib.check(_lib.load().kfac_spd_inverse_batched_f32(
+            self._plan, _lib.ptr_array([m.data_ptr() for m in mats]),
+            _lib.ptr_array([o.data_ptr() for o in outs]), info.data_ptr(), ws.data_ptr(),
+            ws.numel(), _dev.stream_handle(stream)))
+        return outs, info
+
+
+_inverse_plans = {}
+
+
+def inverse_plan(dims):
+    key = tuple(int(d) for d in dims)
+    plan = _inverse_plans.get(key)
+    if plan is None:
+        if len(_inverse_plans) > 64:
+            _inverse_plans.clear()
+        plan = _inverse_plans[key] = InversePlan(key)
+    return plan
+
+
+def spd_inverse_batched(mats, outs=None, info=None, stream=None):
+    """Inverses of a list of SPD matrices (potrf + potri on the GPU)."""
+    return inverse_plan([m.shape[0] for m in mats]).run(mats, outs, info, stream)
+
+
+class DampPlan(object):
+    def __init__(self, dimsA, dimsG):
+        self.dimsA = tuple(int(d) for d in dimsA)
+        self.dimsG = tuple(int(d) for d in dimsG)
+        plan = ctypes.c_void_p()
+        _lib.check(_lib.load().kfac_damp_plan_create(
+            len(self.dimsA), _lib.i32_array(self.dimsA), _lib.i32_array(self.dimsG),
+            ctypes.byref(plan)))
+        self._plan = plan
+
+    def __del__(self):
+        plan = getattr(self, '_plan', None)
+        if plan is not None and _lib._lib is not None:
+            _lib._lib.kfac_damp_plan_destroy(plan)
+            self._plan = None
+
+    def run(self, As, Gs, rW, use_pi=True, pi_out=None, stream=None):
+        for t in list(As) + list(Gs):
+            _dev.require_gpu_tensor(t, 'factor')
+        if pi_out is None:
+            pi_out = torch.empty(len(As), dtype=torch.float32, device=As[0].device)
+        _lib.check(_lib.load().kfac_pi_damp_batched_f32(
+            self._plan, _lib.ptr_array([a.data_ptr() for a in As]),
+            _lib.ptr_array([g.data_ptr() for g in Gs]), _lib.f64_array(rW), int(bool(use_pi)),
+            pi_out.data_ptr(), _dev.stream_handle(stream)))
+        return pi_out
+
+
+_damp_plans = {}
+
+
+def pi_damp_batched(As, Gs, rW, use_pi=True, pi_out=None, stream=None):
+    """In-place trace-norm damping of (A, G) pairs; returns the device vector of pi."""
+    key = (tuple(a.shape[0] for a in As), tuple(g.shape[0] for g in Gs))
+    plan = _damp_plans.get(key)
+    if plan is None:
+        if len(_damp_plans) > 64:
+            _damp_plans.clear()
+        plan = _damp_plans[key] = DampPlan(*key)
+    return plan.run(As, Gs, rW, use_pi, pi_out, stream)
+
+
+def precond_conn(Ginv, Ainv, gradW, gradb=None, kfW=None, kfb=None, stream=None):
+    """(Ginv . [gradW | gradb]) . Ainv split back into the shapes of gradW / gradb."""
+    for t, nm in ((Ginv, 'Ginv'), (Ainv, 'Ainv'), (gradW, 'gradW')):
+        _dev.require_gpu_tensor(t, nm)
+    dG, dA = Ginv.shape[0], Ainv.shape[0]
+    has_b = gradb is not None
+    if gradW.shape[0] != dG or gradW.numel() != dG * (dA - int(has_b)):
+        raise ValueError('gradW shape {} does not match factors ({}, {})'.format(
+            tuple(gradW.shape), dG, dA))
+    if has_b:
+        _dev.require_gpu_tensor(gradb, 'gradb')
+        if gradb.numel() != dG:
+            raise ValueError('gradb size mismatch')
+    kfW = torch.empty_like(gradW) if kfW is None else _dev.require_gpu_tensor(kfW, 'kfW')
+    if has_b:
+        kfb = torch.empty_like(gradb) if kfb is None else _dev.require_gpu_tensor(kfb, 'kfb')
+    lib = _lib.load()
+    nbytes = lib.kfac_precond_conn_workspace_bytes(dG, dA)
+    ws = _dev.workspace('precond', nbytes, Ginv.device)
+    _lib.check(lib.kfac_precond_conn_f32(
+        Ginv.data_ptr(), dG, Ainv.data_ptr(), dA, gradW.data_ptr(), _dev.ptr(gradb),
+        kfW.data_ptr(), _dev.ptr(kfb) if has_b else 0, ws.data_ptr(), ws.numel(),
+        _dev.stream_handle(stream)))
+    return kfW, (kfb if has_b else None)
+
+
+def precond_bn(Finv, g_gamma, g_beta, kf_gamma=None, kf_beta=None, nan_flag=None, stream=None):
+    """Finv . [g_gamma ; g_beta] with the NaN fallback to the raw gradients."""
+    _dev.require_gpu_tensor(Finv, 'Finv')
+    d = Finv.shape[0]
+    ng = 0 if g_gamma is None else g_gamma.numel()
+    nb = 0 if g_beta is None else g_beta.numel()
+    if ng + nb != d:
+        raise ValueError('gradient sizes {}+{} do not match Finv ({})'.format(ng, nb, d))
+    if g_gamma is not None:
+        _dev.require_gpu_tensor(g_gamma, 'g_gamma')
+        kf_gamma = torch.empty_like(g_gamma) if kf_gamma is None else kf_gamma
+    if g_beta is not None:
+        _dev.require_gpu_tensor(g_beta, 'g_beta')
+        kf_beta = torch.empty_like(g_beta) if kf_beta is None else kf_beta
+    if nan_flag is None:
+        nan_flag = torch.empty(1, dtype=torch.int32, device=Finv.device)
+    lib = _lib.load()
+    ws = _dev.workspace('precond_bn', lib.kfac_precond_bn_workspace_bytes(d), Finv.device)
+    _lib.check(lib.kfac_precond_bn_f32(
+        Finv.data_ptr(), d, _dev.ptr(g_gamma), ng, _dev.ptr(g_beta), nb, _dev.ptr(kf_gamma),
+        _dev.ptr(kf_beta), nan_flag.data_ptr(), ws.data_ptr(), ws.numel(),
+        _dev.stream_handle(stream)))
+    return kf_gamma, kf_beta, nan_flag
+
+
+def momentum_update(param, v, grad, lr, momentum, stream=None):
+    """v = momentum*v - lr*grad; param += v (in place)."""
+    for t in (param, v, grad):
+        _dev.require_gpu_tensor(t, 'tensor')
+    _lib.check(_lib.load().kfac_momentum_update_f32(
+        param.data_ptr(), v.data_ptr(), grad.data_ptr(), param.numel(), lr, momentum,
+        _dev.stream_handle(stream)))

@@ -1,0 +1,104 @@
+"""Parity of the HIP covariance kernels with the oracle (rel 1e-4, needs the GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kfac_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4   # covariance tolerance of the north-star spec
+
+
+def rel_err(a, ref):
+    """Norm-wise relative error against a float64 reference."""
+    ref = ref.astype(np.float64)
+    return np.linalg.norm(a.astype(np.float64) - ref) / max(np.linalg.norm(ref), 1e-30)
+
+
+def check(out, ref):
+    out = out.cpu().numpy()
+    assert out.shape == ref.shape
+    assert rel_err(out, ref) < RTOL
+    # element-wise, scaled by the largest entry (cancelling entries can be tiny)
+    assert np.max(np.abs(out - ref)) <= RTOL * np.max(np.abs(ref))
+    assert np.array_equal(out, out.T), 'factor must be exactly symmetric'
+
+
+@pytest.mark.parametrize('n,d_in,bias', [(128, 784, True), (128, 1000, True), (32, 2048, True), (7, 5, True),
+                                         (1, 3, False), (33, 64, False), (128, 10, False), (40, 321, True),
+                                         (128, 4096, True)])
+def test_linear_A(n, d_in, bias):
+    from chainerkfac_amd import ops
+    x = np.random.default_rng(n + d_in).random((n, d_in), dtype=np.float32)
+    A = ops.cov_linear(torch.from_numpy(x).cuda(), bias, 1.0 / n)
+    check(A, O.linear_A(x, bias))
+
+
+@pytest.mark.parametrize('n,d_out', [(128, 1000), (128, 10), (32, 1000), (5, 130)])
+def test_linear_G(n, d_out):
+    from chainerkfac_amd import ops
+    gy = (np.random.default_rng(n * d_out).standard_normal((n, d_out)) / n).astype(np.float32)
+    G = ops.cov_linear(torch.from_numpy(gy).cuda(), False, float(n) ** 2 / n)
+    check(G, O.linear_G(gy))
+
+
+CONV_CASES = [
+    # n, c, h, w, k, s, p, bias
+    (2, 3, 8, 8, 3, 1, 1, True),
+    (3, 2, 7, 6, 3, 2, 1, True),
+    (2, 4, 9, 9, 1, 1, 0, True),        # 1x1: NCHW slab path, 81 pixels (scalar loads)
+    (2, 8, 8, 8, 1, 1, 0, False),       # 1x1, vector loads
+    (2, 5, 8, 8, 1, 2, 0, True),        # strided 1x1 (gather path)
+    (2, 3, 12, 12, 7, 2, 3, True),      # stem-like
+    (2, 3, 10, 10, 5, 1, 0, False),
+    (4, 3, 32, 32, 3, 1, 1, True),      # CIFAR conv1 shape (28)
+    (8, 64, 16, 16, 3, 1, 1, True),     # 577
+    (4, 128, 8, 8, 3, 1, 1, True),      # 1153
+    (2, 40, 6, 6, 3, 1, 1, False),      # 360: two 128-tiles + ragged third
+    (1, 2, 3, 3, 3, 1, 1, True),        # fewer pixels than a panel
+]
+
+
+@pytest.mark.parametrize('n,c,h,w,k,s,p,bias', CONV_CASES)
+def test_conv_A(n, c, h, w, k, s, p, bias):
+    from chainerkfac_amd import ops
+    x = np.random.default_rng(c * h + k).standard_normal((n, c, h, w)).astype(np.float32)
+    A = ops.cov_conv_a(torch.from_numpy(x).cuda(), k, s, p, bias, 1.0 / n)
+    check(A, O.conv_A(x, k, s, p, bias))
+
+
+@pytest.mark.parametrize('n,c,ho,wo', [(2, 5, 3, 3), (4, 64, 16, 16), (3, 130, 7, 7), (2, 256, 4, 4),
+                                       (128, 64, 32, 32), (2, 700, 2, 2)])
+def test_conv_G(n, c, ho, wo):
+    from chainerkfac_amd import ops
+    gy = (np.random.default_rng(c + ho).standard_normal((n, c, ho, wo)) / n).astype(np.float32)
+    G = ops.cov_conv_g(torch.from_numpy(gy).cuda(), float(n) ** 2 / (n * ho * wo))
+    check(G, O.conv_G(gy))
+
+
+def test_running_accumulation_matches_mean_of_covs():
+    """beta = 1, alpha = scale/acc_iters reproduces KFAC.accumulate_covs."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(0)
+    acc_iters = 4
+    xs = [r.standard_normal((2, 6, 8, 8)).astype(np.float32) for _ in range(acc_iters)]
+    acc = None
+    out = None
+    for i, x in enumerate(xs):
+        acc = O.accumulate_covs(acc, [O.conv_A(x, 3, 1, 1, True)], acc_iters)
+        out = ops.cov_conv_a(torch.from_numpy(x).cuda(), 3, 1, 1, True, (1.0 / 2) / acc_iters,
+                             beta=0.0 if i == 0 else 1.0, out=out)
+    check(out, acc[0])
+
+
+def test_workspace_too_small_is_reported():
+    import ctypes
+    from chainerkfac_amd import _lib
+    lib = _lib.load()
+    x = torch.zeros(4, 8, device='cuda')
+    C = torch.zeros(8, 8, device='cuda')
+    rc = lib.kfac_cov_linear_f32(x.data_ptr(), 4, 8, 0, 1.0, 0.0, C.data_ptr(), None, 0, None)
+    assert rc == -3 and b'workspace' in lib.kfac_last_error_string()
+    rc = lib.kfac_cov_linear_f32(x.data_ptr(), 0, 8, 0, 1.0, 0.0, C.data_ptr(), None, 0, None)
+    assert rc == -1
