@@ -25,7 +25,10 @@ struct SyrkPlan {
   int ntile;       // lower-triangle tiles
   int nsplit;
   long long klen;  // reduction length per split (multiple of KT)
+  int nreduced;    // slots after the pre-reduction (0 = none)
 };
+
+constexpr int kFinishSplits = 8;
 
 SyrkPlan plan_syrk(int d, long long rows) {
   SyrkPlan p;
@@ -33,15 +36,53 @@ SyrkPlan plan_syrk(int d, long long rows) {
   p.tiles = kfac::ceil_div(d, p.bm);
   p.ntile = p.tiles * (p.tiles + 1) / 2;
   const long long nk = kfac::ceil_div<long long>(rows > 0 ? rows : 1, KT);
-  const long long target = 1536;  // workgroups wanted in flight (256 CUs)
-  long long ns = kfac::ceil_div<long long>(target, p.ntile);
-  const long long max_ns = nk >= 8 ? nk / 8 : 1;  // at least 8 panels per split
-  if (ns > max_ns) ns = max_ns;
-  if (ns < 1) ns = 1;
+  // Workgroups of one launch do equal work, so the launch takes
+  // ceil(workgroups / resident slots) rounds of (panels per split + fixed
+  // cost).  Pick the split count that minimises that, keeping at least 8
+  // panels per split; the fixed cost stands for the tile prologue, the
+  // partial-tile store and its later reduction.
+  const long long slots = p.bm == 128 ? 512 : 1024;
+  const long long fixed = 4;
+  const long long max_ns = nk >= 8 ? nk / 8 : 1;
+  long long ns = 1, best = -1;
+  for (long long c = 1; c <= max_ns && c <= 4096; ++c) {
+    const long long rounds = kfac::ceil_div<long long>((long long)p.ntile * c, slots);
+    const long long cost = rounds * (kfac::ceil_div(nk, c) + fixed);
+    if (best < 0 || cost < best) {
+      best = cost;
+      ns = c;
+    }
+  }
   const long long per = kfac::ceil_div(nk, ns);
   p.nsplit = (int)kfac::ceil_div(nk, per);
   p.klen = per * KT;
+  // partials are pre-reduced to at most kFinishSplits slots before finishing
+  p.nreduced = p.nsplit > kFinishSplits ? kFinishSplits : 0;
   return p;
+}
+
+size_t syrk_ws_floats(const SyrkPlan &p) {
+  return (size_t)(p.nsplit + p.nreduced) * p.ntile * p.bm * p.bm;
+}
+
+// Sums groups of splits: out slot g = sum of splits [g*per, (g+1)*per).
+__global__ __launch_bounds__(256) void reduce_kernel(const float4 *__restrict__ partial,
+                                                     float4 *__restrict__ out, int nsplit,
+                                                     int per, long long slot4) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= slot4) return;
+  const int g = blockIdx.y;
+  int s = g * per;
+  const int send = (s + per < nsplit) ? s + per : nsplit;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (; s < send; ++s) {
+    const float4 v = partial[(long long)s * slot4 + i];
+    acc.x += v.x;
+    acc.y += v.y;
+    acc.z += v.z;
+    acc.w += v.w;
+  }
+  out[(long long)g * slot4 + i] = acc;
 }
 
 __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
@@ -74,7 +115,10 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_kernel(Loader ld, long long K
   if (kend > K) kend = K;
   floatx16 acc[WM][WM];
   zero_acc<WM, WM>(acc);
-  mainloop<WM, WM>(la, lb, I * BM, J * BM, kbeg, kend, I == J, ldsA, ldsB, acc);
+  if (I == J)
+    mainloop<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
+  else
+    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
   float *out = partial + ((long long)split * ntile + tile) * (BM * BM);
   for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
 }
@@ -129,7 +173,7 @@ template <class L64, class L128>
 int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, float beta,
              float *C, void *ws, size_t ws_bytes, hipStream_t stream) {
   const SyrkPlan p = plan_syrk(d, K);
-  const size_t need = (size_t)p.nsplit * p.ntile * p.bm * p.bm * sizeof(float);
+  const size_t need = syrk_ws_floats(p) * sizeof(float);
   if (ws_bytes < need || ws == nullptr)
     return kfac::fail(KFAC_ENOMEM, "covariance workspace too small: %zu < %zu bytes",
                       ws_bytes, need);
@@ -142,9 +186,22 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, 
     hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
                        p.klen, p.ntile, partial);
   KFAC_HIP_CHECK(hipGetLastError());
+  const float *fin = partial;
+  int nfin = p.nsplit;
+  if (p.nreduced) {
+    const long long slot4 = (long long)p.ntile * p.bm * p.bm / 4;
+    float *red = partial + (size_t)p.nsplit * p.ntile * p.bm * p.bm;
+    const int per = kfac::ceil_div(p.nsplit, p.nreduced);
+    nfin = kfac::ceil_div(p.nsplit, per);
+    hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)kfac::ceil_div<long long>(slot4, 256), nfin),
+                       dim3(256), 0, stream, reinterpret_cast<const float4 *>(partial),
+                       reinterpret_cast<float4 *>(red), p.nsplit, per, slot4);
+    KFAC_HIP_CHECK(hipGetLastError());
+    fin = red;
+  }
   const int sub = kfac::ceil_div(d, 64);
-  hipLaunchKernelGGL(finish_kernel, dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, partial,
-                     p.nsplit, p.ntile, p.bm, d, alpha, beta, C);
+  hipLaunchKernelGGL(finish_kernel, dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, fin, nfin,
+                     p.ntile, p.bm, d, alpha, beta, C);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
@@ -203,8 +260,7 @@ LoaderIM<ROWS> make_im(const float *x, int c, int h, int w, int kh, int kw, int 
 
 extern "C" size_t kfac_cov_workspace_bytes(int d, int64_t rows) {
   if (d <= 0) return 0;
-  const SyrkPlan p = plan_syrk(d, rows);
-  return (size_t)p.nsplit * p.ntile * p.bm * p.bm * sizeof(float);
+  return syrk_ws_floats(plan_syrk(d, rows)) * sizeof(float);
 }
 
 extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_ones,

@@ -40,6 +40,12 @@ struct Panel {
       (ROWS * kRowKStride > KT * kKRowStride) ? ROWS * kRowKStride : KT * kKRowStride;
 };
 
+// Loader protocol: load() issues the global loads of one panel from clamped
+// (always valid) addresses and records which elements are real in bit masks;
+// store() applies the masks and writes the panel to LDS.  Nothing between the
+// two touches the loaded registers, so the loads stay in flight while the
+// matrix cores work on the previous panel.
+
 // ---------------------------------------------------------------------------
 // LoaderKC: element (row, kg) at base + (kg / L) * sample_stride
 //                                     + row * row_stride + (kg % L)
@@ -51,6 +57,8 @@ struct LoaderKC {
   static constexpr int NV = ROWS / 32;
   struct Regs {
     float4 v[NV];
+    unsigned use;   // bit 4*i+e: element e of v[i] is real data
+    unsigned one;   // bit 4*i+e: element reads as 1
   };
   const float *base;
   long long sample_stride;
@@ -67,43 +75,44 @@ struct LoaderKC {
     const int kq = (threadIdx.x & 7) * 4;
     const int rr = threadIdx.x >> 3;
     const long long kg = k0 + kq;
-    if (vec && kg + 3 < k_end) {
-      const long long s = kg / L;
-      const float *p = base + s * sample_stride + (kg - s * L);
+    r.use = 0;
+    r.one = 0;
+    if (vec) {
+      const bool kok = kg + 3 < k_end;
+      const unsigned kc = kok ? (unsigned)kg : 0u;
+      const unsigned s = kc / (unsigned)L;
+      const float *p = base + (long long)s * sample_stride + (kc - s * (unsigned)L);
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int row = row0 + rr + 32 * i;
-        if (row < rows_valid)
-          r.v[i] = *reinterpret_cast<const float4 *>(p + (long long)row * row_stride);
-        else if (row == ones_row)
-          r.v[i] = make_float4(1.f, 1.f, 1.f, 1.f);
-        else
-          r.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        const bool rok = row < rows_valid;
+        r.v[i] = *reinterpret_cast<const float4 *>(p + (long long)(rok ? row : 0) * row_stride);
+        if (rok && kok) r.use |= 0xfu << (4 * i);
+        if (kok && row == ones_row) r.one |= 0xfu << (4 * i);
       }
     } else {
       long long off[4];
-      bool ok[4];
+      unsigned okm = 0;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const long long ke = kg + e;
-        ok[e] = ke < k_end;
-        const long long s = ok[e] ? ke / L : 0;
-        off[e] = ok[e] ? s * sample_stride + (ke - s * L) : 0;
+        const bool ok = ke < k_end;
+        if (ok) okm |= 1u << e;
+        const unsigned kc = ok ? (unsigned)ke : 0u;
+        const unsigned s = kc / (unsigned)L;
+        off[e] = (long long)s * sample_stride + (kc - s * (unsigned)L);
       }
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int row = row0 + rr + 32 * i;
-        float t[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (!ok[e])
-            t[e] = 0.f;
-          else if (row < rows_valid)
-            t[e] = base[off[e] + (long long)row * row_stride];
-          else
-            t[e] = (row == ones_row) ? 1.f : 0.f;
-        }
-        r.v[i] = make_float4(t[0], t[1], t[2], t[3]);
+        const bool rok = row < rows_valid;
+        const long long ro = (long long)(rok ? row : 0) * row_stride;
+        r.v[i].x = base[off[0] + ro];
+        r.v[i].y = base[off[1] + ro];
+        r.v[i].z = base[off[2] + ro];
+        r.v[i].w = base[off[3] + ro];
+        if (rok) r.use |= okm << (4 * i);
+        if (row == ones_row) r.one |= okm << (4 * i);
       }
     }
   }
@@ -114,10 +123,12 @@ struct LoaderKC {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       float *p = lds + (rr + 32 * i) * Panel<ROWS>::kRowKStride + kq;
-      p[0] = r.v[i].x;
-      p[1] = r.v[i].y;
-      p[2] = r.v[i].z;
-      p[3] = r.v[i].w;
+      const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int bit = 4 * i + e;
+        p[e] = ((r.use >> bit) & 1u) ? t[e] : (((r.one >> bit) & 1u) ? 1.f : 0.f);
+      }
     }
   }
 };
@@ -134,6 +145,8 @@ struct LoaderKS {
   static constexpr int NV = KT / KPP;
   struct Regs {
     float4 v[NV];
+    unsigned use;
+    unsigned one;
   };
   const float *base;
   const float *extra;
@@ -149,24 +162,33 @@ struct LoaderKS {
     const int rq = (threadIdx.x % RQ) * 4;
     const int kk = threadIdx.x / RQ;
     const int row = row0 + rq;
+    r.use = 0;
+    r.one = 0;
+    if (vec && row + 3 < rows_valid) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const long long kg = k0 + kk + KPP * i;
-      if (kg >= k_end) {
-        r.v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      } else if (vec && row + 3 < rows_valid) {
-        r.v[i] = *reinterpret_cast<const float4 *>(base + kg * ld + row);
-      } else {
+      for (int i = 0; i < NV; ++i) {
+        const long long kg = k0 + kk + KPP * i;
+        const bool kok = kg < k_end;
+        r.v[i] = *reinterpret_cast<const float4 *>(base + (kok ? kg : 0) * ld + row);
+        if (kok) r.use |= 0xfu << (4 * i);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const long long kg = k0 + kk + KPP * i;
+        const bool kok = kg < k_end;
+        const long long kc = kok ? kg : 0;
         float t[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int re = row + e;
-          if (re < rows_valid)
-            t[e] = base[kg * ld + re];
-          else if (re == rows_valid && has_extra)
-            t[e] = extra ? extra[kg] : 1.f;
-          else
-            t[e] = 0.f;
+          const bool rok = re < rows_valid;
+          const bool ex = re == rows_valid && has_extra;
+          const float *q = base + kc * ld + (rok ? re : 0);
+          if (ex && extra) q = extra + kc;
+          t[e] = *q;
+          if (kok && (rok || (ex && extra))) r.use |= 1u << (4 * i + e);
+          if (kok && ex && !extra) r.one |= 1u << (4 * i + e);
         }
         r.v[i] = make_float4(t[0], t[1], t[2], t[3]);
       }
@@ -177,8 +199,17 @@ struct LoaderKS {
     const int rq = (threadIdx.x % RQ) * 4;
     const int kk = threadIdx.x / RQ;
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
-      *reinterpret_cast<float4 *>(lds + (kk + KPP * i) * Panel<ROWS>::kKRowStride + rq) = r.v[i];
+    for (int i = 0; i < NV; ++i) {
+      const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int bit = 4 * i + e;
+        o[e] = ((r.use >> bit) & 1u) ? t[e] : (((r.one >> bit) & 1u) ? 1.f : 0.f);
+      }
+      *reinterpret_cast<float4 *>(lds + (kk + KPP * i) * Panel<ROWS>::kKRowStride + rq) =
+          make_float4(o[0], o[1], o[2], o[3]);
+    }
   }
 };
 
@@ -193,12 +224,14 @@ struct LoaderIM {
   static constexpr int NV = ROWS / 8;
   struct Regs {
     float v[NV];
+    unsigned use;
+    unsigned one;
   };
   const float *base;
   int C, H, W, kh, kw, sy, sx, ph, pw, ho, wo;
   int d_patch;
   int append_ones;
-  int2 *table;  // LDS, ROWS entries: {offset inside a sample, (i << 16) | j} ; y = -1 zero row, -2 ones row
+  int2 *table;  // LDS, ROWS entries: {offset inside a sample, (i << 16) | j}; y = -1 zero row, -2 ones row
 
   // Build the per-row table for panel rows [row0, row0 + ROWS).
   __device__ __forceinline__ void init(float *lds_table, int row0) {
@@ -226,27 +259,26 @@ struct LoaderIM {
     const int rr = threadIdx.x >> 5;
     const long long kg = k0 + k;
     const bool kok = kg < k_end;
-    const int howo = ho * wo;
-    const long long s = kok ? kg / howo : 0;
-    const int rem = kok ? (int)(kg - s * howo) : 0;
-    const int oy = rem / wo;
-    const int ox = rem - oy * wo;
+    const unsigned kc = kok ? (unsigned)kg : 0u;
+    const unsigned howo = (unsigned)(ho * wo);
+    const unsigned s = kc / howo;
+    const unsigned rem = kc - s * howo;
+    const int oy = (int)(rem / (unsigned)wo);
+    const int ox = (int)rem - oy * wo;
     const int iy0 = oy * sy - ph;
     const int ix0 = ox * sx - pw;
-    const long long idx0 = (s * C * H + iy0) * (long long)W + ix0;
+    const long long idx0 = ((long long)s * C * H + iy0) * (long long)W + ix0;
+    r.use = 0;
+    r.one = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int2 e = table[rr + 8 * i];
-      float val = 0.f;
-      if (e.y >= 0) {
-        const int iy = iy0 + (e.y >> 16);
-        const int ix = ix0 + (e.y & 0xffff);
-        if (kok && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W)
-          val = base[idx0 + e.x];
-      } else if (e.y == -2) {
-        val = kok ? 1.f : 0.f;
-      }
-      r.v[i] = val;
+      const int iy = iy0 + (e.y >> 16);
+      const int ix = ix0 + (e.y & 0xffff);
+      const bool ok = kok && e.y >= 0 && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+      r.v[i] = base[ok ? idx0 + e.x : 0];
+      if (ok) r.use |= 1u << i;
+      if (kok && e.y == -2) r.one |= 1u << i;
     }
   }
 
@@ -255,7 +287,8 @@ struct LoaderIM {
     const int rr = threadIdx.x >> 5;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
-      lds[(rr + 8 * i) * Panel<ROWS>::kRowKStride + k] = r.v[i];
+      lds[(rr + 8 * i) * Panel<ROWS>::kRowKStride + k] =
+          ((r.use >> i) & 1u) ? r.v[i] : (((r.one >> i) & 1u) ? 1.f : 0.f);
   }
 };
 
@@ -270,13 +303,14 @@ __device__ __forceinline__ float fetch(const float *lds, int row, int k) {
 
 // Main loop.  acc[im][in] accumulates the 32x32 block at rows
 // (wave_m * WM + im) * 32 of the A panel and (wave_n * WN + in) * 32 of the B
-// panel.  When `same` (wave-uniform) the B operand is read from the A panel
-// and lb is not used.  ldsA / ldsB hold Panel<64*WM> / Panel<64*WN> floats.
-template <int WM, int WN, class LA, class LB>
+// panel.  With SAME the B operand is read from the A panel (diagonal tile of a
+// SYRK) and lb is not used.  ldsA / ldsB hold Panel<64*WM> / Panel<64*WN>
+// floats.  Operands of step kk+1 are fetched from LDS before the MFMAs of step
+// kk issue, so LDS latency hides behind the matrix pipeline.
+template <int WM, int WN, bool SAME, class LA, class LB>
 __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, int rowB0,
-                                         long long kbeg, long long kend, bool same,
-                                         float *ldsA, float *ldsB,
-                                         floatx16 (&acc)[WM][WN]) {
+                                         long long kbeg, long long kend, float *ldsA,
+                                         float *ldsB, floatx16 (&acc)[WM][WN]) {
   constexpr int RA = 64 * WM, RB = 64 * WN;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -286,35 +320,40 @@ __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, 
   typename LB::Regs rb;
   if (kbeg < kend) {
     la.load(ra, rowA0, kbeg, kend);
-    if (!same) lb.load(rb, rowB0, kbeg, kend);
+    if (!SAME) lb.load(rb, rowB0, kbeg, kend);
   }
-  const float *opB = same ? ldsA : ldsB;
   for (long long k0 = kbeg; k0 < kend; k0 += KT) {
     la.store(ra, ldsA);
-    if (!same) lb.store(rb, ldsB);
+    if (!SAME) lb.store(rb, ldsB);
     __syncthreads();
     if (k0 + KT < kend) {
       la.load(ra, rowA0, k0 + KT, kend);
-      if (!same) lb.load(rb, rowB0, k0 + KT, kend);
+      if (!SAME) lb.load(rb, rowB0, k0 + KT, kend);
     }
-#pragma unroll
-    for (int kk = 0; kk < KT / 2; ++kk) {
-      float a[WM], b[WN];
+    float a[2][WM], b[2][WN];
+    auto fetch_step = [&](int kk, int buf) {
 #pragma unroll
       for (int im = 0; im < WM; ++im)
-        a[im] = fetch<RA, LA::kKRow>(ldsA, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
+        a[buf][im] = fetch<RA, LA::kKRow>(ldsA, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
 #pragma unroll
       for (int in = 0; in < WN; ++in) {
-        if (same)
-          b[in] = fetch<RA, LA::kKRow>(opB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
+        if (SAME)
+          b[buf][in] = fetch<RA, LA::kKRow>(ldsA, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
         else
-          b[in] = fetch<RB, LB::kKRow>(opB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
+          b[buf][in] = fetch<RB, LB::kKRow>(ldsB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
       }
+    };
+    fetch_step(0, 0);
+#pragma unroll
+    for (int kk = 0; kk < KT / 2; ++kk) {
+      const int cur = kk & 1;
+      if (kk + 1 < KT / 2) fetch_step(kk + 1, cur ^ 1);
 #pragma unroll
       for (int im = 0; im < WM; ++im)
 #pragma unroll
         for (int in = 0; in < WN; ++in)
-          acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+          acc[im][in] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][im], b[cur][in], acc[im][in], 0, 0, 0);
     }
     __syncthreads();
   }
