@@ -1,0 +1,179 @@
+// Gradient preconditioning  kf = (G^-1 . [dW | db]) . A^-1  as two FP32 MFMA
+// GEMMs, and the batch-norm block's  kf = F^-1 . [dgamma ; dbeta]  as a GEMV
+// with the NaN fallback.  The [dW | db] concatenation is folded into the
+// operand loader of the first product and the kfgrad split into the epilogue
+// of the second, so no concatenated or sliced copy is made.
+// Replaces compute_kfgrads / update_kfgrads of
+// chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py,
+// fisher_blocks/connection.py:51-61 and normalizations/batch_normalization.py:159-191.
+#include "common.h"
+#include "mma_core.h"
+
+namespace {
+
+using namespace kfac::mma;
+
+// D[i][j] = sum_k Aop(i,k) Bop(j,k), i < M, j < N.  Column j < n_main goes to
+// C0[i*ld0 + j], column n_main (if any) to C1[i].
+template <int W, class LA, class LB>
+__global__ __launch_bounds__(THREADS, 2) void gemm_kernel(LA la, LB lb, int M, int N, int K,
+                                                          int tiles_n, float *__restrict__ C0,
+                                                          long long ld0, int n_main,
+                                                          float *__restrict__ C1) {
+  constexpr int BM = 64 * W;
+  __shared__ float ldsA[Panel<BM>::kFloats];
+  __shared__ float ldsB[Panel<BM>::kFloats];
+  const int ti = blockIdx.x / tiles_n, tj = blockIdx.x % tiles_n;
+  floatx16 acc[W][W];
+  zero_acc<W, W>(acc);
+  mainloop<W, W, false>(la, lb, ti * BM, tj * BM, 0, K, ldsA, ldsB, acc);
+  for_each_acc<W, W>(acc, [&](int r, int c, float v) {
+    const int i = ti * BM + r, j = tj * BM + c;
+    if (i < M && j < N) {
+      if (j < n_main)
+        C0[(long long)i * ld0 + j] = v;
+      else
+        C1[i] = v;
+    }
+  });
+}
+
+template <int ROWS>
+LoaderKC<ROWS> rowmajor_kc(const float *base, int rows, int K, long long ld) {
+  LoaderKC<ROWS> l;
+  l.base = base;
+  l.sample_stride = 0;
+  l.row_stride = ld;
+  l.L = K;
+  l.rows_valid = rows;
+  l.ones_row = -1;
+  l.vec = (ld % 4 == 0) && (K % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+  return l;
+}
+
+template <int ROWS>
+LoaderKS<ROWS> colop_ks(const float *base, long long ld, int rows_valid, const float *extra) {
+  LoaderKS<ROWS> l;
+  l.base = base;
+  l.extra = extra;
+  l.ld = ld;
+  l.rows_valid = rows_valid;
+  l.has_extra = extra != nullptr;
+  l.vec = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+  return l;
+}
+
+// y = F g with g = [g0 ; g1]; one wave per row.
+__global__ __launch_bounds__(256) void gemv_kernel(const float *__restrict__ F, int d,
+                                                   const float *__restrict__ g0, int n0,
+                                                   const float *__restrict__ g1,
+                                                   float *__restrict__ y) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= d) return;
+  const int lane = threadIdx.x & 63;
+  const float *fr = F + (long long)row * d;
+  float acc = 0.f;
+  for (int j = lane; j < d; j += 64) acc += fr[j] * (j < n0 ? g0[j] : g1[j - n0]);
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
+  if (lane == 0) y[row] = acc;
+}
+
+// One workgroup: if any y is NaN the outputs are the raw gradients.
+__global__ __launch_bounds__(1024) void bn_select_kernel(const float *__restrict__ y, int d,
+                                                         const float *__restrict__ g0, int n0,
+                                                         const float *__restrict__ g1,
+                                                         float *__restrict__ k0,
+                                                         float *__restrict__ k1,
+                                                         int *__restrict__ flag) {
+  __shared__ int any;
+  if (threadIdx.x == 0) any = 0;
+  __syncthreads();
+  int mine = 0;
+  for (int i = threadIdx.x; i < d; i += 1024) mine |= (y[i] != y[i]);
+  if (mine) any = 1;
+  __syncthreads();
+  const int bad = any;
+  for (int i = threadIdx.x; i < d; i += 1024) {
+    if (i < n0)
+      k0[i] = bad ? g0[i] : y[i];
+    else
+      k1[i - n0] = bad ? g1[i - n0] : y[i];
+  }
+  if (flag && threadIdx.x == 0) *flag = bad;
+}
+
+template <class LA64, class LB64, class LA128, class LB128>
+int launch_gemm(const LA64 &a64, const LB64 &b64, const LA128 &a128, const LB128 &b128, int M,
+                int N, int K, float *C0, long long ld0, int n_main, float *C1,
+                hipStream_t stream) {
+  const long long t128 = (long long)kfac::ceil_div(M, 128) * kfac::ceil_div(N, 128);
+  if (t128 >= 384) {
+    const int tn = kfac::ceil_div(N, 128);
+    hipLaunchKernelGGL((gemm_kernel<2, LA128, LB128>), dim3((unsigned)t128), dim3(THREADS), 0,
+                       stream, a128, b128, M, N, K, tn, C0, ld0, n_main, C1);
+  } else {
+    const int tn = kfac::ceil_div(N, 64);
+    const int tm = kfac::ceil_div(M, 64);
+    hipLaunchKernelGGL((gemm_kernel<1, LA64, LB64>), dim3(tm * tn), dim3(THREADS), 0, stream, a64,
+                       b64, M, N, K, tn, C0, ld0, n_main, C1);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+}  // namespace
+
+extern "C" size_t kfac_precond_conn_workspace_bytes(int dG, int dA) {
+  if (dG <= 0 || dA <= 0) return 0;
+  return (size_t)dG * dA * sizeof(float) + 256;
+}
+
+extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ainv, int dA,
+                                     const float *gradW, const float *gradb, float *kfW,
+                                     float *kfb, void *ws, size_t ws_bytes, void *stream) {
+  KFAC_REQUIRE(dG > 0 && dA > 0, "bad dimensions dG=%d dA=%d", dG, dA);
+  KFAC_REQUIRE(Ginv && Ainv && gradW && kfW, "null pointer");
+  KFAC_REQUIRE((gradb == nullptr) == (kfb == nullptr), "gradb and kfb must both be given or both null");
+  const int hb = gradb ? 1 : 0;
+  KFAC_REQUIRE(dA - hb > 0, "dA too small");
+  if (ws == nullptr || ws_bytes < kfac_precond_conn_workspace_bytes(dG, dA))
+    return kfac::fail(KFAC_ENOMEM, "preconditioning workspace too small: %zu < %zu bytes",
+                      ws_bytes, kfac_precond_conn_workspace_bytes(dG, dA));
+  hipStream_t s = kfac::as_stream(stream);
+  float *T = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
+  const int dW = dA - hb;
+  // T (dG x dA) = Ginv (dG x dG) . [gradW | gradb] (dG x dA)
+  int rc = launch_gemm(rowmajor_kc<64>(Ginv, dG, dG, dG), colop_ks<64>(gradW, dW, dW, gradb),
+                       rowmajor_kc<128>(Ginv, dG, dG, dG), colop_ks<128>(gradW, dW, dW, gradb), dG,
+                       dA, dG, T, dA, dA, nullptr, s);
+  if (rc != KFAC_OK) return rc;
+  // kf (dG x dA) = T . Ainv (symmetric: column j of Ainv is its row j)
+  return launch_gemm(rowmajor_kc<64>(T, dG, dA, dA), rowmajor_kc<64>(Ainv, dA, dA, dA),
+                     rowmajor_kc<128>(T, dG, dA, dA), rowmajor_kc<128>(Ainv, dA, dA, dA), dG, dA,
+                     dA, kfW, dW, dW, kfb, s);
+}
+
+extern "C" size_t kfac_precond_bn_workspace_bytes(int d) {
+  return d > 0 ? (size_t)d * sizeof(float) : 0;
+}
+
+extern "C" int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamma, int n_gamma,
+                                   const float *g_beta, int n_beta, float *kf_gamma,
+                                   float *kf_beta, int32_t *nan_flag_dev, void *ws,
+                                   size_t ws_bytes, void *stream) {
+  KFAC_REQUIRE(d > 0 && n_gamma >= 0 && n_beta >= 0 && n_gamma + n_beta == d,
+               "sizes %d + %d do not match d = %d", n_gamma, n_beta, d);
+  KFAC_REQUIRE(Finv != nullptr, "Finv is null");
+  KFAC_REQUIRE(n_gamma == 0 || (g_gamma && kf_gamma), "gamma pointers are null");
+  KFAC_REQUIRE(n_beta == 0 || (g_beta && kf_beta), "beta pointers are null");
+  if (ws == nullptr || ws_bytes < kfac_precond_bn_workspace_bytes(d))
+    return kfac::fail(KFAC_ENOMEM, "batch-norm preconditioning workspace too small");
+  hipStream_t s = kfac::as_stream(stream);
+  float *y = static_cast<float *>(ws);
+  hipLaunchKernelGGL(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
+                     n_gamma, g_beta, y);
+  hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
+                     kf_gamma, kf_beta, nan_flag_dev);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}

@@ -1,0 +1,131 @@
+"""Parity of the HIP damped inverse with the oracle (rel 1e-3, needs the GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kfac_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-3   # inverse tolerance of the north-star spec
+
+
+def spd(d, seed):
+    r = np.random.default_rng(seed)
+    X = r.standard_normal((2 * d, d)).astype(np.float32)
+    return (X.T @ X / np.float32(2 * d) + np.float32(1e-3) * np.eye(d, dtype=np.float32)).astype(np.float32)
+
+
+def check_inverse(M, inv):
+    d = M.shape[0]
+    ref = O.inverse(M.copy())
+    ref64 = np.linalg.inv(M.astype(np.float64))
+    nrm = np.linalg.norm(ref64)
+    assert np.linalg.norm(inv - ref) / nrm < RTOL
+    # no worse than a small multiple of the reference formula's own float32 error
+    err_ref = np.linalg.norm(ref - ref64) / nrm
+    err_hip = np.linalg.norm(inv - ref64) / nrm
+    assert err_hip < max(4 * err_ref, 1e-5)
+    resid = np.linalg.norm(M.astype(np.float64) @ inv - np.eye(d)) / np.sqrt(d)
+    assert resid < RTOL
+    assert np.array_equal(inv, inv.T), 'inverse must be exactly symmetric'
+
+
+DIMS = [1, 2, 7, 31, 32, 33, 64, 65, 127, 128, 129, 200, 257, 384, 577, 1000, 1025]
+
+
+def test_batched_inverse_mixed_sizes():
+    from chainerkfac_amd import ops
+    mats = [spd(d, 100 + d) for d in DIMS]
+    dev = [torch.from_numpy(m).cuda() for m in mats]
+    outs, info = ops.spd_inverse_batched(dev)
+    torch.cuda.synchronize()
+    assert info.cpu().tolist() == [0] * len(DIMS)
+    for m, m_dev, o in zip(mats, dev, outs):
+        assert np.array_equal(m_dev.cpu().numpy(), m), 'input must not be modified'
+        check_inverse(m, o.cpu().numpy())
+
+
+@pytest.mark.parametrize('d', [10, 148, 2305])
+def test_single_inverse_free_function(d):
+    from chainerkfac_amd.optimizers.cholesky_inverse import inverse
+    M = spd(d, d)
+    inv = inverse(torch.from_numpy(M).cuda())
+    check_inverse(M, inv.cpu().numpy())
+
+
+def test_special_cases():
+    from chainerkfac_amd import ops
+    diag = np.diag(np.array([1.0, 4.0, 0.5, 2.0, 8.0], dtype=np.float32))
+    one = np.array([[4.0]], dtype=np.float32)
+    ident = np.eye(130, dtype=np.float32)
+    outs, info = ops.spd_inverse_batched([torch.from_numpy(a).cuda() for a in (diag, one, ident)])
+    np.testing.assert_allclose(outs[0].cpu().numpy(), np.diag([1.0, 0.25, 2.0, 0.5, 0.125]), rtol=1e-6)
+    np.testing.assert_allclose(outs[1].cpu().numpy(), [[0.25]], rtol=1e-6)
+    assert np.array_equal(outs[2].cpu().numpy(), ident)
+    assert info.cpu().tolist() == [0, 0, 0]
+    outs, info = ops.spd_inverse_batched([])
+    assert outs == []
+
+
+def test_non_spd_and_nan_are_flagged_per_matrix():
+    """The reference GPU path never reads cuSOLVER's dev_info; here every matrix
+    gets its own code: 1 + index of the first non-positive pivot."""
+    from chainerkfac_amd import ops
+    good = spd(40, 1)
+    bad = np.array([[1.0, 2.0], [2.0, 1.0]], dtype=np.float32)          # pivot 1 is -3
+    late = spd(200, 2); late[150, 150] = -5.0                             # fails at column 150
+    nan = spd(33, 3); nan[0, 0] = np.nan
+    outs, info = ops.spd_inverse_batched([torch.from_numpy(a).cuda() for a in (good, bad, late, nan)])
+    info = info.cpu().tolist()
+    assert info[0] == 0 and info[1] == 2 and info[2] == 151 and info[3] == 1
+    check_inverse(good, outs[0].cpu().numpy())
+    with pytest.raises(np.linalg.LinAlgError):
+        O.inverse(bad)
+
+
+def test_repeated_calls_reuse_plan_and_workspace():
+    from chainerkfac_amd import ops
+    mats = [torch.from_numpy(spd(d, d)).cuda() for d in (300, 50)]
+    outs = [torch.empty_like(m) for m in mats]
+    for _ in range(3):
+        ops.spd_inverse_batched(mats, outs=outs)
+    for m, o in zip(mats, outs):
+        check_inverse(m.cpu().numpy(), o.cpu().numpy())
+
+
+def test_pi_damp_matches_oracle():
+    from chainerkfac_amd import ops
+    layers = [(6, 4), (785, 1000), (1001, 10), (28, 64)]
+    As = [spd(a, a) for a, _ in layers]
+    Gs = [(spd(g, 7 * g) * np.float32(0.01)) for _, g in layers]
+    dampings = [1e-3, 1e-3, 2.5e-4, 0.03]
+    refA = [a.copy() for a in As]; refG = [g.copy() for g in Gs]
+    pis = []
+    for a, g, dmp in zip(refA, refG, dampings):
+        (dA, dG), pi = O.connection_diagvals(a, g, dmp)
+        O.damp_inplace(a, dA); O.damp_inplace(g, dG)
+        pis.append(float(pi))
+    dA = [torch.from_numpy(a).cuda() for a in As]; dG = [torch.from_numpy(g).cuda() for g in Gs]
+    pi = ops.pi_damp_batched(dA, dG, [d ** 0.5 for d in dampings])
+    np.testing.assert_allclose(pi.cpu().numpy(), pis, rtol=1e-5)
+    for got, ref in zip(dA + dG, refA + refG):
+        got = got.cpu().numpy()
+        off = ~np.eye(ref.shape[0], dtype=bool)
+        assert np.array_equal(got[off], ref[off])
+        np.testing.assert_allclose(np.diagonal(got), np.diagonal(ref), rtol=2e-6)
+    # pi_type other than tracenorm: pi = 1
+    a = torch.from_numpy(As[0]).cuda(); g = torch.from_numpy(Gs[0]).cuda()
+    pi = ops.pi_damp_batched([a], [g], [0.1], use_pi=False)
+    assert pi.cpu().tolist() == [1.0]
+    np.testing.assert_allclose(np.diagonal(a.cpu().numpy()), np.diagonal(As[0]) + 0.1, rtol=1e-6)
+
+
+def test_add_diag_batch_norm_halves():
+    from chainerkfac_amd import ops
+    F = spd(10, 4)
+    ref = F.copy()
+    (dv,) = O.bn_diagvals(6, 4, damping=2.5e-4, stab_coeff=16.0, l2_beta=0.5)
+    O.damp_inplace(ref, dv)
+    got = ops.add_diag(torch.from_numpy(F).cuda(), dv[0], dv[-1], split=6).cpu().numpy()
+    assert np.array_equal(got, ref)

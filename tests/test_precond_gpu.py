@@ -1,0 +1,116 @@
+"""Parity of preconditioning, batch-norm statistics and the update rule with the oracle (GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kfac_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-3   # preconditioned-gradient tolerance of the north-star spec
+
+
+def sym(d, seed):
+    r = np.random.default_rng(seed)
+    X = r.standard_normal((d, d)).astype(np.float32)
+    return ((X + X.T) / np.float32(2 * np.sqrt(d))).astype(np.float32)
+
+
+def rel(a, b):
+    return np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30)
+
+
+@pytest.mark.parametrize('dG,wshape,bias', [(10, (10, 1000), True), (1000, (1000, 784), True), (64, (64, 3, 3, 3), True),
+                                             (128, (128, 64, 3, 3), True), (256, (256, 128, 1, 1), False),
+                                             (5, (5, 3), True), (1, (1, 1), False), (130, (130, 70), False),
+                                             (512, (512, 64, 3, 3), False)])
+def test_precondition_connection(dG, wshape, bias):
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(dG)
+    dA = int(np.prod(wshape[1:])) + (1 if bias else 0)
+    Ainv = sym(dA, 1); Ginv = sym(dG, 2)
+    gW = r.standard_normal(wshape).astype(np.float32)
+    gb = r.standard_normal(dG).astype(np.float32) if bias else None
+    kW, kb = O.precondition_conn(Ainv, Ginv, gW, gb)
+    hW, hb = ops.precond_conn(torch.from_numpy(Ginv).cuda(), torch.from_numpy(Ainv).cuda(),
+                              torch.from_numpy(gW).cuda(), None if gb is None else torch.from_numpy(gb).cuda())
+    assert tuple(hW.shape) == wshape
+    assert rel(hW.cpu().numpy(), kW) < RTOL
+    ref64 = (Ginv.astype(np.float64) @ np.column_stack([gW.reshape(dG, -1)] + ([gb] if bias else [])).astype(np.float64)
+             @ Ainv.astype(np.float64))
+    got = np.column_stack([hW.cpu().numpy().reshape(dG, -1)] + ([hb.cpu().numpy()] if bias else []))
+    assert rel(got, ref64) < 1e-5
+    if bias:
+        assert hb.shape == (dG,) and rel(hb.cpu().numpy(), kb) < RTOL
+    else:
+        assert hb is None
+
+
+def test_precondition_identity_returns_gradient():
+    from chainerkfac_amd import ops
+    g = torch.randn(7, 12, device='cuda'); b = torch.randn(7, device='cuda')
+    kW, kb = ops.precond_conn(torch.eye(7, device='cuda'), torch.eye(13, device='cuda'), g, b)
+    assert torch.equal(kW, g) and torch.equal(kb, b)
+
+
+@pytest.mark.parametrize('C', [3, 64, 1024])
+def test_precondition_bn_and_nan_fallback(C):
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(C)
+    Finv = sym(2 * C, 5)
+    gg = r.standard_normal(C).astype(np.float32); gb = r.standard_normal(C).astype(np.float32)
+    kg, kb, _ = O.precondition_bn(Finv, gg, gb)
+    hg, hb, flag = ops.precond_bn(torch.from_numpy(Finv).cuda(), torch.from_numpy(gg).cuda(), torch.from_numpy(gb).cuda())
+    assert flag.item() == 0
+    assert rel(hg.cpu().numpy(), kg) < RTOL and rel(hb.cpu().numpy(), kb) < RTOL
+    Fbad = Finv.copy(); Fbad[1, 2] = np.nan
+    hg, hb, flag = ops.precond_bn(torch.from_numpy(Fbad).cuda(), torch.from_numpy(gg).cuda(), torch.from_numpy(gb).cuda())
+    assert flag.item() == 1
+    assert np.array_equal(hg.cpu().numpy(), gg) and np.array_equal(hb.cpu().numpy(), gb)
+    # gamma only
+    kg, _, _ = O.precondition_bn(Finv[:C, :C].copy(), gg, None)
+    hg, hb, _ = ops.precond_bn(torch.from_numpy(Finv[:C, :C].copy()).cuda(), torch.from_numpy(gg).cuda(), None)
+    assert hb is None and rel(hg.cpu().numpy(), kg) < RTOL
+
+
+@pytest.mark.parametrize('shape', [(6, 4, 5, 3), (8, 5), (32, 64, 8, 8), (4, 130, 7, 7), (16, 1000)])
+def test_bn_factor(shape):
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(sum(shape))
+    x = (r.standard_normal(shape) * 2 + 0.7).astype(np.float32)
+    gy = (r.standard_normal(shape) / shape[0]).astype(np.float32)
+    eps = 2e-5
+    n = shape[0]
+    U = ops.bn_grad_matrix(torch.from_numpy(x).cuda(), torch.from_numpy(gy).cuda(), eps, float(n))
+    Uref = O.bn_grad_matrix(x, gy, eps)
+    assert rel(U.cpu().numpy(), Uref) < 1e-4
+    F = ops.cov_linear(U, False, 1.0 / n)
+    Fref = O.bn_F(x, gy, eps)
+    assert rel(F.cpu().numpy(), Fref) < 1e-4
+    assert np.max(np.abs(F.cpu().numpy() - Fref)) <= 1e-4 * np.max(np.abs(Fref))
+    Ug = ops.bn_grad_matrix(torch.from_numpy(x).cuda(), torch.from_numpy(gy).cuda(), eps, float(n), has_beta=False)
+    assert rel(Ug.cpu().numpy(), O.bn_grad_matrix(x, gy, eps, has_beta=False)) < 1e-4
+    Ub = ops.bn_grad_matrix(torch.from_numpy(x).cuda(), torch.from_numpy(gy).cuda(), eps, float(n), has_gamma=False)
+    assert rel(Ub.cpu().numpy(), O.bn_grad_matrix(x, gy, eps, has_gamma=False)) < 1e-4
+
+
+def test_bn_rejects_other_ranks():
+    from chainerkfac_amd import ops
+    x = torch.zeros(2, 3, 4, device='cuda')
+    with pytest.raises(RuntimeError):
+        ops.bn_grad_matrix(x, x, 1e-5, 1.0)
+
+
+def test_axpby_and_momentum_update():
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(0)
+    x = r.standard_normal(100003).astype(np.float32); y = r.standard_normal(100003).astype(np.float32)
+    got = ops.axpby(torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda(), 0.99, 0.01).cpu().numpy()
+    np.testing.assert_allclose(got, np.float32(0.99) * x + np.float32(0.01) * y, rtol=1e-6, atol=1e-7)
+    p = r.standard_normal(1000).astype(np.float32); v = r.standard_normal(1000).astype(np.float32)
+    g = r.standard_normal(1000).astype(np.float32)
+    pd, vd = torch.from_numpy(p).cuda(), torch.from_numpy(v).cuda()
+    ops.momentum_update(pd, vd, torch.from_numpy(g).cuda(), 0.1, 0.9)
+    O.momentum_update(p, v, g, 0.1, 0.9)
+    np.testing.assert_allclose(vd.cpu().numpy(), v, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(pd.cpu().numpy(), p, rtol=1e-6, atol=1e-7)
