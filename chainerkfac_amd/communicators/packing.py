@@ -63,10 +63,12 @@ class _ArraysInfo(object):
         return self._plan
 
     def __del__(self):
-        plan = getattr(self, '_plan', None)
-        if plan is not None and _lib._lib is not None:
-            _lib._lib.kfac_pack_plan_destroy(plan)
-            self._plan = None
+        try:
+            plan, self._plan = self._plan, None
+            if plan is not None:
+                _lib._lib.kfac_pack_plan_destroy(plan)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
 
     def show(self):
         print('# ainfo: n_arrays: {}'.format(self.n_arrays))

@@ -144,10 +144,12 @@ class InversePlan(object):
         self.workspace_bytes = lib.kfac_inverse_plan_workspace_bytes(plan)
 
     def __del__(self):
-        plan = getattr(self, '_plan', None)
-        if plan is not None and _lib._lib is not None:
-            _lib._lib.kfac_inverse_plan_destroy(plan)
-            self._plan = None
+        try:
+            plan, self._plan = self._plan, None
+            if plan is not None:
+                _lib._lib.kfac_inverse_plan_destroy(plan)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
 
     def run(self, mats, outs=None, info=None, stream=None):
         if len(mats) != len(self.dims):
@@ -204,10 +206,12 @@ class DampPlan(object):
         self._plan = plan
 
     def __del__(self):
-        plan = getattr(self, '_plan', None)
-        if plan is not None and _lib._lib is not None:
-            _lib._lib.kfac_damp_plan_destroy(plan)
-            self._plan = None
+        try:
+            plan, self._plan = self._plan, None
+            if plan is not None:
+                _lib._lib.kfac_damp_plan_destroy(plan)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
 
     def run(self, As, Gs, rW, use_pi=True, pi_out=None, stream=None):
         for t in list(As) + list(Gs):

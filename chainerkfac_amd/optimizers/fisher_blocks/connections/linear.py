@@ -1,0 +1,27 @@
+"""Fisher block of a Linear layer: A = [x, 1]^T [x, 1] / n, G = n * gy^T gy.
+Counterpart of chainerkfac/optimizers/fisher_blocks/connections/linear.py."""
+from chainerkfac_amd import links
+from chainerkfac_amd import ops
+from chainerkfac_amd.optimizers.fisher_blocks.connection import FisherBlockConnection
+
+
+class FisherBlockLinear(FisherBlockConnection):
+
+    @property
+    def funcclass(self):
+        return links.LinearFunction
+
+    def compute_A(self, in_data):
+        x = in_data[0]
+        n, d_in = x.shape
+        has_b = self.link.b is not None
+        d = d_in + (1 if has_b else 0)
+        out, alpha, beta = self._cov_target('A', (d, d), x.device, 1.0 / n)
+        return ops.cov_linear(x, has_b, alpha, beta, out)
+
+    def compute_G(self, in_data, out_grad_data):
+        gy = out_grad_data[0]
+        n, d_out = gy.shape
+        scale = self.gy_scale(n) ** 2 / n
+        out, alpha, beta = self._cov_target('G', (d_out, d_out), gy.device, scale)
+        return ops.cov_linear(gy, False, alpha, beta, out)

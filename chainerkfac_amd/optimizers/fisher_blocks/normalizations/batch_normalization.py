@@ -1,0 +1,131 @@
+"""Fisher block of a BatchNormalization layer: one full (2C x 2C) factor built
+from the per-sample gradients of (gamma, beta).  Counterpart of
+chainerkfac/optimizers/fisher_blocks/normalizations/batch_normalization.py."""
+import warnings
+
+from chainerkfac_amd import links
+from chainerkfac_amd import ops
+from chainerkfac_amd.optimizers.fisher_block import FisherBlock
+
+
+def _same_array(a, b):
+    return a is not None and b is not None and a is b
+
+
+class FisherBlockBatchNormalization(FisherBlock):
+
+    def __init__(self, *args, **kwargs):
+        self._F = None
+        self.nan_flag = None
+        super(FisherBlockBatchNormalization, self).__init__(*args, **kwargs)
+
+    @property
+    def funcclass(self):
+        return links.BatchNormalizationFunction
+
+    @property
+    def cov_forward(self):
+        return None
+
+    @property
+    def cov_backward(self):
+        return self.covs[0]
+
+    @property
+    def inv_forward(self):
+        return None
+
+    @property
+    def inv_backward(self):
+        return self.invs[0]
+
+    def is_mine(self, func, in_data, out_grad_data=None):
+        if not isinstance(func, self.funcclass):
+            return False
+        gamma, beta = self.link.gamma, self.link.beta
+        if not _same_array(in_data[1], None if gamma is None else gamma.data) and \
+                not _same_array(in_data[2], None if beta is None else beta.data):
+            return False
+        return True
+
+    def forward_postprocess(self, func, in_data):
+        pass   # F needs the output gradient
+
+    def backward_preprocess(self, func, in_data, out_grad_data):
+        self._F = self.compute_F(in_data, out_grad_data)
+        self.covs = [self._F]
+
+    def compute_F(self, in_data, out_grad_data):
+        x = in_data[0]
+        gy = out_grad_data[0]
+        if x.ndim not in (2, 4):
+            raise RuntimeError('len(x.shape) must be 2 or 4, not {}.'.format(x.ndim))
+        n = x.shape[0]
+        gy_scale = float(n)
+        if self._loss_scale is not None:
+            gy_scale *= 1.0 / self._loss_scale
+        has_gamma = self.link.gamma is not None
+        has_beta = self.link.beta is not None
+        width = x.shape[1] * (int(has_gamma) + int(has_beta))
+        U = ops.bn_grad_matrix(x, gy, self.link.eps, gy_scale, has_gamma, has_beta,
+                               out=self._buffer('U', (n, width), x.device))
+        out, alpha, beta = self._cov_target('F', (width, width), x.device, 1.0 / n)
+        return ops.cov_linear(U, False, alpha, beta, out)
+
+    def _diag_pair(self):
+        gamma, beta = self.link.gamma, self.link.beta
+        if gamma is None and beta is None:
+            raise RuntimeError('gamma and beta must not be None as the same time')
+        d_gamma = self.get_diagval('gamma')
+        d_beta = self.get_diagval('beta')
+        if d_gamma is not None:
+            d_gamma *= self.stab_coeff
+        if d_beta is not None:
+            d_beta *= self.stab_coeff
+        return d_gamma, d_beta
+
+    def get_diagvals(self):
+        import numpy as np
+        d_gamma, d_beta = self._diag_pair()
+        setattr(self, 'diag_val_backward', d_gamma)
+        gamma, beta = self.link.gamma, self.link.beta
+        if d_beta is None:
+            return [d_gamma * np.ones(gamma.size)]
+        if d_gamma is None:
+            return [d_beta * np.ones(beta.size)]
+        return [np.hstack((d_gamma * np.ones(gamma.size), d_beta * np.ones(beta.size)))]
+
+    def damp(self):
+        d_gamma, d_beta = self._diag_pair()
+        F = self.cov_emas[0]
+        if d_beta is None:
+            ops.add_diag(F, d_gamma)
+        elif d_gamma is None:
+            ops.add_diag(F, d_beta)
+        else:
+            ops.add_diag(F, d_gamma, d_beta, split=self.link.gamma.size)
+
+    def update_kfgrads(self):
+        self.check_attr('invs')
+        gamma, beta = self.link.gamma, self.link.beta
+        g = None if gamma is None else gamma.grad
+        b = None if beta is None else beta.grad
+        kg = None if gamma is None else self._buffer('kf_gamma', gamma.shape, gamma.data.device)
+        kb = None if beta is None else self._buffer('kf_beta', beta.shape, beta.data.device)
+        if self.nan_flag is None:
+            import torch
+            self.nan_flag = torch.zeros(1, dtype=torch.int32, device=self.invs[0].device)
+        # NaN anywhere in F^-1 grad makes the kernel hand back the raw gradients
+        ops.precond_bn(self.invs[0], g, b, kg, kb, self.nan_flag)
+        if gamma is not None:
+            gamma.kfgrad = kg
+        if beta is not None:
+            beta.kfgrad = kb
+        if self.debug() and int(self.nan_flag.item()):
+            warnings.warn('Detected NaN in the kfgrads of the batch normalization layer; '
+                          '``grad`` was substituted for ``kfgrad``')
+
+    def extract_for_reduce_scatter_v(self):
+        arrays = self.extract_attr_from_params('grad')
+        arrays.append((self.cov_backward, True))
+        return arrays

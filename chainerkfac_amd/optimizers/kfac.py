@@ -1,0 +1,346 @@
+"""K-FAC optimizer on the HIP path: the single-GPU ``KFAC`` of the reference
+(chainerkfac/optimizers/kfac.py) with the same constructor, hyper-parameters,
+phase order and attribute names.  ``DistributedKFAC`` and the communicator's
+collectives are not part of this package (one GPU, no inter-GPU traffic).
+
+One step = forward and backward under the function hook (A at forward, G / F at
+backward, computed by the SYRK kernels), then for every Fisher block: moving
+average -> damping -> inverse -> preconditioning, then the momentum update.
+The per-block loop of the reference (``update_kfgrads``) is kept, but damping
+and inversion of all blocks are issued as one batch: the blocks are independent,
+so the results are those of the sequential loop.
+"""
+from chainerkfac_amd import links
+from chainerkfac_amd import ops
+from chainerkfac_amd.optimizers import fisher_blocks as FB
+from chainerkfac_amd.optimizers.fisher_block import PI_TYPE_TRACENORM
+
+
+class Hyperparameter(object):
+    """Attribute bag shared between the optimizer and its update rules."""
+
+    def __init__(self, parent=None):
+        object.__setattr__(self, '_parent', parent)
+
+    def __getattr__(self, name):
+        parent = object.__getattribute__(self, '_parent')
+        if parent is not None:
+            return getattr(parent, name)
+        raise AttributeError(name)
+
+    def get_dict(self):
+        d = {} if self._parent is None else self._parent.get_dict()
+        d.update({k: v for k, v in self.__dict__.items() if k != '_parent'})
+        return d
+
+
+_default_hyperparam = Hyperparameter()
+_default_hyperparam.lr = 0.001
+_default_hyperparam.lr_pre = 0.001
+_default_hyperparam.momentum = 0.9
+_default_hyperparam.cov_ema_decay = 0.99
+_default_hyperparam.damping = 0.03
+
+
+def _proxy(name):
+    return property(lambda self: getattr(self.hyperparam, name),
+                    lambda self, v: setattr(self.hyperparam, name, v))
+
+
+def fblock_constructor(sub_linkname, sub_link, **kwargs):
+    """Fisher block for a link, or None for links K-FAC leaves alone
+    (reference kfac.py:19-30)."""
+    args = (sub_linkname, sub_link)
+    if isinstance(sub_link, links.Linear):
+        return FB.FisherBlockLinear(*args, **kwargs)
+    elif isinstance(sub_link, links.Convolution2D):
+        return FB.FisherBlockConvolution2D(*args, **kwargs)
+    elif isinstance(sub_link, links.BatchNormalization):
+        if sub_link.gamma is None and sub_link.beta is None:
+            return None
+        return FB.FisherBlockBatchNormalization(*args, **kwargs)
+    return None
+
+
+class KFACHook(links.FunctionHook):
+    """Routes each link-function call to the Fisher block that owns it.  The
+    owner is found through the identity of the weight array (a dictionary
+    lookup instead of the reference's scan over all blocks, kfac.py:38-48)."""
+
+    def __init__(self, fblocks):
+        self.fblocks = fblocks
+        self._owner = {}
+        for fb in fblocks:
+            for p in fb.link.params():
+                self._owner[id(p.data)] = fb
+
+    def _find(self, func, in_data, out_grad_data=None):
+        for a in in_data[1:]:
+            fb = self._owner.get(id(a)) if a is not None else None
+            if fb is not None and fb.is_mine(func, in_data, out_grad_data):
+                return fb
+        return None
+
+    def forward_postprocess(self, func, in_data):
+        fb = self._find(func, in_data)
+        if fb is not None:
+            fb.forward_postprocess(func, in_data)
+
+    def backward_preprocess(self, func, in_data, out_grad_data):
+        fb = self._find(func, in_data, out_grad_data)
+        if fb is not None:
+            fb.backward_preprocess(func, in_data, out_grad_data)
+
+
+class KFACUpdateRule(object):
+    """v = momentum * v - lr * kfgrad; param += v (reference kfac.py:51-116)."""
+
+    def __init__(self, parent_hyperparam=None, adjust_momentum=False):
+        self.hyperparam = Hyperparameter(parent_hyperparam or _default_hyperparam)
+        self.adjust_momentum = adjust_momentum
+        self.state = None
+        self.t = 0
+        self.enabled = True
+
+    def init_state(self, param):
+        import torch
+        self.state = {'v': torch.zeros_like(param.data)}
+
+    def update(self, param):
+        if not self.enabled:
+            return
+        self.t += 1
+        if self.state is None:
+            self.init_state(param)
+        if param._loss_scale is not None and getattr(param, 'kfgrad', None) is not None:
+            param.kfgrad /= param._loss_scale
+        self.update_core(param)
+
+    def update_core(self, param):
+        grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
+        if grad is None:
+            return
+        lr = self.hyperparam.lr
+        lr_pre = self.hyperparam.lr_pre
+        momentum = self.hyperparam.momentum
+        if self.adjust_momentum and lr < lr_pre:
+            momentum *= lr / lr_pre
+        ops.momentum_update(param.data, self.state['v'], grad.contiguous(), lr, momentum)
+
+    update_core_gpu = update_core
+
+
+class KFAC(object):
+
+    def __init__(self, lr=_default_hyperparam.lr, momentum=_default_hyperparam.momentum,
+                 cov_ema_decay=_default_hyperparam.cov_ema_decay,
+                 damping=_default_hyperparam.damping, stab_coeff=16.0,
+                 constructor=fblock_constructor, pi_type=PI_TYPE_TRACENORM, use_cholesky=True,
+                 loss_scale=None, adjust_momentum=False, acc_iters=1):
+        self.hyperparam = Hyperparameter()
+        self.hyperparam.lr = lr
+        self.hyperparam.lr_pre = lr
+        self.hyperparam.momentum = momentum
+        self.hyperparam.cov_ema_decay = cov_ema_decay
+        self.hyperparam.damping = damping
+        self.pi_type = pi_type
+        self.constructor = constructor
+        self.adjust_momentum = adjust_momentum
+        self.stab_coeff = stab_coeff
+        self.fblocks = []
+        self.kfhook = None
+        self._loss_scale = loss_scale
+        self.constructor_kwargs = {
+            'cov_ema_decay': self.hyperparam.cov_ema_decay,
+            'damping': self.hyperparam.damping,
+            'use_cholesky': use_cholesky,
+            'pi_type': self.pi_type,
+            'stab_coeff': self.stab_coeff,
+            'loss_scale': self._loss_scale,
+        }
+        assert acc_iters >= 1, 'Accumulation iterations should be 1 or larger'
+        self.acc_iters = acc_iters
+        self.acc_count = 0
+        self.acc_aware_iterations = 0
+        self.only_pic_update_weight = False
+        self.target = None
+        self.t = 0
+        self.observation = {}
+        self._hooks = {'pre': [], 'post': []}
+
+    lr = _proxy('lr')
+    lr_pre = _proxy('lr_pre')
+    momentum = _proxy('momentum')
+    cov_ema_decay = _proxy('cov_ema_decay')
+    damping = _proxy('damping')
+
+    # ---- set-up ---------------------------------------------------------
+    def setup(self, link):
+        self.target = link
+        self.t = 0
+        for param in link.params():
+            param.update_rule = self.create_update_rule()
+        self.fblocks = []
+        for sub_linkname, sub_link in sorted(link.namedlinks(), key=lambda kv: kv[0]):
+            fblock = self.constructor(sub_linkname, sub_link, **self.constructor_kwargs)
+            if fblock is None:
+                continue
+            self.fblocks.append(fblock)
+        self.kfhook = KFACHook(self.fblocks)
+        return self
+
+    def create_update_rule(self):
+        return KFACUpdateRule(self.hyperparam, adjust_momentum=self.adjust_momentum)
+
+    def add_hook(self, hook, name=None, timing='pre'):
+        self._hooks[timing].append(hook)
+
+    def call_hooks(self, timing='pre'):
+        for hook in self._hooks[timing]:
+            hook(self)
+
+    def reallocate_cleared_grads(self):
+        import torch
+        for _, param in self.target.namedparams(False):
+            if hasattr(param, 'kfgrad') and param.kfgrad is None:
+                param.kfgrad = torch.zeros_like(param.data)
+            if param.grad is None:
+                param.grad = torch.zeros_like(param.data)
+
+    # ---- one step -------------------------------------------------------
+    def update(self, lossfun=None, *args, **kwargs):
+        if lossfun is not None:
+            for fblock in self.fblocks:
+                fblock.acc_state = (self.acc_iters, self.acc_count)
+            with self.kfhook:
+                use_cleargrads = getattr(self, '_use_cleargrads', True)
+                loss = lossfun(*args, **kwargs)
+                if use_cleargrads:
+                    self.target.cleargrads()
+                else:
+                    self.target.zerograds()
+                if self._loss_scale is not None:
+                    (loss * self._loss_scale).backward()
+                else:
+                    loss.backward()
+            del loss
+
+        if self.acc_iters > 1:
+            if self.accumulate():
+                return
+
+        self.reallocate_cleared_grads()
+        self.call_hooks('pre')
+        self.t += 1
+        self.update_kfgrads(self.fblocks)
+
+        if not self.only_pic_update_weight:
+            for param in self.target.params():
+                param.update()
+
+        self.reallocate_cleared_grads()
+        self.call_hooks('post')
+        self.acc_aware_iterations += 1
+        self.observation['acc_aware_iterations'] = self.acc_aware_iterations
+
+    # ---- accumulation over acc_iters micro-batches -----------------------
+    def accumulate(self):
+        if self.acc_count == 0:
+            for param in self.target.params():
+                param.acc_grad = None
+            for fblock in self.fblocks:
+                fblock.acc_covs = None
+        self.accumulate_grads()
+        self.accumulate_covs()
+        self.acc_count += 1
+        if self.acc_count == self.acc_iters:
+            self.acc_count = 0
+            for param in self.target.params():
+                param.grad = param.acc_grad
+            for fblock in self.fblocks:
+                fblock.covs = fblock.acc_covs
+            return False
+        elif self.acc_count < self.acc_iters:
+            return True
+        raise ValueError('acc_count {} should not be larger than acc_iters {}'.format(
+            self.acc_count, self.acc_iters))
+
+    def accumulate_grads(self):
+        """acc_grad += grad / acc_iters for every parameter."""
+        for param in self.target.params():
+            if param.grad is None:
+                continue
+            if getattr(param, 'acc_grad', None) is None:
+                buf = getattr(param, '_acc_grad_buf', None)
+                if buf is None or buf.shape != param.grad.shape:
+                    buf = param._acc_grad_buf = param.grad.new_empty(param.grad.shape)
+                param.acc_grad = buf
+                ops.axpby(param.grad.contiguous(), buf, 1 / self.acc_iters, 0.0)
+            else:
+                ops.axpby(param.grad.contiguous(), param.acc_grad, 1 / self.acc_iters, 1.0)
+
+    def accumulate_covs(self):
+        """The covariance kernels already added this micro-batch's factors, scaled
+        by 1/acc_iters, onto the blocks' running buffers; publish them."""
+        for fblock in self.fblocks:
+            fblock.check_attr('covs')
+            fblock.acc_covs = list(fblock.covs)
+
+    # ---- moving average -> damping -> inverse -> preconditioning ----------
+    def update_kfgrads(self, fblocks):
+        for fblock in fblocks:
+            fblock.update_cov_emas()
+        self.update_invs_batched(fblocks)
+        for fblock in fblocks:
+            fblock.update_kfgrads()
+
+    def update_invs_batched(self, fblocks):
+        """``fblock.update_invs()`` for every block, with all damping kernels and
+        all inversions issued together."""
+        conn = [fb for fb in fblocks if isinstance(fb, FB.FisherBlockConnection)]
+        other = [fb for fb in fblocks if not isinstance(fb, FB.FisherBlockConnection)]
+        for fb in fblocks:
+            fb.check_attr('cov_emas')
+        if conn:
+            use_pi = {fb._pi_type == PI_TYPE_TRACENORM for fb in conn}
+            if len(use_pi) == 1:
+                pis = ops.pi_damp_batched([fb.cov_emas[0] for fb in conn],
+                                          [fb.cov_emas[1] for fb in conn],
+                                          [fb._rW() for fb in conn], use_pi=use_pi.pop(),
+                                          pi_out=self._pi_buffer(len(conn), conn[0].cov_emas[0].device))
+                for i, fb in enumerate(conn):
+                    fb.pi = pis[i:i + 1]
+            else:
+                for fb in conn:
+                    fb.damp()
+        for fb in other:
+            fb.damp()
+        mats, outs, owners = [], [], []
+        for fb in fblocks:
+            bufs = fb._inv_buffers()
+            mats.extend(fb.cov_emas)
+            outs.extend(bufs)
+            owners.append((fb, len(bufs)))
+        if not mats:
+            return
+        outs, info = ops.spd_inverse_batched(mats, outs=outs, info=self._info_buffer(len(mats), mats[0].device))
+        self.inv_info = info
+        pos = 0
+        for fb, n in owners:
+            fb.invs = outs[pos:pos + n]
+            fb.inv_info = info[pos:pos + n]
+            pos += n
+
+    def _pi_buffer(self, n, device):
+        import torch
+        buf = getattr(self, '_pi_buf', None)
+        if buf is None or buf.numel() != n or buf.device != device:
+            buf = self._pi_buf = torch.empty(n, dtype=torch.float32, device=device)
+        return buf
+
+    def _info_buffer(self, n, device):
+        import torch
+        buf = getattr(self, '_info_buf', None)
+        if buf is None or buf.numel() != n or buf.device != device:
+            buf = self._info_buf = torch.empty(n, dtype=torch.int32, device=device)
+        return buf
