@@ -1,0 +1,303 @@
+#!/usr/bin/env python
+"""Benchmark of the K-FAC per-layer hot path on one MI355X.
+
+Workload (BASELINE.json configs[2]): ResNet-50 (bottleneck v1, 1000-way FC, all
+convs with bias) K-FAC step on one GPU's share, batch 32 at 224x224, fp32:
+for all 161 Kronecker factors, covariance (fused im2col SYRK) + pi-damped
+Cholesky inverse + gradient preconditioning.  Per-layer activations, output
+gradients and parameter gradients are synthetic N(0,1) tensors of the real
+shapes (output gradients scaled by 1/(batch*sqrt(pixels)), the size a
+mean-reduced loss gives them, which keeps the rank-32 batch-norm factors
+positive definite in float32), resident in HBM before the timed region.  The step is driven through
+the drop-in host classes (FisherBlock*.forward_postprocess /
+backward_preprocess, KFAC.update_kfgrads).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu]
+
+prints ONE JSON line: ms per K-FAC step, per-phase TFLOP/s, the roofline of the
+dominant kernel family (covariance SYRK, timed live with HIP events inside the
+library) and the CPU baseline (the NumPy oracle on a bounded sample of layers).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix peak
+BATCH = 32
+DAMPING = 2.5e-4
+STAB_COEFF = 16.0
+
+
+def build_model(layers, device, gen):
+    """Links with the layer table's shapes plus synthetic per-layer tensors."""
+    import torch
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd import workloads as W
+    model = L.Chain()
+    calls = []
+    for i, layer in enumerate(layers):
+        name = 'l{:03d}_{}'.format(i, layer['name'].replace('/', '_'))
+        if layer['kind'] == 'conv':
+            link = L.Convolution2D(layer['c_in'], layer['c_out'], layer['k'], layer['s'], layer['p'],
+                                   nobias=not layer['bias'], device=device, generator=gen)
+            ho = W.conv_out(layer['h'], layer['k'], layer['s'], layer['p'])
+            x = torch.randn(BATCH, layer['c_in'], layer['h'], layer['w'], device=device, generator=gen)
+            gy = torch.randn(BATCH, layer['c_out'], ho, ho, device=device, generator=gen) / (BATCH * ho)
+            func = L.Convolution2DFunction()
+            in_data = (x, link.W.data) + ((link.b.data,) if layer['bias'] else ())
+        elif layer['kind'] == 'linear':
+            link = L.Linear(layer['d_in'], layer['d_out'], nobias=not layer['bias'], device=device, generator=gen)
+            x = torch.randn(BATCH, layer['d_in'], device=device, generator=gen)
+            gy = torch.randn(BATCH, layer['d_out'], device=device, generator=gen) / BATCH
+            func = L.LinearFunction()
+            in_data = (x, link.W.data) + ((link.b.data,) if layer['bias'] else ())
+        else:
+            link = L.BatchNormalization(layer['c'], device=device)
+            x = torch.randn(BATCH, layer['c'], layer['h'], layer['w'], device=device, generator=gen)
+            gy = torch.randn(BATCH, layer['c'], layer['h'], layer['w'], device=device, generator=gen) / (BATCH * layer['h'])
+            func = L.BatchNormalizationFunction()
+            in_data = (x, link.gamma.data, link.beta.data)
+        setattr(model, name, link)
+        for p in link.params():
+            p.grad = torch.randn(p.shape, device=device, generator=gen)
+        calls.append((name, func, in_data, gy))
+    return model, calls
+
+
+def run_gpu(args):
+    import torch
+    from chainerkfac_amd import _lib
+    from chainerkfac_amd import workloads as W
+    from chainerkfac_amd.optimizers import KFAC
+
+    lib = _lib.load()
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(3)
+    layers = W.resnet50_v1()
+    flops = W.flops(layers, BATCH)
+    model, calls = build_model(layers, dev, gen)
+    opt = KFAC(damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0).setup(model)
+    by_name = {fb.linkname: fb for fb in opt.fblocks}
+    work = [(by_name['/' + name], func, in_data, (gy,)) for name, func, in_data, gy in calls]
+    assert len(opt.fblocks) == len(layers)
+
+    def cov_phase():
+        for fb, func, in_data, gy in work:
+            fb.forward_postprocess(func, in_data)
+            fb.backward_preprocess(func, in_data, gy)
+
+    def inv_phase():
+        for fb in opt.fblocks:
+            fb.update_cov_emas()
+        opt.update_invs_batched(opt.fblocks)
+
+    def pre_phase():
+        for fb in opt.fblocks:
+            fb.update_kfgrads()
+
+    def step():
+        cov_phase()
+        inv_phase()
+        pre_phase()
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+
+    graph = None
+    if not args.no_graph:
+        # the step is a fixed sequence of launches on fixed buffers: replay it
+        # from one HIP graph so the host only pays for a single launch
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+
+    run = graph.replay if graph is not None else step
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-phase split (eager, events on the launch stream)
+    def timed(fn, reps=3):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    phase_ms = {'cov': timed(cov_phase), 'inverse': timed(inv_phase), 'precondition': timed(pre_phase)}
+
+    # dominant kernel family, timed launch by launch inside the library
+    _lib.check(lib.kfac_timing_enable(1))
+    step()
+    torch.cuda.synchronize()
+    fam = {}
+    for name, fid in (('syrk', 0), ('inv_update', 1), ('inv_lauum', 2), ('gemm', 3)):
+        n = ctypes.c_int64()
+        ms = ctypes.c_double()
+        _lib.check(lib.kfac_timing_read(fid, ctypes.byref(n), ctypes.byref(ms)))
+        fam[name] = (n.value, ms.value)
+    _lib.check(lib.kfac_timing_enable(0))
+    info_bad = int((opt.inv_info != 0).sum().item())
+
+    syrk_n, syrk_ms = fam['syrk']
+    achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_ms > 0 else 0.0
+    total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
+    result = {
+        'metric': 'ms per K-FAC step, ResNet-50 bs32/GPU; cov+inv TFLOP/s vs FP32 MFMA peak',
+        'value': round(ms_per_step, 4),
+        'unit': 'ms/step',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': False,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'f32',
+        'data': 'synthetic',
+        'config': {'workload': 'ResNet-50 v1 (bias, 1000-way) K-FAC step, batch 32 @224: 161 factors, '
+                               'cov + damped Cholesky inverse + precondition',
+                   'batch': BATCH, 'factors': len(W.all_factor_dims(layers)), 'damping': DAMPING,
+                   'hip_graph': graph is not None},
+        'tflops': {
+            'step': round(total_flops / ms_per_step / 1e9, 2),
+            'cov_inv': round((flops['cov'] + flops['inverse']) / ((phase_ms['cov'] + phase_ms['inverse'])) / 1e9, 2),
+            'cov': round(flops['cov'] / phase_ms['cov'] / 1e9, 2),
+            'inverse': round(flops['inverse'] / phase_ms['inverse'] / 1e9, 2),
+            'precondition': round(flops['precondition'] / phase_ms['precondition'] / 1e9, 2),
+            'frac_of_fp32_mfma_peak': round(total_flops / ms_per_step / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
+        },
+        'phase_ms': {k: round(v, 3) for k, v in phase_ms.items()},
+        'gflop': {k: round(v / 1e9, 1) for k, v in flops.items()},
+        'kernel_ms': {k: {'launches': n, 'total_ms': round(ms, 3)} for k, (n, ms) in fam.items()},
+        'inverse_info_nonzero': info_bad,
+        'roofline': {
+            'kernel': 'syrk_kernel (covariance, all loaders)',
+            'bound': 'mfma',
+            'achieved': round(achieved, 2),
+            'peak': FP32_MFMA_PEAK_TFLOPS,
+            'unit': 'TFLOP/s',
+            'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+            'launches': syrk_n,
+            'avg_launch_ms': round(syrk_ms / max(syrk_n, 1), 4),
+            'traffic': None,
+        },
+    }
+    return result, layers
+
+
+def run_cpu_baseline(layers, budget_s=20.0):
+    """The NumPy oracle (the restatement of the reference's --no_cuda arithmetic)
+    on a bounded sample of the workload's layers, scaled to the whole step by
+    algorithmic FLOPs."""
+    import numpy as np
+    from chainerkfac_amd import workloads as W
+    from oracle import kfac_oracle as O
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get('num_threads', 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count()
+    rng = np.random.default_rng(3)
+    total = W.flops(layers, BATCH)
+    total_f = sum(total.values())
+    # one bottleneck of stage 4 and one of stage 3 plus the FC: every kernel kind
+    wanted = ('res4/1/', 'res3/1/', 'fc')
+    sample = [l for l in layers if l['name'].startswith(wanted) or l['name'] == 'fc']
+    done_f = 0
+    names = []
+    t_used = 0.0
+    for layer in sample:
+        f = sum(W.flops([layer], BATCH).values())
+        t0 = time.perf_counter()
+        if layer['kind'] == 'conv':
+            ho = W.conv_out(layer['h'], layer['k'], layer['s'], layer['p'])
+            x = rng.standard_normal((BATCH, layer['c_in'], layer['h'], layer['w']), dtype=np.float32)
+            gy = rng.standard_normal((BATCH, layer['c_out'], ho, ho), dtype=np.float32) / (BATCH * ho)
+            gW = rng.standard_normal((layer['c_out'], layer['c_in'], layer['k'], layer['k']), dtype=np.float32)
+            gb = rng.standard_normal(layer['c_out'], dtype=np.float32) if layer['bias'] else None
+            t0 = time.perf_counter()
+            A = O.conv_A(x, layer['k'], layer['s'], layer['p'], layer['bias'])
+            G = O.conv_G(gy)
+        elif layer['kind'] == 'linear':
+            x = rng.standard_normal((BATCH, layer['d_in']), dtype=np.float32)
+            gy = rng.standard_normal((BATCH, layer['d_out']), dtype=np.float32) / BATCH
+            gW = rng.standard_normal((layer['d_out'], layer['d_in']), dtype=np.float32)
+            gb = rng.standard_normal(layer['d_out'], dtype=np.float32)
+            t0 = time.perf_counter()
+            A = O.linear_A(x, True)
+            G = O.linear_G(gy)
+        else:
+            x = rng.standard_normal((BATCH, layer['c'], layer['h'], layer['w']), dtype=np.float32)
+            gy = rng.standard_normal((BATCH, layer['c'], layer['h'], layer['w']), dtype=np.float32) / (BATCH * layer['h'])
+            gg = rng.standard_normal(layer['c'], dtype=np.float32)
+            gb = rng.standard_normal(layer['c'], dtype=np.float32)
+            t0 = time.perf_counter()
+            F = O.bn_F(x, gy, 2e-5)
+        if layer['kind'] == 'bn':
+            (dv,) = O.bn_diagvals(layer['c'], layer['c'], DAMPING, STAB_COEFF)
+            (Finv,) = O.update_invs([F], [dv])
+            O.precondition_bn(Finv, gg, gb)
+        else:
+            dv, _ = O.connection_diagvals(A, G, DAMPING)
+            Ainv, Ginv = O.update_invs([A, G], dv)
+            O.precondition_conn(Ainv, Ginv, gW, gb)
+        t_used += time.perf_counter() - t0
+        done_f += f
+        names.append(layer['name'])
+        if t_used > budget_s:
+            break
+    est_ms = t_used * 1e3 * total_f / done_f
+    return {
+        'value': round(est_ms, 1),
+        'unit': 'ms/step',
+        'cores': int(threads),
+        'kind': 'port',
+        'sample': 'NumPy oracle (cov + damped inverse + precondition) on layers {} = {:.1f} of {:.1f} GFLOP '
+                  'in {:.1f} s, scaled by FLOPs'.format(','.join(names), done_f / 1e9, total_f / 1e9, t_used),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--no-graph', action='store_true', help='launch every kernel from the host each step')
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py measures the single-GPU K-FAC hot path: inter-GPU collectives are outside this '
+                 'build, so --gpus must be 1 (got {})'.format(args.gpus))
+    result, layers = run_gpu(args)
+    if not args.no_cpu:
+        result['cpu_baseline'] = run_cpu_baseline(layers)
+    print(json.dumps(result))
+
+
+if __name__ == '__main__':
+    main()

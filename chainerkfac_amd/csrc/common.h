@@ -77,6 +77,22 @@ class DevTable {
 
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
+// Brackets one kernel launch with HIP events while benchmark timing is on.
+bool timing_on();
+void timing_begin(int family, hipStream_t stream);
+void timing_end(hipStream_t stream);
+
+struct TimedLaunch {
+  hipStream_t stream;
+  bool on;
+  TimedLaunch(int family, hipStream_t s) : stream(s), on(timing_on()) {
+    if (on) timing_begin(family, s);
+  }
+  ~TimedLaunch() {
+    if (on) timing_end(stream);
+  }
+};
+
 template <typename T>
 inline T ceil_div(T a, T b) {
   return (a + b - 1) / b;

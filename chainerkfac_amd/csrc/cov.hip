@@ -179,12 +179,15 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, 
                       ws_bytes, need);
   float *partial = static_cast<float *>(ws);
   const int grid = p.ntile * p.nsplit;
-  if (p.bm == 64)
-    hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
-                       p.klen, p.ntile, partial);
-  else
-    hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
-                       p.klen, p.ntile, partial);
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
+    if (p.bm == 64)
+      hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
+                         p.klen, p.ntile, partial);
+    else
+      hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
+                         p.klen, p.ntile, partial);
+  }
   KFAC_HIP_CHECK(hipGetLastError());
   const float *fin = partial;
   int nfin = p.nsplit;

@@ -9,6 +9,72 @@ char *error_buffer() {
 }
 }  // namespace kfac
 
+namespace kfac {
+namespace {
+struct TimedRec {
+  int family;
+  hipEvent_t start, stop;
+};
+bool g_timing = false;
+std::vector<TimedRec> g_open;
+long long g_launches[KFAC_TIMED_FAMILIES];
+double g_total_ms[KFAC_TIMED_FAMILIES];
+}  // namespace
+
+bool timing_on() { return g_timing; }
+
+void timing_begin(int family, hipStream_t stream) {
+  TimedRec r;
+  r.family = family;
+  if (hipEventCreate(&r.start) != hipSuccess) return;
+  if (hipEventCreate(&r.stop) != hipSuccess) {
+    (void)hipEventDestroy(r.start);
+    return;
+  }
+  (void)hipEventRecord(r.start, stream);
+  g_open.push_back(r);
+}
+
+void timing_end(hipStream_t stream) {
+  if (!g_open.empty()) (void)hipEventRecord(g_open.back().stop, stream);
+}
+
+static void timing_collect() {
+  for (auto &r : g_open) {
+    float ms = 0.f;
+    if (hipEventSynchronize(r.stop) == hipSuccess &&
+        hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+      g_launches[r.family] += 1;
+      g_total_ms[r.family] += ms;
+    }
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_open.clear();
+}
+}  // namespace kfac
+
+extern "C" int kfac_timing_enable(int on) {
+  kfac::timing_collect();
+  if (on) {
+    for (int i = 0; i < KFAC_TIMED_FAMILIES; ++i) {
+      kfac::g_launches[i] = 0;
+      kfac::g_total_ms[i] = 0.0;
+    }
+  }
+  kfac::g_timing = on != 0;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_timing_read(int family, int64_t *launches, double *total_ms) {
+  KFAC_REQUIRE(family >= 0 && family < KFAC_TIMED_FAMILIES, "bad kernel family %d", family);
+  KFAC_REQUIRE(launches && total_ms, "null pointer");
+  kfac::timing_collect();
+  *launches = kfac::g_launches[family];
+  *total_ms = kfac::g_total_ms[family];
+  return KFAC_OK;
+}
+
 extern "C" int kfac_abi_version(void) { return KFAC_ABI_VERSION; }
 extern "C" const char *kfac_last_error_string(void) { return kfac::error_buffer(); }
 

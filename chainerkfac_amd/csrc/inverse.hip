@@ -549,12 +549,17 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(256), kDiagLds, s, tb, k);
     if (plan->panel_total[k] > 0)
       hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), 0, s, tb, k, na);
-    if (plan->update_total[k] > 0)
+    if (plan->update_total[k] > 0) {
+      kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, s);
       hipLaunchKernelGGL(update_kernel, dim3(plan->update_total[k]), dim3(THREADS), 0, s, tb, k,
                          na, plan->update_off[k]);
+    }
   }
   KFAC_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL(lauum_kernel, dim3(plan->total_tiles), dim3(THREADS), 0, s, tb, count);
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_INV_LAUUM, s);
+    hipLaunchKernelGGL(lauum_kernel, dim3(plan->total_tiles), dim3(THREADS), 0, s, tb, count);
+  }
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }

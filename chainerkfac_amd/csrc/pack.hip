@@ -309,6 +309,7 @@ extern "C" int kfac_pack_f32(kfac_pack_plan_t plan, float *buf,
                plan->total_packed);
   if (plan->pack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
+  kfac::TimedLaunch timed(KFAC_TIMED_PACK, kfac::as_stream(stream));
   hipLaunchKernelGGL(pack_kernel, dim3(plan->pack_units), dim3(kThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank);
   KFAC_HIP_CHECK(hipGetLastError());
@@ -325,6 +326,7 @@ extern "C" int kfac_unpack_f32(kfac_pack_plan_t plan, const float *buf,
                plan->total_packed);
   if (plan->unpack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
+  kfac::TimedLaunch timed(KFAC_TIMED_UNPACK, kfac::as_stream(stream));
   hipLaunchKernelGGL(unpack_kernel, dim3(plan->unpack_units), dim3(kThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank,
                      (float)divisor);

@@ -107,6 +107,7 @@ int launch_gemm(const LA64 &a64, const LB64 &b64, const LA128 &a128, const LB128
                 int N, int K, float *C0, long long ld0, int n_main, float *C1,
                 hipStream_t stream) {
   const long long t128 = (long long)kfac::ceil_div(M, 128) * kfac::ceil_div(N, 128);
+  kfac::TimedLaunch timed(KFAC_TIMED_GEMM, stream);
   if (t128 >= 384) {
     const int tn = kfac::ceil_div(N, 128);
     hipLaunchKernelGGL((gemm_kernel<2, LA128, LB128>), dim3((unsigned)t128), dim3(THREADS), 0,

@@ -209,6 +209,24 @@ int kfac_momentum_update_f32(float *param, float *v, const float *grad,
                              int64_t nelems, float lr, float momentum,
                              void *stream);
 
+/* ------------------------------------------------------------------------
+ * Per-kernel timing for benchmarks (no counterpart in the reference, which
+ * has no instrumentation).  While enabled, every launch of the kernel
+ * families below is bracketed by a pair of HIP events on its own stream.
+ * kfac_timing_read waits for the recorded events, adds their elapsed times to
+ * the family totals and returns the totals since the last enable.
+ * --------------------------------------------------------------------- */
+#define KFAC_TIMED_SYRK 0      /* covariance main kernel (all loaders)        */
+#define KFAC_TIMED_INV_UPDATE 1 /* inverse: trailing tile update kernel       */
+#define KFAC_TIMED_INV_LAUUM 2  /* inverse: final U U^T kernel                */
+#define KFAC_TIMED_GEMM 3       /* preconditioning GEMM kernel                */
+#define KFAC_TIMED_PACK 4       /* pack kernel                                */
+#define KFAC_TIMED_UNPACK 5     /* unpack kernel                              */
+#define KFAC_TIMED_FAMILIES 6
+
+int kfac_timing_enable(int on);
+int kfac_timing_read(int family, int64_t *launches, double *total_ms);
+
 #ifdef __cplusplus
 }
 #endif
