@@ -12,6 +12,8 @@
 // Replaces the im2col + transpose + column_stack + GEMM + scale chain of
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py
 // and the batch-norm block's grad^T grad.
+#include <cstdlib>
+
 #include "common.h"
 #include "mma_core.h"
 
@@ -36,22 +38,20 @@ SyrkPlan plan_syrk(int d, long long rows) {
   p.tiles = kfac::ceil_div(d, p.bm);
   p.ntile = p.tiles * (p.tiles + 1) / 2;
   const long long nk = kfac::ceil_div<long long>(rows > 0 ? rows : 1, KT);
-  // Workgroups of one launch do equal work, so the launch takes
-  // ceil(workgroups / resident slots) rounds of (panels per split + fixed
-  // cost).  Pick the split count that minimises that, keeping at least 8
-  // panels per split; the fixed cost stands for the tile prologue, the
-  // partial-tile store and its later reduction.
-  const long long slots = p.bm == 128 ? 512 : 1024;
-  const long long fixed = 4;
-  const long long max_ns = nk >= 8 ? nk / 8 : 1;
-  long long ns = 1, best = -1;
-  for (long long c = 1; c <= max_ns && c <= 4096; ++c) {
-    const long long rounds = kfac::ceil_div<long long>((long long)p.ntile * c, slots);
-    const long long cost = rounds * (kfac::ceil_div(nk, c) + fixed);
-    if (best < 0 || cost < best) {
-      best = cost;
-      ns = c;
-    }
+  // Measured on MI355X: a launch runs best with a few thousand workgroups in
+  // flight-order (several per CU, refilled as they retire), as long as each
+  // keeps at least ~6 panels of work to amortise its prologue and the partial
+  // tile it writes.  Sweeps over ResNet-50 shapes are flat between ~700 and
+  // ~4000 workgroups; aim for 1536.
+  const long long target = 1536;
+  long long ns = kfac::ceil_div<long long>(target, p.ntile);
+  const long long max_ns = nk >= 6 ? nk / 6 : 1;
+  if (ns > max_ns) ns = max_ns;
+  if (ns < 1) ns = 1;
+  // tuning override: KFAC_SYRK_SPLITS=<n> forces the split count
+  if (const char *env = getenv("KFAC_SYRK_SPLITS")) {
+    const long long forced = atoll(env);
+    if (forced >= 1) ns = forced < nk ? forced : nk;
   }
   const long long per = kfac::ceil_div(nk, ns);
   p.nsplit = (int)kfac::ceil_div(nk, per);
@@ -94,7 +94,7 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
 }
 
 template <int WM, class Loader>
-__global__ __launch_bounds__(THREADS, 2) void syrk_kernel(Loader ld, long long K,
+__global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K,
                                                           long long klen, int ntile,
                                                           float *__restrict__ partial) {
   constexpr int BM = 64 * WM;
@@ -214,9 +214,9 @@ LoaderKC<ROWS> make_kc(const float *base, long long sample_stride, long long row
                        int rows_valid, int ones_row) {
   LoaderKC<ROWS> l;
   l.base = base;
-  l.sample_stride = sample_stride;
-  l.row_stride = row_stride;
-  l.L = L;
+  l.sample_stride = (unsigned)sample_stride;
+  l.row_stride = (unsigned)row_stride;
+  l.L = (unsigned)L;
   l.rows_valid = rows_valid;
   l.ones_row = ones_row;
   l.vec = (sample_stride % 4 == 0) && (row_stride % 4 == 0) && (L % 4 == 0) &&
@@ -230,7 +230,7 @@ LoaderKS<ROWS> make_ks(const float *base, long long ld, int rows_valid, int has_
   LoaderKS<ROWS> l;
   l.base = base;
   l.extra = extra;
-  l.ld = ld;
+  l.ld = (unsigned)ld;
   l.rows_valid = rows_valid;
   l.has_extra = has_extra;
   l.vec = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
@@ -270,6 +270,7 @@ extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_o
                                    float alpha, float beta, float *C, void *ws,
                                    size_t ws_bytes, void *stream) {
   KFAC_REQUIRE(n > 0 && d_in > 0, "bad shape n=%d d_in=%d", n, d_in);
+  KFAC_REQUIRE((long long)n * d_in < 0x7fffffffLL, "input too large");
   KFAC_REQUIRE(x && C, "null pointer");
   const int d = d_in + (append_ones ? 1 : 0);
   return run_syrk(make_ks<64>(x, d_in, d_in, append_ones, nullptr),
@@ -281,6 +282,7 @@ extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, floa
                                    float beta, float *C, void *ws, size_t ws_bytes,
                                    void *stream) {
   KFAC_REQUIRE(n > 0 && c > 0 && howo > 0, "bad shape n=%d c=%d howo=%d", n, c, howo);
+  KFAC_REQUIRE((long long)n * c * howo < 0x7fffffffLL, "input too large");
   KFAC_REQUIRE(gy && C, "null pointer");
   const long long K = (long long)n * howo;
   return run_syrk(make_kc<64>(gy, (long long)c * howo, howo, howo, c, -1),
@@ -301,7 +303,7 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
   const int wo = (w + 2 * pw - kw) / sx + 1;
   const long long dl = (long long)c * kh * kw + (append_ones ? 1 : 0);
   KFAC_REQUIRE(dl < 46340, "factor dimension %lld too large", dl);
-  KFAC_REQUIRE((long long)c * h * w < 0x7fffffffLL, "sample too large");
+  KFAC_REQUIRE((long long)n * c * h * w < 0x7fffffffLL, "input too large");
   const int d = (int)dl;
   const long long K = (long long)n * ho * wo;
   hipStream_t s = kfac::as_stream(stream);

@@ -285,11 +285,12 @@ __device__ __forceinline__ LoaderKC<NB> tile_loader(const float *base, long long
   LoaderKC<NB> l;
   l.base = base;
   l.sample_stride = 0;
-  l.row_stride = ld;
+  l.row_stride = (unsigned)ld;
   l.L = NB;
   l.rows_valid = NB;
   l.ones_row = -1;
   l.vec = 1;
+  l.init(nullptr, 0);
   return l;
 }
 

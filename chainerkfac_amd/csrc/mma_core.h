@@ -40,11 +40,15 @@ struct Panel {
       (ROWS * kRowKStride > KT * kKRowStride) ? ROWS * kRowKStride : KT * kKRowStride;
 };
 
-// Loader protocol: load() issues the global loads of one panel from clamped
-// (always valid) addresses and records which elements are real in bit masks;
-// store() applies the masks and writes the panel to LDS.  Nothing between the
-// two touches the loaded registers, so the loads stay in flight while the
-// matrix cores work on the previous panel.
+// Loader protocol: init() fixes the panel (first row) and precomputes what
+// does not change along k (row offsets, row validity); load() issues the
+// global loads of one panel; store() writes it to LDS.  Interior panels (all
+// rows and all k valid: a workgroup-uniform test) take a path without any
+// per-element selects; edge panels load from clamped (always valid) addresses
+// and apply validity masks when storing.  Nothing between load() and store()
+// touches the loaded registers, so the loads stay in flight while the matrix
+// cores work on the previous panel.  Offsets are 32-bit element offsets from
+// the tensor base (tensors hold fewer than 2^31 elements; checked on the host).
 
 // ---------------------------------------------------------------------------
 // LoaderKC: element (row, kg) at base + (kg / L) * sample_stride
@@ -57,62 +61,71 @@ struct LoaderKC {
   static constexpr int NV = ROWS / 32;
   struct Regs {
     float4 v[NV];
-    unsigned use;   // bit 4*i+e: element e of v[i] is real data
-    unsigned one;   // bit 4*i+e: element reads as 1
+    unsigned kmask;  // bit e: k-value e of this thread's quad is inside the range
+    bool fast;       // interior panel: no masks needed
   };
   const float *base;
-  long long sample_stride;
-  long long row_stride;
-  int L;           // k-values per sample
+  unsigned sample_stride;
+  unsigned row_stride;
+  unsigned L;      // k-values per sample
   int rows_valid;
   int ones_row;    // -1 if none
   int vec;         // float4 loads allowed (strides, L multiples of 4, base aligned)
+  // per-thread panel state
+  unsigned rowoff[NV];
+  unsigned rowvalid;  // bit i: row i of this thread is a data row
+  unsigned rowone;    // bit i: row i is the ones row
+  bool full_rows;
 
-  __device__ __forceinline__ void init(float *, int) const {}
-
-  __device__ __forceinline__ void load(Regs &r, int row0, long long k0,
-                                       long long k_end) const {
-    const int kq = (threadIdx.x & 7) * 4;
+  __device__ __forceinline__ void init(float *, int row0) {
     const int rr = threadIdx.x >> 3;
-    const long long kg = k0 + kq;
-    r.use = 0;
-    r.one = 0;
-    if (vec) {
-      const bool kok = kg + 3 < k_end;
-      const unsigned kc = kok ? (unsigned)kg : 0u;
-      const unsigned s = kc / (unsigned)L;
-      const float *p = base + (long long)s * sample_stride + (kc - s * (unsigned)L);
+    rowvalid = 0;
+    rowone = 0;
 #pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        const int row = row0 + rr + 32 * i;
-        const bool rok = row < rows_valid;
-        r.v[i] = *reinterpret_cast<const float4 *>(p + (long long)(rok ? row : 0) * row_stride);
-        if (rok && kok) r.use |= 0xfu << (4 * i);
-        if (kok && row == ones_row) r.one |= 0xfu << (4 * i);
+    for (int i = 0; i < NV; ++i) {
+      const int row = row0 + rr + 32 * i;
+      const bool ok = row < rows_valid;
+      rowoff[i] = (ok ? (unsigned)row : 0u) * row_stride;
+      if (ok) rowvalid |= 1u << i;
+      if (row == ones_row) rowone |= 1u << i;
+    }
+    full_rows = row0 + ROWS <= rows_valid;
+  }
+
+  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
+    const unsigned kq = (threadIdx.x & 7) * 4;
+    const unsigned kg = (unsigned)k0 + kq;
+    const bool full_k = k0 + KT <= k_end;
+    r.fast = full_rows && full_k && vec;
+    if (vec) {
+      const bool kok = full_k || (long long)kg + 3 < k_end;
+      r.kmask = kok ? 0xfu : 0u;
+      const unsigned kc = kok ? kg : 0u;
+      unsigned koff = kc;
+      if (L < (unsigned)k_end) {  // more than one sample
+        const unsigned s = kc / L;
+        koff = s * sample_stride + (kc - s * L);
       }
+      const float *p = base + koff;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + rowoff[i]);
     } else {
-      long long off[4];
-      unsigned okm = 0;
+      unsigned off[4];
+      r.kmask = 0;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const long long ke = kg + e;
-        const bool ok = ke < k_end;
-        if (ok) okm |= 1u << e;
-        const unsigned kc = ok ? (unsigned)ke : 0u;
-        const unsigned s = kc / (unsigned)L;
-        off[e] = (long long)s * sample_stride + (kc - s * (unsigned)L);
+        const bool ok = (long long)kg + e < k_end;
+        if (ok) r.kmask |= 1u << e;
+        const unsigned kc = ok ? kg + e : 0u;
+        const unsigned s = kc / L;
+        off[e] = s * sample_stride + (kc - s * L);
       }
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        const int row = row0 + rr + 32 * i;
-        const bool rok = row < rows_valid;
-        const long long ro = (long long)(rok ? row : 0) * row_stride;
-        r.v[i].x = base[off[0] + ro];
-        r.v[i].y = base[off[1] + ro];
-        r.v[i].z = base[off[2] + ro];
-        r.v[i].w = base[off[3] + ro];
-        if (rok) r.use |= okm << (4 * i);
-        if (row == ones_row) r.one |= okm << (4 * i);
+        r.v[i].x = base[off[0] + rowoff[i]];
+        r.v[i].y = base[off[1] + rowoff[i]];
+        r.v[i].z = base[off[2] + rowoff[i]];
+        r.v[i].w = base[off[3] + rowoff[i]];
       }
     }
   }
@@ -120,14 +133,27 @@ struct LoaderKC {
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
     const int kq = (threadIdx.x & 7) * 4;
     const int rr = threadIdx.x >> 3;
+    if (r.fast) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float *p = lds + (rr + 32 * i) * Panel<ROWS>::kRowKStride + kq;
-      const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+      for (int i = 0; i < NV; ++i) {
+        float *p = lds + (rr + 32 * i) * Panel<ROWS>::kRowKStride + kq;
+        p[0] = r.v[i].x;
+        p[1] = r.v[i].y;
+        p[2] = r.v[i].z;
+        p[3] = r.v[i].w;
+      }
+    } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int bit = 4 * i + e;
-        p[e] = ((r.use >> bit) & 1u) ? t[e] : (((r.one >> bit) & 1u) ? 1.f : 0.f);
+      for (int i = 0; i < NV; ++i) {
+        float *p = lds + (rr + 32 * i) * Panel<ROWS>::kRowKStride + kq;
+        const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+        const bool rv = (rowvalid >> i) & 1u;
+        const float fill = ((rowone >> i) & 1u) ? 1.f : 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool kv = (r.kmask >> e) & 1u;
+          p[e] = kv ? (rv ? t[e] : fill) : 0.f;
+        }
       }
     }
   }
@@ -145,50 +171,53 @@ struct LoaderKS {
   static constexpr int NV = KT / KPP;
   struct Regs {
     float4 v[NV];
-    unsigned use;
-    unsigned one;
+    unsigned kmask;  // bit i: k-value of pass i is inside the range
+    bool fast;
   };
   const float *base;
   const float *extra;
-  long long ld;
+  unsigned ld;
   int rows_valid;
   int has_extra;
   int vec;  // ld multiple of 4 and base 16-byte aligned
+  // per-thread panel state
+  int row;          // first of this thread's four rows
+  bool quad_ok;     // all four rows are data rows and float4 loads are allowed
+  bool full_rows;
 
-  __device__ __forceinline__ void init(float *, int) const {}
+  __device__ __forceinline__ void init(float *, int row0) {
+    row = row0 + (threadIdx.x % RQ) * 4;
+    quad_ok = vec && row + 3 < rows_valid;
+    full_rows = vec && row0 + ROWS <= rows_valid;
+  }
 
-  __device__ __forceinline__ void load(Regs &r, int row0, long long k0,
-                                       long long k_end) const {
-    const int rq = (threadIdx.x % RQ) * 4;
+  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
     const int kk = threadIdx.x / RQ;
-    const int row = row0 + rq;
-    r.use = 0;
-    r.one = 0;
-    if (vec && row + 3 < rows_valid) {
+    const bool full_k = k0 + KT <= k_end;
+    r.fast = full_rows && full_k;
+    r.kmask = 0;
+    if (quad_ok) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const long long kg = k0 + kk + KPP * i;
-        const bool kok = kg < k_end;
-        r.v[i] = *reinterpret_cast<const float4 *>(base + (kok ? kg : 0) * ld + row);
-        if (kok) r.use |= 0xfu << (4 * i);
+        const bool kok = full_k || kg < k_end;
+        if (kok) r.kmask |= 1u << i;
+        r.v[i] = *reinterpret_cast<const float4 *>(base + (unsigned)(kok ? kg : 0) * ld + (unsigned)row);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const long long kg = k0 + kk + KPP * i;
         const bool kok = kg < k_end;
-        const long long kc = kok ? kg : 0;
+        if (kok) r.kmask |= 1u << i;
+        const unsigned kc = (unsigned)(kok ? kg : 0);
         float t[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int re = row + e;
-          const bool rok = re < rows_valid;
-          const bool ex = re == rows_valid && has_extra;
-          const float *q = base + kc * ld + (rok ? re : 0);
-          if (ex && extra) q = extra + kc;
+          const float *q = base + kc * ld + (unsigned)(re < rows_valid ? re : 0);
+          if (re == rows_valid && has_extra && extra) q = extra + kc;
           t[e] = *q;
-          if (kok && (rok || (ex && extra))) r.use |= 1u << (4 * i + e);
-          if (kok && ex && !extra) r.one |= 1u << (4 * i + e);
         }
         r.v[i] = make_float4(t[0], t[1], t[2], t[3]);
       }
@@ -198,17 +227,29 @@ struct LoaderKS {
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
     const int rq = (threadIdx.x % RQ) * 4;
     const int kk = threadIdx.x / RQ;
+    if (r.fast) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
-      float o[4];
+      for (int i = 0; i < NV; ++i)
+        *reinterpret_cast<float4 *>(lds + (kk + KPP * i) * Panel<ROWS>::kKRowStride + rq) = r.v[i];
+    } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int bit = 4 * i + e;
-        o[e] = ((r.use >> bit) & 1u) ? t[e] : (((r.one >> bit) & 1u) ? 1.f : 0.f);
+      for (int i = 0; i < NV; ++i) {
+        const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+        const bool kv = (r.kmask >> i) & 1u;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int re = row + e;
+          float val = 0.f;
+          if (re < rows_valid)
+            val = t[e];
+          else if (re == rows_valid && has_extra)
+            val = extra ? t[e] : 1.f;
+          o[e] = kv ? val : 0.f;
+        }
+        *reinterpret_cast<float4 *>(lds + (kk + KPP * i) * Panel<ROWS>::kKRowStride + rq) =
+            make_float4(o[0], o[1], o[2], o[3]);
       }
-      *reinterpret_cast<float4 *>(lds + (kk + KPP * i) * Panel<ROWS>::kKRowStride + rq) =
-          make_float4(o[0], o[1], o[2], o[3]);
     }
   }
 };
@@ -330,30 +371,24 @@ __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, 
       la.load(ra, rowA0, k0 + KT, kend);
       if (!SAME) lb.load(rb, rowB0, k0 + KT, kend);
     }
-    float a[2][WM], b[2][WN];
-    auto fetch_step = [&](int kk, int buf) {
+#pragma unroll
+    for (int kk = 0; kk < KT / 2; ++kk) {
+      float a[WM], b[WN];
 #pragma unroll
       for (int im = 0; im < WM; ++im)
-        a[buf][im] = fetch<RA, LA::kKRow>(ldsA, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
+        a[im] = fetch<RA, LA::kKRow>(ldsA, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
 #pragma unroll
       for (int in = 0; in < WN; ++in) {
         if (SAME)
-          b[buf][in] = fetch<RA, LA::kKRow>(ldsA, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
+          b[in] = fetch<RA, LA::kKRow>(ldsA, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
         else
-          b[buf][in] = fetch<RB, LB::kKRow>(ldsB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
+          b[in] = fetch<RB, LB::kKRow>(ldsB, (wn * WN + in) * 32 + lrow, 2 * kk + lk);
       }
-    };
-    fetch_step(0, 0);
-#pragma unroll
-    for (int kk = 0; kk < KT / 2; ++kk) {
-      const int cur = kk & 1;
-      if (kk + 1 < KT / 2) fetch_step(kk + 1, cur ^ 1);
 #pragma unroll
       for (int im = 0; im < WM; ++im)
 #pragma unroll
         for (int in = 0; in < WN; ++in)
-          acc[im][in] =
-              __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][im], b[cur][in], acc[im][in], 0, 0, 0);
+          acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
     }
     __syncthreads();
   }

@@ -16,7 +16,7 @@ using namespace kfac::mma;
 // D[i][j] = sum_k Aop(i,k) Bop(j,k), i < M, j < N.  Column j < n_main goes to
 // C0[i*ld0 + j], column n_main (if any) to C1[i].
 template <int W, class LA, class LB>
-__global__ __launch_bounds__(THREADS, 2) void gemm_kernel(LA la, LB lb, int M, int N, int K,
+__global__ __launch_bounds__(THREADS, 2) void gemm_kernel(LA la_in, LB lb_in, int M, int N, int K,
                                                           int tiles_n, float *__restrict__ C0,
                                                           long long ld0, int n_main,
                                                           float *__restrict__ C1) {
@@ -24,6 +24,10 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(LA la, LB lb, int M, i
   __shared__ float ldsA[Panel<BM>::kFloats];
   __shared__ float ldsB[Panel<BM>::kFloats];
   const int ti = blockIdx.x / tiles_n, tj = blockIdx.x % tiles_n;
+  LA la = la_in;
+  LB lb = lb_in;
+  la.init(nullptr, ti * BM);
+  lb.init(nullptr, tj * BM);
   floatx16 acc[W][W];
   zero_acc<W, W>(acc);
   mainloop<W, W, false>(la, lb, ti * BM, tj * BM, 0, K, ldsA, ldsB, acc);
@@ -43,8 +47,8 @@ LoaderKC<ROWS> rowmajor_kc(const float *base, int rows, int K, long long ld) {
   LoaderKC<ROWS> l;
   l.base = base;
   l.sample_stride = 0;
-  l.row_stride = ld;
-  l.L = K;
+  l.row_stride = (unsigned)ld;
+  l.L = (unsigned)K;
   l.rows_valid = rows;
   l.ones_row = -1;
   l.vec = (ld % 4 == 0) && (K % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
@@ -56,7 +60,7 @@ LoaderKS<ROWS> colop_ks(const float *base, long long ld, int rows_valid, const f
   LoaderKS<ROWS> l;
   l.base = base;
   l.extra = extra;
-  l.ld = ld;
+  l.ld = (unsigned)ld;
   l.rows_valid = rows_valid;
   l.has_extra = extra != nullptr;
   l.vec = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
@@ -137,6 +141,9 @@ extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ain
   KFAC_REQUIRE((gradb == nullptr) == (kfb == nullptr), "gradb and kfb must both be given or both null");
   const int hb = gradb ? 1 : 0;
   KFAC_REQUIRE(dA - hb > 0, "dA too small");
+  KFAC_REQUIRE((long long)dG * dA < 0x7fffffffLL && (long long)dA * dA < 0x7fffffffLL &&
+                   (long long)dG * dG < 0x7fffffffLL,
+               "factor too large");
   if (ws == nullptr || ws_bytes < kfac_precond_conn_workspace_bytes(dG, dA))
     return kfac::fail(KFAC_ENOMEM, "preconditioning workspace too small: %zu < %zu bytes",
                       ws_bytes, kfac_precond_conn_workspace_bytes(dG, dA));
