@@ -1,13 +1,16 @@
 // Kronecker-factor construction:  C = beta*C + alpha * P^T P  for the patch /
 // activation / gradient matrix P of one layer, never materialised.
 //
-// Stage 1 (syrk_kernel): each workgroup owns one lower-triangle tile (I >= J)
-// of C and one slice of the reduction index (split-K: the reduction runs over
-// samples x pixels and is far longer than C is wide for most layers), and
-// writes its raw partial tile to the workspace.
-// Stage 2 (finish_kernel): sums the partials of each 64x64 sub-block in a fixed
-// order (deterministic), applies alpha/beta and writes both C[I,J] and its
-// mirror C[J,I] through an LDS transpose, so C is exactly symmetric.
+// syrk_kernel: each workgroup owns one lower-triangle tile (I >= J) of C and one
+// slice of the reduction index (split-K: the reduction runs over samples x
+// pixels and is far longer than C is wide for most layers).
+//   one slice        the tile is scaled and written straight from registers;
+//   more slices      every workgroup stores its raw partial tile; reduce_kernel
+//                    (more than 8 slices: folds them to 8 slots in parallel)
+//                    and finish_kernel (one workgroup per 64x64 block of C, a
+//                    fixed summation order, so deterministic) write C.
+// Tiles are written as C[I,J] plus the mirror C[J,I] through an LDS transpose,
+// so C is exactly symmetric and every store is a contiguous row segment.
 //
 // Replaces the im2col + transpose + column_stack + GEMM + scale chain of
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py
@@ -93,15 +96,62 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
   J = t - r * (r + 1) / 2;
 }
 
+// Writes the finished tile: C[I,J] = alpha*acc + beta*C[I,J] and, for I != J,
+// the mirror C[J,I], 64x64 quadrant by quadrant through an LDS transpose so
+// that every global access is a contiguous row segment.
+template <int WM>
+__device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
+                                           int d, float alpha, float beta,
+                                           float *__restrict__ C) {
+  constexpr int BM = 64 * WM;
+  float(*t)[65] = reinterpret_cast<float(*)[65]>(lds);
+  const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
+  for (int q = 0; q < WM * WM; ++q) {
+    const int qm = q / WM, qn = q % WM;
+    __syncthreads();
+    for_each_acc<WM, WM>(acc, [&](int r, int c, float v) {
+      if (r / 64 == qm && c / 64 == qn) t[r % 64][c % 64] = v;
+    });
+    __syncthreads();
+    const int r0 = I * BM + qm * 64, c0 = J * BM + qn * 64;
+#pragma unroll 4
+    for (int p = 0; p < 16; ++p) {
+      const int lr = lr0 + 4 * p;
+      const int r = r0 + lr, c = c0 + lc;
+      float v = alpha * t[lr][lc];
+      const bool ok = r < d && c < d;
+      if (ok) {
+        if (beta != 0.f) v += beta * C[(long long)r * d + c];
+        C[(long long)r * d + c] = v;
+      }
+      if (beta != 0.f && I != J) t[lr][lc] = v;   // mirror gets the same value
+    }
+    if (I != J) {
+      if (beta != 0.f) __syncthreads();
+#pragma unroll 4
+      for (int p = 0; p < 16; ++p) {
+        const int lr = lr0 + 4 * p;
+        const int mr = c0 + lr, mc = r0 + lc;   // row of the mirrored quadrant = column here
+        if (mr < d && mc < d) C[(long long)mr * d + mc] = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
+      }
+    }
+  }
+}
+
+// With a single k-slice (direct != 0) the tile is scaled and written straight
+// from registers; otherwise the raw partial tile goes to the workspace.
 template <int WM, class Loader>
 __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K,
-                                                          long long klen, int ntile,
-                                                          float *__restrict__ partial) {
+                                                          long long klen, int ntile, int direct,
+                                                          int d, float alpha,
+                                                          float beta, float *__restrict__ partial,
+                                                          float *__restrict__ C) {
   constexpr int BM = 64 * WM;
-  __shared__ float ldsA[Panel<BM>::kFloats];
-  __shared__ float ldsB[Panel<BM>::kFloats];
+  __shared__ float lds[2 * Panel<BM>::kFloats];
   __shared__ int2 tabA[BM];
   __shared__ int2 tabB[BM];
+  float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
+  static_assert(2 * Panel<BM>::kFloats >= 64 * 65, "LDS too small for the epilogue transpose");
   const int tile = blockIdx.x % ntile;
   const int split = blockIdx.x / ntile;
   int I, J;
@@ -119,6 +169,10 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
     mainloop<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
   else
     mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
+  if (direct) {
+    write_tile<WM>(acc, lds, I, J, d, alpha, beta, C);
+    return;
+  }
   float *out = partial + ((long long)split * ntile + tile) * (BM * BM);
   for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
 }
@@ -179,16 +233,18 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, 
                       ws_bytes, need);
   float *partial = static_cast<float *>(ws);
   const int grid = p.ntile * p.nsplit;
+  const int direct = p.nsplit == 1 ? 1 : 0;
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
     if (p.bm == 64)
       hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
-                         p.klen, p.ntile, partial);
+                         p.klen, p.ntile, direct, d, alpha, beta, partial, C);
     else
       hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
-                         p.klen, p.ntile, partial);
+                         p.klen, p.ntile, direct, d, alpha, beta, partial, C);
   }
   KFAC_HIP_CHECK(hipGetLastError());
+  if (direct) return KFAC_OK;
   const float *fin = partial;
   int nfin = p.nsplit;
   if (p.nreduced) {

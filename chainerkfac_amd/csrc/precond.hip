@@ -13,33 +13,102 @@ namespace {
 
 using namespace kfac::mma;
 
-// D[i][j] = sum_k Aop(i,k) Bop(j,k), i < M, j < N.  Column j < n_main goes to
-// C0[i*ld0 + j], column n_main (if any) to C1[i].
+// D[i][j] = sum_k Aop(i,k) Bop(j,k), i < M, j < N, over this workgroup's slice
+// of k.  Without split-K (partial == nullptr) column j < n_main goes to
+// C0[i*ld0 + j] and column n_main (if any) to C1[i]; with split-K the raw tile
+// goes to the workspace and gemm_finish_kernel adds the slices up.
 template <int W, class LA, class LB>
 __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(LA la_in, LB lb_in, int M, int N, int K,
-                                                          int tiles_n, float *__restrict__ C0,
-                                                          long long ld0, int n_main,
-                                                          float *__restrict__ C1) {
+                                                          long long klen, int tiles_n, int ntiles,
+                                                          float *__restrict__ partial,
+                                                          float *__restrict__ C0, long long ld0,
+                                                          int n_main, float *__restrict__ C1) {
   constexpr int BM = 64 * W;
   __shared__ float ldsA[Panel<BM>::kFloats];
   __shared__ float ldsB[Panel<BM>::kFloats];
-  const int ti = blockIdx.x / tiles_n, tj = blockIdx.x % tiles_n;
+  const int tile = blockIdx.x % ntiles;
+  const int split = blockIdx.x / ntiles;
+  const int ti = tile / tiles_n, tj = tile % tiles_n;
   LA la = la_in;
   LB lb = lb_in;
   la.init(nullptr, ti * BM);
   lb.init(nullptr, tj * BM);
+  const long long kbeg = (long long)split * klen;
+  long long kend = kbeg + klen;
+  if (kend > K) kend = K;
   floatx16 acc[W][W];
   zero_acc<W, W>(acc);
-  mainloop<W, W, false>(la, lb, ti * BM, tj * BM, 0, K, ldsA, ldsB, acc);
-  for_each_acc<W, W>(acc, [&](int r, int c, float v) {
-    const int i = ti * BM + r, j = tj * BM + c;
-    if (i < M && j < N) {
-      if (j < n_main)
-        C0[(long long)i * ld0 + j] = v;
-      else
-        C1[i] = v;
-    }
-  });
+  mainloop<W, W, false>(la, lb, ti * BM, tj * BM, kbeg, kend, ldsA, ldsB, acc);
+  if (partial) {
+    float *out = partial + ((long long)split * ntiles + tile) * (BM * BM);
+    for_each_acc<W, W>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
+  } else {
+    for_each_acc<W, W>(acc, [&](int r, int c, float v) {
+      const int i = ti * BM + r, j = tj * BM + c;
+      if (i < M && j < N) {
+        if (j < n_main)
+          C0[(long long)i * ld0 + j] = v;
+        else
+          C1[i] = v;
+      }
+    });
+  }
+}
+
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const float *__restrict__ partial,
+                                                          int nsplit, int ntiles, int tiles_n,
+                                                          int bm, int M, int N,
+                                                          float *__restrict__ C0, long long ld0,
+                                                          int n_main, float *__restrict__ C1) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)M * N) return;
+  const int i = (int)(idx / N), j = (int)(idx - (long long)i * N);
+  const int tile = (i / bm) * tiles_n + j / bm;
+  const float *p = partial + (long long)tile * bm * bm + (i % bm) * bm + (j % bm);
+  const long long stride = (long long)ntiles * bm * bm;
+  float sum = 0.f;
+  for (int s = 0; s < nsplit; ++s) sum += p[s * stride];
+  if (j < n_main)
+    C0[(long long)i * ld0 + j] = sum;
+  else
+    C1[i] = sum;
+}
+
+struct GemmPlan {
+  int w;        // 1: 64x64 tiles, 2: 128x128 tiles
+  int tm, tn;
+  int nsplit;
+  long long klen;
+  size_t partial_floats() const {
+    return nsplit > 1 ? (size_t)nsplit * tm * tn * (64 * w) * (64 * w) : 0;
+  }
+};
+
+// 128x128 tiles with enough k-slices to put ~1000 workgroups in flight; 64x64
+// tiles when even that leaves most CUs idle (small products).
+GemmPlan plan_gemm(int M, int N, int K) {
+  const long long nk = kfac::ceil_div(K, KT);
+  auto splits = [&](long long tiles) {
+    long long ns = kfac::ceil_div<long long>(1024, tiles);
+    const long long max_ns = nk >= 6 ? nk / 6 : 1;
+    if (ns > max_ns) ns = max_ns;
+    return ns < 1 ? 1 : ns;
+  };
+  GemmPlan p;
+  p.w = 2;
+  p.tm = kfac::ceil_div(M, 128);
+  p.tn = kfac::ceil_div(N, 128);
+  long long ns = splits((long long)p.tm * p.tn);
+  if ((long long)p.tm * p.tn * ns < 256) {
+    p.w = 1;
+    p.tm = kfac::ceil_div(M, 64);
+    p.tn = kfac::ceil_div(N, 64);
+    ns = splits((long long)p.tm * p.tn);
+  }
+  const long long per = kfac::ceil_div(nk, ns);
+  p.nsplit = (int)kfac::ceil_div(nk, per);
+  p.klen = per * KT;
+  return p;
 }
 
 template <int ROWS>
@@ -108,29 +177,41 @@ __global__ __launch_bounds__(1024) void bn_select_kernel(const float *__restrict
 
 template <class LA64, class LB64, class LA128, class LB128>
 int launch_gemm(const LA64 &a64, const LB64 &b64, const LA128 &a128, const LB128 &b128, int M,
-                int N, int K, float *C0, long long ld0, int n_main, float *C1,
+                int N, int K, float *partial, float *C0, long long ld0, int n_main, float *C1,
                 hipStream_t stream) {
-  const long long t128 = (long long)kfac::ceil_div(M, 128) * kfac::ceil_div(N, 128);
-  kfac::TimedLaunch timed(KFAC_TIMED_GEMM, stream);
-  if (t128 >= 384) {
-    const int tn = kfac::ceil_div(N, 128);
-    hipLaunchKernelGGL((gemm_kernel<2, LA128, LB128>), dim3((unsigned)t128), dim3(THREADS), 0,
-                       stream, a128, b128, M, N, K, tn, C0, ld0, n_main, C1);
-  } else {
-    const int tn = kfac::ceil_div(N, 64);
-    const int tm = kfac::ceil_div(M, 64);
-    hipLaunchKernelGGL((gemm_kernel<1, LA64, LB64>), dim3(tm * tn), dim3(THREADS), 0, stream, a64,
-                       b64, M, N, K, tn, C0, ld0, n_main, C1);
+  const GemmPlan p = plan_gemm(M, N, K);
+  const int ntiles = p.tm * p.tn;
+  float *part = p.nsplit > 1 ? partial : nullptr;
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_GEMM, stream);
+    if (p.w == 2)
+      hipLaunchKernelGGL((gemm_kernel<2, LA128, LB128>), dim3(ntiles * p.nsplit), dim3(THREADS), 0,
+                         stream, a128, b128, M, N, K, p.klen, p.tn, ntiles, part, C0, ld0, n_main,
+                         C1);
+    else
+      hipLaunchKernelGGL((gemm_kernel<1, LA64, LB64>), dim3(ntiles * p.nsplit), dim3(THREADS), 0,
+                         stream, a64, b64, M, N, K, p.klen, p.tn, ntiles, part, C0, ld0, n_main, C1);
   }
   KFAC_HIP_CHECK(hipGetLastError());
+  if (part) {
+    const long long total = (long long)M * N;
+    hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)kfac::ceil_div<long long>(total, 256)),
+                       dim3(256), 0, stream, part, p.nsplit, ntiles, p.tn, 64 * p.w, M, N, C0, ld0,
+                       n_main, C1);
+    KFAC_HIP_CHECK(hipGetLastError());
+  }
   return KFAC_OK;
 }
+
+size_t align_floats(size_t n) { return (n + 63) & ~(size_t)63; }
 
 }  // namespace
 
 extern "C" size_t kfac_precond_conn_workspace_bytes(int dG, int dA) {
   if (dG <= 0 || dA <= 0) return 0;
-  return (size_t)dG * dA * sizeof(float) + 256;
+  const size_t p1 = plan_gemm(dG, dA, dG).partial_floats();
+  const size_t p2 = plan_gemm(dG, dA, dA).partial_floats();
+  return (align_floats((size_t)dG * dA) + (p1 > p2 ? p1 : p2)) * sizeof(float) + 256;
 }
 
 extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ainv, int dA,
@@ -150,15 +231,16 @@ extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ain
   hipStream_t s = kfac::as_stream(stream);
   float *T = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
   const int dW = dA - hb;
+  float *partial = T + align_floats((size_t)dG * dA);
   // T (dG x dA) = Ginv (dG x dG) . [gradW | gradb] (dG x dA)
   int rc = launch_gemm(rowmajor_kc<64>(Ginv, dG, dG, dG), colop_ks<64>(gradW, dW, dW, gradb),
                        rowmajor_kc<128>(Ginv, dG, dG, dG), colop_ks<128>(gradW, dW, dW, gradb), dG,
-                       dA, dG, T, dA, dA, nullptr, s);
+                       dA, dG, partial, T, dA, dA, nullptr, s);
   if (rc != KFAC_OK) return rc;
   // kf (dG x dA) = T . Ainv (symmetric: column j of Ainv is its row j)
   return launch_gemm(rowmajor_kc<64>(T, dG, dA, dA), rowmajor_kc<64>(Ainv, dA, dA, dA),
                      rowmajor_kc<128>(T, dG, dA, dA), rowmajor_kc<128>(Ainv, dA, dA, dA), dG, dA,
-                     dA, kfW, dW, dW, kfb, s);
+                     dA, partial, kfW, dW, dW, kfb, s);
 }
 
 extern "C" size_t kfac_precond_bn_workspace_bytes(int d) {
