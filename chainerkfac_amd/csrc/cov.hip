@@ -18,6 +18,7 @@
 #include <cstdlib>
 
 #include "common.h"
+#include "conv_halo.h"
 #include "mma_core.h"
 
 namespace {
@@ -35,12 +36,12 @@ struct SyrkPlan {
 
 constexpr int kFinishSplits = 8;
 
-SyrkPlan plan_syrk(int d, long long rows) {
+SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
   SyrkPlan p;
   p.bm = d <= 320 ? 64 : 128;
   p.tiles = kfac::ceil_div(d, p.bm);
   p.ntile = p.tiles * (p.tiles + 1) / 2;
-  const long long nk = kfac::ceil_div<long long>(rows > 0 ? rows : 1, KT);
+  if (nk < 1) nk = 1;
   // Measured on MI355X: a launch runs best with a few thousand workgroups in
   // flight-order (several per CU, refilled as they retire), as long as each
   // keeps at least ~6 panels of work to amortise its prologue and the partial
@@ -58,10 +59,14 @@ SyrkPlan plan_syrk(int d, long long rows) {
   }
   const long long per = kfac::ceil_div(nk, ns);
   p.nsplit = (int)kfac::ceil_div(nk, per);
-  p.klen = per * KT;
+  p.klen = per * panel_len;
   // partials are pre-reduced to at most kFinishSplits slots before finishing
   p.nreduced = p.nsplit > kFinishSplits ? kFinishSplits : 0;
   return p;
+}
+
+SyrkPlan plan_syrk(int d, long long rows) {
+  return plan_syrk_panels(d, kfac::ceil_div<long long>(rows > 0 ? rows : 1, KT), KT);
 }
 
 size_t syrk_ws_floats(const SyrkPlan &p) {
@@ -140,10 +145,49 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
 
 // With a single k-slice (direct != 0) the tile is scaled and written straight
 // from registers; otherwise the raw partial tile goes to the workspace.
+// Workgroup -> (tile, k-slice).  Hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs, each with its own L2.  Every XCD therefore gets a
+// contiguous chunk of the work list, ordered so that the ~100 workgroups an
+// XCD runs at a time share operand panels: one k-slice at a time, tiles in
+// super-rows of 8 tile rows walked column by column (8 tiles share a J panel,
+// the whole super-row shares 8 I panels).
+constexpr int kXcds = 8;
+constexpr int kSuperRows = 8;
+
+__device__ __forceinline__ void work_decode(int bid, int total, int ntile, int tiles, int &split,
+                                            int &tile, int &I, int &J) {
+  const int xcd = bid % kXcds, idx = bid / kXcds;
+  const int base = total / kXcds, rem = total % kXcds;
+  const int w = xcd * base + (xcd < rem ? xcd : rem) + idx;
+  split = w / ntile;
+  const int q = w - split * ntile;
+  int row, dummy;
+  tri_decode(q, row, dummy);
+  const int r = row / kSuperRows;
+  const int I0 = r * kSuperRows;
+  int I1 = I0 + kSuperRows - 1;
+  if (I1 > tiles - 1) I1 = tiles - 1;
+  const int h = I1 - I0 + 1;
+  int qq = q - I0 * (I0 + 1) / 2;
+  if (qq < (I0 + 1) * h) {
+    J = qq / h;
+    I = I0 + (qq - J * h);
+  } else {
+    qq -= (I0 + 1) * h;
+    J = I0 + 1;
+    while (qq >= I1 - J + 1) {
+      qq -= I1 - J + 1;
+      ++J;
+    }
+    I = J + qq;
+  }
+  tile = I * (I + 1) / 2 + J;
+}
+
 template <int WM, class Loader>
 __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K,
-                                                          long long klen, int ntile, int direct,
-                                                          int d, float alpha,
+                                                          long long klen, int ntile, int nsplit,
+                                                          int direct, int d, float alpha,
                                                           float beta, float *__restrict__ partial,
                                                           float *__restrict__ C) {
   constexpr int BM = 64 * WM;
@@ -152,10 +196,8 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
   __shared__ int2 tabB[BM];
   float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
   static_assert(2 * Panel<BM>::kFloats >= 64 * 65, "LDS too small for the epilogue transpose");
-  const int tile = blockIdx.x % ntile;
-  const int split = blockIdx.x / ntile;
-  int I, J;
-  tri_decode(tile, I, J);
+  int split, tile, I, J;
+  work_decode(blockIdx.x, ntile * nsplit, ntile, (d + BM - 1) / BM, split, tile, I, J);
   Loader la = ld, lb = ld;
   la.init(reinterpret_cast<float *>(tabA), I * BM);
   lb.init(reinterpret_cast<float *>(tabB), J * BM);
@@ -171,6 +213,56 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
     mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
   if (direct) {
     write_tile<WM>(acc, lds, I, J, d, alpha, beta, C);
+    return;
+  }
+  float *out = partial + ((long long)split * ntile + tile) * (BM * BM);
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
+}
+
+// Convolution A factor through the LDS halo region (conv_halo.h); `klen` counts
+// reduction steps, not k-values.
+template <int WM, int NKK>
+__global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long long total_steps,
+                                                               long long klen, int ntile,
+                                                               int nsplit, int direct, int d,
+                                                               float alpha,
+                                                               float beta,
+                                                               float *__restrict__ partial,
+                                                               float *__restrict__ C) {
+  constexpr int BM = 64 * WM;
+  extern __shared__ float smem[];
+  const int region = halo_region_floats(g);
+  float *regA = smem;
+  float *regB = smem + region;
+  int *koff_tbl = reinterpret_cast<int *>(smem + 2 * region);
+  int split, tile, I, J;
+  work_decode(blockIdx.x, ntile * nsplit, ntile, (d + BM - 1) / BM, split, tile, I, J);
+  // constant planes (ones, zeros) of both regions and the k -> offset table
+  for (int e = threadIdx.x; e < 2 * g.Rsz; e += THREADS) {
+    const float val = e < g.Rsz ? 1.f : 0.f;
+    regA[g.CH * g.Rsz + e] = val;
+    regB[g.CH * g.Rsz + e] = val;
+  }
+  for (int k = threadIdx.x; k < kHaloMaxK; k += THREADS) {
+    int off = 0;
+    if (k < g.RT * g.WS) {
+      const int orow = k / g.WS, ocol = k - orow * g.WS;
+      off = orow * g.sy * g.Wr + ocol * g.sx;
+    }
+    koff_tbl[k] = off;
+  }
+  __syncthreads();
+  const long long sbeg = (long long)split * klen;
+  long long send = sbeg + klen;
+  if (send > total_steps) send = total_steps;
+  floatx16 acc[WM][WM];
+  zero_acc<WM, WM>(acc);
+  if (I == J)
+    halo_mainloop<WM, NKK, true>(g, I * BM, J * BM, sbeg, send, regA, regB, koff_tbl, acc);
+  else
+    halo_mainloop<WM, NKK, false>(g, I * BM, J * BM, sbeg, send, regA, regB, koff_tbl, acc);
+  if (direct) {
+    write_tile<WM>(acc, smem, I, J, d, alpha, beta, C);
     return;
   }
   float *out = partial + ((long long)split * ntile + tile) * (BM * BM);
@@ -223,28 +315,9 @@ __global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ p
   }
 }
 
-template <class L64, class L128>
-int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, float beta,
-             float *C, void *ws, size_t ws_bytes, hipStream_t stream) {
-  const SyrkPlan p = plan_syrk(d, K);
-  const size_t need = syrk_ws_floats(p) * sizeof(float);
-  if (ws_bytes < need || ws == nullptr)
-    return kfac::fail(KFAC_ENOMEM, "covariance workspace too small: %zu < %zu bytes",
-                      ws_bytes, need);
-  float *partial = static_cast<float *>(ws);
-  const int grid = p.ntile * p.nsplit;
-  const int direct = p.nsplit == 1 ? 1 : 0;
-  {
-    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
-    if (p.bm == 64)
-      hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
-                         p.klen, p.ntile, direct, d, alpha, beta, partial, C);
-    else
-      hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
-                         p.klen, p.ntile, direct, d, alpha, beta, partial, C);
-  }
-  KFAC_HIP_CHECK(hipGetLastError());
-  if (direct) return KFAC_OK;
+// reduce_kernel (more than 8 slices) + finish_kernel on the partial tiles.
+int finish_partials(const SyrkPlan &p, int d, float alpha, float beta, float *C, float *partial,
+                    hipStream_t stream) {
   const float *fin = partial;
   int nfin = p.nsplit;
   if (p.nreduced) {
@@ -265,31 +338,169 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, 
   return KFAC_OK;
 }
 
-template <int ROWS>
-LoaderKC<ROWS> make_kc(const float *base, long long sample_stride, long long row_stride, int L,
-                       int rows_valid, int ones_row) {
-  LoaderKC<ROWS> l;
+int check_ws(const SyrkPlan &p, void *ws, size_t ws_bytes) {
+  const size_t need = syrk_ws_floats(p) * sizeof(float);
+  if (ws_bytes < need || ws == nullptr)
+    return kfac::fail(KFAC_ENOMEM, "covariance workspace too small: %zu < %zu bytes", ws_bytes,
+                      need);
+  return KFAC_OK;
+}
+
+template <class L64, class L128>
+int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, float beta,
+             float *C, void *ws, size_t ws_bytes, hipStream_t stream) {
+  const SyrkPlan p = plan_syrk(d, K);
+  if (int rc = check_ws(p, ws, ws_bytes)) return rc;
+  float *partial = static_cast<float *>(ws);
+  const int grid = p.ntile * p.nsplit;
+  const int direct = p.nsplit == 1 ? 1 : 0;
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
+    if (p.bm == 64)
+      hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
+                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+    else
+      hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
+                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  if (direct) return KFAC_OK;
+  return finish_partials(p, d, alpha, beta, C, partial, stream);
+}
+
+// Geometry of the LDS halo kernel for one convolution; false when the shape
+// does not fit its limits (the element-wise im2col loader is used instead).
+bool make_halo_geom(const float *x, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
+                    int pw, int ho, int wo, int append_ones, ConvGeom *out) {
+  ConvGeom g;
+  g.x = x;
+  g.C = c; g.H = h; g.W = w; g.kh = kh; g.kw = kw; g.sy = sy; g.sx = sx; g.ph = ph; g.pw = pw;
+  g.ho = ho; g.wo = wo;
+  g.d_patch = c * kh * kw;
+  g.append_ones = append_ones;
+  const int khkw = kh * kw;
+  if (khkw < 2 || khkw > 127) return false;
+  g.segs = kfac::ceil_div(wo, kHaloMaxK);
+  g.WS = kfac::ceil_div(wo, g.segs);
+  if (g.WS * g.segs != wo) return false;   // ragged column segments are not handled
+  g.RT = kHaloMaxK / g.WS;
+  if (g.RT > ho) g.RT = ho;
+  if (g.RT < 1) g.RT = 1;
+  g.rgroups = kfac::ceil_div(ho, g.RT);
+  // k-values per step: one of the compiled loop lengths (2 * 25, 28 or 32);
+  // the slots past RT*WS are masked
+  const int span = g.RT * g.WS;
+  if (span < 40) return false;   // tiny images: too few pixels per step to pay off
+  g.nk = span <= 50 ? 50 : (span <= 56 ? 56 : 64);
+  g.Rin = (g.RT - 1) * sy + kh;
+  g.Win = (g.WS - 1) * sx + kw;
+  if (g.Rin > 255 || g.Win > 255) return false;
+  auto round_mod32 = [](int at_least, int residue) {
+    int v = at_least + ((residue - at_least) % 32 + 32) % 32;
+    return v;
+  };
+  g.Wr = round_mod32(g.Win, kw % 32);
+  g.Rsz = round_mod32(g.Rin * g.Wr, khkw % 32);
+  g.CH = 127 / khkw + 2;   // 128 consecutive patch rows touch at most this many channels
+  g.LPR = 16;
+  while (g.LPR < g.Win) g.LPR *= 2;
+  if (g.LPR > THREADS) return false;
+  g.CPP = THREADS / g.LPR;
+  g.passes = kfac::ceil_div(g.CH, g.CPP);
+  g.nq = g.passes * g.Rin;
+  if (g.nq > kHaloMaxQ || g.Rin > 15 || g.passes > 15) return false;
+  g.e_pass = 0;
+  g.e_row = 0;
+  for (int e = 0; e < 16; ++e) {
+    g.goffE[e] = 0;
+    g.loffE[e] = 0;
+  }
+  for (int e = 0; e < g.nq; ++e) {
+    const int ps = e / g.Rin, ry = e % g.Rin;
+    g.e_pass |= (unsigned long long)ps << (4 * e);
+    g.e_row |= (unsigned long long)ry << (4 * e);
+    g.goffE[e] = (ps * g.CPP * h + ry) * w;
+    g.loffE[e] = ps * g.CPP * g.Rsz + ry * g.Wr;
+  }
+  if ((g.CH + 2) * g.Rsz > 0xffff) return false;
+  *out = g;
+  return true;
+}
+
+size_t halo_lds_bytes(const ConvGeom &g) {
+  size_t floats = 2 * (size_t)halo_region_floats(g) + kHaloMaxK;
+  if (floats < 64 * 65) floats = 64 * 65;   // the epilogue transposes through the same memory
+  return floats * sizeof(float);
+}
+
+int run_conv_halo(const ConvGeom &g, int n, int d, float alpha, float beta, float *C, void *ws,
+                  size_t ws_bytes, hipStream_t stream) {
+  const long long total_steps = (long long)n * g.segs * g.rgroups;
+  SyrkPlan p = plan_syrk_panels(d, total_steps, 1);
+  if (p.bm != 128) return 1;   // small factors stay on the generic kernel
+  if (int rc = check_ws(p, ws, ws_bytes)) return rc;
+  const size_t lds = halo_lds_bytes(g);
+  static bool attr_set = false;
+  if (!attr_set) {
+    const void *fns[3] = {reinterpret_cast<const void *>(syrk_conv_kernel<2, 25>),
+                          reinterpret_cast<const void *>(syrk_conv_kernel<2, 28>),
+                          reinterpret_cast<const void *>(syrk_conv_kernel<2, 32>)};
+    for (const void *fn : fns)
+      KFAC_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         160 * 1024));
+    attr_set = true;
+  }
+  float *partial = static_cast<float *>(ws);
+  const int direct = p.nsplit == 1 ? 1 : 0;
+  const dim3 grid(p.ntile * p.nsplit), block(THREADS);
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
+    if (g.nk == 50)
+      hipLaunchKernelGGL((syrk_conv_kernel<2, 25>), grid, block, lds, stream, g, total_steps,
+                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+    else if (g.nk == 56)
+      hipLaunchKernelGGL((syrk_conv_kernel<2, 28>), grid, block, lds, stream, g, total_steps,
+                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+    else
+      hipLaunchKernelGGL((syrk_conv_kernel<2, 32>), grid, block, lds, stream, g, total_steps,
+                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  if (direct) return KFAC_OK;
+  return finish_partials(p, d, alpha, beta, C, partial, stream);
+}
+
+bool kc_vec_ok(const float *base, long long sample_stride, long long row_stride, int L) {
+  return (sample_stride % 4 == 0) && (row_stride % 4 == 0) && (L % 4 == 0) &&
+         (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+}
+
+template <int ROWS, bool VEC>
+LoaderKC<ROWS, VEC> make_kc(const float *base, long long sample_stride, long long row_stride, int L,
+                            int rows_valid, int ones_row) {
+  LoaderKC<ROWS, VEC> l;
   l.base = base;
   l.sample_stride = (unsigned)sample_stride;
   l.row_stride = (unsigned)row_stride;
   l.L = (unsigned)L;
   l.rows_valid = rows_valid;
   l.ones_row = ones_row;
-  l.vec = (sample_stride % 4 == 0) && (row_stride % 4 == 0) && (L % 4 == 0) &&
-          (reinterpret_cast<uintptr_t>(base) % 16 == 0);
   return l;
 }
 
-template <int ROWS>
-LoaderKS<ROWS> make_ks(const float *base, long long ld, int rows_valid, int has_extra,
-                       const float *extra) {
-  LoaderKS<ROWS> l;
+bool ks_vec_ok(const float *base, long long ld) {
+  return (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+}
+
+template <int ROWS, bool VEC>
+LoaderKS<ROWS, VEC> make_ks(const float *base, long long ld, int rows_valid, int has_extra,
+                            const float *extra) {
+  LoaderKS<ROWS, VEC> l;
   l.base = base;
   l.extra = extra;
   l.ld = (unsigned)ld;
   l.rows_valid = rows_valid;
   l.has_extra = has_extra;
-  l.vec = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
   return l;
 }
 
@@ -319,7 +530,11 @@ LoaderIM<ROWS> make_im(const float *x, int c, int h, int w, int kh, int kw, int 
 
 extern "C" size_t kfac_cov_workspace_bytes(int d, int64_t rows) {
   if (d <= 0) return 0;
-  return syrk_ws_floats(plan_syrk(d, rows)) * sizeof(float);
+  // upper bound over every reduction length (the convolution kernels count
+  // their panels differently): the split count never exceeds ceil(1536 / tiles)
+  SyrkPlan p = plan_syrk_panels(d, 1LL << 40, KT);
+  (void)rows;
+  return syrk_ws_floats(p) * sizeof(float);
 }
 
 extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_ones,
@@ -329,9 +544,13 @@ extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_o
   KFAC_REQUIRE((long long)n * d_in < 0x7fffffffLL, "input too large");
   KFAC_REQUIRE(x && C, "null pointer");
   const int d = d_in + (append_ones ? 1 : 0);
-  return run_syrk(make_ks<64>(x, d_in, d_in, append_ones, nullptr),
-                  make_ks<128>(x, d_in, d_in, append_ones, nullptr), d, n, alpha, beta, C, ws,
-                  ws_bytes, kfac::as_stream(stream));
+  if (ks_vec_ok(x, d_in))
+    return run_syrk(make_ks<64, true>(x, d_in, d_in, append_ones, nullptr),
+                    make_ks<128, true>(x, d_in, d_in, append_ones, nullptr), d, n, alpha, beta, C,
+                    ws, ws_bytes, kfac::as_stream(stream));
+  return run_syrk(make_ks<64, false>(x, d_in, d_in, append_ones, nullptr),
+                  make_ks<128, false>(x, d_in, d_in, append_ones, nullptr), d, n, alpha, beta, C,
+                  ws, ws_bytes, kfac::as_stream(stream));
 }
 
 extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, float alpha,
@@ -341,9 +560,13 @@ extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, floa
   KFAC_REQUIRE((long long)n * c * howo < 0x7fffffffLL, "input too large");
   KFAC_REQUIRE(gy && C, "null pointer");
   const long long K = (long long)n * howo;
-  return run_syrk(make_kc<64>(gy, (long long)c * howo, howo, howo, c, -1),
-                  make_kc<128>(gy, (long long)c * howo, howo, howo, c, -1), c, K, alpha, beta,
-                  C, ws, ws_bytes, kfac::as_stream(stream));
+  if (kc_vec_ok(gy, (long long)c * howo, howo, howo))
+    return run_syrk(make_kc<64, true>(gy, (long long)c * howo, howo, howo, c, -1),
+                    make_kc<128, true>(gy, (long long)c * howo, howo, howo, c, -1), c, K, alpha,
+                    beta, C, ws, ws_bytes, kfac::as_stream(stream));
+  return run_syrk(make_kc<64, false>(gy, (long long)c * howo, howo, howo, c, -1),
+                  make_kc<128, false>(gy, (long long)c * howo, howo, howo, c, -1), c, K, alpha,
+                  beta, C, ws, ws_bytes, kfac::as_stream(stream));
 }
 
 extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, int kh, int kw,
@@ -367,9 +590,18 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
     // 1x1 convolution: the patch matrix is the NCHW tensor itself
     const int hw = h * w;
     const int ones = append_ones ? c : -1;
-    return run_syrk(make_kc<64>(x, (long long)c * hw, hw, hw, c, ones),
-                    make_kc<128>(x, (long long)c * hw, hw, hw, c, ones), d, K, alpha, beta, C,
-                    ws, ws_bytes, s);
+    if (kc_vec_ok(x, (long long)c * hw, hw, hw))
+      return run_syrk(make_kc<64, true>(x, (long long)c * hw, hw, hw, c, ones),
+                      make_kc<128, true>(x, (long long)c * hw, hw, hw, c, ones), d, K, alpha, beta,
+                      C, ws, ws_bytes, s);
+    return run_syrk(make_kc<64, false>(x, (long long)c * hw, hw, hw, c, ones),
+                    make_kc<128, false>(x, (long long)c * hw, hw, hw, c, ones), d, K, alpha, beta,
+                    C, ws, ws_bytes, s);
+  }
+  ConvGeom geom;
+  if (make_halo_geom(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones, &geom)) {
+    const int rc = run_conv_halo(geom, n, d, alpha, beta, C, ws, ws_bytes, s);
+    if (rc <= 0) return rc;   // 1 = shape left to the generic kernel
   }
   return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones),
                   make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones), d, K,

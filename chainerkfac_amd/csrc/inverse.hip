@@ -281,15 +281,14 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
 // ---------------------------------------------------------------------------
 // panel and update: 128x128x128 tile products through the shared main loop
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ LoaderKC<NB> tile_loader(const float *base, long long ld) {
-  LoaderKC<NB> l;
+__device__ __forceinline__ LoaderKC<NB, true> tile_loader(const float *base, long long ld) {
+  LoaderKC<NB, true> l;
   l.base = base;
   l.sample_stride = 0;
   l.row_stride = (unsigned)ld;
   l.L = NB;
   l.rows_valid = NB;
   l.ones_row = -1;
-  l.vec = 1;
   l.init(nullptr, 0);
   return l;
 }
@@ -377,8 +376,8 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int cou
   const long long ld = (long long)T * NB;
   const float *M = tb.ws + tb.ws_off[s];
   const int K = (T - I) * NB;
-  LoaderKC<NB> la = tile_loader(M + (long long)I * NB * ld + (long long)I * NB, ld);
-  LoaderKC<NB> lb = tile_loader(M + (long long)J * NB * ld + (long long)I * NB, ld);
+  LoaderKC<NB, true> la = tile_loader(M + (long long)I * NB * ld + (long long)I * NB, ld);
+  LoaderKC<NB, true> lb = tile_loader(M + (long long)J * NB * ld + (long long)I * NB, ld);
   la.L = K;
   lb.L = K;
   floatx16 acc[2][2];

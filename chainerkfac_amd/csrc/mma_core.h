@@ -55,7 +55,10 @@ struct Panel {
 //                                     + row * row_stride + (kg % L)
 // rows >= rows_valid read as 0, except row == ones_row which reads as 1.
 // ---------------------------------------------------------------------------
-template <int ROWS>
+// VEC: float4 loads (strides and L multiples of 4, base 16-byte aligned); a
+// compile-time choice so that the common aligned case carries no scalar-path
+// code or registers.
+template <int ROWS, bool VEC>
 struct LoaderKC {
   static constexpr bool kKRow = false;
   static constexpr int NV = ROWS / 32;
@@ -70,7 +73,6 @@ struct LoaderKC {
   unsigned L;      // k-values per sample
   int rows_valid;
   int ones_row;    // -1 if none
-  int vec;         // float4 loads allowed (strides, L multiples of 4, base aligned)
   // per-thread panel state
   unsigned rowoff[NV];
   unsigned rowvalid;  // bit i: row i of this thread is a data row
@@ -96,8 +98,8 @@ struct LoaderKC {
     const unsigned kq = (threadIdx.x & 7) * 4;
     const unsigned kg = (unsigned)k0 + kq;
     const bool full_k = k0 + KT <= k_end;
-    r.fast = full_rows && full_k && vec;
-    if (vec) {
+    r.fast = full_rows && full_k && VEC;
+    if (VEC) {
       const bool kok = full_k || (long long)kg + 3 < k_end;
       r.kmask = kok ? 0xfu : 0u;
       const unsigned kc = kok ? kg : 0u;
@@ -163,7 +165,7 @@ struct LoaderKC {
 // LoaderKS: element (row, kg) at base + kg * ld + row for row < rows_valid;
 // row == rows_valid reads extra[kg] (or 1 when extra is null) if has_extra.
 // ---------------------------------------------------------------------------
-template <int ROWS>
+template <int ROWS, bool VEC>
 struct LoaderKS {
   static constexpr bool kKRow = true;
   static constexpr int RQ = ROWS / 4;          // row quads per k
@@ -179,7 +181,6 @@ struct LoaderKS {
   unsigned ld;
   int rows_valid;
   int has_extra;
-  int vec;  // ld multiple of 4 and base 16-byte aligned
   // per-thread panel state
   int row;          // first of this thread's four rows
   bool quad_ok;     // all four rows are data rows and float4 loads are allowed
@@ -187,8 +188,8 @@ struct LoaderKS {
 
   __device__ __forceinline__ void init(float *, int row0) {
     row = row0 + (threadIdx.x % RQ) * 4;
-    quad_ok = vec && row + 3 < rows_valid;
-    full_rows = vec && row0 + ROWS <= rows_valid;
+    quad_ok = VEC && row + 3 < rows_valid;
+    full_rows = VEC && row0 + ROWS <= rows_valid;
   }
 
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {

@@ -111,28 +111,34 @@ GemmPlan plan_gemm(int M, int N, int K) {
   return p;
 }
 
-template <int ROWS>
-LoaderKC<ROWS> rowmajor_kc(const float *base, int rows, int K, long long ld) {
-  LoaderKC<ROWS> l;
+bool kc_aligned(const float *base, int K, long long ld) {
+  return (ld % 4 == 0) && (K % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+}
+
+bool ks_aligned(const float *base, long long ld) {
+  return (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+}
+
+template <int ROWS, bool VEC>
+LoaderKC<ROWS, VEC> rowmajor_kc(const float *base, int rows, int K, long long ld) {
+  LoaderKC<ROWS, VEC> l;
   l.base = base;
   l.sample_stride = 0;
   l.row_stride = (unsigned)ld;
   l.L = (unsigned)K;
   l.rows_valid = rows;
   l.ones_row = -1;
-  l.vec = (ld % 4 == 0) && (K % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
   return l;
 }
 
-template <int ROWS>
-LoaderKS<ROWS> colop_ks(const float *base, long long ld, int rows_valid, const float *extra) {
-  LoaderKS<ROWS> l;
+template <int ROWS, bool VEC>
+LoaderKS<ROWS, VEC> colop_ks(const float *base, long long ld, int rows_valid, const float *extra) {
+  LoaderKS<ROWS, VEC> l;
   l.base = base;
   l.extra = extra;
   l.ld = (unsigned)ld;
   l.rows_valid = rows_valid;
   l.has_extra = extra != nullptr;
-  l.vec = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
   return l;
 }
 
@@ -232,15 +238,31 @@ extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ain
   float *T = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
   const int dW = dA - hb;
   float *partial = T + align_floats((size_t)dG * dA);
-  // T (dG x dA) = Ginv (dG x dG) . [gradW | gradb] (dG x dA)
-  int rc = launch_gemm(rowmajor_kc<64>(Ginv, dG, dG, dG), colop_ks<64>(gradW, dW, dW, gradb),
-                       rowmajor_kc<128>(Ginv, dG, dG, dG), colop_ks<128>(gradW, dW, dW, gradb), dG,
-                       dA, dG, partial, T, dA, dA, nullptr, s);
+  // T (dG x dA) = Ginv (dG x dG) . [gradW | gradb] (dG x dA); float4 loads when
+  // both operands are aligned, scalar loads otherwise
+  int rc;
+  if (kc_aligned(Ginv, dG, dG) && ks_aligned(gradW, dW))
+    rc = launch_gemm(rowmajor_kc<64, true>(Ginv, dG, dG, dG), colop_ks<64, true>(gradW, dW, dW, gradb),
+                     rowmajor_kc<128, true>(Ginv, dG, dG, dG),
+                     colop_ks<128, true>(gradW, dW, dW, gradb), dG, dA, dG, partial, T, dA, dA,
+                     nullptr, s);
+  else
+    rc = launch_gemm(rowmajor_kc<64, false>(Ginv, dG, dG, dG),
+                     colop_ks<64, false>(gradW, dW, dW, gradb),
+                     rowmajor_kc<128, false>(Ginv, dG, dG, dG),
+                     colop_ks<128, false>(gradW, dW, dW, gradb), dG, dA, dG, partial, T, dA, dA,
+                     nullptr, s);
   if (rc != KFAC_OK) return rc;
   // kf (dG x dA) = T . Ainv (symmetric: column j of Ainv is its row j)
-  return launch_gemm(rowmajor_kc<64>(T, dG, dA, dA), rowmajor_kc<64>(Ainv, dA, dA, dA),
-                     rowmajor_kc<128>(T, dG, dA, dA), rowmajor_kc<128>(Ainv, dA, dA, dA), dG, dA,
-                     dA, partial, kfW, dW, dW, kfb, s);
+  if (kc_aligned(T, dA, dA) && kc_aligned(Ainv, dA, dA))
+    return launch_gemm(rowmajor_kc<64, true>(T, dG, dA, dA), rowmajor_kc<64, true>(Ainv, dA, dA, dA),
+                       rowmajor_kc<128, true>(T, dG, dA, dA),
+                       rowmajor_kc<128, true>(Ainv, dA, dA, dA), dG, dA, dA, partial, kfW, dW, dW,
+                       kfb, s);
+  return launch_gemm(rowmajor_kc<64, false>(T, dG, dA, dA), rowmajor_kc<64, false>(Ainv, dA, dA, dA),
+                     rowmajor_kc<128, false>(T, dG, dA, dA),
+                     rowmajor_kc<128, false>(Ainv, dA, dA, dA), dG, dA, dA, partial, kfW, dW, dW,
+                     kfb, s);
 }
 
 extern "C" size_t kfac_precond_bn_workspace_bytes(int d) {
