@@ -38,89 +38,44 @@ struct ConvGeom {
   int CH;           // staged channel planes per panel
   // staging: thread t handles column t % LPR of channel t / LPR (+ CPP per
   // pass) for every staged row; element e of a thread is (pass, row) =
-  // (nibble e of e_pass, nibble e of e_row)
+  // (e / Rin, e % Rin), nq = passes * Rin of them
   int LPR, CPP, passes, nq;
-  unsigned long long e_pass, e_row;
-  int goffE[16];    // element e: offset inside the sample, (pass*CPP*H + row) * W
-  int loffE[16];    // element e: offset inside the region, pass*CPP*Rsz + row*Wr
+  unsigned rep;      // sum over passes of 1 << (pass * Rin)
+  unsigned x_bytes;  // size of x in bytes (below 2^31)
 };
 
 constexpr int kHaloMaxQ = 16;   // staged elements per thread and panel
 constexpr int kHaloMaxK = 64;   // k-values per step
+constexpr int kHaloDump = 32;   // floats after each region that absorb stores of idle threads
 
-struct HaloPanel {
-  float v[kHaloMaxQ];
-  unsigned okmask;     // bit e: element e of this step is inside the image
-  // thread constants of the panel
-  int rx;
-  bool rx_in;
-  unsigned g_thread;   // chq*H*W + rx
-  unsigned l_thread;   // chq*Rsz + rx
-  unsigned chreal;     // bit p: channel of pass p exists in the input
-  unsigned chlive;     // bit p: channel of pass p has a plane in the region
-  int c_lo;
-
-  __device__ __forceinline__ void init(const ConvGeom &g, int row0) {
-    c_lo = row0 / (g.kh * g.kw);
-    const int chq = threadIdx.x / g.LPR;
-    rx = threadIdx.x - chq * g.LPR;
-    rx_in = rx < g.Win;
-    g_thread = (unsigned)(chq * g.H * g.W + rx);
-    l_thread = (unsigned)(chq * g.Rsz + rx);
-    chreal = 0;
-    chlive = 0;
-    for (int p = 0; p < g.passes; ++p) {
-      const int ch = p * g.CPP + chq;
-      if (ch < g.CH) chlive |= 1u << p;
-      if (ch < g.CH && c_lo + ch < g.C) chreal |= 1u << p;
-    }
-  }
-
-  // Issue the loads of the region for the step whose first tap is input pixel
-  // (iy0, ix0) of the sample at `sample_base`.  Element offsets are uniform
-  // across the workgroup apart from the per-thread base.
-  __device__ __forceinline__ void load(const ConvGeom &g, long long sample_base, int iy0, int ix0) {
-    const float *p = g.x + sample_base + (long long)c_lo * g.H * g.W + (long long)iy0 * g.W + ix0 +
-                     g_thread;
-    const bool col_ok = rx_in && (unsigned)(ix0 + rx) < (unsigned)g.W;
-    okmask = 0;
-#pragma unroll
-    for (int e = 0; e < kHaloMaxQ; ++e) {
-      const int ps = (int)((g.e_pass >> (4 * e)) & 15), ry = (int)((g.e_row >> (4 * e)) & 15);
-      const bool ok = e < g.nq && col_ok && ((chreal >> ps) & 1u) &&
-                      (unsigned)(iy0 + ry) < (unsigned)g.H;
-      const float *addr = ok ? p + g.goffE[e] : g.x;   // always valid
-      v[e] = *addr;
-      if (ok) okmask |= 1u << e;
-    }
-  }
-
-  __device__ __forceinline__ void store(const ConvGeom &g, float *region) const {
-#pragma unroll
-    for (int e = 0; e < kHaloMaxQ; ++e) {
-      const int ps = (int)((g.e_pass >> (4 * e)) & 15);
-      if (e < g.nq && rx_in && ((chlive >> ps) & 1u))
-        region[l_thread + g.loffE[e]] = ((okmask >> e) & 1u) ? v[e] : 0.f;
-    }
-  }
-};
-
-// LDS floats: two regions of (CH + 2) planes, the koff table, the row tables.
-__host__ __device__ inline int halo_region_floats(const ConvGeom &g) { return (g.CH + 2) * g.Rsz; }
+// LDS floats of one region: CH channel planes, the ones plane, the zero plane
+// and the dump slots.
+__host__ __device__ inline int halo_region_floats(const ConvGeom &g) {
+  return (g.CH + 2) * g.Rsz + kHaloDump;
+}
 
 // NKK = k-values per step / 2, a compile-time constant so that the MFMA loop is
 // fully unrolled and the per-lane k offsets live in registers.
-template <int WM, int NKK, bool SAME>
+//
+// Staging is branch-free per element: the input is read through a raw buffer
+// descriptor, and an element outside the image (zero padding, a channel past
+// the end of the input) gets bit 31 set in its byte offset, which puts it past
+// the descriptor's size so that the load returns 0 without touching memory.
+// Everything about an element that does not change from step to step (its
+// offset inside a sample, its LDS slot, whether its channel and column exist)
+// is computed once per workgroup and kept in registers.
+template <int WM, int NKK, bool SAME, bool MASK>
 __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int row0B,
-                                              long long sbeg, long long send, float *regA,
-                                              float *regB, const int *koff_tbl,
+                                              long long sbeg, long long send, float *smem,
+                                              int regA, int regB, const int *koff_tbl,
                                               floatx16 (&acc)[WM][WM]) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane & 31, lk = lane >> 5;
   const int khkw = g.kh * g.kw;
-  const int steps_per_sample = g.segs * g.rgroups;
+  const int HW = g.H * g.W;
 
   // operand row offsets of this lane (floats): plane of the row's channel + tap
   auto row_offset = [&](int row0, int r) {
@@ -139,54 +94,113 @@ __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int 
   int offA[WM], offB[WM];
 #pragma unroll
   for (int im = 0; im < WM; ++im) {
-    offA[im] = row_offset(row0A, (wm * WM + im) * 32 + lrow);
-    offB[im] = row_offset(row0B, (wn * WM + im) * 32 + lrow);
+    offA[im] = regA + row_offset(row0A, (wm * WM + im) * 32 + lrow);
+    offB[im] = (SAME ? regA : regB) + row_offset(row0B, (wn * WM + im) * 32 + lrow);
   }
-  const float *opB = SAME ? regA : regB;
   // per-lane k offsets (k = 2t + lk)
   int ko[NKK];
 #pragma unroll
   for (int t = 0; t < NKK; ++t) ko[t] = koff_tbl[2 * t + lk];
 
-  HaloPanel pa, pb;
-  pa.init(g, row0A);
-  if (!SAME) pb.init(g, row0B);
+  // ---- per-thread staging constants
+  const int c_loA = row0A / khkw, c_loB = row0B / khkw;
+  const int chq = tid / g.LPR;
+  const int rx = tid - chq * g.LPR;
+  int goff[kHaloMaxQ];   // byte offset of the element inside a sample, from channel c_lo
+  int loff[kHaloMaxQ];   // float offset of its LDS slot inside a region
+  unsigned tmaskA = 0, tmaskB = 0;
+  {
+    const int dump = (g.CH + 2) * g.Rsz + (tid & (kHaloDump - 1));
+    int ps = 0, ry = 0;
+#pragma unroll
+    for (int e = 0; e < kHaloMaxQ; ++e) {
+      const int ch = ps * g.CPP + chq;
+      const bool live = e < g.nq && rx < g.Win && ch < g.CH;
+      goff[e] = (ch * HW + ry * g.W + rx) * 4;
+      loff[e] = live ? ch * g.Rsz + ry * g.Wr + rx : dump;
+      if (live && c_loA + ch < g.C) tmaskA |= 1u << e;
+      if (live && c_loB + ch < g.C) tmaskB |= 1u << e;
+      if (++ry == g.Rin) { ry = 0; ++ps; }
+    }
+  }
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(g.x), (short)0, (int)g.x_bytes, 0x00020000);
 
-  auto decode = [&](long long s, long long &sample_base, int &iy0, int &ix0, int &orow0, int &ocol0) {
-    const long long smp = s / steps_per_sample;
-    const int rem = (int)(s - smp * steps_per_sample);
-    const int rg = rem / g.segs;
-    const int sg = rem - rg * g.segs;
-    orow0 = rg * g.RT;
-    ocol0 = sg * g.WS;
-    iy0 = orow0 * g.sy - g.ph;
-    ix0 = ocol0 * g.sx - g.pw;
-    sample_base = smp * (long long)g.C * g.H * g.W;
+  // ---- step state (uniform): position inside the sample and byte offset of the sample
+  const int steps_per_sample = g.segs * g.rgroups;
+  const long long smp0 = sbeg / steps_per_sample;
+  int rg, sg;
+  {
+    const int rem = (int)(sbeg - smp0 * steps_per_sample);
+    rg = rem / g.segs;
+    sg = rem - rg * g.segs;
+  }
+  int sample4 = (int)(smp0 * g.C * HW * 4);
+  const int sample_stride4 = g.C * HW * 4;
+
+  float va[kHaloMaxQ], vb[kHaloMaxQ];
+  auto issue = [&](float (&v)[kHaloMaxQ], unsigned tmask, int c_lo) {
+    const int iy0 = rg * g.RT * g.sy - g.ph, ix0 = sg * g.WS * g.sx - g.pw;
+    // rows of the region inside the image: [rlo, rhi)
+    const int rlo = iy0 < 0 ? -iy0 : 0;
+    int rhi = g.H - iy0;
+    if (rhi > g.Rin) rhi = g.Rin;
+    const unsigned rowbits = rhi > rlo ? (1u << rhi) - (1u << rlo) : 0u;
+    const unsigned emask = rowbits * g.rep;
+    const bool col_ok = (unsigned)(ix0 + rx) < (unsigned)g.W;
+    const unsigned ninv = col_ok ? ~(tmask & emask) : ~0u;
+    const int step4 = sample4 + (c_lo * HW + iy0 * g.W + ix0) * 4;
+#pragma unroll
+    for (int e0 = 0; e0 < kHaloMaxQ; e0 += 4) {
+      if (e0 < g.nq) {
+#pragma unroll
+        for (int e = e0; e < e0 + 4; ++e) {
+          const unsigned bad = ninv << (31 - e);
+          const unsigned voff = ((unsigned)(goff[e] + step4) & 0x7fffffffu) | (bad & 0x80000000u);
+          v[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff, 0, 0));
+        }
+      }
+    }
+  };
+  auto stash = [&](const float (&v)[kHaloMaxQ], int reg) {
+#pragma unroll
+    for (int e0 = 0; e0 < kHaloMaxQ; e0 += 4) {
+      if (e0 < g.nq) {
+#pragma unroll
+        for (int e = e0; e < e0 + 4; ++e) smem[reg + loff[e]] = v[e];
+      }
+    }
+  };
+  auto advance = [&]() {
+    if (++sg == g.segs) {
+      sg = 0;
+      if (++rg == g.rgroups) {
+        rg = 0;
+        sample4 += sample_stride4;
+      }
+    }
   };
 
-  long long sample_base;
-  int iy0, ix0, orow0, ocol0;
   if (sbeg < send) {
-    decode(sbeg, sample_base, iy0, ix0, orow0, ocol0);
-    pa.load(g, sample_base, iy0, ix0);
-    if (!SAME) pb.load(g, sample_base, iy0, ix0);
+    issue(va, tmaskA, c_loA);
+    if (!SAME) issue(vb, tmaskB, c_loB);
   }
   for (long long s = sbeg; s < send; ++s) {
-    pa.store(g, regA);
-    if (!SAME) pb.store(g, regB);
+    stash(va, regA);
+    if (!SAME) stash(vb, regB);
     // k-values at or past kcut lie below the image (row group hanging over the
     // bottom edge) or past the end of the step; their A operand is zeroed
-    int kcut = (g.ho - orow0) * g.WS;
+    int kcut = (g.ho - rg * g.RT) * g.WS;
     if (kcut > g.RT * g.WS) kcut = g.RT * g.WS;
     __syncthreads();
     if (s + 1 < send) {
-      decode(s + 1, sample_base, iy0, ix0, orow0, ocol0);
-      pa.load(g, sample_base, iy0, ix0);
-      if (!SAME) pb.load(g, sample_base, iy0, ix0);
+      advance();
+      issue(va, tmaskA, c_loA);
+      if (!SAME) issue(vb, tmaskB, c_loB);
     }
     // Opaque copies of the operand row offsets: without them the compiler
     // hoists all NKK * 2 * WM operand addresses out of the step loop and
-    // spills.  (Offsets, not pointers, so the reads stay LDS instructions.)
+    // spills.
     int qA[WM], qB[WM];
 #pragma unroll
     for (int im = 0; im < WM; ++im) {
@@ -194,21 +208,34 @@ __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int 
       qB[im] = offB[im];
       asm volatile("" : "+v"(qA[im]), "+v"(qB[im]));
     }
-#pragma unroll
-    for (int t = 0; t < NKK; ++t) {
-      float a[WM], b[WM];
+    // two-stage software pipeline: the operands of step t+1 are fetched from
+    // LDS before the MFMAs of step t issue
+    float a[2][WM], b[2][WM];
+    auto fetch_t = [&](int t, int buf) {
+      const bool kv = !MASK || lk < kcut - 2 * t;
 #pragma unroll
       for (int im = 0; im < WM; ++im) {
-        const float x = regA[qA[im] + ko[t]];
-        a[im] = (2 * t + lk < kcut) ? x : 0.f;
+        const float x = smem[qA[im] + ko[t]];
+        a[buf][im] = kv ? x : 0.f;
       }
 #pragma unroll
-      for (int in = 0; in < WM; ++in) b[in] = opB[qB[in] + ko[t]];
+      for (int in = 0; in < WM; ++in) b[buf][in] = smem[qB[in] + ko[t]];
+    };
+    fetch_t(0, 0);
+#pragma unroll
+    for (int t = 0; t < NKK; ++t) {
+      const int cur = t & 1;
+      if (t + 1 < NKK) fetch_t(t + 1, cur ^ 1);
+      // keep the scheduler from sinking those reads below the MFMAs (it does,
+      // to save three registers, and then every MFMA waits for its operand)
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int im = 0; im < WM; ++im)
 #pragma unroll
         for (int in = 0; in < WM; ++in)
-          acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+          acc[im][in] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][im], b[cur][in], acc[im][in], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
   }

@@ -221,7 +221,7 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
 
 // Convolution A factor through the LDS halo region (conv_halo.h); `klen` counts
 // reduction steps, not k-values.
-template <int WM, int NKK>
+template <int WM, int NKK, bool MASK>
 __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long long total_steps,
                                                                long long klen, int ntile,
                                                                int nsplit, int direct, int d,
@@ -232,16 +232,15 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
   constexpr int BM = 64 * WM;
   extern __shared__ float smem[];
   const int region = halo_region_floats(g);
-  float *regA = smem;
-  float *regB = smem + region;
+  const int regA = 0, regB = region;
   int *koff_tbl = reinterpret_cast<int *>(smem + 2 * region);
   int split, tile, I, J;
   work_decode(blockIdx.x, ntile * nsplit, ntile, (d + BM - 1) / BM, split, tile, I, J);
   // constant planes (ones, zeros) of both regions and the k -> offset table
   for (int e = threadIdx.x; e < 2 * g.Rsz; e += THREADS) {
     const float val = e < g.Rsz ? 1.f : 0.f;
-    regA[g.CH * g.Rsz + e] = val;
-    regB[g.CH * g.Rsz + e] = val;
+    smem[regA + g.CH * g.Rsz + e] = val;
+    smem[regB + g.CH * g.Rsz + e] = val;
   }
   for (int k = threadIdx.x; k < kHaloMaxK; k += THREADS) {
     int off = 0;
@@ -258,9 +257,9 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
   floatx16 acc[WM][WM];
   zero_acc<WM, WM>(acc);
   if (I == J)
-    halo_mainloop<WM, NKK, true>(g, I * BM, J * BM, sbeg, send, regA, regB, koff_tbl, acc);
+    halo_mainloop<WM, NKK, true, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc);
   else
-    halo_mainloop<WM, NKK, false>(g, I * BM, J * BM, sbeg, send, regA, regB, koff_tbl, acc);
+    halo_mainloop<WM, NKK, false, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc);
   if (direct) {
     write_tile<WM>(acc, smem, I, J, d, alpha, beta, C);
     return;
@@ -370,7 +369,7 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, 
 
 // Geometry of the LDS halo kernel for one convolution; false when the shape
 // does not fit its limits (the element-wise im2col loader is used instead).
-bool make_halo_geom(const float *x, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
+bool make_halo_geom(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
                     int pw, int ho, int wo, int append_ones, ConvGeom *out) {
   ConvGeom g;
   g.x = x;
@@ -408,21 +407,14 @@ bool make_halo_geom(const float *x, int c, int h, int w, int kh, int kw, int sy,
   g.CPP = THREADS / g.LPR;
   g.passes = kfac::ceil_div(g.CH, g.CPP);
   g.nq = g.passes * g.Rin;
-  if (g.nq > kHaloMaxQ || g.Rin > 15 || g.passes > 15) return false;
-  g.e_pass = 0;
-  g.e_row = 0;
-  for (int e = 0; e < 16; ++e) {
-    g.goffE[e] = 0;
-    g.loffE[e] = 0;
-  }
-  for (int e = 0; e < g.nq; ++e) {
-    const int ps = e / g.Rin, ry = e % g.Rin;
-    g.e_pass |= (unsigned long long)ps << (4 * e);
-    g.e_row |= (unsigned long long)ry << (4 * e);
-    g.goffE[e] = (ps * g.CPP * h + ry) * w;
-    g.loffE[e] = ps * g.CPP * g.Rsz + ry * g.Wr;
-  }
-  if ((g.CH + 2) * g.Rsz > 0xffff) return false;
+  if (g.nq > kHaloMaxQ) return false;
+  g.rep = 0;
+  for (int p = 0; p < g.passes; ++p) g.rep |= 1u << (p * g.Rin);
+  // the staging loads address x through a 32-bit byte offset whose top bit
+  // marks elements outside the image
+  const long long x_bytes = (long long)n * c * h * w * (long long)sizeof(float);
+  if (x_bytes >= (1ll << 31)) return false;
+  g.x_bytes = (unsigned)x_bytes;
   *out = g;
   return true;
 }
@@ -440,30 +432,32 @@ int run_conv_halo(const ConvGeom &g, int n, int d, float alpha, float beta, floa
   if (p.bm != 128) return 1;   // small factors stay on the generic kernel
   if (int rc = check_ws(p, ws, ws_bytes)) return rc;
   const size_t lds = halo_lds_bytes(g);
+  // the masked variants zero operands of k-values past the image's bottom edge
+  // or past the end of a step; most shapes do not need them
+  const bool mask = (g.RT * g.WS != g.nk) || (g.ho % g.RT != 0);
+  using Kern = void (*)(ConvGeom, long long, long long, int, int, int, int, float, float, float *,
+                        float *);
+  static const Kern kerns[3][2] = {
+      {syrk_conv_kernel<2, 25, false>, syrk_conv_kernel<2, 25, true>},
+      {syrk_conv_kernel<2, 28, false>, syrk_conv_kernel<2, 28, true>},
+      {syrk_conv_kernel<2, 32, false>, syrk_conv_kernel<2, 32, true>}};
   static bool attr_set = false;
   if (!attr_set) {
-    const void *fns[3] = {reinterpret_cast<const void *>(syrk_conv_kernel<2, 25>),
-                          reinterpret_cast<const void *>(syrk_conv_kernel<2, 28>),
-                          reinterpret_cast<const void *>(syrk_conv_kernel<2, 32>)};
-    for (const void *fn : fns)
-      KFAC_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         160 * 1024));
+    for (int i = 0; i < 3; ++i)
+      for (int j = 0; j < 2; ++j)
+        KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kerns[i][j]),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           160 * 1024));
     attr_set = true;
   }
   float *partial = static_cast<float *>(ws);
   const int direct = p.nsplit == 1 ? 1 : 0;
   const dim3 grid(p.ntile * p.nsplit), block(THREADS);
+  const Kern kern = kerns[g.nk == 50 ? 0 : (g.nk == 56 ? 1 : 2)][mask ? 1 : 0];
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
-    if (g.nk == 50)
-      hipLaunchKernelGGL((syrk_conv_kernel<2, 25>), grid, block, lds, stream, g, total_steps,
-                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
-    else if (g.nk == 56)
-      hipLaunchKernelGGL((syrk_conv_kernel<2, 28>), grid, block, lds, stream, g, total_steps,
-                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
-    else
-      hipLaunchKernelGGL((syrk_conv_kernel<2, 32>), grid, block, lds, stream, g, total_steps,
-                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, g, total_steps, p.klen, p.ntile, p.nsplit,
+                       direct, d, alpha, beta, partial, C);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (direct) return KFAC_OK;
@@ -599,7 +593,7 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
                     C, ws, ws_bytes, s);
   }
   ConvGeom geom;
-  if (make_halo_geom(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones, &geom)) {
+  if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones, &geom)) {
     const int rc = run_conv_halo(geom, n, d, alpha, beta, C, ws, ws_bytes, s);
     if (rc <= 0) return rc;   // 1 = shape left to the generic kernel
   }
