@@ -2,28 +2,41 @@
 // followed by the triangular inverse and L^-T L^-1 (potri), FP32 MFMA.
 //
 // All matrices of a batch advance together.  Each is copied (lower tiles
-// only) into a zero/identity padded workspace of NB x NB tiles (NB = 128) and
-// swept once, block column k = 0 .. T-1, with three launches per step that
-// cover every matrix that still has a block column k:
+// only) into a zero/identity padded workspace of NB x NB tiles (NB = 128),
+// stored tile by tile (tile (I,J) of a T x T grid is the contiguous 64 KB block
+// number I*T + J), so that every operand panel and every tile that is read and
+// written back is one dense block instead of 128 short rows a matrix row apart.
+// The strictly lower tiles end up holding L, the upper tiles U = L^-T (the
+// triangular inverse, stored transposed), the diagonal tiles U_kk = L_kk^-T.
+// With M(a,j) the tile in slot (a,j), every product of the sweep has one form,
 //
-//   diag(k)    one workgroup per matrix: Cholesky of the updated diagonal
-//              tile, its inverse W = L_kk^-1 and Z = W^T W (= A_kk^-1), all
-//              inside LDS on 32x32 MFMA blocks.
-//   panel(k)   L(m,k) = A(m,k) W^T                     (m > k)   "trsm"
-//              X^T(k,m) = -Z A(m,k)^T                  (m > k)   trtri seed
-//              U(n,k) = X^T(n,k) W^T                   (n < k)   trtri row finish
-//   update(k)  A(m,n) -= L(m,k) L(n,k)^T               (k < n <= m)  potrf
-//              X^T(n,m) -= U(n,k) L(m,k)^T             (n < k < m)   trtri
+//     C(a,b) -= sum_{j = j_lo .. j_hi} M(a,j) M(b,j)^T                   (*)
 //
-// The strictly lower tiles hold L, the upper tiles hold U = L^-T (the running
-// right-looking triangular inverse, stored transposed), so potrf and trtri
-// share one sweep and every product is a k-contiguous "NT" tile GEMM.  A final
-// launch forms  out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T  (lauum) and writes the
-// full symmetric inverse.  Tasks of a launch are found with one wave-uniform
-// binary search over per-step cumulative tables built once per plan.
+//   a >= b   potrf:  A(a,b) -= sum_j L(a,j) L(b,j)^T                (j < b)
+//   a <  b   trtri:  X^T(a,b) = -sum_j U(a,j) L(b,j)^T         (a <= j < b)
+//            followed by U(a,b) = X^T(a,b) L_bb^-T once the sum is complete,
+//
+// both k-contiguous "NT" tile GEMMs over row slabs of the workspace.  Block
+// columns are processed in groups of kGroup: inside a group the sweep is
+// left-looking (column k receives the products of the group's earlier columns
+// just before it is factored, K up to (kGroup-1)*NB), and after a group every
+// column to its right receives the whole group at once (K = kGroup*NB), which
+// reads and writes each trailing tile once per group instead of once per
+// column.  Per block column k:
+//
+//   column(k)  (*) for the tiles of column k, j over the group's columns < k
+//   diag(k)    one workgroup per matrix: Cholesky of the diagonal tile and
+//              its inverse W = L_kk^-1 inside LDS on 32x32 MFMA blocks
+//   panel(k)   M(x,k) = M(x,k) W^T for x != k  (L(x,k) below, U(x,k) above)
+//
+// and after the group's last column  trailing(g): (*) for all tiles right of
+// the group.  A final launch forms  out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T
+// (lauum) and writes the full symmetric inverse.  The tiles of every launch are
+// listed in a task table built once per plan.
 //
 // Replaces chainerkfac/optimizers/cholesky_inverse.py:16-102 (potrf + potrs
 // against the identity, one matrix at a time).
+#include <cstdlib>
 #include <algorithm>
 #include <numeric>
 
@@ -47,9 +60,9 @@ struct InvTables {
   const long long *ws_off;   // [count] float offset of the padded matrix
   const int *tile_cs;        // [count+1] cumulative lower-tile counts
   const int *panel_cs;       // [count+1] cumulative (nt-1)
-  const int *update_cs;      // flat per-step cumulative update-task counts
+  const int2 *tasks;         // update tasks of all launches: {slot, a | b << 16}
   float *ws;                 // padded matrices
-  float *side;               // per slot: W (NB*NB) then Z (NB*NB)
+  float *side;               // per slot: W (NB*NB)
   int *info;
 };
 
@@ -73,6 +86,40 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
   J = t - r * (r + 1) / 2;
 }
 
+__device__ __forceinline__ float *tile_ptr(const InvTables &tb, int s, int I, int J) {
+  return tb.ws + tb.ws_off[s] + ((long long)I * tb.nt[s] + J) * (NB * NB);
+}
+
+// Operand loader of the shared main loop for a run of consecutive tiles of one
+// tile row: k-value k is column k % NB of tile k / NB.  A 128 x 32 panel is
+// 128 rows of 128 contiguous bytes inside one tile; no edge masks are needed
+// (the workspace is padded).
+struct LoaderTile {
+  static constexpr bool kKRow = false;
+  struct Regs {
+    float4 v[NB / 32];
+  };
+  const float *base;   // first tile of the run
+  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long) const {
+    const unsigned k = (unsigned)k0 + (threadIdx.x & 7) * 4;
+    const float *p = base + (size_t)(k / NB) * (NB * NB) + (k % NB) + (threadIdx.x >> 3) * NB;
+#pragma unroll
+    for (int i = 0; i < NB / 32; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + 32 * i * NB);
+  }
+  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
+    const int kq = (threadIdx.x & 7) * 4;
+    const int rr = threadIdx.x >> 3;
+#pragma unroll
+    for (int i = 0; i < NB / 32; ++i) {
+      float *p = lds + (rr + 32 * i) * Panel<NB>::kRowKStride + kq;
+      p[0] = r.v[i].x;
+      p[1] = r.v[i].y;
+      p[2] = r.v[i].z;
+      p[3] = r.v[i].w;
+    }
+  }
+};
+
 // ---------------------------------------------------------------------------
 // copy-in: lower tiles of in -> padded workspace (identity on the padding)
 // ---------------------------------------------------------------------------
@@ -81,14 +128,14 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
   int I, J;
   tri_decode(blockIdx.x - tb.tile_cs[s], I, J);
   const int d = tb.dim[s];
-  const long long ld = (long long)tb.nt[s] * NB;
   const float *__restrict__ src = tb.in[s];
-  float *__restrict__ dst = tb.ws + tb.ws_off[s];
+  float *__restrict__ dst = tile_ptr(tb, s, I, J);
   const int c4 = (threadIdx.x & 31) * 4;
   const int r0 = threadIdx.x >> 5;
 #pragma unroll 4
   for (int p = 0; p < NB / 8; ++p) {
-    const int r = I * NB + r0 + 8 * p;
+    const int rl = r0 + 8 * p;
+    const int r = I * NB + rl;
     const int c = J * NB + c4;
     float v[4];
 #pragma unroll
@@ -98,7 +145,7 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
       if (r < d && ce < d) x = src[(long long)r * d + ce];
       v[e] = x;
     }
-    *reinterpret_cast<float4 *>(dst + (long long)r * ld + c) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4 *>(dst + rl * NB + c4) = make_float4(v[0], v[1], v[2], v[3]);
   }
 }
 
@@ -178,8 +225,8 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   float *scratch = smem + NB * LS;      // 4 waves x SB x LS
   const int s = blockIdx.x;
   const int d = tb.dim[s];
-  const long long ld = (long long)tb.nt[s] * NB;
-  float *tile = tb.ws + tb.ws_off[s] + (long long)k * NB * ld + (long long)k * NB;
+  constexpr int ld = NB;
+  float *tile = tile_ptr(tb, s, k, k);
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   {
@@ -187,7 +234,7 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
 #pragma unroll 4
     for (int p = 0; p < NB / 8; ++p) {
       const int r = r0 + 8 * p;
-      const float4 v = *reinterpret_cast<const float4 *>(tile + (long long)r * ld + c4);
+      const float4 v = *reinterpret_cast<const float4 *>(tile + r * ld + c4);
       S[r * LS + c4 + 0] = v.x;
       S[r * LS + c4 + 1] = v.y;
       S[r * LS + c4 + 2] = v.z;
@@ -250,8 +297,7 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   }
 
   // ---- outputs
-  float *Wg = tb.side + (long long)s * 2 * NB * NB;
-  float *Zg = Wg + NB * NB;
+  float *Wg = tb.side + (long long)s * NB * NB;
   {
     // U -> diagonal tile of the workspace (zeros below the diagonal);
     // W = U^T -> side buffer (zeros above the diagonal)
@@ -260,108 +306,59 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
     for (int p = 0; p < NB / 2; ++p) {
       const int r = r0 + 2 * p;
       const bool up = (c / SB > r / SB) || (c / SB == r / SB && c >= r);
-      tile[(long long)r * ld + c] = up ? S[r * LS + c] : 0.f;
+      tile[r * ld + c] = up ? S[r * LS + c] : 0.f;
       const bool lo = (r / SB > c / SB) || (c / SB == r / SB && r >= c);
       Wg[r * NB + c] = lo ? S[c * LS + r] : 0.f;
     }
-  }
-  // Z = U U^T on lower blocks, mirrored
-  for (int t = wave; t < 10; t += 4) {
-    int bi, bj;
-    tri_decode(t, bi, bj);
-    const floatx16 z = wave_gemm<false>(S + (bi * SB) * LS + bi * SB,
-                                        S + (bj * SB) * LS + bi * SB, NB - bi * SB, zero);
-    wave_visit(z, [&](int r, int c, float v) {
-      Zg[(bi * SB + r) * NB + bj * SB + c] = v;
-      if (bi != bj) Zg[(bj * SB + c) * NB + bi * SB + r] = v;
-    });
   }
 }
 
 // ---------------------------------------------------------------------------
 // panel and update: 128x128x128 tile products through the shared main loop
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ LoaderKC<NB, true> tile_loader(const float *base, long long ld) {
-  LoaderKC<NB, true> l;
-  l.base = base;
-  l.sample_stride = 0;
-  l.row_stride = (unsigned)ld;
-  l.L = NB;
-  l.rows_valid = NB;
-  l.ones_row = -1;
-  l.init(nullptr, 0);
-  return l;
-}
-
+// M(x,k) = M(x,k) W^T in place for every x != k.
 __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, int nactive) {
   __shared__ float ldsA[Panel<NB>::kFloats];
   __shared__ float ldsB[Panel<NB>::kFloats];
   const int s = find_slot(tb.panel_cs, nactive, blockIdx.x);
   const int local = blockIdx.x - tb.panel_cs[s];
-  const int T = tb.nt[s];
-  const long long ld = (long long)T * NB;
-  float *M = tb.ws + tb.ws_off[s];
-  const float *Wg = tb.side + (long long)s * 2 * NB * NB;
-  const float *Zg = Wg + NB * NB;
-  const int r = T - k - 1;
+  const int x = local < k ? local : local + 1;
+  float *tile = tile_ptr(tb, s, x, k);
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
-  if (local < r) {
-    const int m = k + 1 + local;
-    float *Amk = M + (long long)m * NB * ld + (long long)k * NB;   // lower slot (m,k)
-    float *Xkm = M + (long long)k * NB * ld + (long long)m * NB;   // upper slot (k,m)
-    // X^T(k,m) = -Z A(m,k)^T
-    mainloop<2, 2, false>(tile_loader(Zg, NB), tile_loader(Amk, ld), 0, 0, 0, NB, ldsA, ldsB, acc);
-    for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { Xkm[(long long)rr * ld + cc] = -v; });
-    // L(m,k) = A(m,k) W^T, in place
-    zero_acc<2, 2>(acc);
-    mainloop<2, 2, false>(tile_loader(Amk, ld), tile_loader(Wg, NB), 0, 0, 0, NB, ldsA, ldsB, acc);
-    for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { Amk[(long long)rr * ld + cc] = v; });
-  } else {
-    const int n = local - r;
-    float *Unk = M + (long long)n * NB * ld + (long long)k * NB;   // upper slot (n,k)
-    // U(n,k) = X^T(n,k) W^T, in place
-    mainloop<2, 2, false>(tile_loader(Unk, ld), tile_loader(Wg, NB), 0, 0, 0, NB, ldsA, ldsB, acc);
-    for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { Unk[(long long)rr * ld + cc] = v; });
-  }
+  mainloop<2, 2, false>(LoaderTile{tile}, LoaderTile{tb.side + (long long)s * NB * NB}, 0, 0, 0, NB,
+                        ldsA, ldsB, acc);
+  for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { tile[rr * NB + cc] = v; });
 }
 
-__global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int k, int nactive,
-                                                            int cs_off) {
+// One task of (*): tile (a,b) of matrix `slot`, products over the block
+// columns [k0, k1] clipped to the tile's own range.  The accumulators start
+// from -C, so the tile is read while the first operand panels are in flight and
+// the epilogue is a plain store.  An upper tile whose row lies inside [k0, k1]
+// receives its first product here and is overwritten (it holds stale data).
+__global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0, int k0, int k1) {
   __shared__ float ldsA[Panel<NB>::kFloats];
   __shared__ float ldsB[Panel<NB>::kFloats];
-  const int *cs = tb.update_cs + cs_off;
-  const int s = find_slot(cs, nactive, blockIdx.x);
-  const int local = blockIdx.x - cs[s];
-  const int T = tb.nt[s];
-  const long long ld = (long long)T * NB;
-  float *M = tb.ws + tb.ws_off[s];
-  const int r = T - k - 1;
-  const int ntri = r * (r + 1) / 2;
+  const int2 task = tb.tasks[task0 + blockIdx.x];
+  const int s = task.x;
+  const int a = task.y & 0xffff, b = task.y >> 16;
+  const bool upper = a < b;
+  const int j_lo = upper && a > k0 ? a : k0;
+  const int j_hi = upper && b - 1 < k1 ? b - 1 : k1;
+  const int K = (j_hi - j_lo + 1) * NB;
+  const bool first = upper && a >= k0;
+  float *C = tile_ptr(tb, s, a, b);
   floatx16 acc[2][2];
-  zero_acc<2, 2>(acc);
-  float *C;
-  if (local < ntri) {
-    int a, b;
-    tri_decode(local, a, b);
-    const int m = k + 1 + a, n = k + 1 + b;
-    const float *Lm = M + (long long)m * NB * ld + (long long)k * NB;
-    const float *Ln = M + (long long)n * NB * ld + (long long)k * NB;
-    C = M + (long long)m * NB * ld + (long long)n * NB;
-    if (m == n)
-      mainloop<2, 2, true>(tile_loader(Lm, ld), tile_loader(Ln, ld), 0, 0, 0, NB, ldsA, ldsB, acc);
-    else
-      mainloop<2, 2, false>(tile_loader(Lm, ld), tile_loader(Ln, ld), 0, 0, 0, NB, ldsA, ldsB, acc);
-  } else {
-    const int q = local - ntri;
-    const int a = q / k, n = q - a * k;
-    const int m = k + 1 + a;
-    const float *Unk = M + (long long)n * NB * ld + (long long)k * NB;
-    const float *Lm = M + (long long)m * NB * ld + (long long)k * NB;
-    C = M + (long long)n * NB * ld + (long long)m * NB;  // upper slot (n,m)
-    mainloop<2, 2, false>(tile_loader(Unk, ld), tile_loader(Lm, ld), 0, 0, 0, NB, ldsA, ldsB, acc);
-  }
-  for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[(long long)rr * ld + cc] -= v; });
+  if (first)
+    zero_acc<2, 2>(acc);
+  else
+    fill_acc<2, 2>(acc, [&](int rr, int cc) { return -C[rr * NB + cc]; });
+  const LoaderTile la{tile_ptr(tb, s, a, j_lo)}, lb{tile_ptr(tb, s, b, j_lo)};
+  if (a == b)
+    mainloop<2, 2, true>(la, lb, 0, 0, 0, K, ldsA, ldsB, acc);
+  else
+    mainloop<2, 2, false>(la, lb, 0, 0, 0, K, ldsA, ldsB, acc);
+  for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[rr * NB + cc] = -v; });
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
@@ -373,13 +370,8 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int cou
   tri_decode(blockIdx.x - tb.tile_cs[s], I, J);
   const int T = tb.nt[s];
   const int d = tb.dim[s];
-  const long long ld = (long long)T * NB;
-  const float *M = tb.ws + tb.ws_off[s];
   const int K = (T - I) * NB;
-  LoaderKC<NB, true> la = tile_loader(M + (long long)I * NB * ld + (long long)I * NB, ld);
-  LoaderKC<NB, true> lb = tile_loader(M + (long long)J * NB * ld + (long long)I * NB, ld);
-  la.L = K;
-  lb.L = K;
+  const LoaderTile la{tile_ptr(tb, s, I, I)}, lb{tile_ptr(tb, s, J, I)};
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
   if (I == J)
@@ -400,22 +392,62 @@ constexpr size_t kDiagLds = (size_t)(NB * LS + 4 * SB * LS) * sizeof(float);
 
 }  // namespace
 
+struct UpdateLaunch {
+  int task0 = 0, count = 0;   // range in the task table
+  int k0 = 0, k1 = 0;         // block columns whose products are applied
+};
+
 struct kfac_inverse_plan {
   int count = 0;
   int max_t = 0;
+  int group = 4;                   // block columns per trailing update
   std::vector<int> order;          // slot -> caller index
   std::vector<int> nt;             // per slot
   std::vector<int> nactive;        // per step
   std::vector<int> panel_total;    // per step
-  std::vector<int> update_total;   // per step
-  std::vector<int> update_off;     // per step offset into update_cs
+  std::vector<UpdateLaunch> column;    // per step: left-looking update of column k
+  // per step, set on the last column of a group: the tiles of the next group's
+  // columns ("urgent") and everything right of them ("rest")
+  std::vector<UpdateLaunch> urgent, rest;
+  // The rest of a trailing update touches nothing the next group's sweep needs,
+  // so it runs on a second stream beside that sweep.
+  bool lookahead = true;
+  hipStream_t side = nullptr;
+  std::vector<hipEvent_t> ev_main, ev_side;   // per group
+  ~kfac_inverse_plan() {
+    for (hipEvent_t e : ev_main) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ev_side) (void)hipEventDestroy(e);
+    if (side) (void)hipStreamDestroy(side);
+  }
   int total_tiles = 0;
   size_t ws_floats = 0;            // padded matrices
   size_t side_floats = 0;
   std::vector<const void *> in_sorted, out_sorted;
-  kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_off, d_tile, d_panel, d_update;
+  kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_off, d_tile, d_panel, d_tasks;
   bool attr_set = false;
 };
+
+namespace {
+
+// Workgroup i of a launch runs on XCD i % 8.  Deal the tasks out so that each
+// XCD receives one contiguous run of the natural order (neighbouring tasks
+// share operand row slabs, which then stay in that XCD's L2).
+void append_tasks(std::vector<int2> &table, const std::vector<int2> &natural) {
+  const size_t n = natural.size();
+  const size_t chunk = (n + 7) / 8;
+  std::vector<int2> dealt;
+  dealt.reserve(n);
+  // position p of XCD x holds natural[x * chunk + p]; emit in launch order
+  // (p major, x minor) and skip the holes of a ragged last chunk
+  for (size_t p = 0; p < chunk; ++p)
+    for (size_t x = 0; x < 8; ++x) {
+      const size_t i = x * chunk + p;
+      if (i < n) dealt.push_back(natural[i]);
+    }
+  table.insert(table.end(), dealt.begin(), dealt.end());
+}
+
+}  // namespace
 
 extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
                                         kfac_inverse_plan_t *plan_out) {
@@ -427,6 +459,10 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     KFAC_REQUIRE(dims[i] > 0 && dims[i] <= 46340, "matrix %d: bad dimension %d", i, dims[i]);
   auto *p = new (std::nothrow) kfac_inverse_plan;
   if (!p) return kfac::fail(KFAC_ENOMEM, "out of host memory");
+  if (const char *e = getenv("KFAC_INVERSE_GROUP")) {   // tuning override
+    const int g = atoi(e);
+    if (g >= 1 && g <= 64) p->group = g;
+  }
   p->count = count;
   p->order.resize(count);
   std::iota(p->order.begin(), p->order.end(), 0);
@@ -446,26 +482,65 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     panel_cs[s + 1] = panel_cs[s] + (T - 1);
   }
   p->ws_floats = total;
-  p->side_floats = (size_t)count * 2 * NB * NB;
+  p->side_floats = (size_t)count * NB * NB;
   p->total_tiles = tile_cs[count];
   p->max_t = count ? p->nt[0] : 0;
-  std::vector<int> update_cs;
+  std::vector<int2> tasks, natural;
+  p->column.resize(p->max_t);
+  p->urgent.resize(p->max_t);
+  p->rest.resize(p->max_t);
+  if (const char *e = getenv("KFAC_INVERSE_LOOKAHEAD")) p->lookahead = atoi(e) != 0;
+  auto pack = [](int s, int a, int b) { return make_int2(s, a | (b << 16)); };
   for (int k = 0; k < p->max_t; ++k) {
     int na = 0;
     while (na < count && p->nt[na] > k) ++na;
     p->nactive.push_back(na);
     p->panel_total.push_back(panel_cs[na]);
-    p->update_off.push_back((int)update_cs.size());
-    int run = 0;
-    update_cs.push_back(0);
-    for (int s = 0; s < na; ++s) {
-      const int r = p->nt[s] - k - 1;
-      run += r * (r + 1) / 2 + r * k;
-      update_cs.push_back(run);
+    const int k0 = k / p->group * p->group;
+    const int k1 = std::min(k0 + p->group - 1, p->max_t - 1);
+    if (k > k0) {
+      // column k of every active matrix: products of columns k0 .. k-1
+      natural.clear();
+      for (int s = 0; s < na; ++s) {
+        for (int m = k; m < p->nt[s]; ++m) natural.push_back(pack(s, m, k));
+        for (int a = 0; a < k; ++a) natural.push_back(pack(s, a, k));
+      }
+      p->column[k].task0 = (int)tasks.size();
+      p->column[k].count = (int)natural.size();
+      p->column[k].k0 = k0;
+      p->column[k].k1 = k - 1;
+      append_tasks(tasks, natural);
     }
-    p->update_total.push_back(run);
+    if (k == k1) {
+      // every column right of the group: products of columns k0 .. k1, split at
+      // the end of the next group; the upper tiles whose row lies inside the
+      // group have shorter sums and go last
+      const int ku = k1 + p->group;   // last urgent column
+      for (int part = 0; part < 2; ++part) {
+        natural.clear();
+        std::vector<int2> tail;
+        for (int s = 0; s < count && p->nt[s] > k1 + 1; ++s) {
+          const int T = p->nt[s];
+          const int c_lo = part == 0 ? k1 + 1 : ku + 1;
+          const int c_hi = part == 0 ? std::min(ku, T - 1) : T - 1;
+          for (int n = c_lo; n <= c_hi; ++n)
+            for (int m = n; m < T; ++m) natural.push_back(pack(s, m, n));
+          for (int a = 0; a < k0; ++a)
+            for (int b = c_lo; b <= c_hi; ++b) natural.push_back(pack(s, a, b));
+          for (int a = k0; a <= k1; ++a)
+            for (int b = c_lo; b <= c_hi; ++b) tail.push_back(pack(s, a, b));
+        }
+        UpdateLaunch &u = part == 0 ? p->urgent[k] : p->rest[k];
+        u.task0 = (int)tasks.size();
+        u.count = (int)(natural.size() + tail.size());
+        u.k0 = k0;
+        u.k1 = k1;
+        append_tasks(tasks, natural);
+        append_tasks(tasks, tail);
+      }
+    }
   }
-  if (update_cs.empty()) update_cs.push_back(0);
+  if (tasks.empty()) tasks.push_back(make_int2(0, 0));
   int rc = KFAC_OK;
   auto up = [&](kfac::DevTable &t, const void *h, size_t b) {
     if (rc == KFAC_OK) rc = t.set(h, b, nullptr);
@@ -476,7 +551,21 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_off, off.data(), sizeof(long long) * count);
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
   up(p->d_panel, panel_cs.data(), sizeof(int) * (count + 1));
-  up(p->d_update, update_cs.data(), sizeof(int) * update_cs.size());
+  up(p->d_tasks, tasks.data(), sizeof(int2) * tasks.size());
+  if (rc == KFAC_OK && p->lookahead && p->max_t > p->group) {
+    const int groups = kfac::ceil_div(p->max_t, p->group);
+    bool ok = hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess;
+    for (int g = 0; ok && g < groups; ++g) {
+      hipEvent_t a = nullptr, b = nullptr;
+      ok = hipEventCreateWithFlags(&a, hipEventDisableTiming) == hipSuccess;
+      if (ok) p->ev_main.push_back(a);
+      ok = ok && hipEventCreateWithFlags(&b, hipEventDisableTiming) == hipSuccess;
+      if (ok && b) p->ev_side.push_back(b);
+    }
+    if (!ok) rc = kfac::fail(KFAC_EHIP, "cannot create the look-ahead stream or its events");
+  } else {
+    p->lookahead = false;
+  }
   if (rc != KFAC_OK) {
     delete p;
     return rc;
@@ -536,7 +625,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.ws_off = plan->d_off.as<const long long>();
   tb.tile_cs = plan->d_tile.as<const int>();
   tb.panel_cs = plan->d_panel.as<const int>();
-  tb.update_cs = plan->d_update.as<const int>();
+  tb.tasks = plan->d_tasks.as<const int2>();
   uintptr_t base = (reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255;
   tb.ws = reinterpret_cast<float *>(base);
   tb.side = tb.ws + plan->ws_floats;
@@ -544,17 +633,36 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
 
   hipLaunchKernelGGL(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
   KFAC_HIP_CHECK(hipGetLastError());
+  auto update = [&](const UpdateLaunch &u, hipStream_t st) {
+    if (u.count == 0) return;
+    kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
+    hipLaunchKernelGGL(update_kernel, dim3(u.count), dim3(THREADS), 0, st, tb, u.task0, u.k0, u.k1);
+  };
+  int pending = -1;   // group whose rest is still running on the side stream
   for (int k = 0; k < plan->max_t; ++k) {
     const int na = plan->nactive[k];
+    update(plan->column[k], s);
     hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(256), kDiagLds, s, tb, k);
     if (plan->panel_total[k] > 0)
       hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), 0, s, tb, k, na);
-    if (plan->update_total[k] > 0) {
-      kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, s);
-      hipLaunchKernelGGL(update_kernel, dim3(plan->update_total[k]), dim3(THREADS), 0, s, tb, k,
-                         na, plan->update_off[k]);
+    if (plan->urgent[k].count == 0) continue;
+    // the urgent tiles were also targets of the previous group's rest
+    if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
+    pending = -1;
+    update(plan->urgent[k], s);
+    if (plan->rest[k].count == 0) continue;
+    if (!plan->lookahead) {
+      update(plan->rest[k], s);
+      continue;
     }
+    const int g = k / plan->group;
+    KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[g], s));
+    KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_main[g], 0));
+    update(plan->rest[k], plan->side);
+    KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[g], plan->side));
+    pending = g;
   }
+  if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
   KFAC_HIP_CHECK(hipGetLastError());
   {
     kfac::TimedLaunch timed(KFAC_TIMED_INV_LAUUM, s);

@@ -395,6 +395,25 @@ __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, 
   }
 }
 
+// Set every accumulator element of this lane to f(row, col), row / col relative
+// to the workgroup tile.
+template <int WM, int WN, class F>
+__device__ __forceinline__ void fill_acc(floatx16 (&acc)[WM][WN], F f) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int im = 0; im < WM; ++im)
+#pragma unroll
+    for (int in = 0; in < WN; ++in)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = (wm * WM + im) * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int col = (wn * WN + in) * 32 + (lane & 31);
+        acc[im][in][v] = f(row, col);
+      }
+}
+
 // Visit every accumulator element of this lane: f(row, col, value) with row /
 // col relative to the workgroup tile.
 template <int WM, int WN, class F>
