@@ -26,8 +26,8 @@
 //
 //   column(k)  (*) for the tiles of column k, j over the group's columns < k
 //   diag(k)    one workgroup per matrix: Cholesky of the diagonal tile and
-//              its inverse W = L_kk^-1 inside LDS on 32x32 MFMA blocks
-//   panel(k)   M(x,k) = M(x,k) W^T for x != k  (L(x,k) below, U(x,k) above)
+//              U_kk = L_kk^-T inside LDS on 32x32 MFMA blocks
+//   panel(k)   M(x,k) = M(x,k) U_kk for x != k  (L(x,k) below, U(x,k) above)
 //
 // and after the group's last column  trailing(g): (*) for all tiles right of
 // the group.  A final launch forms  out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T
@@ -62,7 +62,6 @@ struct InvTables {
   const int *panel_cs;       // [count+1] cumulative (nt-1)
   const int2 *tasks;         // update tasks of all launches: {slot, a | b << 16}
   float *ws;                 // padded matrices
-  float *side;               // per slot: W (NB*NB)
   int *info;
 };
 
@@ -120,6 +119,28 @@ struct LoaderTile {
   }
 };
 
+// The same tile read as its transpose: operand row c, k-value q is element
+// (q, c).  Rows of the tile are contiguous in c, so the panel goes to LDS in the
+// k-major layout.
+struct LoaderTileT {
+  static constexpr bool kKRow = true;
+  struct Regs {
+    float4 v[KT / 8];
+  };
+  const float *base;
+  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long) const {
+    const float *p = base + ((int)k0 + (threadIdx.x >> 5)) * NB + (threadIdx.x & 31) * 4;
+#pragma unroll
+    for (int i = 0; i < KT / 8; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + 8 * i * NB);
+  }
+  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
+    float *p = lds + (threadIdx.x >> 5) * Panel<NB>::kKRowStride + (threadIdx.x & 31) * 4;
+#pragma unroll
+    for (int i = 0; i < KT / 8; ++i)
+      *reinterpret_cast<float4 *>(p + 8 * i * Panel<NB>::kKRowStride) = r.v[i];
+  }
+};
+
 // ---------------------------------------------------------------------------
 // copy-in: lower tiles of in -> padded workspace (identity on the padding)
 // ---------------------------------------------------------------------------
@@ -150,7 +171,7 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
 }
 
 // ---------------------------------------------------------------------------
-// diagonal tile: Cholesky + inverse + Z inside LDS
+// diagonal tile: Cholesky + triangular inverse inside LDS
 // ---------------------------------------------------------------------------
 
 // acc += A(32 x K) * B^T, A at a[row*LS + k]; B at b[row*LS + k] or, when BT,
@@ -179,42 +200,41 @@ __device__ __forceinline__ float lane_bcast(float x, int lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), lane));
 }
 
-// Wave 0: factor the 32x32 block at S[b0.., b0..] (lower) in registers, then
-// overwrite the block with U32 = (L32^-1)^T (upper triangular, zeros below).
+// Wave 0: factor the 32x32 block at S[b0.., b0..] (lower) in registers and
+// overwrite it with U32 = (L32^-1)^T (upper triangular, zeros below).
+//
+// Lanes 0..31 hold the rows of A, lanes 32..63 the columns of the identity: the
+// column operations of the right-looking Cholesky (scale column j by
+// 1/sqrt(pivot), subtract l_cj times it from column c) turn the first into L
+// and, applied to the identity with the same multipliers, are exactly the
+// forward substitution that turns the second into the columns of L^-1.  One
+// broadcast of l_cj feeds both halves in the same instruction.
 // Returns 0 or 1 + the local index of the first non-positive pivot.
 __device__ __forceinline__ int chol_inv_32(float *S, int b0) {
   const int lane = threadIdx.x & 63;
   const int i = lane & 31;
-  float a[SB];
+  const bool chol = lane < SB;
+  float x[SB];
 #pragma unroll
-  for (int c = 0; c < SB; ++c) a[c] = S[(b0 + i) * LS + b0 + c];
+  for (int c = 0; c < SB; ++c) {
+    const float a = S[(b0 + i) * LS + b0 + c];
+    x[c] = chol ? a : (c == i ? 1.f : 0.f);
+  }
   int bad = 0;
 #pragma unroll
   for (int j = 0; j < SB; ++j) {
-    const float piv = lane_bcast(a[j], j);
+    const float piv = lane_bcast(x[j], j);
     if (!(piv > 0.f) && bad == 0) bad = j + 1;
-    const float root = sqrtf(piv);
-    const float rinv = 1.0f / root;
-    a[j] = (i == j) ? root : a[j] * rinv;
+    float rinv = __builtin_amdgcn_rsqf(piv);
+    rinv = rinv * (1.5f - 0.5f * piv * rinv * rinv);   // one Newton step on the hardware estimate
+    x[j] *= rinv;
 #pragma unroll
-    for (int c = j + 1; c < SB; ++c) {
-      const float lcj = lane_bcast(a[j], c);
-      a[c] -= a[j] * lcj;
-    }
+    for (int c = j + 1; c < SB; ++c) x[c] -= x[j] * lane_bcast(x[j], c);
   }
-  // lane c solves L w = e_c: w[i] = (delta_ic - sum_{k<i} l_ik w_k) / l_ii
-  float w[SB];
+  // lane 32 + m holds column m of W = row m of U; entries with r < m are exact zeros
+  if (!chol) {
 #pragma unroll
-  for (int r = 0; r < SB; ++r) {
-    float s = (r == i) ? 1.f : 0.f;
-#pragma unroll
-    for (int k = 0; k < r; ++k) s -= lane_bcast(a[k], r) * w[k];
-    w[r] = s / lane_bcast(a[r], r);
-  }
-  // lane c holds column c of W = row c of U; entries with r < c are exact zeros
-  if (lane < SB) {
-#pragma unroll
-    for (int r = 0; r < SB; ++r) S[(b0 + i) * LS + b0 + r] = w[r];
+    for (int r = 0; r < SB; ++r) S[(b0 + i) * LS + b0 + r] = x[r];
   }
   return bad;
 }
@@ -297,18 +317,20 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   }
 
   // ---- outputs
-  float *Wg = tb.side + (long long)s * NB * NB;
+  // U -> diagonal tile of the workspace, exact zeros below the diagonal
   {
-    // U -> diagonal tile of the workspace (zeros below the diagonal);
-    // W = U^T -> side buffer (zeros above the diagonal)
-    const int c = threadIdx.x & 127;
-    const int r0 = threadIdx.x >> 7;
-    for (int p = 0; p < NB / 2; ++p) {
-      const int r = r0 + 2 * p;
-      const bool up = (c / SB > r / SB) || (c / SB == r / SB && c >= r);
-      tile[r * ld + c] = up ? S[r * LS + c] : 0.f;
-      const bool lo = (r / SB > c / SB) || (c / SB == r / SB && r >= c);
-      Wg[r * NB + c] = lo ? S[c * LS + r] : 0.f;
+    const int c4 = (threadIdx.x & 31) * 4, r0 = threadIdx.x >> 5;
+#pragma unroll 4
+    for (int p = 0; p < NB / 8; ++p) {
+      const int r = r0 + 8 * p;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int c = c4 + e;
+        const bool up = (c / SB > r / SB) || (c / SB == r / SB && c >= r);
+        v[e] = up ? S[r * LS + c] : 0.f;
+      }
+      *reinterpret_cast<float4 *>(tile + r * ld + c4) = make_float4(v[0], v[1], v[2], v[3]);
     }
   }
 }
@@ -316,7 +338,8 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
 // ---------------------------------------------------------------------------
 // panel and update: 128x128x128 tile products through the shared main loop
 // ---------------------------------------------------------------------------
-// M(x,k) = M(x,k) W^T in place for every x != k.
+// M(x,k) = M(x,k) W^T = M(x,k) U_kk in place for every x != k; the operand
+// W^T is the diagonal tile itself, read transposed.
 __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, int nactive) {
   __shared__ float ldsA[Panel<NB>::kFloats];
   __shared__ float ldsB[Panel<NB>::kFloats];
@@ -326,8 +349,8 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, 
   float *tile = tile_ptr(tb, s, x, k);
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
-  mainloop<2, 2, false>(LoaderTile{tile}, LoaderTile{tb.side + (long long)s * NB * NB}, 0, 0, 0, NB,
-                        ldsA, ldsB, acc);
+  mainloop<2, 2, false>(LoaderTile{tile}, LoaderTileT{tile_ptr(tb, s, k, k)}, 0, 0, 0, NB, ldsA,
+                        ldsB, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { tile[rr * NB + cc] = v; });
 }
 
@@ -421,7 +444,6 @@ struct kfac_inverse_plan {
   }
   int total_tiles = 0;
   size_t ws_floats = 0;            // padded matrices
-  size_t side_floats = 0;
   std::vector<const void *> in_sorted, out_sorted;
   kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_off, d_tile, d_panel, d_tasks;
   bool attr_set = false;
@@ -482,7 +504,6 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     panel_cs[s + 1] = panel_cs[s] + (T - 1);
   }
   p->ws_floats = total;
-  p->side_floats = (size_t)count * NB * NB;
   p->total_tiles = tile_cs[count];
   p->max_t = count ? p->nt[0] : 0;
   std::vector<int2> tasks, natural;
@@ -576,7 +597,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
 
 extern "C" size_t kfac_inverse_plan_workspace_bytes(kfac_inverse_plan_t plan) {
   if (!plan) return 0;
-  return (plan->ws_floats + plan->side_floats) * sizeof(float) + 256;
+  return plan->ws_floats * sizeof(float) + 256;
 }
 
 extern "C" int kfac_inverse_plan_destroy(kfac_inverse_plan_t plan) {
@@ -628,7 +649,6 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.tasks = plan->d_tasks.as<const int2>();
   uintptr_t base = (reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255;
   tb.ws = reinterpret_cast<float *>(base);
-  tb.side = tb.ws + plan->ws_floats;
   tb.info = info_dev;
 
   hipLaunchKernelGGL(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
