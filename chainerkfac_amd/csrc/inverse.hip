@@ -50,6 +50,7 @@ using namespace kfac::mma;
 constexpr int NB = 128;
 constexpr int SB = 32;
 constexpr int LS = NB + 1;  // LDS row stride of the diagonal-tile kernel
+constexpr int PS = SB + 1;  // row stride of a wave's private 32x32 block
 
 struct InvTables {
   const float *const *in;    // [count] sorted slot -> input matrix
@@ -174,15 +175,15 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
 // diagonal tile: Cholesky + triangular inverse inside LDS
 // ---------------------------------------------------------------------------
 
-// acc += A(32 x K) * B^T, A at a[row*LS + k]; B at b[row*LS + k] or, when BT,
+// acc += A(32 x K) * B^T, A at a[row*AS + k]; B at b[row*LS + k] or, when BT,
 // at b[k*LS + row].
-template <bool BT>
+template <bool BT, int AS = LS>
 __device__ __forceinline__ floatx16 wave_gemm(const float *a, const float *b, int K,
                                               floatx16 acc) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
   for (int k = 0; k < K; k += 2) {
-    const float av = a[r * LS + k + h];
+    const float av = a[r * AS + k + h];
     const float bv = BT ? b[(k + h) * LS + r] : b[r * LS + k + h];
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
   }
@@ -242,7 +243,7 @@ __device__ __forceinline__ int chol_inv_32(float *S, int b0) {
 __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   extern __shared__ float smem[];
   float *S = smem;                      // NB x LS working tile
-  float *scratch = smem + NB * LS;      // 4 waves x SB x LS
+  float *scratch = smem + NB * LS;      // 4 waves x SB x PS
   const int s = blockIdx.x;
   const int d = tb.dim[s];
   constexpr int ld = NB;
@@ -300,16 +301,16 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   }
 
   // ---- trtri: U(jb,ib) = -[sum_kb U(jb,kb) L(ib,kb)^T] U32(ib), by distance
-  float *P = scratch + wave * SB * LS;
+  float *P = scratch + wave * SB * PS;
   for (int dd = 1; dd < NB / SB; ++dd) {
     for (int jb = wave; jb + dd < NB / SB; jb += 4) {
       const int ib = jb + dd;
       const floatx16 p = wave_gemm<false>(S + (jb * SB) * LS + jb * SB,
                                           S + (ib * SB) * LS + jb * SB, dd * SB, zero);
-      wave_visit(p, [&](int r, int c, float v) { P[r * LS + c] = v; });
+      wave_visit(p, [&](int r, int c, float v) { P[r * PS + c] = v; });
       // the same wave re-reads P: LDS accesses of one wave execute in order
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      const floatx16 u = wave_gemm<true>(P, S + (ib * SB) * LS + ib * SB, SB, zero);
+      const floatx16 u = wave_gemm<true, PS>(P, S + (ib * SB) * LS + ib * SB, SB, zero);
       float *blk = S + (jb * SB) * LS + ib * SB;
       wave_visit(u, [&](int r, int c, float v) { blk[r * LS + c] = -v; });
     }
@@ -411,7 +412,10 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int cou
   });
 }
 
-constexpr size_t kDiagLds = (size_t)(NB * LS + 4 * SB * LS) * sizeof(float);
+// 83 KB: small enough to share a CU with two workgroups of the tile kernels,
+// so a diagonal step does not have to wait for a CU to drain while a trailing
+// update runs beside the sweep.
+constexpr size_t kDiagLds = (size_t)(NB * LS + 4 * SB * PS) * sizeof(float);
 
 }  // namespace
 
@@ -436,7 +440,7 @@ struct kfac_inverse_plan {
   // so it runs on a second stream beside that sweep.
   bool lookahead = true;
   hipStream_t side = nullptr;
-  std::vector<hipEvent_t> ev_main, ev_side;   // per group
+  std::vector<hipEvent_t> ev_main, ev_side;   // per step
   ~kfac_inverse_plan() {
     for (hipEvent_t e : ev_main) (void)hipEventDestroy(e);
     for (hipEvent_t e : ev_side) (void)hipEventDestroy(e);
@@ -574,9 +578,8 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_panel, panel_cs.data(), sizeof(int) * (count + 1));
   up(p->d_tasks, tasks.data(), sizeof(int2) * tasks.size());
   if (rc == KFAC_OK && p->lookahead && p->max_t > p->group) {
-    const int groups = kfac::ceil_div(p->max_t, p->group);
     bool ok = hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess;
-    for (int g = 0; ok && g < groups; ++g) {
+    for (int g = 0; ok && g < p->max_t; ++g) {
       hipEvent_t a = nullptr, b = nullptr;
       ok = hipEventCreateWithFlags(&a, hipEventDisableTiming) == hipSuccess;
       if (ok) p->ev_main.push_back(a);
@@ -658,29 +661,30 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
     hipLaunchKernelGGL(update_kernel, dim3(u.count), dim3(THREADS), 0, st, tb, u.task0, u.k0, u.k1);
   };
-  int pending = -1;   // group whose rest is still running on the side stream
+  // Side stream: after the last column of a group, the rest of its trailing update.
+  int pending = -1;   // step of the latest work queued on the side stream
   for (int k = 0; k < plan->max_t; ++k) {
     const int na = plan->nactive[k];
     update(plan->column[k], s);
     hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(256), kDiagLds, s, tb, k);
     if (plan->panel_total[k] > 0)
       hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), 0, s, tb, k, na);
-    if (plan->urgent[k].count == 0) continue;
-    // the urgent tiles were also targets of the previous group's rest
-    if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
-    pending = -1;
-    update(plan->urgent[k], s);
+    if (plan->urgent[k].count > 0) {
+      // the urgent tiles were also targets of the previous group's rest
+      if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
+      pending = -1;
+      update(plan->urgent[k], s);
+    }
     if (plan->rest[k].count == 0) continue;
     if (!plan->lookahead) {
       update(plan->rest[k], s);
       continue;
     }
-    const int g = k / plan->group;
-    KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[g], s));
-    KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_main[g], 0));
+    KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
+    KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_main[k], 0));
     update(plan->rest[k], plan->side);
-    KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[g], plan->side));
-    pending = g;
+    KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[k], plan->side));
+    pending = k;
   }
   if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
   KFAC_HIP_CHECK(hipGetLastError());
