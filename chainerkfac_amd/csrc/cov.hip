@@ -83,6 +83,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const float4 *__restrict__ 
   int s = g * per;
   const int send = (s + per < nsplit) ? s + per : nsplit;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
   for (; s < send; ++s) {
     const float4 v = partial[(long long)s * slot4 + i];
     acc.x += v.x;
@@ -268,10 +269,12 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
   for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
 }
 
-// One workgroup per 64x64 sub-block (si >= sj) of C.
-__global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ partial,
-                                                     int nsplit, int ntile, int bm, int d,
-                                                     float alpha, float beta,
+// One workgroup per 64x64 sub-block (si >= sj) of C.  The number of slices is a
+// compile-time constant so that all loads of a thread are issued before the
+// first sum needs one (with a run-time loop every slice costs a trip to memory).
+template <int NS>
+__global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ partial, int ntile,
+                                                     int bm, int d, float alpha, float beta,
                                                      float *__restrict__ C) {
   __shared__ float tile[64][65];
   int si, sj;
@@ -283,13 +286,14 @@ __global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ p
   const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
   const long long tile_stride = (long long)bm * bm;
   const float *p0 = partial + (long long)t * tile_stride + (long long)r_in * bm + c_in;
+  const long long split_stride = (long long)ntile * tile_stride;
   float sum[16];
 #pragma unroll
-  for (int p = 0; p < 16; ++p) sum[p] = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float *ps = p0 + (long long)s * ntile * tile_stride;
+  for (int p = 0; p < 16; ++p) {
+    float a = 0.f;
 #pragma unroll
-    for (int p = 0; p < 16; ++p) sum[p] += ps[(lr0 + 4 * p) * bm + lc];
+    for (int s = 0; s < NS; ++s) a += p0[s * split_stride + (lr0 + 4 * p) * bm + lc];
+    sum[p] = a;
   }
 #pragma unroll
   for (int p = 0; p < 16; ++p) {
@@ -331,8 +335,13 @@ int finish_partials(const SyrkPlan &p, int d, float alpha, float beta, float *C,
     fin = red;
   }
   const int sub = kfac::ceil_div(d, 64);
-  hipLaunchKernelGGL(finish_kernel, dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, fin, nfin,
-                     p.ntile, p.bm, d, alpha, beta, C);
+  using Kern = void (*)(const float *, int, int, int, float, float, float *);
+  static const Kern kerns[kFinishSplits] = {finish_kernel<1>, finish_kernel<2>, finish_kernel<3>,
+                                            finish_kernel<4>, finish_kernel<5>, finish_kernel<6>,
+                                            finish_kernel<7>, finish_kernel<8>};
+  if (nfin < 1 || nfin > kFinishSplits) return kfac::fail(KFAC_EINVAL, "bad slice count %d", nfin);
+  hipLaunchKernelGGL(kerns[nfin - 1], dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, fin, p.ntile,
+                     p.bm, d, alpha, beta, C);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
