@@ -30,6 +30,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix peak
+# HBM bytes per covariance SYRK launch (average over the 161 launches of a step):
+# hardware counters FETCH_SIZE and WRITE_SIZE collected with `rocprofv3 --pmc` on
+# this script (--no-graph --calibrate-copy), each scaled by what it reads for the
+# 256 MiB calibration copy; the counter summary is kept under profiles/.
+SYRK_HBM_BYTES_PER_LAUNCH = 51.6e6
 BATCH = 32
 DAMPING = 2.5e-4
 STAB_COEFF = 16.0
@@ -81,6 +86,13 @@ def run_gpu(args):
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(3)
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.add(src, 0.0, out=dst)   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     layers = W.resnet50_v1()
     flops = W.flops(layers, BATCH)
     model, calls = build_model(layers, dev, gen)
@@ -204,7 +216,8 @@ def run_gpu(args):
             'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
             'launches': syrk_n,
             'avg_launch_ms': round(syrk_ms / max(syrk_n, 1), 4),
-            'traffic': None,
+            'traffic': SYRK_HBM_BYTES_PER_LAUNCH,
+            'traffic_unit': 'bytes/launch',
         },
     }
     return result, layers
@@ -289,6 +302,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--no-graph', action='store_true', help='launch every kernel from the host each step')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='first run one 256 MiB device-to-device elementwise copy (a kernel of known traffic, '
+                         'the reference point for hardware byte counters collected under rocprofv3 --pmc)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures the single-GPU K-FAC hot path: inter-GPU collectives are outside this '
