@@ -57,9 +57,10 @@ struct Panel {
 // ---------------------------------------------------------------------------
 // VEC: float4 loads (strides and L multiples of 4, base 16-byte aligned); a
 // compile-time choice so that the common aligned case carries no scalar-path
-// code or registers.
+// code or registers.  The primary template is the float4 variant.
 template <int ROWS, bool VEC>
 struct LoaderKC {
+  static_assert(VEC, "the scalar variant is the specialisation below");
   static constexpr bool kKRow = false;
   static constexpr int NV = ROWS / 32;
   struct Regs {
@@ -98,38 +99,18 @@ struct LoaderKC {
     const unsigned kq = (threadIdx.x & 7) * 4;
     const unsigned kg = (unsigned)k0 + kq;
     const bool full_k = k0 + KT <= k_end;
-    r.fast = full_rows && full_k && VEC;
-    if (VEC) {
-      const bool kok = full_k || (long long)kg + 3 < k_end;
-      r.kmask = kok ? 0xfu : 0u;
-      const unsigned kc = kok ? kg : 0u;
-      unsigned koff = kc;
-      if (L < (unsigned)k_end) {  // more than one sample
-        const unsigned s = kc / L;
-        koff = s * sample_stride + (kc - s * L);
-      }
-      const float *p = base + koff;
-#pragma unroll
-      for (int i = 0; i < NV; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + rowoff[i]);
-    } else {
-      unsigned off[4];
-      r.kmask = 0;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool ok = (long long)kg + e < k_end;
-        if (ok) r.kmask |= 1u << e;
-        const unsigned kc = ok ? kg + e : 0u;
-        const unsigned s = kc / L;
-        off[e] = s * sample_stride + (kc - s * L);
-      }
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        r.v[i].x = base[off[0] + rowoff[i]];
-        r.v[i].y = base[off[1] + rowoff[i]];
-        r.v[i].z = base[off[2] + rowoff[i]];
-        r.v[i].w = base[off[3] + rowoff[i]];
-      }
+    r.fast = full_rows && full_k;
+    const bool kok = full_k || (long long)kg + 3 < k_end;
+    r.kmask = kok ? 0xfu : 0u;
+    const unsigned kc = kok ? kg : 0u;
+    unsigned koff = kc;
+    if (L < (unsigned)k_end) {  // more than one sample
+      const unsigned s = kc / L;
+      koff = s * sample_stride + (kc - s * L);
     }
+    const float *p = base + koff;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + rowoff[i]);
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
@@ -157,6 +138,67 @@ struct LoaderKC {
           p[e] = kv ? (rv ? t[e] : fill) : 0.f;
         }
       }
+    }
+  }
+};
+
+// Unaligned tensors (odd row strides such as d = 9C + 1): dword loads with the 32
+// lanes of a half-wave on 32 consecutive k-values of one row, so that every
+// load instruction reads whole 128-byte row segments whatever their alignment.
+template <int ROWS>
+struct LoaderKC<ROWS, false> {
+  static constexpr bool kKRow = false;
+  static constexpr int NR = ROWS / 8;   // rows per thread
+  struct Regs {
+    float v[NR];
+    bool kvalid;   // this thread's k-value is inside the range
+  };
+  const float *base;
+  unsigned sample_stride;
+  unsigned row_stride;
+  unsigned L;      // k-values per sample
+  int rows_valid;
+  int ones_row;    // -1 if none
+  // per-thread panel state: row i of the thread is first_row + 8 i; rows past
+  // the end load from the last data row (masked when stored)
+  int first_row;
+  unsigned last_off;
+
+  __device__ __forceinline__ void init(float *, int row0) {
+    first_row = row0 + (threadIdx.x >> 5);
+    last_off = (unsigned)(rows_valid > 0 ? rows_valid - 1 : 0) * row_stride;
+  }
+
+  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
+    const long long kg = k0 + (threadIdx.x & 31);
+    r.kvalid = kg < k_end;
+    const unsigned kc = r.kvalid ? (unsigned)kg : 0u;
+    unsigned koff = kc;
+    if (L < (unsigned)k_end) {  // more than one sample
+      const unsigned s = kc / L;
+      koff = s * sample_stride + (kc - s * L);
+    }
+    const float *p = base + koff;
+    // The row offsets are cheap to recompute and expensive to keep: hide the
+    // row from the optimiser so that it does not hoist NR offsets per operand
+    // out of the k loop (which spills under a 3-workgroup register budget).
+    int fr = first_row;
+    asm volatile("" : "+v"(fr));
+    const unsigned off0 = (unsigned)fr * row_stride;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const unsigned off = off0 + (unsigned)(8 * i) * row_stride;
+      r.v[i] = p[off < last_off ? off : last_off];
+    }
+  }
+
+  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
+    float *p = lds + (threadIdx.x >> 5) * Panel<ROWS>::kRowKStride + (threadIdx.x & 31);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int row = first_row + 8 * i;
+      const float fill = row == ones_row ? 1.f : 0.f;
+      p[8 * i * Panel<ROWS>::kRowKStride] = r.kvalid ? (row < rows_valid ? r.v[i] : fill) : 0.f;
     }
   }
 };
