@@ -1,9 +1,9 @@
 // Per-sample gradient matrix of a batch-normalisation layer,
 //   U[s] = [ sum_hw gy'[s] * h[s] | sum_hw gy'[s] ],   h = (x - mean) / sqrt(var + eps),
-// with the batch mean and biased variance recomputed from x (two passes, as
-// numpy's mean/var do), gy' = gy * gy_scale.  The activation and its gradient
-// are each read from HBM once more than strictly needed (x twice, gy once) and
-// nothing of their size is written.  One wave owns one (sample, channel) slab.
+// with the batch mean and biased variance recomputed from x (centred second
+// moments, as numpy's var computes them), gy' = gy * gy_scale.  The activation
+// and its gradient are each read from HBM once and nothing of their size is
+// written.  One wave owns one (sample, channel) slab.
 // Replaces chainerkfac/optimizers/fisher_blocks/normalizations/
 // batch_normalization.py:86-119.
 #include "common.h"
@@ -11,55 +11,51 @@
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
 
-__device__ __forceinline__ float wave_sum(float v) {
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
-  return __shfl(v, 0, 64);
+// Sum over a group of LPS consecutive lanes, delivered to every lane of the group.
+template <int LPS>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = LPS / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, LPS);
+  return v;
 }
 
-// s1[slab] = sum x
-__global__ __launch_bounds__(kThreads) void bn_sum_kernel(const float *__restrict__ x,
-                                                          int nslab, int hw,
-                                                          float *__restrict__ s1) {
-  const int slab = blockIdx.x * kWaves + (threadIdx.x >> 6);
-  if (slab >= nslab) return;
-  const int lane = threadIdx.x & 63;
-  const float *p = x + (long long)slab * hw;
+// LPS lanes (a wave, or a quarter wave for small images) per (sample, channel)
+// slab of hw pixels: the slab's mean, its
+// centred second moment, sum gy and sum gy (x - slab mean).  The second sweep
+// over the slab hits cache; per-channel batch statistics are assembled from
+// these exactly (pairwise combination of means and centred moments), so x and
+// gy are each read from HBM once.
+template <int LPS>
+__global__ __launch_bounds__(kThreads) void bn_stats_kernel(
+    const float *__restrict__ x, const float *__restrict__ gy, int nslab, int hw,
+    float *__restrict__ smean, float *__restrict__ sm2, float *__restrict__ sg,
+    float *__restrict__ sgx) {
+  // idle groups of the last workgroup redo the last slab, so that every lane
+  // takes part in the shuffles
+  int slab = (blockIdx.x * kThreads + threadIdx.x) / LPS;
+  if (slab >= nslab) slab = nslab - 1;
+  const int lane = threadIdx.x % LPS;
+  const float *px = x + (long long)slab * hw;
+  const float *pg = gy + (long long)slab * hw;
+  const bool vec =
+      (hw & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gy)) & 15) == 0;
   float acc = 0.f;
-  if ((hw & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-    const float4 *p4 = reinterpret_cast<const float4 *>(p);
-    for (int i = lane; i < hw / 4; i += 64) {
-      const float4 v = p4[i];
+  if (vec) {
+    const float4 *x4 = reinterpret_cast<const float4 *>(px);
+    for (int i = lane; i < hw / 4; i += LPS) {
+      const float4 v = x4[i];
       acc += (v.x + v.y) + (v.z + v.w);
     }
   } else {
-    for (int i = lane; i < hw; i += 64) acc += p[i];
+    for (int i = lane; i < hw; i += LPS) acc += px[i];
   }
-  acc = wave_sum(acc);
-  if (lane == 0) s1[slab] = acc;
-}
-
-// per slab: ss = sum (x-mean)^2, sg = sum gy, sgx = sum gy (x-mean)
-__global__ __launch_bounds__(kThreads) void bn_moments_kernel(
-    const float *__restrict__ x, const float *__restrict__ gy, int n, int c, int hw,
-    const float *__restrict__ s1, float *__restrict__ ss, float *__restrict__ sg,
-    float *__restrict__ sgx) {
-  const int nslab = n * c;
-  const int slab = blockIdx.x * kWaves + (threadIdx.x >> 6);
-  if (slab >= nslab) return;
-  const int lane = threadIdx.x & 63;
-  const int ch = slab % c;
-  float tot = 0.f;
-  for (int s = lane; s < n; s += 64) tot += s1[s * c + ch];
-  const float mean = wave_sum(tot) / ((float)n * (float)hw);
-  const float *px = x + (long long)slab * hw;
-  const float *pg = gy + (long long)slab * hw;
+  const float mean = group_sum<LPS>(acc) / (float)hw;
   float a = 0.f, b = 0.f, g = 0.f;
-  if ((hw & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gy)) & 15) == 0) {
+  if (vec) {
     const float4 *x4 = reinterpret_cast<const float4 *>(px);
     const float4 *g4 = reinterpret_cast<const float4 *>(pg);
-    for (int i = lane; i < hw / 4; i += 64) {
+    for (int i = lane; i < hw / 4; i += LPS) {
       const float4 xv = x4[i];
       const float4 gv = g4[i];
       const float d0 = xv.x - mean, d1 = xv.y - mean, d2 = xv.z - mean, d3 = xv.w - mean;
@@ -68,7 +64,7 @@ __global__ __launch_bounds__(kThreads) void bn_moments_kernel(
       g += (gv.x * d0 + gv.y * d1) + (gv.z * d2 + gv.w * d3);
     }
   } else {
-    for (int i = lane; i < hw; i += 64) {
+    for (int i = lane; i < hw; i += LPS) {
       const float dv = px[i] - mean;
       const float gv = pg[i];
       a += dv * dv;
@@ -76,33 +72,66 @@ __global__ __launch_bounds__(kThreads) void bn_moments_kernel(
       g += gv * dv;
     }
   }
-  a = wave_sum(a);
-  b = wave_sum(b);
-  g = wave_sum(g);
+  a = group_sum<LPS>(a);
+  b = group_sum<LPS>(b);
+  g = group_sum<LPS>(g);
   if (lane == 0) {
-    ss[slab] = a;
+    smean[slab] = mean;
+    sm2[slab] = a;
     sg[slab] = b;
     sgx[slab] = g;
   }
 }
 
-// U[s][ch] = gy_scale * rstd[ch] * sgx ; U[s][off_beta + ch] = gy_scale * sg
-__global__ __launch_bounds__(kThreads) void bn_finish_kernel(
+// 64 channels per workgroup (lanes on consecutive channels, so every access is
+// coalesced), the samples dealt to the 4 waves: batch mean and variance of the
+// channel from the slab statistics, then the channel's column(s) of U.
+//   sum_hw gy (x - mean_c) = sgx_s + (mean_s - mean_c) sg_s
+__global__ __launch_bounds__(256) void bn_finish_kernel(
     int n, int c, int hw, float eps, float gy_scale, int has_gamma, int has_beta,
-    const float *__restrict__ ss, const float *__restrict__ sg, const float *__restrict__ sgx,
-    float *__restrict__ U) {
-  const int idx = blockIdx.x * kThreads + threadIdx.x;
-  if (idx >= n * c) return;
-  const int ch = idx % c, s = idx / c;
+    const float *__restrict__ smean, const float *__restrict__ sm2, const float *__restrict__ sg,
+    const float *__restrict__ sgx, float *__restrict__ U) {
+  __shared__ float part[2][4][64];
+  const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int ch = blockIdx.x * 64 + lane;
+  const bool live = ch < c;
   const int width = c * (has_gamma + has_beta);
+  float mean = 0.f, rstd = 0.f;
   if (has_gamma) {
     float tot = 0.f;
-    for (int t = 0; t < n; ++t) tot += ss[t * c + ch];
-    const float var = tot / ((float)n * (float)hw);
-    const float rstd = 1.0f / sqrtf(var + eps);
-    U[(long long)s * width + ch] = gy_scale * (sgx[idx] * rstd);
+    if (live) {
+#pragma unroll 8
+      for (int s = grp; s < n; s += 4) tot += smean[s * c + ch];
+    }
+    part[0][grp][lane] = tot;
+    __syncthreads();
+    mean = ((part[0][0][lane] + part[0][1][lane]) + (part[0][2][lane] + part[0][3][lane])) / (float)n;
+    float m2 = 0.f, dev = 0.f;
+    if (live) {
+#pragma unroll 8
+      for (int s = grp; s < n; s += 4) {
+        const float dm = smean[s * c + ch] - mean;
+        m2 += sm2[s * c + ch];
+        dev += dm * dm;
+      }
+    }
+    part[1][grp][lane] = m2 + (float)hw * dev;
+    __syncthreads();
+    const float var = ((part[1][0][lane] + part[1][1][lane]) + (part[1][2][lane] + part[1][3][lane])) /
+                      ((float)n * (float)hw);
+    rstd = 1.0f / sqrtf(var + eps);
   }
-  if (has_beta) U[(long long)s * width + (has_gamma ? c : 0) + ch] = gy_scale * sg[idx];
+  if (!live) return;
+#pragma unroll 8
+  for (int s = grp; s < n; s += 4) {
+    const int idx = s * c + ch;
+    const float b = sg[idx];
+    if (has_gamma) {
+      const float g = sgx[idx] + (smean[idx] - mean) * b;
+      U[(long long)s * width + ch] = gy_scale * (g * rstd);
+    }
+    if (has_beta) U[(long long)s * width + (has_gamma ? c : 0) + ch] = gy_scale * b;
+  }
 }
 
 }  // namespace
@@ -124,14 +153,16 @@ extern "C" int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, i
                       kfac_bn_workspace_bytes(n, c));
   hipStream_t s = kfac::as_stream(stream);
   const int nslab = n * c;
-  float *s1 = static_cast<float *>(ws);
-  float *ss = s1 + nslab, *sg = ss + nslab, *sgx = sg + nslab;
-  const int grid = kfac::ceil_div(nslab, kWaves);
-  hipLaunchKernelGGL(bn_sum_kernel, dim3(grid), dim3(kThreads), 0, s, x, nslab, hw, s1);
-  hipLaunchKernelGGL(bn_moments_kernel, dim3(grid), dim3(kThreads), 0, s, x, gy, n, c, hw, s1, ss,
-                     sg, sgx);
-  hipLaunchKernelGGL(bn_finish_kernel, dim3(kfac::ceil_div(nslab, kThreads)), dim3(kThreads), 0, s,
-                     n, c, hw, eps, gy_scale, has_gamma ? 1 : 0, has_beta ? 1 : 0, ss, sg, sgx, U);
+  float *smean = static_cast<float *>(ws);
+  float *sm2 = smean + nslab, *sg = sm2 + nslab, *sgx = sg + nslab;
+  if (hw <= 256)
+    hipLaunchKernelGGL(bn_stats_kernel<16>, dim3(kfac::ceil_div(nslab, kThreads / 16)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  else
+    hipLaunchKernelGGL(bn_stats_kernel<64>, dim3(kfac::ceil_div(nslab, kThreads / 64)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  hipLaunchKernelGGL(bn_finish_kernel, dim3(kfac::ceil_div(c, 64)), dim3(256), 0, s, n, c, hw, eps,
+                     gy_scale, has_gamma ? 1 : 0, has_beta ? 1 : 0, smean, sm2, sg, sgx, U);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
