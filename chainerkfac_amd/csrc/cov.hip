@@ -39,6 +39,9 @@ constexpr int kFinishSplits = 8;
 SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
   SyrkPlan p;
   p.bm = d <= 320 ? 64 : 128;
+  // A short reduction (batch-norm blocks: K = batch size) is all output traffic:
+  // 64-tiles spread the stores over four times as many workgroups.
+  if (panel_len == KT && nk <= 4 && kfac::ceil_div(d, 128) <= 32) p.bm = 64;
   p.tiles = kfac::ceil_div(d, p.bm);
   p.ntile = p.tiles * (p.tiles + 1) / 2;
   if (nk < 1) nk = 1;
