@@ -152,7 +152,29 @@ __global__ __launch_bounds__(256) void gemv_kernel(const float *__restrict__ F, 
   const int lane = threadIdx.x & 63;
   const float *fr = F + (long long)row * d;
   float acc = 0.f;
-  for (int j = lane; j < d; j += 64) acc += fr[j] * (j < n0 ? g0[j] : g1[j - n0]);
+  const bool vec = ((d | n0) & 3) == 0 &&
+                   ((reinterpret_cast<uintptr_t>(F) | reinterpret_cast<uintptr_t>(g0) |
+                     reinterpret_cast<uintptr_t>(g1)) & 15) == 0;
+  if (vec) {
+    // float4 loads, four independent partial sums per lane
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    const float4 *f4 = reinterpret_cast<const float4 *>(fr);
+    const float4 *g04 = reinterpret_cast<const float4 *>(g0);
+    const float4 *g14 = reinterpret_cast<const float4 *>(g1);
+    const int q0 = n0 / 4, q = d / 4;
+#pragma unroll 4
+    for (int j = lane; j < q; j += 64) {
+      const float4 f = f4[j];
+      const float4 g = j < q0 ? g04[j] : g14[j - q0];
+      a0 += f.x * g.x;
+      a1 += f.y * g.y;
+      a2 += f.z * g.z;
+      a3 += f.w * g.w;
+    }
+    acc = (a0 + a1) + (a2 + a3);
+  } else {
+    for (int j = lane; j < d; j += 64) acc += fr[j] * (j < n0 ? g0[j] : g1[j - n0]);
+  }
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
   if (lane == 0) y[row] = acc;
 }
