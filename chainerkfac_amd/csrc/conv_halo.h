@@ -64,11 +64,14 @@ __host__ __device__ inline int halo_region_floats(const ConvGeom &g) {
 // Everything about an element that does not change from step to step (its
 // offset inside a sample, its LDS slot, whether its channel and column exist)
 // is computed once per workgroup and kept in registers.
+// With SAME (diagonal tile) the lane also sums the A operand values it feeds to
+// the matrix cores into rs[im] (half of the row sum of row (wave_m * WM + im) *
+// 32 + lane % 32: the other half is in lane ^ 32).
 template <int WM, int NKK, bool SAME, bool MASK>
 __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int row0B,
                                               long long sbeg, long long send, float *smem,
                                               int regA, int regB, const int *koff_tbl,
-                                              floatx16 (&acc)[WM][WM]) {
+                                              floatx16 (&acc)[WM][WM], float (&rs)[WM]) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -229,6 +232,10 @@ __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int 
       // keep the scheduler from sinking those reads below the MFMAs (it does,
       // to save three registers, and then every MFMA waits for its operand)
       __builtin_amdgcn_sched_barrier(0);
+      if (SAME) {
+#pragma unroll
+        for (int im = 0; im < WM; ++im) rs[im] += a[cur][im];
+      }
 #pragma unroll
       for (int im = 0; im < WM; ++im)
 #pragma unroll

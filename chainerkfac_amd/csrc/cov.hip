@@ -11,6 +11,11 @@
 //                    fixed summation order, so deterministic) write C.
 // Tiles are written as C[I,J] plus the mirror C[J,I] through an LDS transpose,
 // so C is exactly symmetric and every store is a contiguous row segment.
+// A bias ("ones") column is kept out of the tile grid: d = 9C + 1 would pay a
+// whole extra tile row for it.  Its row of C is the vector of row sums of the
+// operand, which the diagonal tiles' workgroups accumulate on the side from the
+// operand values they feed to the matrix cores anyway, and its corner entry is
+// the reduction length.
 //
 // Replaces the im2col + transpose + column_stack + GEMM + scale chain of
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py
@@ -72,8 +77,14 @@ SyrkPlan plan_syrk(int d, long long rows) {
   return plan_syrk_panels(d, kfac::ceil_div<long long>(rows > 0 ? rows : 1, KT), KT);
 }
 
+// Floats of one k-slice in the workspace: the partial tiles, then one row-sum
+// slot per tile row (used when there is a ones column).
+size_t syrk_slot_floats(const SyrkPlan &p) {
+  return (size_t)p.ntile * p.bm * p.bm + (size_t)p.tiles * p.bm;
+}
+
 size_t syrk_ws_floats(const SyrkPlan &p) {
-  return (size_t)(p.nsplit + p.nreduced) * p.ntile * p.bm * p.bm;
+  return (size_t)(p.nsplit + p.nreduced) * syrk_slot_floats(p);
 }
 
 // Sums groups of splits: out slot g = sum of splits [g*per, (g+1)*per).
@@ -108,9 +119,10 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
 // Writes the finished tile: C[I,J] = alpha*acc + beta*C[I,J] and, for I != J,
 // the mirror C[J,I], 64x64 quadrant by quadrant through an LDS transpose so
 // that every global access is a contiguous row segment.
+// Rows and columns below dt (the tiled part); d is the leading dimension of C.
 template <int WM>
 __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
-                                           int d, float alpha, float beta,
+                                           int dt, int d, float alpha, float beta,
                                            float *__restrict__ C) {
   constexpr int BM = 64 * WM;
   float(*t)[65] = reinterpret_cast<float(*)[65]>(lds);
@@ -128,7 +140,7 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
       const int lr = lr0 + 4 * p;
       const int r = r0 + lr, c = c0 + lc;
       float v = alpha * t[lr][lc];
-      const bool ok = r < d && c < d;
+      const bool ok = r < dt && c < dt;
       if (ok) {
         if (beta != 0.f) v += beta * C[(long long)r * d + c];
         C[(long long)r * d + c] = v;
@@ -141,9 +153,43 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
       for (int p = 0; p < 16; ++p) {
         const int lr = lr0 + 4 * p;
         const int mr = c0 + lr, mc = r0 + lc;   // row of the mirrored quadrant = column here
-        if (mr < d && mc < d) C[(long long)mr * d + mc] = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
+        if (mr < dt && mc < dt) C[(long long)mr * d + mc] = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
       }
     }
+  }
+}
+
+// Ones column of a diagonal tile's rows.  rs[im] holds this lane's half of the
+// row sums (see the main loops); after adding the other half, lanes 0..31 of the
+// waves with wave_n == 0 own row (wave_m * WM + im) * 32 + lane of the tile.
+// direct: C[d-1, row] = C[row, d-1] = alpha * sum + beta * C[d-1, row], and the
+// first tile also writes the corner alpha * count + beta * C[d-1, d-1];
+// otherwise the sums go to the k-slice's row-sum slot.
+template <int WM>
+__device__ __forceinline__ void write_rowsums(float (&rs)[WM], int I, int dt, int d, int direct,
+                                              float count, float alpha, float beta,
+                                              float *__restrict__ vec, float *__restrict__ C) {
+  constexpr int BM = 64 * WM;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int im = 0; im < WM; ++im) {
+    const float tot = rs[im] + __shfl_xor(rs[im], 32, 64);
+    if (wn != 0 || lane >= 32) continue;
+    const int row = I * BM + (wm * WM + im) * 32 + lane;
+    if (!direct) {
+      vec[row] = tot;
+    } else if (row < dt) {
+      float v = alpha * tot;
+      if (beta != 0.f) v += beta * C[(long long)(d - 1) * d + row];
+      C[(long long)(d - 1) * d + row] = v;
+      C[(long long)row * d + d - 1] = v;
+    }
+  }
+  if (direct && I == 0 && threadIdx.x == 0) {
+    float v = alpha * count;
+    if (beta != 0.f) v += beta * C[(long long)(d - 1) * d + d - 1];
+    C[(long long)(d - 1) * d + d - 1] = v;
   }
 }
 
@@ -191,8 +237,9 @@ __device__ __forceinline__ void work_decode(int bid, int total, int ntile, int t
 template <int WM, class Loader>
 __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K,
                                                           long long klen, int ntile, int nsplit,
-                                                          int direct, int d, float alpha,
-                                                          float beta, float *__restrict__ partial,
+                                                          int direct, int d, int ones,
+                                                          float alpha, float beta,
+                                                          float *__restrict__ partial,
                                                           float *__restrict__ C) {
   constexpr int BM = 64 * WM;
   __shared__ float lds[2 * Panel<BM>::kFloats];
@@ -200,8 +247,10 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
   __shared__ int2 tabB[BM];
   float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
   static_assert(2 * Panel<BM>::kFloats >= 64 * 65, "LDS too small for the epilogue transpose");
+  const int dt = d - ones;   // rows of the tile grid
+  const int tiles = (dt + BM - 1) / BM;
   int split, tile, I, J;
-  work_decode(blockIdx.x, ntile * nsplit, ntile, (d + BM - 1) / BM, split, tile, I, J);
+  work_decode(blockIdx.x, ntile * nsplit, ntile, tiles, split, tile, I, J);
   Loader la = ld, lb = ld;
   la.init(reinterpret_cast<float *>(tabA), I * BM);
   lb.init(reinterpret_cast<float *>(tabB), J * BM);
@@ -211,15 +260,22 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
   if (kend > K) kend = K;
   floatx16 acc[WM][WM];
   zero_acc<WM, WM>(acc);
+  float rs[WM];
+#pragma unroll
+  for (int im = 0; im < WM; ++im) rs[im] = 0.f;
   if (I == J)
-    mainloop<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
+    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs);
   else
     mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
+  const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
+  float *mine = partial + split * slot;
+  if (ones && I == J)
+    write_rowsums<WM>(rs, I, dt, d, direct, (float)K, alpha, beta, mine + (long long)ntile * (BM * BM), C);
   if (direct) {
-    write_tile<WM>(acc, lds, I, J, d, alpha, beta, C);
+    write_tile<WM>(acc, lds, I, J, dt, d, alpha, beta, C);
     return;
   }
-  float *out = partial + ((long long)split * ntile + tile) * (BM * BM);
+  float *out = mine + (long long)tile * (BM * BM);
   for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
 }
 
@@ -229,8 +285,8 @@ template <int WM, int NKK, bool MASK>
 __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long long total_steps,
                                                                long long klen, int ntile,
                                                                int nsplit, int direct, int d,
-                                                               float alpha,
-                                                               float beta,
+                                                               int ones, float count,
+                                                               float alpha, float beta,
                                                                float *__restrict__ partial,
                                                                float *__restrict__ C) {
   constexpr int BM = 64 * WM;
@@ -238,8 +294,10 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
   const int region = halo_region_floats(g);
   const int regA = 0, regB = region;
   int *koff_tbl = reinterpret_cast<int *>(smem + 2 * region);
+  const int dt = d - ones;   // rows of the tile grid
+  const int tiles = (dt + BM - 1) / BM;
   int split, tile, I, J;
-  work_decode(blockIdx.x, ntile * nsplit, ntile, (d + BM - 1) / BM, split, tile, I, J);
+  work_decode(blockIdx.x, ntile * nsplit, ntile, tiles, split, tile, I, J);
   // constant planes (ones, zeros) of both regions and the k -> offset table
   for (int e = threadIdx.x; e < 2 * g.Rsz; e += THREADS) {
     const float val = e < g.Rsz ? 1.f : 0.f;
@@ -260,15 +318,22 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
   if (send > total_steps) send = total_steps;
   floatx16 acc[WM][WM];
   zero_acc<WM, WM>(acc);
+  float rs[WM];
+#pragma unroll
+  for (int im = 0; im < WM; ++im) rs[im] = 0.f;
   if (I == J)
-    halo_mainloop<WM, NKK, true, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc);
+    halo_mainloop<WM, NKK, true, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc, rs);
   else
-    halo_mainloop<WM, NKK, false, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc);
+    halo_mainloop<WM, NKK, false, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc, rs);
+  const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
+  float *mine = partial + split * slot;
+  if (ones && I == J)
+    write_rowsums<WM>(rs, I, dt, d, direct, count, alpha, beta, mine + (long long)ntile * (BM * BM), C);
   if (direct) {
-    write_tile<WM>(acc, smem, I, J, d, alpha, beta, C);
+    write_tile<WM>(acc, smem, I, J, dt, d, alpha, beta, C);
     return;
   }
-  float *out = partial + ((long long)split * ntile + tile) * (BM * BM);
+  float *out = mine + (long long)tile * (BM * BM);
   for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
 }
 
@@ -277,8 +342,9 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
 // first sum needs one (with a run-time loop every slice costs a trip to memory).
 template <int NS>
 __global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ partial, int ntile,
-                                                     int bm, int d, float alpha, float beta,
-                                                     float *__restrict__ C) {
+                                                     int bm, long long slot, int dt, int d,
+                                                     int ones, float count, float alpha,
+                                                     float beta, float *__restrict__ C) {
   __shared__ float tile[64][65];
   int si, sj;
   tri_decode(blockIdx.x, si, sj);
@@ -289,21 +355,39 @@ __global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ p
   const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
   const long long tile_stride = (long long)bm * bm;
   const float *p0 = partial + (long long)t * tile_stride + (long long)r_in * bm + c_in;
-  const long long split_stride = (long long)ntile * tile_stride;
   float sum[16];
 #pragma unroll
   for (int p = 0; p < 16; ++p) {
     float a = 0.f;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) a += p0[s * split_stride + (lr0 + 4 * p) * bm + lc];
+    for (int s = 0; s < NS; ++s) a += p0[s * slot + (lr0 + 4 * p) * bm + lc];
     sum[p] = a;
+  }
+  // ones column: the diagonal sub-blocks finish their 64 row sums
+  if (ones && si == sj && threadIdx.x < 64) {
+    const int row = si * 64 + threadIdx.x;
+    const float *v0 = partial + (long long)ntile * tile_stride + row;
+    float a = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) a += v0[s * slot];
+    if (row < dt) {
+      float v = alpha * a;
+      if (beta != 0.f) v += beta * C[(long long)(d - 1) * d + row];
+      C[(long long)(d - 1) * d + row] = v;
+      C[(long long)row * d + d - 1] = v;
+    }
+    if (row == 0) {
+      float v = alpha * count;
+      if (beta != 0.f) v += beta * C[(long long)(d - 1) * d + d - 1];
+      C[(long long)(d - 1) * d + d - 1] = v;
+    }
   }
 #pragma unroll
   for (int p = 0; p < 16; ++p) {
     const int lr = lr0 + 4 * p;
     const int r = si * 64 + lr, c = sj * 64 + lc;
     float v = alpha * sum[p];
-    if (beta != 0.f && r < d && c < d) v += beta * C[(long long)r * d + c];
+    if (beta != 0.f && r < dt && c < dt) v += beta * C[(long long)r * d + c];
     tile[lr][lc] = v;
   }
   __syncthreads();
@@ -312,23 +396,26 @@ __global__ __launch_bounds__(256) void finish_kernel(const float *__restrict__ p
     const int lr = lr0 + 4 * p;
     const int r = si * 64 + lr, c = sj * 64 + lc;
     if (si == sj) {
-      if (r < d && c < d) C[(long long)r * d + c] = (lc <= lr) ? tile[lr][lc] : tile[lc][lr];
+      if (r < dt && c < dt) C[(long long)r * d + c] = (lc <= lr) ? tile[lr][lc] : tile[lc][lr];
     } else {
-      if (r < d && c < d) C[(long long)r * d + c] = tile[lr][lc];
+      if (r < dt && c < dt) C[(long long)r * d + c] = tile[lr][lc];
       const int mr = sj * 64 + lr, mc = si * 64 + lc;
-      if (mr < d && mc < d) C[(long long)mr * d + mc] = tile[lc][lr];
+      if (mr < dt && mc < dt) C[(long long)mr * d + mc] = tile[lc][lr];
     }
   }
 }
 
 // reduce_kernel (more than 8 slices) + finish_kernel on the partial tiles.
-int finish_partials(const SyrkPlan &p, int d, float alpha, float beta, float *C, float *partial,
-                    hipStream_t stream) {
+// d is the dimension of C, ones = 1 if its last row/column is the ones column,
+// count the reduction length (the corner entry).
+int finish_partials(const SyrkPlan &p, int d, int ones, float count, float alpha, float beta,
+                    float *C, float *partial, hipStream_t stream) {
   const float *fin = partial;
   int nfin = p.nsplit;
+  const long long slot = (long long)syrk_slot_floats(p);
   if (p.nreduced) {
-    const long long slot4 = (long long)p.ntile * p.bm * p.bm / 4;
-    float *red = partial + (size_t)p.nsplit * p.ntile * p.bm * p.bm;
+    const long long slot4 = slot / 4;
+    float *red = partial + (size_t)p.nsplit * slot;
     const int per = kfac::ceil_div(p.nsplit, p.nreduced);
     nfin = kfac::ceil_div(p.nsplit, per);
     hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)kfac::ceil_div<long long>(slot4, 256), nfin),
@@ -337,14 +424,16 @@ int finish_partials(const SyrkPlan &p, int d, float alpha, float beta, float *C,
     KFAC_HIP_CHECK(hipGetLastError());
     fin = red;
   }
-  const int sub = kfac::ceil_div(d, 64);
-  using Kern = void (*)(const float *, int, int, int, float, float, float *);
+  const int dt = d - ones;
+  const int sub = kfac::ceil_div(dt, 64);
+  using Kern = void (*)(const float *, int, int, long long, int, int, int, float, float, float,
+                        float *);
   static const Kern kerns[kFinishSplits] = {finish_kernel<1>, finish_kernel<2>, finish_kernel<3>,
                                             finish_kernel<4>, finish_kernel<5>, finish_kernel<6>,
                                             finish_kernel<7>, finish_kernel<8>};
   if (nfin < 1 || nfin > kFinishSplits) return kfac::fail(KFAC_EINVAL, "bad slice count %d", nfin);
   hipLaunchKernelGGL(kerns[nfin - 1], dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, fin, p.ntile,
-                     p.bm, d, alpha, beta, C);
+                     p.bm, slot, dt, d, ones, count, alpha, beta, C);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
@@ -357,10 +446,13 @@ int check_ws(const SyrkPlan &p, void *ws, size_t ws_bytes) {
   return KFAC_OK;
 }
 
+// d: dimension of C; ones = 1 if its last row/column is a ones column, which
+// the loaders must then not supply (their rows end at d - 1).
 template <class L64, class L128>
-int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, float beta,
-             float *C, void *ws, size_t ws_bytes, hipStream_t stream) {
-  const SyrkPlan p = plan_syrk(d, K);
+int run_syrk(const L64 &l64, const L128 &l128, int d, int ones, long long K, float alpha,
+             float beta, float *C, void *ws, size_t ws_bytes, hipStream_t stream) {
+  if (d - ones == 0) return kfac::fail(KFAC_EINVAL, "empty factor");
+  const SyrkPlan p = plan_syrk(d - ones, K);
   if (int rc = check_ws(p, ws, ws_bytes)) return rc;
   float *partial = static_cast<float *>(ws);
   const int grid = p.ntile * p.nsplit;
@@ -369,14 +461,14 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, long long K, float alpha, 
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
     if (p.bm == 64)
       hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
-                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+                         p.klen, p.ntile, p.nsplit, direct, d, ones, alpha, beta, partial, C);
     else
       hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
-                         p.klen, p.ntile, p.nsplit, direct, d, alpha, beta, partial, C);
+                         p.klen, p.ntile, p.nsplit, direct, d, ones, alpha, beta, partial, C);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (direct) return KFAC_OK;
-  return finish_partials(p, d, alpha, beta, C, partial, stream);
+  return finish_partials(p, d, ones, (float)K, alpha, beta, C, partial, stream);
 }
 
 // Geometry of the LDS halo kernel for one convolution; false when the shape
@@ -437,18 +529,19 @@ size_t halo_lds_bytes(const ConvGeom &g) {
   return floats * sizeof(float);
 }
 
-int run_conv_halo(const ConvGeom &g, int n, int d, float alpha, float beta, float *C, void *ws,
-                  size_t ws_bytes, hipStream_t stream) {
+int run_conv_halo(const ConvGeom &g, int n, int d, int ones, float alpha, float beta, float *C,
+                  void *ws, size_t ws_bytes, hipStream_t stream) {
   const long long total_steps = (long long)n * g.segs * g.rgroups;
-  SyrkPlan p = plan_syrk_panels(d, total_steps, 1);
+  const float count = (float)((long long)n * g.ho * g.wo);
+  SyrkPlan p = plan_syrk_panels(d - ones, total_steps, 1);
   if (p.bm != 128) return 1;   // small factors stay on the generic kernel
   if (int rc = check_ws(p, ws, ws_bytes)) return rc;
   const size_t lds = halo_lds_bytes(g);
   // the masked variants zero operands of k-values past the image's bottom edge
   // or past the end of a step; most shapes do not need them
   const bool mask = (g.RT * g.WS != g.nk) || (g.ho % g.RT != 0);
-  using Kern = void (*)(ConvGeom, long long, long long, int, int, int, int, float, float, float *,
-                        float *);
+  using Kern = void (*)(ConvGeom, long long, long long, int, int, int, int, int, float, float,
+                        float, float *, float *);
   static const Kern kerns[3][2] = {
       {syrk_conv_kernel<2, 25, false>, syrk_conv_kernel<2, 25, true>},
       {syrk_conv_kernel<2, 28, false>, syrk_conv_kernel<2, 28, true>},
@@ -469,11 +562,11 @@ int run_conv_halo(const ConvGeom &g, int n, int d, float alpha, float beta, floa
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
     hipLaunchKernelGGL(kern, grid, block, lds, stream, g, total_steps, p.klen, p.ntile, p.nsplit,
-                       direct, d, alpha, beta, partial, C);
+                       direct, d, ones, count, alpha, beta, partial, C);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (direct) return KFAC_OK;
-  return finish_partials(p, d, alpha, beta, C, partial, stream);
+  return finish_partials(p, d, ones, count, alpha, beta, C, partial, stream);
 }
 
 bool kc_vec_ok(const float *base, long long sample_stride, long long row_stride, int L) {
@@ -538,9 +631,13 @@ extern "C" size_t kfac_cov_workspace_bytes(int d, int64_t rows) {
   if (d <= 0) return 0;
   // upper bound over every reduction length (the convolution kernels count
   // their panels differently): the split count never exceeds ceil(1536 / tiles)
-  SyrkPlan p = plan_syrk_panels(d, 1LL << 40, KT);
   (void)rows;
-  return syrk_ws_floats(p) * sizeof(float);
+  size_t need = syrk_ws_floats(plan_syrk_panels(d, 1LL << 40, KT));
+  if (d > 1) {   // with a ones column the tile grid covers d - 1 rows
+    const size_t alt = syrk_ws_floats(plan_syrk_panels(d - 1, 1LL << 40, KT));
+    if (alt > need) need = alt;
+  }
+  return need * sizeof(float);
 }
 
 extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_ones,
@@ -549,14 +646,15 @@ extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_o
   KFAC_REQUIRE(n > 0 && d_in > 0, "bad shape n=%d d_in=%d", n, d_in);
   KFAC_REQUIRE((long long)n * d_in < 0x7fffffffLL, "input too large");
   KFAC_REQUIRE(x && C, "null pointer");
-  const int d = d_in + (append_ones ? 1 : 0);
+  const int ones = append_ones ? 1 : 0;
+  const int d = d_in + ones;
   if (ks_vec_ok(x, d_in))
-    return run_syrk(make_ks<64, true>(x, d_in, d_in, append_ones, nullptr),
-                    make_ks<128, true>(x, d_in, d_in, append_ones, nullptr), d, n, alpha, beta, C,
-                    ws, ws_bytes, kfac::as_stream(stream));
-  return run_syrk(make_ks<64, false>(x, d_in, d_in, append_ones, nullptr),
-                  make_ks<128, false>(x, d_in, d_in, append_ones, nullptr), d, n, alpha, beta, C,
-                  ws, ws_bytes, kfac::as_stream(stream));
+    return run_syrk(make_ks<64, true>(x, d_in, d_in, 0, nullptr),
+                    make_ks<128, true>(x, d_in, d_in, 0, nullptr), d, ones, n, alpha, beta, C, ws,
+                    ws_bytes, kfac::as_stream(stream));
+  return run_syrk(make_ks<64, false>(x, d_in, d_in, 0, nullptr),
+                  make_ks<128, false>(x, d_in, d_in, 0, nullptr), d, ones, n, alpha, beta, C, ws,
+                  ws_bytes, kfac::as_stream(stream));
 }
 
 extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, float alpha,
@@ -568,10 +666,10 @@ extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, floa
   const long long K = (long long)n * howo;
   if (kc_vec_ok(gy, (long long)c * howo, howo, howo))
     return run_syrk(make_kc<64, true>(gy, (long long)c * howo, howo, howo, c, -1),
-                    make_kc<128, true>(gy, (long long)c * howo, howo, howo, c, -1), c, K, alpha,
+                    make_kc<128, true>(gy, (long long)c * howo, howo, howo, c, -1), c, 0, K, alpha,
                     beta, C, ws, ws_bytes, kfac::as_stream(stream));
   return run_syrk(make_kc<64, false>(gy, (long long)c * howo, howo, howo, c, -1),
-                  make_kc<128, false>(gy, (long long)c * howo, howo, howo, c, -1), c, K, alpha,
+                  make_kc<128, false>(gy, (long long)c * howo, howo, howo, c, -1), c, 0, K, alpha,
                   beta, C, ws, ws_bytes, kfac::as_stream(stream));
 }
 
@@ -590,26 +688,26 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
   KFAC_REQUIRE(dl < 46340, "factor dimension %lld too large", dl);
   KFAC_REQUIRE((long long)n * c * h * w < 0x7fffffffLL, "input too large");
   const int d = (int)dl;
+  const int ones = append_ones ? 1 : 0;
   const long long K = (long long)n * ho * wo;
   hipStream_t s = kfac::as_stream(stream);
   if (kh == 1 && kw == 1 && sy == 1 && sx == 1 && ph == 0 && pw == 0) {
     // 1x1 convolution: the patch matrix is the NCHW tensor itself
     const int hw = h * w;
-    const int ones = append_ones ? c : -1;
     if (kc_vec_ok(x, (long long)c * hw, hw, hw))
-      return run_syrk(make_kc<64, true>(x, (long long)c * hw, hw, hw, c, ones),
-                      make_kc<128, true>(x, (long long)c * hw, hw, hw, c, ones), d, K, alpha, beta,
-                      C, ws, ws_bytes, s);
-    return run_syrk(make_kc<64, false>(x, (long long)c * hw, hw, hw, c, ones),
-                    make_kc<128, false>(x, (long long)c * hw, hw, hw, c, ones), d, K, alpha, beta,
-                    C, ws, ws_bytes, s);
+      return run_syrk(make_kc<64, true>(x, (long long)c * hw, hw, hw, c, -1),
+                      make_kc<128, true>(x, (long long)c * hw, hw, hw, c, -1), d, ones, K, alpha,
+                      beta, C, ws, ws_bytes, s);
+    return run_syrk(make_kc<64, false>(x, (long long)c * hw, hw, hw, c, -1),
+                    make_kc<128, false>(x, (long long)c * hw, hw, hw, c, -1), d, ones, K, alpha,
+                    beta, C, ws, ws_bytes, s);
   }
   ConvGeom geom;
-  if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones, &geom)) {
-    const int rc = run_conv_halo(geom, n, d, alpha, beta, C, ws, ws_bytes, s);
+  if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, 0, &geom)) {
+    const int rc = run_conv_halo(geom, n, d, ones, alpha, beta, C, ws, ws_bytes, s);
     if (rc <= 0) return rc;   // 1 = shape left to the generic kernel
   }
-  return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones),
-                  make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, append_ones), d, K,
-                  alpha, beta, C, ws, ws_bytes, s);
+  return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, 0),
+                  make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, 0), d, ones, K, alpha,
+                  beta, C, ws, ws_bytes, s);
 }

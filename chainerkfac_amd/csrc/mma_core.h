@@ -391,10 +391,13 @@ __device__ __forceinline__ float fetch(const float *lds, int row, int k) {
 // SYRK) and lb is not used.  ldsA / ldsB hold Panel<64*WM> / Panel<64*WN>
 // floats.  Operands of step kk+1 are fetched from LDS before the MFMAs of step
 // kk issue, so LDS latency hides behind the matrix pipeline.
-template <int WM, int WN, bool SAME, class LA, class LB>
-__device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, int rowB0,
-                                         long long kbeg, long long kend, float *ldsA,
-                                         float *ldsB, floatx16 (&acc)[WM][WN]) {
+// With RS the lane also sums the A operand values it feeds to the matrix cores:
+// rs[im] ends as the sum over this lane's k-values (k = lane / 32 mod 2) of row
+// (wave_m * WM + im) * 32 + lane % 32, i.e. half of that row's sum.
+template <int WM, int WN, bool SAME, bool RS, class LA, class LB>
+__device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int rowA0, int rowB0,
+                                              long long kbeg, long long kend, float *ldsA,
+                                              float *ldsB, floatx16 (&acc)[WM][WN], float *rs) {
   constexpr int RA = 64 * WM, RB = 64 * WN;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -420,6 +423,10 @@ __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, 
 #pragma unroll
       for (int im = 0; im < WM; ++im)
         a[im] = fetch<RA, LA::kKRow>(ldsA, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
+      if (RS) {
+#pragma unroll
+        for (int im = 0; im < WM; ++im) rs[im] += a[im];
+      }
 #pragma unroll
       for (int in = 0; in < WN; ++in) {
         if (SAME)
@@ -435,6 +442,21 @@ __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, 
     }
     __syncthreads();
   }
+}
+
+template <int WM, int WN, bool SAME, class LA, class LB>
+__device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, int rowB0,
+                                         long long kbeg, long long kend, float *ldsA,
+                                         float *ldsB, floatx16 (&acc)[WM][WN]) {
+  mainloop_impl<WM, WN, SAME, false>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, nullptr);
+}
+
+template <int WM, int WN, bool SAME, class LA, class LB>
+__device__ __forceinline__ void mainloop_rowsum(const LA &la, const LB &lb, int rowA0, int rowB0,
+                                                long long kbeg, long long kend, float *ldsA,
+                                                float *ldsB, floatx16 (&acc)[WM][WN],
+                                                float (&rs)[WM]) {
+  mainloop_impl<WM, WN, SAME, true>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, rs);
 }
 
 // Set every accumulator element of this lane to f(row, col), row / col relative

@@ -101,6 +101,35 @@ def test_running_accumulation_matches_mean_of_covs():
     check(out, acc[0])
 
 
+@pytest.mark.parametrize('shape', ['conv3x3_region', 'conv1x1_slab', 'linear'])
+def test_accumulation_with_ones_column(shape):
+    """beta != 0 on the ones row/column and the corner entry, for the kernels that keep the ones column
+    outside the tile grid (k-sliced and single-slice epilogues)."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(5)
+    acc = None
+    out = None
+    for i in range(3):
+        if shape == 'conv3x3_region':      # d = 577, 2048 pixels: several k-slices + finish kernel
+            x = r.standard_normal((8, 64, 16, 16)).astype(np.float32)
+            ref = O.conv_A(x, 3, 1, 1, True)
+            run = lambda b, o: ops.cov_conv_a(torch.from_numpy(x).cuda(), 3, 1, 1, True, (1.0 / 8) / 3, beta=b, out=o)
+        elif shape == 'conv1x1_slab':      # d = 41, odd pixel count: scalar slab loader
+            x = r.standard_normal((4, 40, 7, 7)).astype(np.float32)
+            ref = O.conv_A(x, 1, 1, 0, True)
+            run = lambda b, o: ops.cov_conv_a(torch.from_numpy(x).cuda(), 1, 1, 0, True, (1.0 / 4) / 3, beta=b, out=o)
+        else:                              # one 32-row panel: written straight from registers
+            x = r.random((16, 200), dtype=np.float32)
+            ref = O.linear_A(x, True)
+            run = lambda b, o: ops.cov_linear(torch.from_numpy(x).cuda(), True, (1.0 / 16) / 3, b, o)
+        acc = O.accumulate_covs(acc, [ref], 3)
+        out = run(0.0 if i == 0 else 1.0, out)
+    check(out, acc[0])
+    got = out.cpu().numpy()
+    assert np.array_equal(got, got.T)
+    assert abs(got[-1, -1] - acc[0][-1, -1]) <= 1e-6 * abs(acc[0][-1, -1])
+
+
 def test_workspace_too_small_is_reported():
     import ctypes
     from chainerkfac_amd import _lib
