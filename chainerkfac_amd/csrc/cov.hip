@@ -60,6 +60,26 @@ SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
   const long long max_ns = nk >= 6 ? nk / 6 : 1;
   if (ns > max_ns) ns = max_ns;
   if (ns < 1) ns = 1;
+  if (panel_len != KT) {
+    // Region kernel (panel = one step of <= 64 pixels): its workgroups are all
+    // alike and 2 fit a CU, so a launch runs in rounds of 512 and a round that
+    // is nearly empty still costs a full workgroup.  Pick the slice count with
+    // the least rounds x (steps per slice + fixed cost), near the target above.
+    const long long slots = 512;
+    double best = 0;
+    long long best_ns = ns;
+    for (long long c = 1; c <= max_ns && c <= 4 * ns; ++c) {
+      const long long per = kfac::ceil_div(nk, c);
+      const long long eff = kfac::ceil_div(nk, per);
+      const long long rounds = kfac::ceil_div(p.ntile * eff, slots);
+      const double cost = (double)rounds * ((double)per + 3.0) + 0.25 * (double)eff;
+      if (c == 1 || cost < best) {
+        best = cost;
+        best_ns = c;
+      }
+    }
+    ns = best_ns;
+  }
   // tuning override: KFAC_SYRK_SPLITS=<n> forces the split count
   if (const char *env = getenv("KFAC_SYRK_SPLITS")) {
     const long long forced = atoll(env);
