@@ -17,7 +17,7 @@
 //            followed by U(a,b) = X^T(a,b) L_bb^-T once the sum is complete,
 //
 // both k-contiguous "NT" tile GEMMs over row slabs of the workspace.  Block
-// columns are processed in groups of kGroup: inside a group the sweep is
+// columns are processed in groups of kGroup (2): inside a group the sweep is
 // left-looking (column k receives the products of the group's earlier columns
 // just before it is factored, K up to (kGroup-1)*NB), and after a group every
 // column to its right receives the whole group at once (K = kGroup*NB), which
@@ -141,6 +141,73 @@ struct LoaderTileT {
       *reinterpret_cast<float4 *>(p + 8 * i * Panel<NB>::kKRowStride) = r.v[i];
   }
 };
+
+// Main loop of the tile kernels: the shared loop with 64 k-values (two LDS
+// panels per operand) per pass instead of 32.  The products of this file are
+// short (K = 128 .. 512) and often one workgroup per CU, so what counts is how
+// many loads are in flight and how few barrier-to-barrier round trips a product
+// needs: K = 128 takes two passes instead of four.  K must be a multiple of 64.
+// lds: 4 panels (A0, A1, B0, B1) of Panel<NB>::kFloats.
+constexpr int kTileLdsFloats = 4 * Panel<NB>::kFloats;
+constexpr size_t kTileLdsBytes = kTileLdsFloats * sizeof(float);
+
+template <bool SAME, class LA, class LB>
+__device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K, float *lds,
+                                              floatx16 (&acc)[2][2]) {
+  constexpr int PF = Panel<NB>::kFloats;
+  float *ldsA = lds, *ldsB = lds + 2 * PF;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane & 31, lk = lane >> 5;
+  typename LA::Regs ra[2];
+  typename LB::Regs rb[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    la.load(ra[h], 0, KT * h, K);
+    if (!SAME) lb.load(rb[h], 0, KT * h, K);
+  }
+  for (int k0 = 0; k0 < K; k0 += 2 * KT) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      la.store(ra[h], ldsA + h * PF);
+      if (!SAME) lb.store(rb[h], ldsB + h * PF);
+    }
+    __syncthreads();
+    if (k0 + 2 * KT < K) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        la.load(ra[h], 0, k0 + 2 * KT + KT * h, K);
+        if (!SAME) lb.load(rb[h], 0, k0 + 2 * KT + KT * h, K);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float *pa = ldsA + h * PF;
+      const float *pb = SAME ? pa : ldsB + h * PF;
+#pragma unroll
+      for (int kk = 0; kk < KT / 2; ++kk) {
+        float a[2], b[2];
+#pragma unroll
+        for (int im = 0; im < 2; ++im)
+          a[im] = fetch<NB, LA::kKRow>(pa, (wm * 2 + im) * 32 + lrow, 2 * kk + lk);
+#pragma unroll
+        for (int in = 0; in < 2; ++in) {
+          if (SAME)
+            b[in] = fetch<NB, LA::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
+          else
+            b[in] = fetch<NB, LB::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
+        }
+#pragma unroll
+        for (int im = 0; im < 2; ++im)
+#pragma unroll
+          for (int in = 0; in < 2; ++in)
+            acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+}
 
 // ---------------------------------------------------------------------------
 // copy-in: lower tiles of in -> padded workspace (identity on the padding)
@@ -342,16 +409,14 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
 // M(x,k) = M(x,k) W^T = M(x,k) U_kk in place for every x != k; the operand
 // W^T is the diagonal tile itself, read transposed.
 __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, int nactive) {
-  __shared__ float ldsA[Panel<NB>::kFloats];
-  __shared__ float ldsB[Panel<NB>::kFloats];
+  extern __shared__ float lds[];
   const int s = find_slot(tb.panel_cs, nactive, blockIdx.x);
   const int local = blockIdx.x - tb.panel_cs[s];
   const int x = local < k ? local : local + 1;
   float *tile = tile_ptr(tb, s, x, k);
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
-  mainloop<2, 2, false>(LoaderTile{tile}, LoaderTileT{tile_ptr(tb, s, k, k)}, 0, 0, 0, NB, ldsA,
-                        ldsB, acc);
+  tile_mainloop<false>(LoaderTile{tile}, LoaderTileT{tile_ptr(tb, s, k, k)}, NB, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { tile[rr * NB + cc] = v; });
 }
 
@@ -361,8 +426,7 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, 
 // the epilogue is a plain store.  An upper tile whose row lies inside [k0, k1]
 // receives its first product here and is overwritten (it holds stale data).
 __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0, int k0, int k1) {
-  __shared__ float ldsA[Panel<NB>::kFloats];
-  __shared__ float ldsB[Panel<NB>::kFloats];
+  extern __shared__ float lds[];
   const int2 task = tb.tasks[task0 + blockIdx.x];
   const int s = task.x;
   const int a = task.y & 0xffff, b = task.y >> 16;
@@ -379,16 +443,15 @@ __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int ta
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -C[rr * NB + cc]; });
   const LoaderTile la{tile_ptr(tb, s, a, j_lo)}, lb{tile_ptr(tb, s, b, j_lo)};
   if (a == b)
-    mainloop<2, 2, true>(la, lb, 0, 0, 0, K, ldsA, ldsB, acc);
+    tile_mainloop<true>(la, lb, K, lds, acc);
   else
-    mainloop<2, 2, false>(la, lb, 0, 0, 0, K, ldsA, ldsB, acc);
+    tile_mainloop<false>(la, lb, K, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[rr * NB + cc] = -v; });
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
 __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int count) {
-  __shared__ float ldsA[Panel<NB>::kFloats];
-  __shared__ float ldsB[Panel<NB>::kFloats];
+  extern __shared__ float lds[];
   const int s = find_slot(tb.tile_cs, count, blockIdx.x);
   int I, J;
   tri_decode(blockIdx.x - tb.tile_cs[s], I, J);
@@ -399,9 +462,9 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int cou
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
   if (I == J)
-    mainloop<2, 2, true>(la, lb, 0, 0, 0, K, ldsA, ldsB, acc);
+    tile_mainloop<true>(la, lb, K, lds, acc);
   else
-    mainloop<2, 2, false>(la, lb, 0, 0, 0, K, ldsA, ldsB, acc);
+    tile_mainloop<false>(la, lb, K, lds, acc);
   float *__restrict__ out = tb.out[s];
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) {
     const int r = I * NB + rr, c = J * NB + cc;
@@ -427,7 +490,7 @@ struct UpdateLaunch {
 struct kfac_inverse_plan {
   int count = 0;
   int max_t = 0;
-  int group = 4;                   // block columns per trailing update
+  int group = 2;                   // block columns per trailing update (measured best of 1..8)
   std::vector<int> order;          // slot -> caller index
   std::vector<int> nt;             // per slot
   std::vector<int> nactive;        // per step
@@ -638,6 +701,11 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(diag_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)kDiagLds));
+    for (const void *f : {reinterpret_cast<const void *>(panel_kernel),
+                          reinterpret_cast<const void *>(update_kernel),
+                          reinterpret_cast<const void *>(lauum_kernel)})
+      KFAC_HIP_CHECK(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)kTileLdsBytes));
     plan->attr_set = true;
   }
   InvTables tb;
@@ -659,7 +727,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   auto update = [&](const UpdateLaunch &u, hipStream_t st) {
     if (u.count == 0) return;
     kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
-    hipLaunchKernelGGL(update_kernel, dim3(u.count), dim3(THREADS), 0, st, tb, u.task0, u.k0, u.k1);
+    hipLaunchKernelGGL(update_kernel, dim3(u.count), dim3(THREADS), kTileLdsBytes, st, tb, u.task0,
+                       u.k0, u.k1);
   };
   // Side stream: after the last column of a group, the rest of its trailing update.
   int pending = -1;   // step of the latest work queued on the side stream
@@ -668,7 +737,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     update(plan->column[k], s);
     hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(256), kDiagLds, s, tb, k);
     if (plan->panel_total[k] > 0)
-      hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), 0, s, tb, k, na);
+      hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), kTileLdsBytes, s,
+                         tb, k, na);
     if (plan->urgent[k].count > 0) {
       // the urgent tiles were also targets of the previous group's rest
       if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
@@ -690,7 +760,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   KFAC_HIP_CHECK(hipGetLastError());
   {
     kfac::TimedLaunch timed(KFAC_TIMED_INV_LAUUM, s);
-    hipLaunchKernelGGL(lauum_kernel, dim3(plan->total_tiles), dim3(THREADS), 0, s, tb, count);
+    hipLaunchKernelGGL(lauum_kernel, dim3(plan->total_tiles), dim3(THREADS), kTileLdsBytes, s, tb,
+                       count);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
