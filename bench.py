@@ -34,7 +34,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix peak
 # hardware counters FETCH_SIZE and WRITE_SIZE collected with `rocprofv3 --pmc` on
 # this script (--no-graph --calibrate-copy), each scaled by what it reads for the
 # 256 MiB calibration copy; the counter summary is kept under profiles/.
-SYRK_HBM_BYTES_PER_LAUNCH = 51.6e6
+SYRK_HBM_BYTES_PER_LAUNCH = 44.1e6
 BATCH = 32
 DAMPING = 2.5e-4
 STAB_COEFF = 16.0
