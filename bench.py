@@ -10,7 +10,12 @@ shapes (output gradients scaled by 1/(batch*sqrt(pixels)), the size a
 mean-reduced loss gives them, which keeps the rank-32 batch-norm factors
 positive definite in float32), resident in HBM before the timed region.  The step is driven through
 the drop-in host classes (FisherBlock*.forward_postprocess /
-backward_preprocess, KFAC.update_kfgrads).
+backward_preprocess, KFAC.update_kfgrads).  The 53 batch-norm blocks, whose
+factor is the rank-32 matrix U^T U / 32 of this batch, are inverted through
+their Woodbury form (the same dense damped inverse as the Cholesky path, which
+--dense-bn-inverse forces); the JSON states which path ran and reports the
+inverse rate both against the reference's 161 dense inversions and against
+the dense work actually executed.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu]
 
@@ -96,7 +101,9 @@ def run_gpu(args):
     layers = W.resnet50_v1()
     flops = W.flops(layers, BATCH)
     model, calls = build_model(layers, dev, gen)
-    opt = KFAC(damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0).setup(model)
+    opt = KFAC(damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0)
+    opt.bn_lowrank_inverse = not args.dense_bn_inverse
+    opt = opt.setup(model)
     by_name = {fb.linkname: fb for fb in opt.fblocks}
     work = [(by_name['/' + name], func, in_data, (gy,)) for name, func, in_data, gy in calls]
     assert len(opt.fblocks) == len(layers)
@@ -174,10 +181,16 @@ def run_gpu(args):
         fam[name] = (n.value, ms.value)
     _lib.check(lib.kfac_timing_enable(0))
     info_bad = int((opt.inv_info != 0).sum().item())
+    lowrank = [fb for fb in opt.fblocks if getattr(fb, 'lowrank_inverse_args', lambda: None)() is not None] \
+        if opt.bn_lowrank_inverse else []
+    info_bad += sum(int((fb.inv_info != 0).sum().item()) for fb in lowrank)
+    # d^3 of the factors that went through the dense Cholesky path (the reference inverts all 161 densely)
+    dense_inverse_flops = flops['inverse'] - sum(float(fb.cov_emas[0].shape[0]) ** 3 for fb in lowrank)
 
     syrk_n, syrk_ms = fam['syrk']
     achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_ms > 0 else 0.0
     total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
+    executed_flops = flops['cov'] + dense_inverse_flops + flops['precondition']
     result = {
         'metric': 'ms per K-FAC step, ResNet-50 bs32/GPU; cov+inv TFLOP/s vs FP32 MFMA peak',
         'value': round(ms_per_step, 4),
@@ -194,17 +207,23 @@ def run_gpu(args):
         'config': {'workload': 'ResNet-50 v1 (bias, 1000-way) K-FAC step, batch 32 @224: 161 factors, '
                                'cov + damped Cholesky inverse + precondition',
                    'batch': BATCH, 'factors': len(W.all_factor_dims(layers)), 'damping': DAMPING,
-                   'hip_graph': graph is not None},
+                   'hip_graph': graph is not None,
+                   'bn_inverse': 'woodbury rank-32 ({} blocks)'.format(len(lowrank)) if lowrank else 'dense'},
+        # rates use the flops actually executed; the *_reference_work entries divide the work of the
+        # reference's algorithm (all 161 factors inverted densely) by the same times
         'tflops': {
-            'step': round(total_flops / ms_per_step / 1e9, 2),
-            'cov_inv': round((flops['cov'] + flops['inverse']) / ((phase_ms['cov'] + phase_ms['inverse'])) / 1e9, 2),
+            'step': round(executed_flops / ms_per_step / 1e9, 2),
+            'cov_inv': round((flops['cov'] + dense_inverse_flops) / ((phase_ms['cov'] + phase_ms['inverse'])) / 1e9, 2),
             'cov': round(flops['cov'] / phase_ms['cov'] / 1e9, 2),
-            'inverse': round(flops['inverse'] / phase_ms['inverse'] / 1e9, 2),
+            'inverse': round(dense_inverse_flops / phase_ms['inverse'] / 1e9, 2),
             'precondition': round(flops['precondition'] / phase_ms['precondition'] / 1e9, 2),
-            'frac_of_fp32_mfma_peak': round(total_flops / ms_per_step / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
+            'frac_of_fp32_mfma_peak': round(executed_flops / ms_per_step / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
+            'step_reference_work': round(total_flops / ms_per_step / 1e9, 2),
+            'inverse_reference_work': round(flops['inverse'] / phase_ms['inverse'] / 1e9, 2),
         },
         'phase_ms': {k: round(v, 3) for k, v in phase_ms.items()},
-        'gflop': {k: round(v / 1e9, 1) for k, v in flops.items()},
+        'gflop': dict({k: round(v / 1e9, 1) for k, v in flops.items()},
+                      inverse_executed=round(dense_inverse_flops / 1e9, 1)),
         'kernel_ms': {k: {'launches': n, 'total_ms': round(ms, 3)} for k, (n, ms) in fam.items()},
         'inverse_info_nonzero': info_bad,
         'roofline': {
@@ -302,6 +321,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--no-graph', action='store_true', help='launch every kernel from the host each step')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--dense-bn-inverse', action='store_true',
+                    help='invert the batch-norm blocks with the dense Cholesky path as well (default: their '
+                         'rank-32 Woodbury form, which yields the same dense inverse)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='first run one 256 MiB device-to-device elementwise copy (a kernel of known traffic, '
                          'the reference point for hardware byte counters collected under rocprofv3 --pmc)')

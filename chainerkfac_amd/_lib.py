@@ -47,6 +47,10 @@ PROTOTYPES = {
     'kfac_damp_plan_create': (c_int, [c_int, c_i32p, c_i32p, c_vpp]),
     'kfac_damp_plan_destroy': (c_int, [c_vp]),
     'kfac_pi_damp_batched_f32': (c_int, [c_vp, c_vpp, c_vpp, c_dp, c_int, c_vp, c_vp]),
+    'kfac_bn_lowrank_plan_create': (c_int, [c_int, c_int, c_i32p, c_i32p, c_vpp]),
+    'kfac_bn_lowrank_workspace_bytes': (c_sz, [c_vp]),
+    'kfac_bn_lowrank_plan_destroy': (c_int, [c_vp]),
+    'kfac_bn_lowrank_inverse_batched_f32': (c_int, [c_vp, c_vpp, c_vpp, c_dp, c_dp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_add_diag_f32': (c_int, [c_vp, c_int, c_int, c_d, c_d, c_vp]),
     'kfac_precond_conn_workspace_bytes': (c_sz, [c_int, c_int]),
     'kfac_precond_conn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),

@@ -40,6 +40,7 @@
 #include <algorithm>
 #include <numeric>
 
+#include "chol32.h"
 #include "common.h"
 #include "mma_core.h"
 
@@ -264,49 +265,6 @@ __device__ __forceinline__ void wave_visit(const floatx16 &acc, F f) {
   for (int v = 0; v < 16; ++v) f(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), lane & 31, acc[v]);
 }
 
-__device__ __forceinline__ float lane_bcast(float x, int lane) {
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), lane));
-}
-
-// Wave 0: factor the 32x32 block at S[b0.., b0..] (lower) in registers and
-// overwrite it with U32 = (L32^-1)^T (upper triangular, zeros below).
-//
-// Lanes 0..31 hold the rows of A, lanes 32..63 the columns of the identity: the
-// column operations of the right-looking Cholesky (scale column j by
-// 1/sqrt(pivot), subtract l_cj times it from column c) turn the first into L
-// and, applied to the identity with the same multipliers, are exactly the
-// forward substitution that turns the second into the columns of L^-1.  One
-// broadcast of l_cj feeds both halves in the same instruction.
-// Returns 0 or 1 + the local index of the first non-positive pivot.
-__device__ __forceinline__ int chol_inv_32(float *S, int b0) {
-  const int lane = threadIdx.x & 63;
-  const int i = lane & 31;
-  const bool chol = lane < SB;
-  float x[SB];
-#pragma unroll
-  for (int c = 0; c < SB; ++c) {
-    const float a = S[(b0 + i) * LS + b0 + c];
-    x[c] = chol ? a : (c == i ? 1.f : 0.f);
-  }
-  int bad = 0;
-#pragma unroll
-  for (int j = 0; j < SB; ++j) {
-    const float piv = lane_bcast(x[j], j);
-    if (!(piv > 0.f) && bad == 0) bad = j + 1;
-    float rinv = __builtin_amdgcn_rsqf(piv);
-    rinv = rinv * (1.5f - 0.5f * piv * rinv * rinv);   // one Newton step on the hardware estimate
-    x[j] *= rinv;
-#pragma unroll
-    for (int c = j + 1; c < SB; ++c) x[c] -= x[j] * lane_bcast(x[j], c);
-  }
-  // lane 32 + m holds column m of W = row m of U; entries with r < m are exact zeros
-  if (!chol) {
-#pragma unroll
-    for (int r = 0; r < SB; ++r) S[(b0 + i) * LS + b0 + r] = x[r];
-  }
-  return bad;
-}
-
 __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   extern __shared__ float smem[];
   float *S = smem;                      // NB x LS working tile
@@ -337,7 +295,7 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
   // ---- potrf on 32x32 blocks
   for (int jb = 0; jb < NB / SB; ++jb) {
     if (wave == 0) {
-      const int bad = chol_inv_32(S, jb * SB);
+      const int bad = kfac::chol_inv_32<LS>(S, jb * SB);
       if (lane == 0) {
         int *pinfo = &tb.info[tb.orig[s]];
         if (k == 0 && jb == 0) *pinfo = 0;

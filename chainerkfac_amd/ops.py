@@ -195,6 +195,71 @@ def spd_inverse_batched(mats, outs=None, info=None, stream=None):
     return inverse_plan([m.shape[0] for m in mats]).run(mats, outs, info, stream)
 
 
+class BnLowrankPlan(object):
+    """Schedule for the low-rank damped inverses of a fixed list of batch-norm blocks."""
+
+    def __init__(self, n, widths, splits):
+        self.n = int(n)
+        self.widths = tuple(int(w) for w in widths)
+        self.splits = tuple(int(v) for v in splits)
+        lib = _lib.load()
+        plan = ctypes.c_void_p()
+        _lib.check(lib.kfac_bn_lowrank_plan_create(
+            len(self.widths), self.n, _lib.i32_array(self.widths), _lib.i32_array(self.splits),
+            ctypes.byref(plan)))
+        self._plan = plan
+        self.workspace_bytes = lib.kfac_bn_lowrank_workspace_bytes(plan)
+
+    def __del__(self):
+        try:
+            plan, self._plan = self._plan, None
+            if plan is not None:
+                _lib._lib.kfac_bn_lowrank_plan_destroy(plan)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+    def run(self, Us, d_gamma, d_beta, outs=None, info=None, stream=None):
+        if len(Us) != len(self.widths):
+            raise ValueError('expected {} gradient matrices'.format(len(self.widths)))
+        for U, w in zip(Us, self.widths):
+            _dev.require_gpu_tensor(U, 'U')
+            if tuple(U.shape) != (self.n, w):
+                raise ValueError('U shape {} != ({}, {})'.format(tuple(U.shape), self.n, w))
+        if not Us:
+            return [], info
+        dev = Us[0].device
+        if outs is None:
+            outs = [torch.empty((w, w), dtype=torch.float32, device=dev) for w in self.widths]
+        for o, w in zip(outs, self.widths):
+            _dev.require_gpu_tensor(o, 'out')
+            if tuple(o.shape) != (w, w):
+                raise ValueError('out shape mismatch')
+        if info is None:
+            info = torch.empty(len(Us), dtype=torch.int32, device=dev)
+        ws = _dev.workspace('bn_lowrank', self.workspace_bytes, dev)
+        _lib.check(_lib.load().kfac_bn_lowrank_inverse_batched_f32(
+            self._plan, _lib.ptr_array([U.data_ptr() for U in Us]),
+            _lib.ptr_array([o.data_ptr() for o in outs]),
+            _lib.f64_array([0.0 if v is None else v for v in d_gamma]),
+            _lib.f64_array([0.0 if v is None else v for v in d_beta]),
+            info.data_ptr(), ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
+        return outs, info
+
+
+_bn_lowrank_plans = {}
+
+
+def bn_lowrank_inverse_batched(Us, splits, d_gamma, d_beta, outs=None, info=None, stream=None):
+    """(U^T U / n + diag(d_gamma | d_beta))^-1 for a list of (n, w) gradient matrices."""
+    key = (Us[0].shape[0], tuple(U.shape[1] for U in Us), tuple(int(v) for v in splits))
+    plan = _bn_lowrank_plans.get(key)
+    if plan is None:
+        if len(_bn_lowrank_plans) > 64:
+            _bn_lowrank_plans.clear()
+        plan = _bn_lowrank_plans[key] = BnLowrankPlan(*key)
+    return plan.run(Us, d_gamma, d_beta, outs, info, stream)
+
+
 class DampPlan(object):
     def __init__(self, dimsA, dimsG):
         self.dimsA = tuple(int(d) for d in dimsA)

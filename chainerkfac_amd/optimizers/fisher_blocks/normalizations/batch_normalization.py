@@ -14,8 +14,16 @@ def _same_array(a, b):
 
 class FisherBlockBatchNormalization(FisherBlock):
 
+    #: largest batch size the low-rank inverse handles (one 32 x 32 Cholesky per block)
+    LOWRANK_MAX_BATCH = 32
+
     def __init__(self, *args, **kwargs):
         self._F = None
+        self._U = None
+        self._ema_is_single_factor = False
+        #: cleared by whoever replaces ``covs`` by something that is not this
+        #: process's own single-batch factor (e.g. an average over ranks)
+        self.factor_is_local = True
         self.nan_flag = None
         super(FisherBlockBatchNormalization, self).__init__(*args, **kwargs)
 
@@ -69,8 +77,35 @@ class FisherBlockBatchNormalization(FisherBlock):
         width = x.shape[1] * (int(has_gamma) + int(has_beta))
         U = ops.bn_grad_matrix(x, gy, self.link.eps, gy_scale, has_gamma, has_beta,
                                out=self._buffer('U', (n, width), x.device))
+        self._U = U
         out, alpha, beta = self._cov_target('F', (width, width), x.device, 1.0 / n)
         return ops.cov_linear(U, False, alpha, beta, out)
+
+    def update_cov_emas(self):
+        first = self.cov_emas is None
+        super(FisherBlockBatchNormalization, self).update_cov_emas()
+        self._ema_is_single_factor = first or self.cov_ema_decay == 1.0
+
+    def lowrank_inverse_args(self):
+        """``(U, split, d_gamma, d_beta)`` when the damped moving average is exactly
+        ``U^T U / n + diag(d_gamma | d_beta)`` with U this step's per-sample
+        gradient matrix, so that its inverse can be taken by the Woodbury identity
+        (an n x n Cholesky) instead of a dense factorisation; ``None`` otherwise
+        (accumulation over micro-batches, a moving average with history, factors
+        that were averaged over ranks, batches larger than LOWRANK_MAX_BATCH)."""
+        U = self._U
+        if U is None or not self._ema_is_single_factor or not self.factor_is_local:
+            return None
+        if self.acc_state[0] != 1 or U.shape[0] > self.LOWRANK_MAX_BATCH:
+            return None
+        if self.cov_emas is None or self.cov_emas[0].shape[0] != U.shape[1]:
+            return None
+        d_gamma, d_beta = self._diag_pair()
+        for d in (d_gamma, d_beta):
+            if d is not None and not d > 0.0:
+                return None
+        split = 0 if self.link.gamma is None else self.link.gamma.size
+        return U, split, d_gamma, d_beta
 
     def _diag_pair(self):
         gamma, beta = self.link.gamma, self.link.beta

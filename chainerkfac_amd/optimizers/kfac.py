@@ -132,6 +132,11 @@ class KFACUpdateRule(object):
 
 class KFAC(object):
 
+    #: invert batch-norm blocks from their rank-n form when that is exact (see
+    #: FisherBlockBatchNormalization.lowrank_inverse_args); False forces the
+    #: dense Cholesky path for every block
+    bn_lowrank_inverse = True
+
     def __init__(self, lr=_default_hyperparam.lr, momentum=_default_hyperparam.momentum,
                  cov_ema_decay=_default_hyperparam.cov_ema_decay,
                  damping=_default_hyperparam.damping, stab_coeff=16.0,
@@ -315,8 +320,32 @@ class KFAC(object):
                     fb.damp()
         for fb in other:
             fb.damp()
+        # batch-norm blocks whose factor is this step's rank-n matrix U^T U / n:
+        # Woodbury inverse (the same dense result, an n x n Cholesky each)
+        lowrank = []
+        if self.bn_lowrank_inverse:
+            by_batch = {}
+            for fb in other:
+                args = getattr(fb, 'lowrank_inverse_args', lambda: None)()
+                if args is not None:
+                    by_batch.setdefault(args[0].shape[0], []).append((fb, args))
+            for group in by_batch.values():
+                fbs = [fb for fb, _ in group]
+                bufs = [fb._inv_buffers()[0] for fb in fbs]
+                info = self._info_buffer(len(fbs), bufs[0].device, key='_info_lowrank_{}'.format(
+                    group[0][1][0].shape[0]))
+                ops.bn_lowrank_inverse_batched(
+                    [a[0] for _, a in group], [a[1] for _, a in group], [a[2] for _, a in group],
+                    [a[3] for _, a in group], outs=bufs, info=info)
+                for i, fb in enumerate(fbs):
+                    fb.invs = [bufs[i]]
+                    fb.inv_info = info[i:i + 1]
+                lowrank.extend(fbs)
+        done = set(id(fb) for fb in lowrank)
         mats, outs, owners = [], [], []
         for fb in fblocks:
+            if id(fb) in done:
+                continue
             bufs = fb._inv_buffers()
             mats.extend(fb.cov_emas)
             outs.extend(bufs)
@@ -338,9 +367,10 @@ class KFAC(object):
             buf = self._pi_buf = torch.empty(n, dtype=torch.float32, device=device)
         return buf
 
-    def _info_buffer(self, n, device):
+    def _info_buffer(self, n, device, key='_info_buf'):
         import torch
-        buf = getattr(self, '_info_buf', None)
+        buf = getattr(self, key, None)
         if buf is None or buf.numel() != n or buf.device != device:
-            buf = self._info_buf = torch.empty(n, dtype=torch.int32, device=device)
+            buf = torch.empty(n, dtype=torch.int32, device=device)
+            setattr(self, key, buf)
         return buf

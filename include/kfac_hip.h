@@ -170,6 +170,32 @@ int kfac_pi_damp_batched_f32(kfac_damp_plan_t plan, float *const *A_ptrs,
                              float *const *G_ptrs, const double *rW, int use_pi,
                              float *pi_out_dev, void *stream);
 
+/* Damped inverses of `count` batch-norm blocks from their low-rank form:
+ * block i has the (n x widths[i]) per-sample gradient matrix U_i (row-major,
+ * as written by kfac_bn_grad_matrix_f32) with factor F_i = U_i^T U_i / n, and
+ *   out_i = (F_i + diag(d_gamma[i] for columns < splits[i], d_beta[i] after))^-1
+ * as a dense symmetric (w x w) matrix, by the Woodbury identity (an n x n
+ * Cholesky instead of a w^3 one).  n <= 32; the damping value of a half that
+ * has columns must be positive.  info_dev[i] = 0, or 1 + the index of the
+ * first non-positive pivot of the n x n matrix.  Mathematically the result of
+ * update_invs (fisher_block.py:165-179, cholesky_inverse.py:16-102) on the
+ * factor of normalizations/batch_normalization.py:121-131 damped per
+ * batch_normalization.py:133-157; valid only while the block's moving average
+ * is that single factor (cov_ema_decay == 1 or first step, no accumulation).
+ * Workspace: kfac_bn_lowrank_workspace_bytes(plan). */
+typedef struct kfac_bn_lowrank_plan *kfac_bn_lowrank_plan_t;
+int kfac_bn_lowrank_plan_create(int count, int n, const int32_t *widths,
+                                const int32_t *splits,
+                                kfac_bn_lowrank_plan_t *plan_out);
+size_t kfac_bn_lowrank_workspace_bytes(kfac_bn_lowrank_plan_t plan);
+int kfac_bn_lowrank_plan_destroy(kfac_bn_lowrank_plan_t plan);
+int kfac_bn_lowrank_inverse_batched_f32(kfac_bn_lowrank_plan_t plan,
+                                        const float *const *U_ptrs,
+                                        float *const *out_ptrs,
+                                        const double *d_gamma, const double *d_beta,
+                                        int32_t *info_dev, void *ws, size_t ws_bytes,
+                                        void *stream);
+
 /* diag(M)[i] += (i < split ? v0 : v1), float64 sum rounded to float32.
  * Batch-norm damping (normalizations/batch_normalization.py:133-157 with
  * fisher_block.py:175). */

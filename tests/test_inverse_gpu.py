@@ -129,3 +129,45 @@ def test_add_diag_batch_norm_halves():
     O.damp_inplace(ref, dv)
     got = ops.add_diag(torch.from_numpy(F).cuda(), dv[0], dv[-1], split=6).cpu().numpy()
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('n', [32, 7, 1])
+def test_bn_lowrank_inverse_matches_dense_oracle(n):
+    """(U^T U / n + D)^-1 by the Woodbury identity against the dense float64 inverse and the
+    float32 oracle formula, for gamma+beta, gamma-only and beta-only blocks of ragged widths."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(40 + n)
+    widths = [128, 600, 2, 257, 64]
+    splits = [64, 300, 1, 257, 0]          # 257: gamma only, 0: beta only
+    d_gamma = [4e-3, 1e-2, 0.5, 2e-3, None]
+    d_beta = [4e-3, 3e-3, 0.25, None, 1e-3]
+    Us = [(r.standard_normal((n, w)) * r.uniform(0.1, 3.0, size=w)).astype(np.float32) for w in widths]
+    outs, info = ops.bn_lowrank_inverse_batched([torch.from_numpy(U).cuda() for U in Us], splits, d_gamma, d_beta)
+    assert int((info != 0).sum()) == 0
+    for U, w, sp, dg, db, out in zip(Us, widths, splits, d_gamma, d_beta, outs):
+        diag = np.concatenate([np.full(sp, dg if dg is not None else 0.0), np.full(w - sp, db if db is not None else 0.0)])
+        F = U.astype(np.float64).T @ U.astype(np.float64) / n + np.diag(diag)
+        ref64 = np.linalg.inv(F)
+        got = out.cpu().numpy()
+        assert np.array_equal(got, got.T)
+        err = np.linalg.norm(got - ref64) / np.linalg.norm(ref64)
+        ref32 = O.inverse(F.astype(np.float32)).astype(np.float64)
+        err_ref = np.linalg.norm(ref32 - ref64) / np.linalg.norm(ref64)
+        assert err < 1e-3 and err <= 4 * err_ref + 1e-6, (w, err, err_ref)
+        # residual no worse than a small multiple of the reference formula's own (both grow with
+        # the condition number lambda_max / damping of these rank-deficient factors)
+        resid = np.linalg.norm(F @ got - np.eye(w)) / np.sqrt(w)
+        resid_ref = np.linalg.norm(F @ ref32 - np.eye(w)) / np.sqrt(w)
+        assert resid < max(4 * resid_ref, 1e-4), (w, resid, resid_ref)
+
+
+@pytest.mark.gpu
+def test_bn_lowrank_rejects_bad_arguments():
+    from chainerkfac_amd import ops, _lib
+    U = torch.zeros(40, 8, device='cuda')
+    with pytest.raises(_lib.KfacHipError):
+        ops.bn_lowrank_inverse_batched([U], [4], [1e-3], [1e-3])       # batch larger than 32
+    U = torch.zeros(4, 8, device='cuda')
+    with pytest.raises(_lib.KfacHipError):
+        ops.bn_lowrank_inverse_batched([U], [4], [0.0], [1e-3])        # non-positive damping
