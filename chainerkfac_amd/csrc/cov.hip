@@ -20,6 +20,7 @@
 // Replaces the im2col + transpose + column_stack + GEMM + scale chain of
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py
 // and the batch-norm block's grad^T grad.
+#include <algorithm>
 #include <cstdlib>
 
 #include "common.h"
@@ -491,38 +492,27 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, int ones, long long K, flo
   return finish_partials(p, d, ones, (float)K, alpha, beta, C, partial, stream);
 }
 
-// Geometry of the LDS halo kernel for one convolution; false when the shape
-// does not fit its limits (the element-wise im2col loader is used instead).
-bool make_halo_geom(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
-                    int pw, int ho, int wo, int append_ones, ConvGeom *out) {
-  ConvGeom g;
-  g.x = x;
-  g.C = c; g.H = h; g.W = w; g.kh = kh; g.kw = kw; g.sy = sy; g.sx = sx; g.ph = ph; g.pw = pw;
-  g.ho = ho; g.wo = wo;
-  g.d_patch = c * kh * kw;
-  g.append_ones = append_ones;
-  const int khkw = kh * kw;
-  if (khkw < 2 || khkw > 127) return false;
-  g.segs = kfac::ceil_div(wo, kHaloMaxK);
-  g.WS = kfac::ceil_div(wo, g.segs);
-  if (g.WS * g.segs != wo) return false;   // ragged column segments are not handled
-  g.RT = kHaloMaxK / g.WS;
-  if (g.RT > ho) g.RT = ho;
-  if (g.RT < 1) g.RT = 1;
-  g.rgroups = kfac::ceil_div(ho, g.RT);
+// Fills the fields of g that depend on the step shape (WS output columns x RT
+// output rows); false if that shape does not fit the kernel's limits.
+bool halo_step_shape(ConvGeom &g, int WS, int RT) {
+  const int khkw = g.kh * g.kw;
+  if (WS < 1 || RT < 1 || g.wo % WS != 0) return false;   // ragged column segments are not handled
+  g.WS = WS;
+  g.RT = RT;
+  g.segs = g.wo / WS;
+  g.rgroups = kfac::ceil_div(g.ho, RT);
   // k-values per step: one of the compiled loop lengths (2 * 25, 28 or 32);
   // the slots past RT*WS are masked
-  const int span = g.RT * g.WS;
-  if (span < 40) return false;   // tiny images: too few pixels per step to pay off
+  const int span = RT * WS;
+  if (span < 40 || span > kHaloMaxK) return false;   // too few pixels per step do not pay off
   g.nk = span <= 50 ? 50 : (span <= 56 ? 56 : 64);
-  g.Rin = (g.RT - 1) * sy + kh;
-  g.Win = (g.WS - 1) * sx + kw;
+  g.Rin = (RT - 1) * g.sy + g.kh;
+  g.Win = (WS - 1) * g.sx + g.kw;
   if (g.Rin > 255 || g.Win > 255) return false;
   auto round_mod32 = [](int at_least, int residue) {
-    int v = at_least + ((residue - at_least) % 32 + 32) % 32;
-    return v;
+    return at_least + ((residue - at_least) % 32 + 32) % 32;
   };
-  g.Wr = round_mod32(g.Win, kw % 32);
+  g.Wr = round_mod32(g.Win, g.kw % 32);
   g.Rsz = round_mod32(g.Rin * g.Wr, khkw % 32);
   g.CH = 127 / khkw + 2;   // 128 consecutive patch rows touch at most this many channels
   g.LPR = 16;
@@ -534,13 +524,50 @@ bool make_halo_geom(const float *x, int n, int c, int h, int w, int kh, int kw, 
   if (g.nq > kHaloMaxQ) return false;
   g.rep = 0;
   for (int p = 0; p < g.passes; ++p) g.rep |= 1u << (p * g.Rin);
+  return true;
+}
+
+// Geometry of the LDS halo kernel for one convolution; false when the shape
+// does not fit its limits (the element-wise im2col loader is used instead).
+// Among the step shapes that fit, the one with the fewest k-slots per sample
+// (padding of a step to its loop length and row groups hanging over the bottom
+// edge both cost matrix-core work), then the fewest steps.
+bool make_halo_geom(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
+                    int pw, int ho, int wo, int append_ones, ConvGeom *out) {
+  ConvGeom g;
+  g.x = x;
+  g.C = c; g.H = h; g.W = w; g.kh = kh; g.kw = kw; g.sy = sy; g.sx = sx; g.ph = ph; g.pw = pw;
+  g.ho = ho; g.wo = wo;
+  g.d_patch = c * kh * kw;
+  g.append_ones = append_ones;
+  const int khkw = kh * kw;
+  if (khkw < 2 || khkw > 127) return false;
   // the staging loads address x through a 32-bit byte offset whose top bit
   // marks elements outside the image
   const long long x_bytes = (long long)n * c * h * w * (long long)sizeof(float);
   if (x_bytes >= (1ll << 31)) return false;
   g.x_bytes = (unsigned)x_bytes;
-  *out = g;
-  return true;
+  bool found = false;
+  long long best_slots = 0, best_steps = 0;
+  for (int segs = 1; segs <= wo; ++segs) {
+    if (wo % segs != 0) continue;
+    const int WS = wo / segs;
+    if (WS > kHaloMaxK) continue;
+    const int rt_max = std::min(ho, kHaloMaxK / WS);
+    for (int RT = 1; RT <= rt_max; ++RT) {
+      ConvGeom t = g;
+      if (!halo_step_shape(t, WS, RT)) continue;
+      const long long steps = (long long)t.segs * t.rgroups;
+      const long long slots = steps * t.nk;
+      if (!found || slots < best_slots || (slots == best_slots && steps < best_steps)) {
+        found = true;
+        best_slots = slots;
+        best_steps = steps;
+        *out = t;
+      }
+    }
+  }
+  return found;
 }
 
 size_t halo_lds_bytes(const ConvGeom &g) {
