@@ -44,7 +44,9 @@ constexpr int kFinishSplits = 8;
 
 SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
   SyrkPlan p;
-  p.bm = d <= 320 ? 64 : 128;
+  int bm64_max = 520;   // measured: 64-tiles win up to d = 512 (more workgroups, 4x smaller partial tiles)
+  if (const char *env = getenv("KFAC_SYRK_BM64_MAX")) bm64_max = atoi(env);   // tuning override
+  p.bm = d <= bm64_max ? 64 : 128;
   // A short reduction (batch-norm blocks: K = batch size) is all output traffic:
   // 64-tiles spread the stores over four times as many workgroups.
   if (panel_len == KT && nk <= 4 && kfac::ceil_div(d, 128) <= 32) p.bm = 64;

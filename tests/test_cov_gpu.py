@@ -55,16 +55,17 @@ CONV_CASES = [
     (4, 3, 32, 32, 3, 1, 1, True),      # CIFAR conv1 shape (28)
     (8, 64, 16, 16, 3, 1, 1, True),     # 577
     (4, 128, 8, 8, 3, 1, 1, True),      # 1153
-    (2, 40, 6, 6, 3, 1, 1, False),      # 360: two 128-tiles + ragged third
+    (2, 40, 6, 6, 3, 1, 1, False),      # 360: six 64-tiles, the last ragged
+    (2, 70, 6, 6, 3, 1, 1, False),      # 630: 128-tiles, ragged fifth, element-gather loader
     (1, 2, 3, 3, 3, 1, 1, True),        # fewer pixels than a panel
-    # shapes that take the LDS-staged input-region kernel (d > 320, >= 40 pixels per step)
+    # shapes that take the LDS-staged input-region kernel (d > 520, >= 40 pixels per step)
     (2, 64, 29, 29, 3, 2, 1, True),     # stride 2, 15x15 outputs: 4-row steps hang over the bottom edge
-    (2, 20, 14, 14, 5, 1, 2, True),     # 5x5 taps, 14-wide rows, ragged last row group
-    (1, 40, 56, 56, 3, 1, 1, True),     # one 56-wide output row per step, four staging passes
-    (2, 48, 28, 28, 3, 1, 1, False),    # two 28-wide rows per step, no bias row
+    (2, 24, 14, 14, 5, 1, 2, True),     # 5x5 taps, 14-wide rows, ragged last row group
+    (1, 64, 56, 56, 3, 1, 1, True),     # one 56-wide output row per step, four staging passes
+    (2, 64, 28, 28, 3, 1, 1, False),    # two 28-wide rows per step, no bias row
     (4, 64, 7, 7, 3, 1, 1, True),       # whole 7x7 image per step (49 of 50 k slots used)
-    (1, 36, 20, 112, 3, 1, 1, True),    # rows wider than a step: two column segments
-    (2, 8, 38, 38, 7, 2, 3, True),      # 7x7 stride 2, 19x19 outputs
+    (1, 60, 20, 112, 3, 1, 1, True),    # rows wider than a step: two column segments
+    (2, 12, 38, 38, 7, 2, 3, True),     # 7x7 stride 2, 19x19 outputs
     (3, 130, 9, 9, 3, 1, 0, True),      # no padding, 7x7 outputs, last panel past the channel count
 ]
 
