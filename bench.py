@@ -257,9 +257,11 @@ def run_cpu_baseline(layers, budget_s=20.0):
     rng = np.random.default_rng(3)
     total = W.flops(layers, BATCH)
     total_f = sum(total.values())
-    # one bottleneck of stage 4 and one of stage 3 plus the FC: every kernel kind
-    wanted = ('res4/1/', 'res3/1/', 'fc')
-    sample = [l for l in layers if l['name'].startswith(wanted) or l['name'] == 'fc']
+    # one bottleneck of every stage plus the FC (every kernel kind and every factor size class), in an
+    # order that puts the big stage-5 factors last, where the time budget cuts the sample off
+    sample = []
+    for prefix in ('res3/1/', 'res4/1/', 'fc', 'res2/1/', 'res5/1/', 'res4/2/', 'res5/2/', 'res3/2/'):
+        sample += [l for l in layers if l['name'].startswith(prefix) or l['name'] == prefix]
     done_f = 0
     names = []
     t_used = 0.0
