@@ -7,13 +7,14 @@
 // A 3x3 patch row re-reads each staged input element nine times from LDS, so
 // global loads and their address arithmetic drop ~9x compared with gathering
 // the patch matrix element by element; zero padding is written into the region
-// when it is staged, the ones column is a constant plane next to it.
+// when it is staged.  (A bias column never reaches this loop: the caller takes
+// it from the row sums the diagonal tiles accumulate.)
 //
 // Region layout per panel (128 rows of (c,i,j)): plane ch (input channel
 // c_lo + ch) at ch*Rsz, element (ry, rx) at ry*Wr + rx, with Wr = kw and
 // Rsz = kh*kw (mod 32): the 32 consecutive patch rows an MFMA operand fetch
-// touches then fall into 32 different LDS banks.  Two extra planes hold ones
-// (bias column) and zeros (rows past the end of the factor).
+// touches then fall into 32 different LDS banks.  One extra plane holds zeros
+// (rows past the end of the factor).
 //
 // One "step" of the reduction covers RT output rows x WS output columns of one
 // sample (RT*WS <= 64, rounded up to even for the 2-deep MFMA).
@@ -28,7 +29,6 @@ struct ConvGeom {
   const float *x;
   int C, H, W, kh, kw, sy, sx, ph, pw, ho, wo;
   int d_patch;      // C*kh*kw
-  int append_ones;
   int WS, RT;       // output columns / rows per step
   int segs;         // column segments per output row
   int rgroups;      // row groups per sample
@@ -48,10 +48,9 @@ constexpr int kHaloMaxQ = 16;   // staged elements per thread and panel
 constexpr int kHaloMaxK = 64;   // k-values per step
 constexpr int kHaloDump = 32;   // floats after each region that absorb stores of idle threads
 
-// LDS floats of one region: CH channel planes, the ones plane, the zero plane
-// and the dump slots.
+// LDS floats of one region: CH channel planes, the zero plane and the dump slots.
 __host__ __device__ inline int halo_region_floats(const ConvGeom &g) {
-  return (g.CH + 2) * g.Rsz + kHaloDump;
+  return (g.CH + 1) * g.Rsz + kHaloDump;
 }
 
 // NKK = k-values per step / 2, a compile-time constant so that the MFMA loop is
@@ -91,8 +90,7 @@ __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int 
       const int j = rem - i * g.kw;
       return (c - c_lo) * g.Rsz + i * g.Wr + j;
     }
-    if (grow == g.d_patch && g.append_ones) return g.CH * g.Rsz;   // ones plane
-    return (g.CH + 1) * g.Rsz;                                     // zero plane
+    return g.CH * g.Rsz;   // zero plane
   };
   int offA[WM], offB[WM];
 #pragma unroll
@@ -113,7 +111,7 @@ __device__ __forceinline__ void halo_mainloop(const ConvGeom &g, int row0A, int 
   int loff[kHaloMaxQ];   // float offset of its LDS slot inside a region
   unsigned tmaskA = 0, tmaskB = 0;
   {
-    const int dump = (g.CH + 2) * g.Rsz + (tid & (kHaloDump - 1));
+    const int dump = (g.CH + 1) * g.Rsz + (tid & (kHaloDump - 1));
     int ps = 0, ry = 0;
 #pragma unroll
     for (int e = 0; e < kHaloMaxQ; ++e) {

@@ -321,11 +321,10 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
   const int tiles = (dt + BM - 1) / BM;
   int split, tile, I, J;
   work_decode(blockIdx.x, ntile * nsplit, ntile, tiles, split, tile, I, J);
-  // constant planes (ones, zeros) of both regions and the k -> offset table
-  for (int e = threadIdx.x; e < 2 * g.Rsz; e += THREADS) {
-    const float val = e < g.Rsz ? 1.f : 0.f;
-    smem[regA + g.CH * g.Rsz + e] = val;
-    smem[regB + g.CH * g.Rsz + e] = val;
+  // zero plane of both regions and the k -> offset table
+  for (int e = threadIdx.x; e < g.Rsz; e += THREADS) {
+    smem[regA + g.CH * g.Rsz + e] = 0.f;
+    smem[regB + g.CH * g.Rsz + e] = 0.f;
   }
   for (int k = threadIdx.x; k < kHaloMaxK; k += THREADS) {
     int off = 0;
@@ -535,13 +534,12 @@ bool halo_step_shape(ConvGeom &g, int WS, int RT) {
 // (padding of a step to its loop length and row groups hanging over the bottom
 // edge both cost matrix-core work), then the fewest steps.
 bool make_halo_geom(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
-                    int pw, int ho, int wo, int append_ones, ConvGeom *out) {
+                    int pw, int ho, int wo, ConvGeom *out) {
   ConvGeom g;
   g.x = x;
   g.C = c; g.H = h; g.W = w; g.kh = kh; g.kw = kw; g.sy = sy; g.sx = sx; g.ph = ph; g.pw = pw;
   g.ho = ho; g.wo = wo;
   g.d_patch = c * kh * kw;
-  g.append_ones = append_ones;
   const int khkw = kh * kw;
   if (khkw < 2 || khkw > 127) return false;
   // the staging loads address x through a 32-bit byte offset whose top bit
@@ -625,14 +623,13 @@ bool kc_vec_ok(const float *base, long long sample_stride, long long row_stride,
 
 template <int ROWS, bool VEC>
 LoaderKC<ROWS, VEC> make_kc(const float *base, long long sample_stride, long long row_stride, int L,
-                            int rows_valid, int ones_row) {
+                            int rows_valid) {
   LoaderKC<ROWS, VEC> l;
   l.base = base;
   l.sample_stride = (unsigned)sample_stride;
   l.row_stride = (unsigned)row_stride;
   l.L = (unsigned)L;
   l.rows_valid = rows_valid;
-  l.ones_row = ones_row;
   return l;
 }
 
@@ -654,7 +651,7 @@ LoaderKS<ROWS, VEC> make_ks(const float *base, long long ld, int rows_valid, int
 
 template <int ROWS>
 LoaderIM<ROWS> make_im(const float *x, int c, int h, int w, int kh, int kw, int sy, int sx,
-                       int ph, int pw, int ho, int wo, int append_ones) {
+                       int ph, int pw, int ho, int wo) {
   LoaderIM<ROWS> l;
   l.base = x;
   l.C = c;
@@ -669,7 +666,6 @@ LoaderIM<ROWS> make_im(const float *x, int c, int h, int w, int kh, int kw, int 
   l.ho = ho;
   l.wo = wo;
   l.d_patch = c * kh * kw;
-  l.append_ones = append_ones;
   l.table = nullptr;
   return l;
 }
@@ -714,11 +710,11 @@ extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, floa
   KFAC_REQUIRE(gy && C, "null pointer");
   const long long K = (long long)n * howo;
   if (kc_vec_ok(gy, (long long)c * howo, howo, howo))
-    return run_syrk(make_kc<64, true>(gy, (long long)c * howo, howo, howo, c, -1),
-                    make_kc<128, true>(gy, (long long)c * howo, howo, howo, c, -1), c, 0, K, alpha,
+    return run_syrk(make_kc<64, true>(gy, (long long)c * howo, howo, howo, c),
+                    make_kc<128, true>(gy, (long long)c * howo, howo, howo, c), c, 0, K, alpha,
                     beta, C, ws, ws_bytes, kfac::as_stream(stream));
-  return run_syrk(make_kc<64, false>(gy, (long long)c * howo, howo, howo, c, -1),
-                  make_kc<128, false>(gy, (long long)c * howo, howo, howo, c, -1), c, 0, K, alpha,
+  return run_syrk(make_kc<64, false>(gy, (long long)c * howo, howo, howo, c),
+                  make_kc<128, false>(gy, (long long)c * howo, howo, howo, c), c, 0, K, alpha,
                   beta, C, ws, ws_bytes, kfac::as_stream(stream));
 }
 
@@ -744,19 +740,19 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
     // 1x1 convolution: the patch matrix is the NCHW tensor itself
     const int hw = h * w;
     if (kc_vec_ok(x, (long long)c * hw, hw, hw))
-      return run_syrk(make_kc<64, true>(x, (long long)c * hw, hw, hw, c, -1),
-                      make_kc<128, true>(x, (long long)c * hw, hw, hw, c, -1), d, ones, K, alpha,
+      return run_syrk(make_kc<64, true>(x, (long long)c * hw, hw, hw, c),
+                      make_kc<128, true>(x, (long long)c * hw, hw, hw, c), d, ones, K, alpha,
                       beta, C, ws, ws_bytes, s);
-    return run_syrk(make_kc<64, false>(x, (long long)c * hw, hw, hw, c, -1),
-                    make_kc<128, false>(x, (long long)c * hw, hw, hw, c, -1), d, ones, K, alpha,
+    return run_syrk(make_kc<64, false>(x, (long long)c * hw, hw, hw, c),
+                    make_kc<128, false>(x, (long long)c * hw, hw, hw, c), d, ones, K, alpha,
                     beta, C, ws, ws_bytes, s);
   }
   ConvGeom geom;
-  if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, 0, &geom)) {
+  if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, &geom)) {
     const int rc = run_conv_halo(geom, n, d, ones, alpha, beta, C, ws, ws_bytes, s);
     if (rc <= 0) return rc;   // 1 = shape left to the generic kernel
   }
-  return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, 0),
-                  make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, 0), d, ones, K, alpha,
+  return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo),
+                  make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo), d, ones, K, alpha,
                   beta, C, ws, ws_bytes, s);
 }

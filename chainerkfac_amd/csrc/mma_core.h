@@ -53,7 +53,7 @@ struct Panel {
 // ---------------------------------------------------------------------------
 // LoaderKC: element (row, kg) at base + (kg / L) * sample_stride
 //                                     + row * row_stride + (kg % L)
-// rows >= rows_valid read as 0, except row == ones_row which reads as 1.
+// rows >= rows_valid read as 0.
 // ---------------------------------------------------------------------------
 // VEC: float4 loads (strides and L multiples of 4, base 16-byte aligned); a
 // compile-time choice so that the common aligned case carries no scalar-path
@@ -73,24 +73,20 @@ struct LoaderKC {
   unsigned row_stride;
   unsigned L;      // k-values per sample
   int rows_valid;
-  int ones_row;    // -1 if none
   // per-thread panel state
   unsigned rowoff[NV];
   unsigned rowvalid;  // bit i: row i of this thread is a data row
-  unsigned rowone;    // bit i: row i is the ones row
   bool full_rows;
 
   __device__ __forceinline__ void init(float *, int row0) {
     const int rr = threadIdx.x >> 3;
     rowvalid = 0;
-    rowone = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int row = row0 + rr + 32 * i;
       const bool ok = row < rows_valid;
       rowoff[i] = (ok ? (unsigned)row : 0u) * row_stride;
       if (ok) rowvalid |= 1u << i;
-      if (row == ones_row) rowone |= 1u << i;
     }
     full_rows = row0 + ROWS <= rows_valid;
   }
@@ -131,11 +127,10 @@ struct LoaderKC {
         float *p = lds + (rr + 32 * i) * Panel<ROWS>::kRowKStride + kq;
         const float t[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
         const bool rv = (rowvalid >> i) & 1u;
-        const float fill = ((rowone >> i) & 1u) ? 1.f : 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const bool kv = (r.kmask >> e) & 1u;
-          p[e] = kv ? (rv ? t[e] : fill) : 0.f;
+          p[e] = (kv && rv) ? t[e] : 0.f;
         }
       }
     }
@@ -158,7 +153,6 @@ struct LoaderKC<ROWS, false> {
   unsigned row_stride;
   unsigned L;      // k-values per sample
   int rows_valid;
-  int ones_row;    // -1 if none
   // per-thread panel state: row i of the thread is first_row + 8 i; rows past
   // the end load from the last data row (masked when stored)
   int first_row;
@@ -197,8 +191,7 @@ struct LoaderKC<ROWS, false> {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       const int row = first_row + 8 * i;
-      const float fill = row == ones_row ? 1.f : 0.f;
-      p[8 * i * Panel<ROWS>::kRowKStride] = r.kvalid ? (row < rows_valid ? r.v[i] : fill) : 0.f;
+      p[8 * i * Panel<ROWS>::kRowKStride] = (r.kvalid && row < rows_valid) ? r.v[i] : 0.f;
     }
   }
 };
@@ -299,8 +292,8 @@ struct LoaderKS {
 
 // ---------------------------------------------------------------------------
 // LoaderIM: implicit im2col over an NCHW tensor.
-//   row = (c * kh + i) * kw + j  for row < d_patch, row == d_patch is the ones
-//   column when append_ones; kg = (sample * ho + oy) * wo + ox.
+//   row = (c * kh + i) * kw + j  for row < d_patch (rows past it read as 0);
+//   kg = (sample * ho + oy) * wo + ox.
 // ---------------------------------------------------------------------------
 template <int ROWS>
 struct LoaderIM {
@@ -309,13 +302,11 @@ struct LoaderIM {
   struct Regs {
     float v[NV];
     unsigned use;
-    unsigned one;
   };
   const float *base;
   int C, H, W, kh, kw, sy, sx, ph, pw, ho, wo;
   int d_patch;
-  int append_ones;
-  int2 *table;  // LDS, ROWS entries: {offset inside a sample, (i << 16) | j}; y = -1 zero row, -2 ones row
+  int2 *table;  // LDS, ROWS entries: {offset inside a sample, (i << 16) | j}; y = -1: row past the end
 
   // Build the per-row table for panel rows [row0, row0 + ROWS).
   __device__ __forceinline__ void init(float *lds_table, int row0) {
@@ -332,7 +323,7 @@ struct LoaderIM {
         e.y = (i << 16) | j;
       } else {
         e.x = 0;
-        e.y = (row == d_patch && append_ones) ? -2 : -1;
+        e.y = -1;
       }
       table[t] = e;
     }
@@ -353,7 +344,6 @@ struct LoaderIM {
     const int ix0 = ox * sx - pw;
     const long long idx0 = ((long long)s * C * H + iy0) * (long long)W + ix0;
     r.use = 0;
-    r.one = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int2 e = table[rr + 8 * i];
@@ -362,7 +352,6 @@ struct LoaderIM {
       const bool ok = kok && e.y >= 0 && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
       r.v[i] = base[ok ? idx0 + e.x : 0];
       if (ok) r.use |= 1u << i;
-      if (kok && e.y == -2) r.one |= 1u << i;
     }
   }
 
@@ -371,8 +360,7 @@ struct LoaderIM {
     const int rr = threadIdx.x >> 5;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
-      lds[(rr + 8 * i) * Panel<ROWS>::kRowKStride + k] =
-          ((r.use >> i) & 1u) ? r.v[i] : (((r.one >> i) & 1u) ? 1.f : 0.f);
+      lds[(rr + 8 * i) * Panel<ROWS>::kRowKStride + k] = ((r.use >> i) & 1u) ? r.v[i] : 0.f;
   }
 };
 

@@ -127,7 +127,6 @@ LoaderKC<ROWS, VEC> rowmajor_kc(const float *base, int rows, int K, long long ld
   l.row_stride = (unsigned)ld;
   l.L = (unsigned)K;
   l.rows_valid = rows;
-  l.ones_row = -1;
   return l;
 }
 
