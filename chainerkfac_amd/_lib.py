@@ -32,6 +32,8 @@ PROTOTYPES = {
     'kfac_pack_plan_destroy': (c_int, [c_vp]),
     'kfac_pack_f32': (c_int, [c_vp, c_vp, c_i64, c_int, c_vp]),
     'kfac_unpack_f32': (c_int, [c_vp, c_vp, c_i64, c_int, c_int, c_vp]),
+    'kfac_pack_f16': (c_int, [c_vp, c_vp, c_i64, c_int, c_vp]),
+    'kfac_unpack_f16': (c_int, [c_vp, c_vp, c_i64, c_int, c_int, c_vp]),
     'kfac_cov_workspace_bytes': (c_sz, [c_int, c_i64]),
     'kfac_cov_linear_f32': (c_int, [c_vp, c_int, c_int, c_int, c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
     'kfac_cov_conv_a_f32': (c_int, [c_vp] + [c_int] * 11 + [c_f, c_f, c_vp, c_vp, c_sz, c_vp]),

@@ -28,6 +28,9 @@ class _ArraysInfo(object):
             for array, triangular in local_arrays:
                 if isinstance(array, torch.Tensor) and array.dtype not in (torch.float16, torch.float32):
                     raise ValueError('dtype must be float16 or float32.')
+                if isinstance(array, torch.Tensor) and array.dtype == torch.float16:
+                    raise NotImplementedError('float16 arrays are not supported (float32 arrays, float32 or '
+                                              'float16 buffer)')
                 _dev.require_gpu_tensor(array, 'array')
                 if triangular:
                     if array.ndim != 2 or array.shape[0] != array.shape[1]:
@@ -111,28 +114,39 @@ class ArrayPacker(object):
 
     @staticmethod
     def _check_buf(gpu_buf, buf_dtype, need):
-        if buf_dtype is not None and np.dtype(buf_dtype) != np.float32:
-            raise ValueError('only a float32 buffer is supported, not {}'.format(buf_dtype))
-        _dev.require_gpu_tensor(gpu_buf, 'gpu_buf')
+        """Returns 'f32' or 'f16': the element type of the wire buffer.  The
+        arrays themselves are float32; float16 is the reference's optional
+        communication dtype (pure_nccl_communicator.py:32-33)."""
+        dt = np.dtype(np.float32 if buf_dtype is None else buf_dtype)
+        if dt == np.float32:
+            kind, tdtype = 'f32', torch.float32
+        elif dt == np.float16:
+            kind, tdtype = 'f16', torch.float16
+        else:
+            raise ValueError('the buffer must be float32 or float16, not {}'.format(buf_dtype))
+        _dev.require_gpu_tensor(gpu_buf, 'gpu_buf', dtype=tdtype)
         if gpu_buf.numel() < need:
             raise ValueError('gpu_buf holds {} elements, {} needed'.format(gpu_buf.numel(), need))
+        return kind
 
     def _pack_arrays_to_buffer(self, arrays, gpu_buf, buf_dtype=np.float32, target=-1,
                                stream=None, debug=False):
         info = self._info(arrays)
         if debug and self.rank == 0:
             info.show()
-        self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
-        _lib.check(_lib.load().kfac_pack_f32(
-            info.plan, gpu_buf.data_ptr(), gpu_buf.numel(), int(target),
-            _dev.stream_handle(stream)))
+        kind = self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
+        lib = _lib.load()
+        fn = lib.kfac_pack_f16 if kind == 'f16' else lib.kfac_pack_f32
+        _lib.check(fn(info.plan, gpu_buf.data_ptr(), gpu_buf.numel(), int(target),
+                      _dev.stream_handle(stream)))
 
     def _unpack_arrays_from_buffer(self, arrays, gpu_buf, buf_dtype=np.float32, target=-1,
                                    divisor=1, stream=None, debug=False):
         info = self._info(arrays)
         if debug and self.rank == 0:
             info.show()
-        self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
-        _lib.check(_lib.load().kfac_unpack_f32(
-            info.plan, gpu_buf.data_ptr(), gpu_buf.numel(), int(target), int(divisor),
-            _dev.stream_handle(stream)))
+        kind = self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
+        lib = _lib.load()
+        fn = lib.kfac_unpack_f16 if kind == 'f16' else lib.kfac_unpack_f32
+        _lib.check(fn(info.plan, gpu_buf.data_ptr(), gpu_buf.numel(), int(target), int(divisor),
+                      _dev.stream_handle(stream)))

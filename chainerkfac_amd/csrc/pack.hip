@@ -18,6 +18,8 @@
 //           directly and to M[J, I] through an LDS transpose, so every global
 //           access is a contiguous 256-byte run per wave.  Flat arrays use
 //           4096-element chunks.
+#include <hip/hip_fp16.h>
+
 #include "common.h"
 
 namespace {
@@ -61,8 +63,23 @@ __device__ __forceinline__ int tri_row(long long t) {
   return (int)r;
 }
 
-__global__ __launch_bounds__(kThreads) void pack_kernel(PackTables tb,
-                                                        float *__restrict__ buf,
+// Element type of the packed buffer: float, or __half for the float16 wire
+// format (the arrays stay float32).  Conversions follow the reference kernels:
+// pack stores (half)value, round to nearest even; unpack divides in the
+// buffer's type, half / (half)divisor rounded to half, then widens.
+__device__ __forceinline__ void to_buf(float v, float &out) { out = v; }
+__device__ __forceinline__ void to_buf(float v, __half &out) { out = __float2half_rn(v); }
+
+__device__ __forceinline__ float from_buf(float v, int divisor) {
+  return divisor != 1 ? v / (float)divisor : v;
+}
+__device__ __forceinline__ float from_buf(__half v, int divisor) {
+  // the float quotient of two halves rounds to the correctly rounded half quotient
+  return __half2float(__float2half_rn(__half2float(v) / __half2float(__int2half_rn(divisor))));
+}
+
+template <class B>
+__global__ __launch_bounds__(kThreads) void pack_kernel(PackTables tb, B *__restrict__ buf,
                                                         int target) {
   const int unit = blockIdx.x;
   const int j = find_array(tb.pack_csum, tb.n, unit);
@@ -70,7 +87,7 @@ __global__ __launch_bounds__(kThreads) void pack_kernel(PackTables tb,
   const long long nel = tb.nel[j];
   const long long t0 = (long long)(unit - tb.pack_csum[j]) * kChunk + threadIdx.x;
   const float *__restrict__ src = tb.ptrs[j];
-  float *__restrict__ dst = buf + tb.buf_off[j];
+  B *__restrict__ dst = buf + tb.buf_off[j];
   const int d = tb.tri[j];
   float val[kPerThread];
   if (d > 0) {
@@ -99,34 +116,34 @@ __global__ __launch_bounds__(kThreads) void pack_kernel(PackTables tb,
 #pragma unroll
   for (int i = 0; i < kPerThread; ++i) {
     const long long t = t0 + (long long)i * kThreads;
-    if (t < nel) dst[t] = val[i];
+    if (t < nel) to_buf(val[i], dst[t]);
   }
 }
 
-__global__ __launch_bounds__(kThreads) void unpack_kernel(
-    PackTables tb, const float *__restrict__ buf, int target, float divisor) {
+template <class B>
+__global__ __launch_bounds__(kThreads) void unpack_kernel(PackTables tb, const B *__restrict__ buf,
+                                                          int target, int divisor) {
   __shared__ float tile[kTile][kTile + 1];
   const int unit = blockIdx.x;
   const int j = find_array(tb.unpack_csum, tb.n, unit);
   if (target >= 0 && tb.rank[j] != target) return;
   const int local = unit - tb.unpack_csum[j];
   float *__restrict__ dst = const_cast<float *>(tb.ptrs[j]);
-  const float *__restrict__ src = buf + tb.buf_off[j];
+  const B *__restrict__ src = buf + tb.buf_off[j];
   const int d = tb.tri[j];
-  const bool divide = divisor != 1.0f;
   if (d == 0) {
     const long long nel = tb.nel[j];
     const long long t0 = (long long)local * kChunk + threadIdx.x;
-    float val[kPerThread];
+    B val[kPerThread];
 #pragma unroll
     for (int i = 0; i < kPerThread; ++i) {
       const long long t = t0 + (long long)i * kThreads;
-      val[i] = (t < nel) ? src[t] : 0.f;
+      if (t < nel) val[i] = src[t];
     }
 #pragma unroll
     for (int i = 0; i < kPerThread; ++i) {
       const long long t = t0 + (long long)i * kThreads;
-      if (t < nel) dst[t] = divide ? val[i] / divisor : val[i];
+      if (t < nel) dst[t] = from_buf(val[i], divisor);
     }
     return;
   }
@@ -137,18 +154,20 @@ __global__ __launch_bounds__(kThreads) void unpack_kernel(
   const int lr0 = threadIdx.x / kTile;  // 0..3
   constexpr int kRowsPerPass = kThreads / kTile;
   constexpr int kPasses = kTile / kRowsPerPass;
-  float val[kPasses];
+  B val[kPasses];
+  bool have[kPasses];
 #pragma unroll
   for (int p = 0; p < kPasses; ++p) {
     const int lr = lr0 + p * kRowsPerPass;
     const int r = I * kTile + lr;
     const int c = J * kTile + lc;
-    val[p] = (r < d && c <= r) ? src[(long long)r * (r + 1) / 2 + c] : 0.f;
+    have[p] = r < d && c <= r;
+    if (have[p]) val[p] = src[(long long)r * (r + 1) / 2 + c];
   }
 #pragma unroll
   for (int p = 0; p < kPasses; ++p) {
     const int lr = lr0 + p * kRowsPerPass;
-    tile[lr][lc] = divide ? val[p] / divisor : val[p];
+    tile[lr][lc] = have[p] ? from_buf(val[p], divisor) : 0.f;
   }
   __syncthreads();
   if (I == J) {
@@ -301,8 +320,10 @@ extern "C" int kfac_pack_plan_destroy(kfac_pack_plan_t plan) {
   return KFAC_OK;
 }
 
-extern "C" int kfac_pack_f32(kfac_pack_plan_t plan, float *buf,
-                             int64_t buf_nelems, int target_rank, void *stream) {
+namespace {
+
+template <class B>
+int run_pack(kfac_pack_plan_t plan, B *buf, int64_t buf_nelems, int target_rank, void *stream) {
   KFAC_REQUIRE(plan != nullptr, "plan is null");
   KFAC_REQUIRE(buf_nelems >= plan->total_packed,
                "buffer holds %lld elements, %lld needed", (long long)buf_nelems,
@@ -310,15 +331,15 @@ extern "C" int kfac_pack_f32(kfac_pack_plan_t plan, float *buf,
   if (plan->pack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
   kfac::TimedLaunch timed(KFAC_TIMED_PACK, kfac::as_stream(stream));
-  hipLaunchKernelGGL(pack_kernel, dim3(plan->pack_units), dim3(kThreads), 0,
+  hipLaunchKernelGGL(pack_kernel<B>, dim3(plan->pack_units), dim3(kThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
 
-extern "C" int kfac_unpack_f32(kfac_pack_plan_t plan, const float *buf,
-                               int64_t buf_nelems, int target_rank, int divisor,
-                               void *stream) {
+template <class B>
+int run_unpack(kfac_pack_plan_t plan, const B *buf, int64_t buf_nelems, int target_rank,
+               int divisor, void *stream) {
   KFAC_REQUIRE(plan != nullptr, "plan is null");
   KFAC_REQUIRE(divisor != 0, "divisor is 0");
   KFAC_REQUIRE(buf_nelems >= plan->total_packed,
@@ -327,9 +348,31 @@ extern "C" int kfac_unpack_f32(kfac_pack_plan_t plan, const float *buf,
   if (plan->unpack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
   kfac::TimedLaunch timed(KFAC_TIMED_UNPACK, kfac::as_stream(stream));
-  hipLaunchKernelGGL(unpack_kernel, dim3(plan->unpack_units), dim3(kThreads), 0,
-                     kfac::as_stream(stream), plan->tables(), buf, target_rank,
-                     (float)divisor);
+  hipLaunchKernelGGL(unpack_kernel<B>, dim3(plan->unpack_units), dim3(kThreads), 0,
+                     kfac::as_stream(stream), plan->tables(), buf, target_rank, divisor);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
+}
+
+}  // namespace
+
+extern "C" int kfac_pack_f32(kfac_pack_plan_t plan, float *buf, int64_t buf_nelems,
+                             int target_rank, void *stream) {
+  return run_pack(plan, buf, buf_nelems, target_rank, stream);
+}
+
+extern "C" int kfac_unpack_f32(kfac_pack_plan_t plan, const float *buf, int64_t buf_nelems,
+                               int target_rank, int divisor, void *stream) {
+  return run_unpack(plan, buf, buf_nelems, target_rank, divisor, stream);
+}
+
+extern "C" int kfac_pack_f16(kfac_pack_plan_t plan, void *buf, int64_t buf_nelems,
+                             int target_rank, void *stream) {
+  return run_pack(plan, static_cast<__half *>(buf), buf_nelems, target_rank, stream);
+}
+
+extern "C" int kfac_unpack_f16(kfac_pack_plan_t plan, const void *buf, int64_t buf_nelems,
+                               int target_rank, int divisor, void *stream) {
+  return run_unpack(plan, static_cast<const __half *>(buf), buf_nelems, target_rank, divisor,
+                    stream);
 }

@@ -76,6 +76,16 @@ int kfac_pack_f32(kfac_pack_plan_t plan, float *buf, int64_t buf_nelems,
 int kfac_unpack_f32(kfac_pack_plan_t plan, const float *buf, int64_t buf_nelems,
                     int target_rank, int divisor, void *stream);
 
+/* The same with a float16 buffer (the arrays stay float32), the reference's
+ * fp16 communication dtype: pack stores (half)value, round to nearest even
+ * (pure_nccl_communicator.py:354-363); unpack divides in half precision,
+ * buf[i] / (half)divisor, then widens (pure_nccl_communicator.py:438-449).
+ * buf_nelems counts halves. */
+int kfac_pack_f16(kfac_pack_plan_t plan, void *buf, int64_t buf_nelems,
+                  int target_rank, void *stream);
+int kfac_unpack_f16(kfac_pack_plan_t plan, const void *buf, int64_t buf_nelems,
+                    int target_rank, int divisor, void *stream);
+
 /* ------------------------------------------------------------------------
  * (1) Kronecker-factor construction:  C = beta*C + alpha * P^T P
  *     beta = 1, alpha = scale/acc_iters gives the running accumulation of

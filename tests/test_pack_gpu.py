@@ -127,3 +127,66 @@ def test_resnet50d_factor_list_round_trip_bit_exact(pack_oracle_c):
     ref = np.zeros(O.get_nelems(host), np.float32)
     pack_oracle_c.pack(host, ref)
     assert np.array_equal(buf[n - ref.size:].cpu().numpy(), ref)
+
+
+def _half_stress_values(n, seed):
+    """float32 values that exercise float16 rounding: ties, subnormals, overflow, signed zeros."""
+    r = np.random.default_rng(seed)
+    v = (r.standard_normal(n) * np.exp(r.uniform(-12, 12, n))).astype(np.float32)
+    special = np.array([0.0, -0.0, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 65504.0, 65520.0, 65519.9, 1e6, -1e6,
+                        2.0 ** -24, 2.0 ** -25, 3 * 2.0 ** -25, 6.1e-5, -5.96e-8, 2049.0, 2051.0], np.float32)
+    v[:special.size] = special[:min(special.size, n)]
+    return v
+
+
+@pytest.mark.parametrize('target', [-1, 1, 4])
+def test_pack_float16_buffer_matches_oracle(target):
+    """Round to nearest even into a half buffer (pure_nccl_communicator.py:354-363)."""
+    from chainerkfac_amd.communicators import ArrayPacker
+    host = make(5, RAGGED)
+    for la in host:
+        for a, _ in la:
+            a.reshape(-1)[:] = _half_stress_values(a.size, a.size)
+    dev = to_dev(host)
+    n = O.get_nelems(host)
+    ref = np.full(n, -3.0, np.float16)
+    with np.errstate(over='ignore'):
+        O.pack(host, ref, target)
+    small = [[la[0]] if la else [] for la in host]
+    assert np.array_equal(O.pack(small, np.zeros(O.get_nelems(small), np.float16)).view(np.uint16),
+                          O.pack_bruteforce(small, np.zeros(O.get_nelems(small), np.float16)).view(np.uint16))
+    buf = torch.full((n,), -3.0, dtype=torch.float16, device='cuda')
+    ArrayPacker()._pack_arrays_to_buffer(dev, buf, np.float16, target, None)
+    got = buf.cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize('target,divisor', [(-1, 1), (-1, 4), (1, 3), (-1, 7), (4, 2048)])
+def test_unpack_float16_buffer_matches_oracle(target, divisor):
+    """buf[i] / (half)divisor in half precision, then widened (pure_nccl_communicator.py:438-449)."""
+    from chainerkfac_amd.communicators import ArrayPacker
+    host = make(6, RAGGED)
+    n = O.get_nelems(host)
+    with np.errstate(over='ignore'):
+        bufh = _half_stress_values(n, 8).astype(np.float16)   # values past 65504 become inf on purpose
+    ref = [[(np.full_like(a, 9.0), t) for a, t in la] for la in host]
+    O.unpack(ref, bufh, target, divisor)
+    dev = [[(torch.full_like(torch.from_numpy(a), 9.0).cuda(), t) for a, t in la] for la in host]
+    ArrayPacker()._unpack_arrays_from_buffer(dev, torch.from_numpy(bufh).cuda(), np.float16, target, divisor, None)
+    for lr, ld in zip(ref, dev):
+        for (a, _), (b, _) in zip(lr, ld):
+            assert np.array_equal(a.view(np.uint32), b.cpu().numpy().view(np.uint32))
+
+
+def test_float16_arrays_and_wrong_buffer_dtype_are_rejected():
+    from chainerkfac_amd.communicators import ArrayPacker
+    p = ArrayPacker()
+    with pytest.raises(NotImplementedError):
+        p._pack_arrays_to_buffer([[(torch.zeros(4, dtype=torch.float16, device='cuda'), False)]],
+                                 torch.zeros(4, device='cuda'))
+    with pytest.raises(ValueError):
+        p._pack_arrays_to_buffer([[(torch.zeros(4, device='cuda'), False)]],
+                                 torch.zeros(4, device='cuda'), np.float16)   # float32 tensor, float16 declared
+    with pytest.raises(ValueError):
+        p._pack_arrays_to_buffer([[(torch.zeros(4, device='cuda'), False)]],
+                                 torch.zeros(4, dtype=torch.float64, device='cuda'), np.float64)
