@@ -35,6 +35,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix peak
+HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E peak
 # HBM bytes per covariance SYRK launch (average over the 161 launches of a step):
 # hardware counters FETCH_SIZE and WRITE_SIZE collected with `rocprofv3 --pmc` on
 # this script (--no-graph --calibrate-copy), each scaled by what it reads for the
@@ -169,6 +170,26 @@ def run_gpu(args):
 
     phase_ms = {'cov': timed(cov_phase), 'inverse': timed(inv_phase), 'precondition': timed(pre_phase)}
 
+    # wire format of the factors (outside the step: what a communicator would do with them): pack the
+    # lower triangles of all 161 factors into one buffer and unpack them again, HBM-bound
+    from chainerkfac_amd.communicators import ArrayPacker
+    packer = ArrayPacker()
+    arrays = [[(cov, True) for fb in opt.fblocks for cov in fb.covs]]
+    nel = packer.get_nelems(arrays)
+    wire = torch.empty(nel, dtype=torch.float32, device=dev)
+    full = sum(c.numel() for c, _ in arrays[0])
+    packer._pack_arrays_to_buffer(arrays, wire)
+    packer._unpack_arrays_from_buffer(arrays, wire)
+    pack_ms = timed(lambda: packer._pack_arrays_to_buffer(arrays, wire), reps=10)
+    unpack_ms = timed(lambda: packer._unpack_arrays_from_buffer(arrays, wire), reps=10)
+    wire_stats = {
+        'pack': {'ms': round(pack_ms, 4), 'GBps': round(8.0 * nel / pack_ms / 1e6, 1),
+                 'frac_of_hbm_peak': round(8.0 * nel / pack_ms / 1e6 / HBM_PEAK_GBPS, 3)},
+        'unpack': {'ms': round(unpack_ms, 4), 'GBps': round(4.0 * (nel + full) / unpack_ms / 1e6, 1),
+                   'frac_of_hbm_peak': round(4.0 * (nel + full) / unpack_ms / 1e6 / HBM_PEAK_GBPS, 3)},
+        'packed_MB': round(4.0 * nel / 1e6, 1), 'full_MB': round(4.0 * full / 1e6, 1),
+    }
+
     # dominant kernel family, timed launch by launch inside the library
     _lib.check(lib.kfac_timing_enable(1))
     step()
@@ -226,6 +247,7 @@ def run_gpu(args):
                       inverse_executed=round(dense_inverse_flops / 1e9, 1)),
         'kernel_ms': {k: {'launches': n, 'total_ms': round(ms, 3)} for k, (n, ms) in fam.items()},
         'inverse_info_nonzero': info_bad,
+        'wire_format': wire_stats,
         'roofline': {
             'kernel': 'syrk_kernel (covariance, all loaders)',
             'bound': 'mfma',
