@@ -40,7 +40,7 @@ HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E peak
 # hardware counters FETCH_SIZE and WRITE_SIZE collected with `rocprofv3 --pmc` on
 # this script (--no-graph --calibrate-copy), each scaled by what it reads for the
 # 256 MiB calibration copy; the counter summary is kept under profiles/.
-SYRK_HBM_BYTES_PER_LAUNCH = 44.1e6
+SYRK_HBM_BYTES_PER_LAUNCH = 41.6e6
 BATCH = 32
 DAMPING = 2.5e-4
 STAB_COEFF = 16.0
