@@ -22,16 +22,21 @@
 // just before it is factored, K up to (kGroup-1)*NB), and after a group every
 // column to its right receives the whole group at once (K = kGroup*NB), which
 // reads and writes each trailing tile once per group instead of once per
-// column.  Per block column k:
+// column.  Per block column k, two dependent launches:
 //
-//   column(k)  (*) for the tiles of column k, j over the group's columns < k
-//   diag(k)    one workgroup per matrix: Cholesky of the diagonal tile and
-//              U_kk = L_kk^-T inside LDS on 32x32 MFMA blocks
+//   step(k)    one workgroup per matrix gives the diagonal tile the products it
+//              is still owed, then does its Cholesky and U_kk = L_kk^-T inside
+//              LDS on 32x32 MFMA blocks; the other workgroups of the launch
+//              apply (*) to the rest of column k (inside a group: the group's
+//              earlier columns; on a group's first column: the previous group,
+//              for both columns of this group)
 //   panel(k)   M(x,k) = M(x,k) U_kk for x != k  (L(x,k) below, U(x,k) above)
 //
-// and after the group's last column  trailing(g): (*) for all tiles right of
-// the group.  A final launch forms  out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T
-// (lauum) and writes the full symmetric inverse.  The tiles of every launch are
+// and after a group's last column, on a second stream beside the next group's
+// sweep, rest(g): (*) for all tiles right of the next group.  A final launch
+// forms  out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T  (lauum) and writes the full
+// symmetric inverse.  Matrices of different sizes end their sweeps together (a
+// matrix of T tiles joins at step max_T - T).  The tiles of every launch are
 // listed in a task table built once per plan.
 //
 // Replaces chainerkfac/optimizers/cholesky_inverse.py:16-102 (potrf + potrs
@@ -59,6 +64,7 @@ struct InvTables {
   const int *orig;           // [count] slot -> caller index
   const int *dim;            // [count]
   const int *nt;             // [count] tiles per side
+  const int *shift;          // [count] sweep step at which the matrix starts
   const long long *ws_off;   // [count] float offset of the padded matrix
   const int *tile_cs;        // [count+1] cumulative lower-tile counts
   const int *panel_cs;       // [count+1] cumulative (nt-1)
@@ -265,17 +271,26 @@ __device__ __forceinline__ void wave_visit(const floatx16 &acc, F f) {
   for (int v = 0; v < 16; ++v) f(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), lane & 31, acc[v]);
 }
 
-__global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
-  extern __shared__ float smem[];
+// Diagonal tile (k,k) of matrix s: first the products it is still owed,
+//   C(k,k) -= sum_{j = lo .. hi} M(k,j) M(k,j)^T        (nothing when hi < lo),
+// through the shared main loop (the other tiles of the column receive theirs
+// from the update workgroups of the same launch), then the factorisation.
+__device__ __forceinline__ void diag_role(const InvTables &tb, int s, int k, int lo, int hi,
+                                          float *smem) {
   float *S = smem;                      // NB x LS working tile
-  float *scratch = smem + NB * LS;      // 4 waves x SB x PS
-  const int s = blockIdx.x;
+  float *scratch = smem + NB * LS;      // 3 waves x SB x PS
   const int d = tb.dim[s];
   constexpr int ld = NB;
   float *tile = tile_ptr(tb, s, k, k);
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  {
+  if (hi >= lo) {
+    floatx16 acc[2][2];
+    fill_acc<2, 2>(acc, [&](int rr, int cc) { return -tile[rr * NB + cc]; });
+    const LoaderTile la{tile_ptr(tb, s, k, lo)};
+    tile_mainloop<true>(la, la, (hi - lo + 1) * NB, smem, acc);   // ends with a barrier
+    for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { S[rr * LS + cc] = -v; });
+  } else {
     const int c4 = (threadIdx.x & 31) * 4, r0 = threadIdx.x >> 5;
 #pragma unroll 4
     for (int p = 0; p < NB / 8; ++p) {
@@ -366,9 +381,10 @@ __global__ __launch_bounds__(256) void diag_kernel(InvTables tb, int k) {
 // ---------------------------------------------------------------------------
 // M(x,k) = M(x,k) W^T = M(x,k) U_kk in place for every x != k; the operand
 // W^T is the diagonal tile itself, read transposed.
-__global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, int nactive) {
+__global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int step, int nactive) {
   extern __shared__ float lds[];
   const int s = find_slot(tb.panel_cs, nactive, blockIdx.x);
+  const int k = step - tb.shift[s];
   const int local = blockIdx.x - tb.panel_cs[s];
   const int x = local < k ? local : local + 1;
   float *tile = tile_ptr(tb, s, x, k);
@@ -383,9 +399,8 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int k, 
 // from -C, so the tile is read while the first operand panels are in flight and
 // the epilogue is a plain store.  An upper tile whose row lies inside [k0, k1]
 // receives its first product here and is overwritten (it holds stale data).
-__global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0, int k0, int k1) {
-  extern __shared__ float lds[];
-  const int2 task = tb.tasks[task0 + blockIdx.x];
+__device__ __forceinline__ void update_role(const InvTables &tb, int2 task, int k0, int k1,
+                                            float *lds) {
   const int s = task.x;
   const int a = task.y & 0xffff, b = task.y >> 16;
   const bool upper = a < b;
@@ -405,6 +420,46 @@ __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int ta
   else
     tile_mainloop<false>(la, lb, K, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[rr * NB + cc] = -v; });
+}
+
+// The group's block columns [step0, step1] in matrix s's own numbering (a
+// matrix that starts inside the group has a shorter first group).
+__device__ __forceinline__ void local_range(const InvTables &tb, int s, int step0, int step1,
+                                            int &k0, int &k1) {
+  const int shift = tb.shift[s];
+  k0 = step0 > shift ? step0 - shift : 0;
+  k1 = step1 - shift;
+}
+
+// One launch per sweep step: workgroups [0, ndiag) factor the diagonal tile of
+// their matrix (after giving it the products of columns [step0, step1]), the
+// others apply the same columns to the tiles the next panel step reads.  The
+// diagonal workgroups come first in launch order, so the serial part starts at
+// once and the updates fill the rest of the GPU beside it.
+__global__ __launch_bounds__(THREADS, 2) void step_kernel(InvTables tb, int step, int ndiag,
+                                                          int task0, int step0, int step1) {
+  extern __shared__ float lds[];
+  if ((int)blockIdx.x < ndiag) {
+    const int s = blockIdx.x;
+    int k0, k1;
+    local_range(tb, s, step0, step1, k0, k1);
+    diag_role(tb, s, step - tb.shift[s], k0, k1, lds);
+  } else {
+    const int2 task = tb.tasks[task0 + blockIdx.x - ndiag];
+    int k0, k1;
+    local_range(tb, task.x, step0, step1, k0, k1);
+    update_role(tb, task, k0, k1, lds);
+  }
+}
+
+// The part of a trailing update that the next group's sweep does not read.
+__global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0, int step0,
+                                                            int step1) {
+  extern __shared__ float lds[];
+  const int2 task = tb.tasks[task0 + blockIdx.x];
+  int k0, k1;
+  local_range(tb, task.x, step0, step1, k0, k1);
+  update_role(tb, task, k0, k1, lds);
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
@@ -433,10 +488,15 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int cou
   });
 }
 
-// 83 KB: small enough to share a CU with two workgroups of the tile kernels,
-// so a diagonal step does not have to wait for a CU to drain while a trailing
-// update runs beside the sweep.
-constexpr size_t kDiagLds = (size_t)(NB * LS + 4 * SB * PS) * sizeof(float);
+// Dynamic LDS of the step kernel: the diagonal role's working tile and three
+// private blocks (at most three waves are busy in a pass of the triangular
+// inverse), 77 KB, so that two workgroups share a CU like the other tile kernels.
+constexpr size_t kDiagLds = (size_t)(NB * LS + 3 * SB * PS) * sizeof(float);
+constexpr size_t kStepLds = kDiagLds > kTileLdsBytes ? kDiagLds : kTileLdsBytes;
+static_assert(2 * kStepLds <= 160 * 1024, "two step workgroups must fit a CU");
+constexpr size_t kRestLdsBytes = 81 * 1024;
+static_assert(2 * kRestLdsBytes > 160 * 1024 && kRestLdsBytes + kStepLds <= 160 * 1024,
+              "one rest workgroup per CU, with room for a step workgroup");
 
 }  // namespace
 
@@ -453,13 +513,17 @@ struct kfac_inverse_plan {
   std::vector<int> nt;             // per slot
   std::vector<int> nactive;        // per step
   std::vector<int> panel_total;    // per step
-  std::vector<UpdateLaunch> column;    // per step: left-looking update of column k
-  // per step, set on the last column of a group: the tiles of the next group's
-  // columns ("urgent") and everything right of them ("rest")
-  std::vector<UpdateLaunch> urgent, rest;
+  // per step: the update tasks that share the launch with the diagonal tiles:
+  // inside a group the left-looking update of column k, on a group's first
+  // column the previous group's trailing update of this group's columns
+  std::vector<UpdateLaunch> with_diag;
+  // per step, set on the last column of a group: its trailing update of
+  // everything right of the next group
+  std::vector<UpdateLaunch> rest;
   // The rest of a trailing update touches nothing the next group's sweep needs,
   // so it runs on a second stream beside that sweep.
   bool lookahead = true;
+  size_t rest_lds = 0;
   hipStream_t side = nullptr;
   std::vector<hipEvent_t> ev_main, ev_side;   // per step
   ~kfac_inverse_plan() {
@@ -470,7 +534,7 @@ struct kfac_inverse_plan {
   int total_tiles = 0;
   size_t ws_floats = 0;            // padded matrices
   std::vector<const void *> in_sorted, out_sorted;
-  kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_off, d_tile, d_panel, d_tasks;
+  kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_shift, d_off, d_tile, d_panel, d_tasks;
   bool attr_set = false;
 };
 
@@ -532,58 +596,97 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   p->total_tiles = tile_cs[count];
   p->max_t = count ? p->nt[0] : 0;
   std::vector<int2> tasks, natural;
-  p->column.resize(p->max_t);
-  p->urgent.resize(p->max_t);
+  p->with_diag.resize(p->max_t);
   p->rest.resize(p->max_t);
   if (const char *e = getenv("KFAC_INVERSE_LOOKAHEAD")) p->lookahead = atoi(e) != 0;
+  // The rest asks for more LDS than it uses, 81 KB: then one of its workgroups
+  // fits a CU, not two, and a step or panel workgroup always finds room beside
+  // it instead of queueing behind the rest for a slot (measured: the rest alone
+  // loses 14 %, the sweep as a whole gains).  KFAC_INVERSE_REST_LDS overrides.
+  p->rest_lds = kRestLdsBytes;
+  if (const char *e = getenv("KFAC_INVERSE_REST_LDS")) {
+    const long v = atol(e);
+    if (v >= (long)kTileLdsBytes && v <= 160 * 1024) p->rest_lds = (size_t)v;
+  }
   auto pack = [](int s, int a, int b) { return make_int2(s, a | (b << 16)); };
-  for (int k = 0; k < p->max_t; ++k) {
+  // Matrix s joins the sweep at step shift[s] and runs nt[s] steps.  Aligning
+  // the ends (shift = max_t - nt) puts the short sweeps of the small matrices
+  // beside the late steps of the largest ones, which on their own leave most of
+  // the GPU idle (few tiles, one dependent launch after another); aligning the
+  // starts piles all matrices onto the early steps, which are the ones that are
+  // already throughput-bound.  KFAC_INVERSE_ALIGN=<percent> (0 = starts, 100 =
+  // ends) is a tuning override.
+  int align = 100;
+  if (const char *e = getenv("KFAC_INVERSE_ALIGN")) align = std::min(100, std::max(0, atoi(e)));
+  std::vector<int> shift(count);
+  for (int s = 0; s < count; ++s) shift[s] = (p->max_t - p->nt[s]) * align / 100;
+  // Tiles right of the source group [s0, s1] (sweep steps) that receive its
+  // products: the columns of the following group when `next`, otherwise
+  // everything right of those.  The upper tiles whose row lies inside the source
+  // group have shorter sums and go to `tail`.  The following group's first
+  // diagonal tile is left to its diagonal workgroup.
+  auto trailing = [&](bool next, int s0, int s1, std::vector<int2> &body, std::vector<int2> &tail) {
+    for (int s = 0; s < count; ++s) {
+      const int T = p->nt[s];
+      const int k1 = s1 - shift[s];
+      if (k1 < 0 || k1 >= T) continue;   // not in the sweep during the source group
+      const int k0 = std::max(s0 - shift[s], 0);
+      const int ku = k1 + p->group;
+      const int c_lo = next ? k1 + 1 : ku + 1;
+      const int c_hi = next ? std::min(ku, T - 1) : T - 1;
+      for (int n = c_lo; n <= c_hi; ++n)
+        for (int m = n; m < T; ++m)
+          if (!(next && m == c_lo)) body.push_back(pack(s, m, n));
+      for (int a = 0; a < k0; ++a)
+        for (int b = c_lo; b <= c_hi; ++b) body.push_back(pack(s, a, b));
+      for (int a = k0; a <= k1; ++a)
+        for (int b = c_lo; b <= c_hi; ++b) tail.push_back(pack(s, a, b));
+    }
+  };
+  for (int g = 0; g < p->max_t; ++g) {
+    // active matrices: shift <= g < shift + nt; a prefix of the sorted order
+    // (shift grows and shift + nt shrinks with the slot number)
     int na = 0;
-    while (na < count && p->nt[na] > k) ++na;
+    while (na < count && shift[na] <= g && g < shift[na] + p->nt[na]) ++na;
     p->nactive.push_back(na);
     p->panel_total.push_back(panel_cs[na]);
-    const int k0 = k / p->group * p->group;
-    const int k1 = std::min(k0 + p->group - 1, p->max_t - 1);
-    if (k > k0) {
-      // column k of every active matrix: products of columns k0 .. k-1
-      natural.clear();
+    const int g0 = g / p->group * p->group;
+    const int g1 = std::min(g0 + p->group - 1, p->max_t - 1);
+    UpdateLaunch &w = p->with_diag[g];
+    std::vector<int2> tail;
+    natural.clear();
+    if (g > g0) {
+      // column g - shift of every active matrix: products of the group's earlier
+      // columns (the diagonal tile takes its own inside the diagonal workgroup)
+      w.k0 = g0;
+      w.k1 = g - 1;
       for (int s = 0; s < na; ++s) {
-        for (int m = k; m < p->nt[s]; ++m) natural.push_back(pack(s, m, k));
+        const int k = g - shift[s], k0 = std::max(g0 - shift[s], 0);
+        if (k <= k0) continue;
+        for (int m = k + 1; m < p->nt[s]; ++m) natural.push_back(pack(s, m, k));
         for (int a = 0; a < k; ++a) natural.push_back(pack(s, a, k));
       }
-      p->column[k].task0 = (int)tasks.size();
-      p->column[k].count = (int)natural.size();
-      p->column[k].k0 = k0;
-      p->column[k].k1 = k - 1;
-      append_tasks(tasks, natural);
+    } else {
+      // first column of a group: the previous group's products for this group's columns
+      w.k0 = g0 - p->group;
+      w.k1 = g0 - 1;
+      if (g > 0) trailing(true, w.k0, w.k1, natural, tail);
     }
-    if (k == k1) {
-      // every column right of the group: products of columns k0 .. k1, split at
-      // the end of the next group; the upper tiles whose row lies inside the
-      // group have shorter sums and go last
-      const int ku = k1 + p->group;   // last urgent column
-      for (int part = 0; part < 2; ++part) {
-        natural.clear();
-        std::vector<int2> tail;
-        for (int s = 0; s < count && p->nt[s] > k1 + 1; ++s) {
-          const int T = p->nt[s];
-          const int c_lo = part == 0 ? k1 + 1 : ku + 1;
-          const int c_hi = part == 0 ? std::min(ku, T - 1) : T - 1;
-          for (int n = c_lo; n <= c_hi; ++n)
-            for (int m = n; m < T; ++m) natural.push_back(pack(s, m, n));
-          for (int a = 0; a < k0; ++a)
-            for (int b = c_lo; b <= c_hi; ++b) natural.push_back(pack(s, a, b));
-          for (int a = k0; a <= k1; ++a)
-            for (int b = c_lo; b <= c_hi; ++b) tail.push_back(pack(s, a, b));
-        }
-        UpdateLaunch &u = part == 0 ? p->urgent[k] : p->rest[k];
-        u.task0 = (int)tasks.size();
-        u.count = (int)(natural.size() + tail.size());
-        u.k0 = k0;
-        u.k1 = k1;
-        append_tasks(tasks, natural);
-        append_tasks(tasks, tail);
-      }
+    w.task0 = (int)tasks.size();
+    w.count = (int)(natural.size() + tail.size());
+    append_tasks(tasks, natural);
+    append_tasks(tasks, tail);
+    if (g == g1 && g1 + 1 < p->max_t) {
+      natural.clear();
+      tail.clear();
+      trailing(false, g0, g1, natural, tail);
+      UpdateLaunch &u = p->rest[g];
+      u.task0 = (int)tasks.size();
+      u.count = (int)(natural.size() + tail.size());
+      u.k0 = g0;
+      u.k1 = g1;
+      append_tasks(tasks, natural);
+      append_tasks(tasks, tail);
     }
   }
   if (tasks.empty()) tasks.push_back(make_int2(0, 0));
@@ -594,6 +697,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_orig, p->order.data(), sizeof(int) * count);
   up(p->d_dim, dim.data(), sizeof(int) * count);
   up(p->d_nt, p->nt.data(), sizeof(int) * count);
+  up(p->d_shift, shift.data(), sizeof(int) * count);
   up(p->d_off, off.data(), sizeof(long long) * count);
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
   up(p->d_panel, panel_cs.data(), sizeof(int) * (count + 1));
@@ -656,14 +760,15 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   rc = plan->d_out.set(plan->out_sorted.data(), sizeof(void *) * count, s);
   if (rc != KFAC_OK) return rc;
   if (!plan->attr_set) {
-    KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(diag_kernel),
+    KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(step_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kDiagLds));
+                                       (int)kStepLds));
     for (const void *f : {reinterpret_cast<const void *>(panel_kernel),
-                          reinterpret_cast<const void *>(update_kernel),
                           reinterpret_cast<const void *>(lauum_kernel)})
       KFAC_HIP_CHECK(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize,
                                          (int)kTileLdsBytes));
+    KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(update_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     plan->attr_set = true;
   }
   InvTables tb;
@@ -672,6 +777,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.orig = plan->d_orig.as<const int>();
   tb.dim = plan->d_dim.as<const int>();
   tb.nt = plan->d_nt.as<const int>();
+  tb.shift = plan->d_shift.as<const int>();
   tb.ws_off = plan->d_off.as<const long long>();
   tb.tile_cs = plan->d_tile.as<const int>();
   tb.panel_cs = plan->d_panel.as<const int>();
@@ -682,38 +788,58 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
 
   hipLaunchKernelGGL(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
   KFAC_HIP_CHECK(hipGetLastError());
-  auto update = [&](const UpdateLaunch &u, hipStream_t st) {
-    if (u.count == 0) return;
-    kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
-    hipLaunchKernelGGL(update_kernel, dim3(u.count), dim3(THREADS), kTileLdsBytes, st, tb, u.task0,
-                       u.k0, u.k1);
+  // Side stream: after the last column of a group, the rest of its trailing
+  // update.  It is queued just after the next step's launch, so that the step's
+  // workgroups (the serial part of the sweep) are placed first and the rest
+  // fills the GPU around them.
+  int pending = -1;    // step of the latest work queued on the side stream
+  int deferred = -1;   // step whose rest is still to be queued
+  auto queue_rest = [&]() -> int {
+    if (deferred < 0) return KFAC_OK;
+    const UpdateLaunch &r = plan->rest[deferred];
+    hipStream_t st = s;
+    if (plan->lookahead) {
+      KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_main[deferred], 0));
+      st = plan->side;
+    }
+    {
+      kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
+      hipLaunchKernelGGL(update_kernel, dim3(r.count), dim3(THREADS), plan->rest_lds, st, tb,
+                         r.task0, r.k0, r.k1);
+    }
+    if (plan->lookahead) {
+      KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[deferred], plan->side));
+      pending = deferred;
+    }
+    deferred = -1;
+    return KFAC_OK;
   };
-  // Side stream: after the last column of a group, the rest of its trailing update.
-  int pending = -1;   // step of the latest work queued on the side stream
   for (int k = 0; k < plan->max_t; ++k) {
     const int na = plan->nactive[k];
-    update(plan->column[k], s);
-    hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(256), kDiagLds, s, tb, k);
+    const UpdateLaunch &w = plan->with_diag[k];
+    // A group's first step applies the previous group to this group's columns,
+    // tiles that the rest of the group before that one (two back) also updated.
+    // The rest of the previous group itself only touches columns further right
+    // and runs beside this group's sweep.
+    const int two_back = k - 1 - plan->group;
+    if (plan->lookahead && k % plan->group == 0 && two_back >= 0 && plan->rest[two_back].count > 0)
+      KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[two_back], 0));
+    if (!plan->lookahead)
+      if (int rc2 = queue_rest()) return rc2;   // one stream: keep the program order
+    {
+      kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, s);
+      hipLaunchKernelGGL(step_kernel, dim3(na + w.count), dim3(THREADS), kStepLds, s, tb, k, na,
+                         w.task0, w.k0, w.k1);
+    }
+    if (int rc2 = queue_rest()) return rc2;
     if (plan->panel_total[k] > 0)
       hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), kTileLdsBytes, s,
                          tb, k, na);
-    if (plan->urgent[k].count > 0) {
-      // the urgent tiles were also targets of the previous group's rest
-      if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
-      pending = -1;
-      update(plan->urgent[k], s);
-    }
     if (plan->rest[k].count == 0) continue;
-    if (!plan->lookahead) {
-      update(plan->rest[k], s);
-      continue;
-    }
-    KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
-    KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_main[k], 0));
-    update(plan->rest[k], plan->side);
-    KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[k], plan->side));
-    pending = k;
+    if (plan->lookahead) KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
+    deferred = k;
   }
+  if (int rc2 = queue_rest()) return rc2;
   if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
   KFAC_HIP_CHECK(hipGetLastError());
   {
@@ -724,3 +850,4 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
+
