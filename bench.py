@@ -104,24 +104,25 @@ def run_gpu(args):
     model, calls = build_model(layers, dev, gen)
     opt = KFAC(damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0)
     opt.bn_lowrank_inverse = not args.dense_bn_inverse
+    opt.lanes = args.lanes
     opt = opt.setup(model)
-    by_name = {fb.linkname: fb for fb in opt.fblocks}
-    work = [(by_name['/' + name], func, in_data, (gy,)) for name, func, in_data, gy in calls]
+    work = [(func, in_data, (gy,)) for _, func, in_data, gy in calls]
     assert len(opt.fblocks) == len(layers)
+    hook = opt.kfhook
 
+    # the calls the function hooks make during forward/backward, then KFAC.update_kfgrads in its three parts
     def cov_phase():
-        for fb, func, in_data, gy in work:
-            fb.forward_postprocess(func, in_data)
-            fb.backward_preprocess(func, in_data, gy)
+        for func, in_data, gy in work:
+            hook.forward_postprocess(func, in_data)
+            hook.backward_preprocess(func, in_data, gy)
+        opt._lanes.join()
 
     def inv_phase():
-        for fb in opt.fblocks:
-            fb.update_cov_emas()
+        opt.update_cov_emas(opt.fblocks)
         opt.update_invs_batched(opt.fblocks)
 
     def pre_phase():
-        for fb in opt.fblocks:
-            fb.update_kfgrads()
+        opt.precondition(opt.fblocks)
 
     def step():
         cov_phase()
@@ -132,23 +133,23 @@ def run_gpu(args):
         step()
     torch.cuda.synchronize()
 
-    graph = None
-    if not args.no_graph:
-        # the step is a fixed sequence of launches on fixed buffers: replay it
-        # from one HIP graph so the host only pays for a single launch
+    def capture(fn):
+        """The launches of ``fn`` as one HIP graph (fixed sequence, fixed buffers):
+        the host then pays for a single launch per replay."""
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            step()
+            fn()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-        graph.replay()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        g.replay()
         torch.cuda.synchronize()
+        return g.replay
 
-    run = graph.replay if graph is not None else step
+    run = step if args.no_graph else capture(step)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -156,7 +157,7 @@ def run_gpu(args):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # per-phase split (eager, events on the launch stream)
+    # per-phase split: each phase launched the same way as the step (its own graph), timed with events
     def timed(fn, reps=3):
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
@@ -168,7 +169,8 @@ def run_gpu(args):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / reps
 
-    phase_ms = {'cov': timed(cov_phase), 'inverse': timed(inv_phase), 'precondition': timed(pre_phase)}
+    phases = {'cov': cov_phase, 'inverse': inv_phase, 'precondition': pre_phase}
+    phase_ms = {k: timed(fn if args.no_graph else capture(fn)) for k, fn in phases.items()}
 
     # wire format of the factors (outside the step: what a communicator would do with them): pack the
     # lower triangles of all 161 factors into one buffer and unpack them again, HBM-bound
@@ -191,9 +193,12 @@ def run_gpu(args):
     }
 
     # dominant kernel family, timed launch by launch inside the library
+    # (one stream: with lanes, launches overlap and the time between a launch's events is shared with others)
+    opt._lanes.n = 0
     _lib.check(lib.kfac_timing_enable(1))
     step()
     torch.cuda.synchronize()
+    opt._lanes.n = args.lanes
     fam = {}
     for name, fid in (('syrk', 0), ('inv_update', 1), ('inv_lauum', 2), ('gemm', 3)):
         n = ctypes.c_int64()
@@ -228,7 +233,8 @@ def run_gpu(args):
         'config': {'workload': 'ResNet-50 v1 (bias, 1000-way) K-FAC step, batch 32 @224: 161 factors, '
                                'cov + damped Cholesky inverse + precondition',
                    'batch': BATCH, 'factors': len(W.all_factor_dims(layers)), 'damping': DAMPING,
-                   'hip_graph': graph is not None,
+                   'hip_graph': not args.no_graph,
+            'lanes': args.lanes,
                    'bn_inverse': 'woodbury rank-32 ({} blocks)'.format(len(lowrank)) if lowrank else 'dense'},
         # rates use the flops actually executed; the *_reference_work entries divide the work of the
         # reference's algorithm (all 161 factors inverted densely) by the same times
@@ -348,6 +354,8 @@ def main():
     ap.add_argument('--dense-bn-inverse', action='store_true',
                     help='invert the batch-norm blocks with the dense Cholesky path as well (default: their '
                          'rank-32 Woodbury form, which yields the same dense inverse)')
+    ap.add_argument('--lanes', type=int, default=3,
+                    help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='first run one 256 MiB device-to-device elementwise copy (a kernel of known traffic, '
                          'the reference point for hardware byte counters collected under rocprofv3 --pmc)')

@@ -49,10 +49,76 @@ class Workspace(object):
 
 
 _default_workspaces = {}
+_current_lane = None   # index of the lane whose work is being queued (None: the caller's stream)
 
 
 def workspace(kind, nbytes, device):
-    ws = _default_workspaces.get(kind)
+    """Scratch buffer of ``kind`` for the lane being queued on (work on
+    different lanes runs concurrently and must not share scratch memory)."""
+    key = (kind, _current_lane)
+    ws = _default_workspaces.get(key)
     if ws is None:
-        ws = _default_workspaces[kind] = Workspace()
+        ws = _default_workspaces[key] = Workspace()
     return ws.get(nbytes, device)
+
+
+class Lanes(object):
+    """Side streams for per-layer work that does not depend on other layers.
+
+    The factor kernels of one layer (and later its preconditioning products) are
+    often too small to fill the GPU and each waits for the previous one to drain
+    when they share a stream.  ``run`` deals such work onto ``n`` streams in
+    turn; every piece first waits for what the caller's stream has queued so far
+    (its inputs), and ``join`` makes the caller's stream wait for all of it.
+    With ``n`` = 0 everything runs on the caller's stream.
+    """
+
+    def __init__(self, n=0):
+        self.n = int(n)
+        self._streams = {}
+        self._turn = 0
+        self._busy = []
+
+    def _pool(self, device):
+        pool = self._streams.get(device)
+        if pool is None:
+            pool = self._streams[device] = [torch.cuda.Stream(device=device) for _ in range(self.n)]
+        return pool
+
+    def run(self, fn, tensors=()):
+        """Calls ``fn()`` with the next lane as the current stream.  ``tensors``
+        are the arrays it reads: their memory is kept from reuse until the lane
+        has passed this point."""
+        if self.n <= 0:
+            return fn()
+        main = torch.cuda.current_stream()
+        pool = self._pool(main.device)
+        global _current_lane
+        index = self._turn % self.n
+        lane = pool[index]
+        self._turn += 1
+        lane.wait_stream(main)
+        outer = _current_lane
+        _current_lane = index
+        try:
+            with torch.cuda.stream(lane):
+                out = fn()
+        finally:
+            _current_lane = outer
+        for t in tensors:
+            if isinstance(t, torch.Tensor) and t.is_cuda:
+                t.record_stream(lane)
+        if lane not in self._busy:
+            self._busy.append(lane)
+        return out
+
+    def join(self):
+        # every phase deals its work the same way each time it runs (the scratch
+        # buffers of a lane then keep their sizes, which a captured graph needs)
+        self._turn = 0
+        if not self._busy:
+            return
+        main = torch.cuda.current_stream()
+        for lane in self._busy:
+            main.wait_stream(lane)
+        self._busy = []

@@ -10,6 +10,7 @@ The per-block loop of the reference (``update_kfgrads``) is kept, but damping
 and inversion of all blocks are issued as one batch: the blocks are independent,
 so the results are those of the sequential loop.
 """
+from chainerkfac_amd import device as _dev
 from chainerkfac_amd import links
 from chainerkfac_amd import ops
 from chainerkfac_amd.optimizers import fisher_blocks as FB
@@ -67,8 +68,9 @@ class KFACHook(links.FunctionHook):
     owner is found through the identity of the weight array (a dictionary
     lookup instead of the reference's scan over all blocks, kfac.py:38-48)."""
 
-    def __init__(self, fblocks):
+    def __init__(self, fblocks, lanes=None):
         self.fblocks = fblocks
+        self.lanes = lanes
         self._owner = {}
         for fb in fblocks:
             for p in fb.link.params():
@@ -81,15 +83,21 @@ class KFACHook(links.FunctionHook):
                 return fb
         return None
 
+    def _run(self, fn, tensors):
+        if self.lanes is None:
+            return fn()
+        return self.lanes.run(fn, tensors)
+
     def forward_postprocess(self, func, in_data):
         fb = self._find(func, in_data)
         if fb is not None:
-            fb.forward_postprocess(func, in_data)
+            self._run(lambda: fb.forward_postprocess(func, in_data), in_data[:1])
 
     def backward_preprocess(self, func, in_data, out_grad_data):
         fb = self._find(func, in_data, out_grad_data)
         if fb is not None:
-            fb.backward_preprocess(func, in_data, out_grad_data)
+            self._run(lambda: fb.backward_preprocess(func, in_data, out_grad_data),
+                      tuple(in_data[:1]) + tuple(out_grad_data))
 
 
 class KFACUpdateRule(object):
@@ -136,6 +144,12 @@ class KFAC(object):
     #: FisherBlockBatchNormalization.lowrank_inverse_args); False forces the
     #: dense Cholesky path for every block
     bn_lowrank_inverse = True
+
+    #: number of side streams the per-layer factor and preconditioning kernels
+    #: are dealt onto (layers are independent of each other and most of their
+    #: kernels are too small to fill the GPU alone); 0 keeps everything on the
+    #: caller's stream.  Read at ``setup``.
+    lanes = 3
 
     def __init__(self, lr=_default_hyperparam.lr, momentum=_default_hyperparam.momentum,
                  cov_ema_decay=_default_hyperparam.cov_ema_decay,
@@ -191,7 +205,8 @@ class KFAC(object):
             if fblock is None:
                 continue
             self.fblocks.append(fblock)
-        self.kfhook = KFACHook(self.fblocks)
+        self._lanes = _dev.Lanes(self.lanes)
+        self.kfhook = KFACHook(self.fblocks, self._lanes)
         return self
 
     def create_update_rule(self):
@@ -229,6 +244,8 @@ class KFAC(object):
                 else:
                     loss.backward()
             del loss
+        # the factor kernels of this pass ran on the side streams
+        self._lanes.join()
 
         if self.acc_iters > 1:
             if self.accumulate():
@@ -293,11 +310,20 @@ class KFAC(object):
 
     # ---- moving average -> damping -> inverse -> preconditioning ----------
     def update_kfgrads(self, fblocks):
+        self.update_cov_emas(fblocks)
+        self.update_invs_batched(fblocks)
+        self.precondition(fblocks)
+
+    def update_cov_emas(self, fblocks):
+        self._lanes.join()   # factors computed by the hooks
         for fblock in fblocks:
             fblock.update_cov_emas()
-        self.update_invs_batched(fblocks)
+
+    def precondition(self, fblocks):
+        """``fblock.update_kfgrads()`` for every block, independent blocks side by side."""
         for fblock in fblocks:
-            fblock.update_kfgrads()
+            self._lanes.run(fblock.update_kfgrads)
+        self._lanes.join()
 
     def update_invs_batched(self, fblocks):
         """``fblock.update_invs()`` for every block, with all damping kernels and

@@ -194,6 +194,49 @@ def test_accumulation_over_micro_batches():
     assert opt.t == 2 and opt.acc_aware_iterations == 2 and opt.acc_count == 0
 
 
+def test_side_streams_do_not_change_results(monkeypatch):
+    """The per-layer kernels dealt onto side streams are the same launches on the
+    same data: factors, inverses and preconditioned gradients are bit-identical to
+    the one-stream run.  (Driven through the hook calls on fixed tensors: the
+    network's own backward pass is not bit-reproducible from run to run.)"""
+    import bench
+    from chainerkfac_amd.optimizers import KFAC
+    layers = [
+        dict(kind='conv', name='c1', c_in=3, c_out=16, k=3, s=1, p=1, bias=True, h=16, w=16),
+        dict(kind='bn', name='b1', c=16, h=16, w=16),
+        dict(kind='conv', name='c2', c_in=16, c_out=72, k=1, s=1, p=0, bias=True, h=16, w=16),
+        dict(kind='bn', name='b2', c=72, h=16, w=16),
+        dict(kind='conv', name='c3', c_in=72, c_out=40, k=3, s=2, p=1, bias=False, h=16, w=16),
+        dict(kind='conv', name='c4', c_in=40, c_out=40, k=1, s=2, p=0, bias=True, h=8, w=8),
+        dict(kind='linear', name='fc', d_in=640, d_out=10, bias=True),
+    ]
+    outs = []
+    for lanes in (0, 3, 2):
+        monkeypatch.setattr(KFAC, 'lanes', lanes)
+        gen = torch.Generator(device='cuda').manual_seed(11)
+        model, calls = bench.build_model(layers, torch.device('cuda:0'), gen)
+        opt = KFAC(damping=1e-2, cov_ema_decay=0.9).setup(model)
+        assert opt._lanes.n == lanes
+        for _ in range(2):   # the second pass runs the moving average
+            for _, func, in_data, gy in calls:
+                opt.kfhook.forward_postprocess(func, in_data)
+                opt.kfhook.backward_preprocess(func, in_data, (gy,))
+            opt.reallocate_cleared_grads()
+            opt.update_kfgrads(opt.fblocks)
+        torch.cuda.synchronize()
+        got = []
+        for fb in opt.fblocks:
+            got += [(fb.linkname, 'cov', c.cpu().numpy()) for c in fb.cov_emas]
+            got += [(fb.linkname, 'inv', c.cpu().numpy()) for c in fb.invs]
+        got += [(n, 'kfgrad', p.kfgrad.cpu().numpy()) for n, p in sorted(model.namedparams())]
+        outs.append(got)
+    for other in outs[1:]:
+        assert len(other) == len(outs[0])
+        for (n0, k0, a0), (n1, k1, a1) in zip(outs[0], other):
+            assert (n0, k0) == (n1, k1)
+            assert np.array_equal(a0, a1), (n0, k0)
+
+
 def test_constructor_defaults_and_plugin_seam():
     from chainerkfac_amd import links as L
     from chainerkfac_amd.optimizers import KFAC, fblock_constructor
