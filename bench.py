@@ -345,6 +345,8 @@ def run_cpu_baseline(layers, budget_s=20.0):
 
 
 def main():
+    import faulthandler
+    faulthandler.enable()   # a crash inside a native call still names the Python line it came from
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)

@@ -139,49 +139,6 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
   J = t - r * (r + 1) / 2;
 }
 
-// Writes the finished tile: C[I,J] = alpha*acc + beta*C[I,J] and, for I != J,
-// the mirror C[J,I], 64x64 quadrant by quadrant through an LDS transpose so
-// that every global access is a contiguous row segment.
-// Rows and columns below dt (the tiled part); d is the leading dimension of C.
-template <int WM>
-__device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
-                                           int dt, int d, float alpha, float beta,
-                                           float *__restrict__ C) {
-  constexpr int BM = 64 * WM;
-  float(*t)[65] = reinterpret_cast<float(*)[65]>(lds);
-  const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
-  for (int q = 0; q < WM * WM; ++q) {
-    const int qm = q / WM, qn = q % WM;
-    __syncthreads();
-    for_each_acc<WM, WM>(acc, [&](int r, int c, float v) {
-      if (r / 64 == qm && c / 64 == qn) t[r % 64][c % 64] = v;
-    });
-    __syncthreads();
-    const int r0 = I * BM + qm * 64, c0 = J * BM + qn * 64;
-#pragma unroll 4
-    for (int p = 0; p < 16; ++p) {
-      const int lr = lr0 + 4 * p;
-      const int r = r0 + lr, c = c0 + lc;
-      float v = alpha * t[lr][lc];
-      const bool ok = r < dt && c < dt;
-      if (ok) {
-        if (beta != 0.f) v += beta * C[(long long)r * d + c];
-        C[(long long)r * d + c] = v;
-      }
-      if (beta != 0.f && I != J) t[lr][lc] = v;   // mirror gets the same value
-    }
-    if (I != J) {
-      if (beta != 0.f) __syncthreads();
-#pragma unroll 4
-      for (int p = 0; p < 16; ++p) {
-        const int lr = lr0 + 4 * p;
-        const int mr = c0 + lr, mc = r0 + lc;   // row of the mirrored quadrant = column here
-        if (mr < dt && mc < dt) C[(long long)mr * d + mc] = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
-      }
-    }
-  }
-}
-
 // Ones column of a diagonal tile's rows.  rs[im] holds this lane's half of the
 // row sums (see the main loops); after adding the other half, lanes 0..31 of the
 // waves with wave_n == 0 own row (wave_m * WM + im) * 32 + lane of the tile.
@@ -746,6 +703,15 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
     return run_syrk(make_kc<64, false>(x, (long long)c * hw, hw, hw, c),
                     make_kc<128, false>(x, (long long)c * hw, hw, hw, c), d, ones, K, alpha,
                     beta, C, ws, ws_bytes, s);
+  }
+  if (kh == 1 && kw == 1 && ph == 0 && pw == 0) {
+    // strided 1x1 convolution: the same slab, every sx-th pixel of every sy-th line
+    auto l64 = make_kc<64, false>(x, (long long)c * h * w, (long long)h * w, ho * wo, c);
+    auto l128 = make_kc<128, false>(x, (long long)c * h * w, (long long)h * w, ho * wo, c);
+    l64.line_len = l128.line_len = (unsigned)wo;
+    l64.line_stride = l128.line_stride = (unsigned)(sy * w);
+    l64.px_stride = l128.px_stride = (unsigned)sx;
+    return run_syrk(l64, l128, d, ones, K, alpha, beta, C, ws, ws_bytes, s);
   }
   ConvGeom geom;
   if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, &geom)) {

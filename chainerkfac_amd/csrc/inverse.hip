@@ -478,14 +478,8 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int cou
     tile_mainloop<true>(la, lb, K, lds, acc);
   else
     tile_mainloop<false>(la, lb, K, lds, acc);
-  float *__restrict__ out = tb.out[s];
-  for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) {
-    const int r = I * NB + rr, c = J * NB + cc;
-    if (r < d && c < d) {
-      out[(long long)r * d + c] = v;
-      if (I != J) out[(long long)c * d + r] = v;
-    }
-  });
+  // through an LDS transpose, so that the mirror is written in row segments too
+  write_tile<2>(acc, lds, I, J, d, d, 1.f, 0.f, tb.out[s]);
 }
 
 // Dynamic LDS of the step kernel: the diagonal role's working tile and three

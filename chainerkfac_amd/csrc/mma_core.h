@@ -153,6 +153,11 @@ struct LoaderKC<ROWS, false> {
   unsigned row_stride;
   unsigned L;      // k-values per sample
   int rows_valid;
+  // Subsampled rows (a strided 1x1 convolution reads every sx-th pixel of every
+  // sy-th image line): k-value p of a sample is pixel (p / line_len) *
+  // line_stride + (p % line_len) * px_stride of the row.  line_len = 0: k-values
+  // are consecutive elements.
+  unsigned line_len = 0, line_stride = 0, px_stride = 1;
   // per-thread panel state: row i of the thread is first_row + 8 i; rows past
   // the end load from the last data row (masked when stored)
   int first_row;
@@ -168,9 +173,14 @@ struct LoaderKC<ROWS, false> {
     r.kvalid = kg < k_end;
     const unsigned kc = r.kvalid ? (unsigned)kg : 0u;
     unsigned koff = kc;
-    if (L < (unsigned)k_end) {  // more than one sample
+    if (L < (unsigned)k_end || line_len) {  // more than one sample, or subsampled rows
       const unsigned s = kc / L;
-      koff = s * sample_stride + (kc - s * L);
+      unsigned pix = kc - s * L;
+      if (line_len) {
+        const unsigned line = pix / line_len;
+        pix = line * line_stride + (pix - line * line_len) * px_stride;
+      }
+      koff = s * sample_stride + pix;
     }
     const float *p = base + koff;
     // The row offsets are cheap to recompute and expensive to keep: hide the
@@ -493,6 +503,49 @@ __device__ __forceinline__ void zero_acc(floatx16 (&acc)[WM][WN]) {
     for (int in = 0; in < WN; ++in)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[im][in][v] = 0.f;
+}
+
+// Writes the finished tile: C[I,J] = alpha*acc + beta*C[I,J] and, for I != J,
+// the mirror C[J,I], 64x64 quadrant by quadrant through an LDS transpose so
+// that every global access is a contiguous row segment.
+// Rows and columns below dt (the tiled part); d is the leading dimension of C.
+template <int WM>
+__device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
+                                           int dt, int d, float alpha, float beta,
+                                           float *__restrict__ C) {
+  constexpr int BM = 64 * WM;
+  float(*t)[65] = reinterpret_cast<float(*)[65]>(lds);
+  const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
+  for (int q = 0; q < WM * WM; ++q) {
+    const int qm = q / WM, qn = q % WM;
+    __syncthreads();
+    for_each_acc<WM, WM>(acc, [&](int r, int c, float v) {
+      if (r / 64 == qm && c / 64 == qn) t[r % 64][c % 64] = v;
+    });
+    __syncthreads();
+    const int r0 = I * BM + qm * 64, c0 = J * BM + qn * 64;
+#pragma unroll 4
+    for (int p = 0; p < 16; ++p) {
+      const int lr = lr0 + 4 * p;
+      const int r = r0 + lr, c = c0 + lc;
+      float v = alpha * t[lr][lc];
+      const bool ok = r < dt && c < dt;
+      if (ok) {
+        if (beta != 0.f) v += beta * C[(long long)r * d + c];
+        C[(long long)r * d + c] = v;
+      }
+      if (beta != 0.f && I != J) t[lr][lc] = v;   // mirror gets the same value
+    }
+    if (I != J) {
+      if (beta != 0.f) __syncthreads();
+#pragma unroll 4
+      for (int p = 0; p < 16; ++p) {
+        const int lr = lr0 + 4 * p;
+        const int mr = c0 + lr, mc = r0 + lc;   // row of the mirrored quadrant = column here
+        if (mr < dt && mc < dt) C[(long long)mr * d + mc] = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
+      }
+    }
+  }
 }
 
 }  // namespace mma

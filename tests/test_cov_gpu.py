@@ -49,7 +49,10 @@ CONV_CASES = [
     (3, 2, 7, 6, 3, 2, 1, True),
     (2, 4, 9, 9, 1, 1, 0, True),        # 1x1: NCHW slab path, 81 pixels (scalar loads)
     (2, 8, 8, 8, 1, 1, 0, False),       # 1x1, vector loads
-    (2, 5, 8, 8, 1, 2, 0, True),        # strided 1x1 (gather path)
+    (2, 5, 8, 8, 1, 2, 0, True),        # strided 1x1: the slab, subsampled
+    (3, 70, 9, 7, 1, 2, 0, True),       # strided 1x1, odd sizes (5x4 outputs), two 64-tiles
+    (2, 600, 6, 6, 1, 2, 0, True),      # strided 1x1, 128-tiles
+    (2, 40, 9, 9, 1, 3, 0, False),      # stride 3
     (2, 3, 12, 12, 7, 2, 3, True),      # stem-like
     (2, 3, 10, 10, 5, 1, 0, False),
     (4, 3, 32, 32, 3, 1, 1, True),      # CIFAR conv1 shape (28)
