@@ -463,11 +463,13 @@ __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int ta
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
-__global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int count) {
+// One task per tile; the table deals whole tile rows to XCDs (see the plan).
+__global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int task0) {
   extern __shared__ float lds[];
-  const int s = find_slot(tb.tile_cs, count, blockIdx.x);
-  int I, J;
-  tri_decode(blockIdx.x - tb.tile_cs[s], I, J);
+  const int2 task = tb.tasks[task0 + blockIdx.x];
+  const int s = task.x;
+  if (s < 0) return;   // padding of an XCD's shorter list
+  const int I = task.y & 0xffff, J = task.y >> 16;
   const int T = tb.nt[s];
   const int d = tb.dim[s];
   const int K = (T - I) * NB;
@@ -526,6 +528,7 @@ struct kfac_inverse_plan {
     if (side) (void)hipStreamDestroy(side);
   }
   int total_tiles = 0;
+  int lauum_task0 = 0, lauum_count = 0;
   size_t ws_floats = 0;            // padded matrices
   std::vector<const void *> in_sorted, out_sorted;
   kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_shift, d_off, d_tile, d_panel, d_tasks;
@@ -683,6 +686,43 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
       append_tasks(tasks, tail);
     }
   }
+  // Final products out(I,J) = sum_k U(I,k) U(J,k)^T: the I + 1 tiles of tile row I
+  // all read the row U(I, I..T-1).  A whole row goes to one XCD (workgroup i of a
+  // launch runs on XCD i % 8), so that the row stays in that XCD's L2 while its
+  // tiles stream the U(J, .) rows; rows are dealt longest first to the XCD with
+  // the least work, and each XCD runs its long-K rows first.
+  {
+    struct Row { int s, I; double cost; };
+    std::vector<Row> rows;
+    for (int s = 0; s < count; ++s)
+      for (int I = 0; I < p->nt[s]; ++I)
+        rows.push_back({s, I, (double)(I + 1) * (p->nt[s] - I) + 0.5 * (I + 1)});
+    std::stable_sort(rows.begin(), rows.end(), [](const Row &a, const Row &b) { return a.cost > b.cost; });
+    std::vector<Row> mine[8];
+    double load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (const Row &r : rows) {
+      int x = 0;
+      for (int i = 1; i < 8; ++i)
+        if (load[i] < load[x]) x = i;
+      mine[x].push_back(r);
+      load[x] += r.cost;
+    }
+    std::vector<int2> list[8];
+    size_t longest = 0;
+    for (int x = 0; x < 8; ++x) {
+      std::stable_sort(mine[x].begin(), mine[x].end(), [&](const Row &a, const Row &b) {
+        return p->nt[a.s] - a.I > p->nt[b.s] - b.I;
+      });
+      for (const Row &r : mine[x])
+        for (int J = 0; J <= r.I; ++J) list[x].push_back(pack(r.s, r.I, J));
+      longest = std::max(longest, list[x].size());
+    }
+    p->lauum_task0 = (int)tasks.size();
+    for (size_t i = 0; i < longest; ++i)
+      for (int x = 0; x < 8; ++x)
+        tasks.push_back(i < list[x].size() ? list[x][i] : make_int2(-1, 0));
+    p->lauum_count = (int)(longest * 8);
+  }
   if (tasks.empty()) tasks.push_back(make_int2(0, 0));
   int rc = KFAC_OK;
   auto up = [&](kfac::DevTable &t, const void *h, size_t b) {
@@ -838,8 +878,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   KFAC_HIP_CHECK(hipGetLastError());
   {
     kfac::TimedLaunch timed(KFAC_TIMED_INV_LAUUM, s);
-    hipLaunchKernelGGL(lauum_kernel, dim3(plan->total_tiles), dim3(THREADS), kTileLdsBytes, s, tb,
-                       count);
+    hipLaunchKernelGGL(lauum_kernel, dim3(plan->lauum_count), dim3(THREADS), kTileLdsBytes, s, tb,
+                       plan->lauum_task0);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
