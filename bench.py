@@ -40,7 +40,7 @@ HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E peak
 # hardware counters FETCH_SIZE and WRITE_SIZE collected with `rocprofv3 --pmc` on
 # this script (--no-graph --calibrate-copy), each scaled by what it reads for the
 # 256 MiB calibration copy; the counter summary is kept under profiles/.
-SYRK_HBM_BYTES_PER_LAUNCH = 41.6e6
+SYRK_HBM_BYTES_PER_LAUNCH = 41.4e6
 BATCH = 32
 DAMPING = 2.5e-4
 STAB_COEFF = 16.0
@@ -213,8 +213,19 @@ def run_gpu(args):
     # d^3 of the factors that went through the dense Cholesky path (the reference inverts all 161 densely)
     dense_inverse_flops = flops['inverse'] - sum(float(fb.cov_emas[0].shape[0]) ** 3 for fb in lowrank)
 
-    syrk_n, syrk_ms = fam['syrk']
-    achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_ms > 0 else 0.0
+    # What a pair of events adds to the launch it brackets (the time between an
+    # event and the neighbouring kernel's edge): bracket nothing, many times.
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(200)]
+    torch.cuda.synchronize()
+    for e0, e1 in pairs:
+        e0.record()
+        e1.record()
+    torch.cuda.synchronize()
+    bracket_ms = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[len(pairs) // 2]
+
+    syrk_n, syrk_raw_ms = fam['syrk']
+    syrk_ms = max(syrk_raw_ms - syrk_n * bracket_ms, 1e-9)
+    achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
     total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
     executed_flops = flops['cov'] + dense_inverse_flops + flops['precondition']
     result = {
@@ -263,6 +274,9 @@ def run_gpu(args):
             'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
             'launches': syrk_n,
             'avg_launch_ms': round(syrk_ms / max(syrk_n, 1), 4),
+            'avg_launch_ms_with_event_bracket': round(syrk_raw_ms / max(syrk_n, 1), 4),
+            'event_bracket_ms': round(bracket_ms, 4),
+            'timed': 'launches on one stream (--lanes 0 for this pass), HIP events around each launch, empty bracket subtracted',
             'traffic': SYRK_HBM_BYTES_PER_LAUNCH,
             'traffic_unit': 'bytes/launch',
         },
