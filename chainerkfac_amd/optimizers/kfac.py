@@ -360,9 +360,10 @@ class KFAC(object):
                 bufs = [fb._inv_buffers()[0] for fb in fbs]
                 info = self._info_buffer(len(fbs), bufs[0].device, key='_info_lowrank_{}'.format(
                     group[0][1][0].shape[0]))
-                ops.bn_lowrank_inverse_batched(
+                # beside the dense inversions below (a lane of its own; joined at the end)
+                self._lanes.run(lambda group=group, bufs=bufs, info=info: ops.bn_lowrank_inverse_batched(
                     [a[0] for _, a in group], [a[1] for _, a in group], [a[2] for _, a in group],
-                    [a[3] for _, a in group], outs=bufs, info=info)
+                    [a[3] for _, a in group], outs=bufs, info=info))
                 for i, fb in enumerate(fbs):
                     fb.invs = [bufs[i]]
                     fb.inv_info = info[i:i + 1]
@@ -377,6 +378,7 @@ class KFAC(object):
             outs.extend(bufs)
             owners.append((fb, len(bufs)))
         if not mats:
+            self._lanes.join()
             return
         outs, info = ops.spd_inverse_batched(mats, outs=outs, info=self._info_buffer(len(mats), mats[0].device))
         self.inv_info = info
@@ -385,6 +387,7 @@ class KFAC(object):
             fb.invs = outs[pos:pos + n]
             fb.inv_info = info[pos:pos + n]
             pos += n
+        self._lanes.join()
 
     def _pi_buffer(self, n, device):
         import torch
