@@ -101,17 +101,19 @@ __device__ __forceinline__ float *tile_ptr(const InvTables &tb, int s, int I, in
 // tile row: k-value k is column k % NB of tile k / NB.  A 128 x 32 panel is
 // 128 rows of 128 contiguous bytes inside one tile; no edge masks are needed
 // (the workspace is padded).
+typedef float vfloat4 __attribute__((ext_vector_type(4)));   // register arrays of HIP's float4 struct can end up in scratch
+
 struct LoaderTile {
   static constexpr bool kKRow = false;
   struct Regs {
-    float4 v[NB / 32];
+    vfloat4 v[NB / 32];
   };
   const float *base;   // first tile of the run
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long) const {
     const unsigned k = (unsigned)k0 + (threadIdx.x & 7) * 4;
     const float *p = base + (size_t)(k / NB) * (NB * NB) + (k % NB) + (threadIdx.x >> 3) * NB;
 #pragma unroll
-    for (int i = 0; i < NB / 32; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + 32 * i * NB);
+    for (int i = 0; i < NB / 32; ++i) r.v[i] = *reinterpret_cast<const vfloat4 *>(p + 32 * i * NB);
   }
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
     const int kq = (threadIdx.x & 7) * 4;
@@ -133,19 +135,19 @@ struct LoaderTile {
 struct LoaderTileT {
   static constexpr bool kKRow = true;
   struct Regs {
-    float4 v[KT / 8];
+    vfloat4 v[KT / 8];
   };
   const float *base;
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long) const {
     const float *p = base + ((int)k0 + (threadIdx.x >> 5)) * NB + (threadIdx.x & 31) * 4;
 #pragma unroll
-    for (int i = 0; i < KT / 8; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + 8 * i * NB);
+    for (int i = 0; i < KT / 8; ++i) r.v[i] = *reinterpret_cast<const vfloat4 *>(p + 8 * i * NB);
   }
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
     float *p = lds + (threadIdx.x >> 5) * Panel<NB>::kKRowStride + (threadIdx.x & 31) * 4;
 #pragma unroll
     for (int i = 0; i < KT / 8; ++i)
-      *reinterpret_cast<float4 *>(p + 8 * i * Panel<NB>::kKRowStride) = r.v[i];
+      *reinterpret_cast<vfloat4 *>(p + 8 * i * Panel<NB>::kKRowStride) = r.v[i];
   }
 };
 
@@ -158,61 +160,75 @@ struct LoaderTileT {
 constexpr int kTileLdsFloats = 4 * Panel<NB>::kFloats;
 constexpr size_t kTileLdsBytes = kTileLdsFloats * sizeof(float);
 
-template <bool SAME, class LA, class LB>
+template <bool SAME, int D, class LA, class LB>
 __device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K, float *lds,
                                               floatx16 (&acc)[2][2]) {
   constexpr int PF = Panel<NB>::kFloats;
+  // D: passes of 64 k-values held in registers ahead of the one in LDS.  With
+  // one, a third of the passes of a full GPU wait 2-4 us for their operands
+  // (measured with time stamps); two cover that where the registers allow it.
   float *ldsA = lds, *ldsB = lds + 2 * PF;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane & 31, lk = lane >> 5;
-  typename LA::Regs ra[2];
-  typename LB::Regs rb[2];
+  typename LA::Regs ra[D][2];
+  typename LB::Regs rb[D][2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    la.load(ra[h], 0, KT * h, K);
-    if (!SAME) lb.load(rb[h], 0, KT * h, K);
-  }
-  for (int k0 = 0; k0 < K; k0 += 2 * KT) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      la.store(ra[h], ldsA + h * PF);
-      if (!SAME) lb.store(rb[h], ldsB + h * PF);
-    }
-    __syncthreads();
-    if (k0 + 2 * KT < K) {
+  for (int d = 0; d < D; ++d) {
+    if (d * 2 * KT < K) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        la.load(ra[h], 0, k0 + 2 * KT + KT * h, K);
-        if (!SAME) lb.load(rb[h], 0, k0 + 2 * KT + KT * h, K);
+        la.load(ra[d][h], 0, d * 2 * KT + KT * h, K);
+        if (!SAME) lb.load(rb[d][h], 0, d * 2 * KT + KT * h, K);
       }
     }
+  }
+  for (int kb = 0; kb < K; kb += D * 2 * KT) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const float *pa = ldsA + h * PF;
-      const float *pb = SAME ? pa : ldsB + h * PF;
+    for (int d = 0; d < D; ++d) {
+      const int k0 = kb + d * 2 * KT;
+      if (k0 < K) {
 #pragma unroll
-      for (int kk = 0; kk < KT / 2; ++kk) {
-        float a[2], b[2];
+      for (int h = 0; h < 2; ++h) {
+        la.store(ra[d][h], ldsA + h * PF);
+        if (!SAME) lb.store(rb[d][h], ldsB + h * PF);
+      }
+      __syncthreads();
+      if (k0 + D * 2 * KT < K) {
 #pragma unroll
-        for (int im = 0; im < 2; ++im)
-          a[im] = fetch<NB, LA::kKRow>(pa, (wm * 2 + im) * 32 + lrow, 2 * kk + lk);
-#pragma unroll
-        for (int in = 0; in < 2; ++in) {
-          if (SAME)
-            b[in] = fetch<NB, LA::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
-          else
-            b[in] = fetch<NB, LB::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
+        for (int h = 0; h < 2; ++h) {
+          la.load(ra[d][h], 0, k0 + D * 2 * KT + KT * h, K);
+          if (!SAME) lb.load(rb[d][h], 0, k0 + D * 2 * KT + KT * h, K);
         }
+      }
 #pragma unroll
-        for (int im = 0; im < 2; ++im)
+      for (int h = 0; h < 2; ++h) {
+        const float *pa = ldsA + h * PF;
+        const float *pb = SAME ? pa : ldsB + h * PF;
 #pragma unroll
-          for (int in = 0; in < 2; ++in)
-            acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+        for (int kk = 0; kk < KT / 2; ++kk) {
+          float a[2], b[2];
+#pragma unroll
+          for (int im = 0; im < 2; ++im)
+            a[im] = fetch<NB, LA::kKRow>(pa, (wm * 2 + im) * 32 + lrow, 2 * kk + lk);
+#pragma unroll
+          for (int in = 0; in < 2; ++in) {
+            if (SAME)
+              b[in] = fetch<NB, LA::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
+            else
+              b[in] = fetch<NB, LB::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
+          }
+#pragma unroll
+          for (int im = 0; im < 2; ++im)
+#pragma unroll
+            for (int in = 0; in < 2; ++in)
+              acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+        }
+      }
+      __syncthreads();
       }
     }
-    __syncthreads();
   }
 }
 
@@ -288,7 +304,7 @@ __device__ __forceinline__ void diag_role(const InvTables &tb, int s, int k, int
     floatx16 acc[2][2];
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -tile[rr * NB + cc]; });
     const LoaderTile la{tile_ptr(tb, s, k, lo)};
-    tile_mainloop<true>(la, la, (hi - lo + 1) * NB, smem, acc);   // ends with a barrier
+    tile_mainloop<true, 1>(la, la, (hi - lo + 1) * NB, smem, acc);   // ends with a barrier
     for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { S[rr * LS + cc] = -v; });
   } else {
     const int c4 = (threadIdx.x & 31) * 4, r0 = threadIdx.x >> 5;
@@ -390,7 +406,7 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int ste
   float *tile = tile_ptr(tb, s, x, k);
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
-  tile_mainloop<false>(LoaderTile{tile}, LoaderTileT{tile_ptr(tb, s, k, k)}, NB, lds, acc);
+  tile_mainloop<false, 1>(LoaderTile{tile}, LoaderTileT{tile_ptr(tb, s, k, k)}, NB, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { tile[rr * NB + cc] = v; });
 }
 
@@ -399,6 +415,7 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int ste
 // from -C, so the tile is read while the first operand panels are in flight and
 // the epilogue is a plain store.  An upper tile whose row lies inside [k0, k1]
 // receives its first product here and is overwritten (it holds stale data).
+template <int D>
 __device__ __forceinline__ void update_role(const InvTables &tb, int2 task, int k0, int k1,
                                             float *lds) {
   const int s = task.x;
@@ -416,9 +433,9 @@ __device__ __forceinline__ void update_role(const InvTables &tb, int2 task, int 
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -C[rr * NB + cc]; });
   const LoaderTile la{tile_ptr(tb, s, a, j_lo)}, lb{tile_ptr(tb, s, b, j_lo)};
   if (a == b)
-    tile_mainloop<true>(la, lb, K, lds, acc);
+    tile_mainloop<true, D>(la, lb, K, lds, acc);
   else
-    tile_mainloop<false>(la, lb, K, lds, acc);
+    tile_mainloop<false, D>(la, lb, K, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[rr * NB + cc] = -v; });
 }
 
@@ -448,7 +465,7 @@ __global__ __launch_bounds__(THREADS, 2) void step_kernel(InvTables tb, int step
     const int2 task = tb.tasks[task0 + blockIdx.x - ndiag];
     int k0, k1;
     local_range(tb, task.x, step0, step1, k0, k1);
-    update_role(tb, task, k0, k1, lds);
+    update_role<1>(tb, task, k0, k1, lds);
   }
 }
 
@@ -459,7 +476,7 @@ __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int ta
   const int2 task = tb.tasks[task0 + blockIdx.x];
   int k0, k1;
   local_range(tb, task.x, step0, step1, k0, k1);
-  update_role(tb, task, k0, k1, lds);
+  update_role<1>(tb, task, k0, k1, lds);
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
@@ -477,9 +494,9 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int tas
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
   if (I == J)
-    tile_mainloop<true>(la, lb, K, lds, acc);
+    tile_mainloop<true, 2>(la, lb, K, lds, acc);
   else
-    tile_mainloop<false>(la, lb, K, lds, acc);
+    tile_mainloop<false, 2>(la, lb, K, lds, acc);
   // through an LDS transpose, so that the mirror is written in row segments too
   write_tile<2>(acc, lds, I, J, d, d, 1.f, 0.f, tb.out[s]);
 }
