@@ -46,6 +46,26 @@ def test_batched_inverse_mixed_sizes():
         check_inverse(m, o.cpu().numpy())
 
 
+@pytest.mark.parametrize('env,extra', [({'KFAC_INVERSE_ALIGN': '0'}, 3), ({'KFAC_INVERSE_ALIGN': '50'}, 4),
+                                       ({'KFAC_INVERSE_GROUP': '3'}, 5), ({'KFAC_INVERSE_GROUP': '1'}, 6),
+                                       ({'KFAC_INVERSE_LOOKAHEAD': '0'}, 8),
+                                       ({'KFAC_INVERSE_GROUP': '4', 'KFAC_INVERSE_ALIGN': '30'}, 9)])
+def test_schedule_overrides_do_not_change_results(monkeypatch, env, extra):
+    """The tuning overrides (where a matrix joins the sweep, block columns per
+    group, second stream) only reorder launches.  A plan reads them when it is
+    created; `extra` makes the size list, and with it the plan, unique to the case."""
+    from chainerkfac_amd import ops
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    dims = [900, 641, 640, 385, 300, 129, 128, 40, extra]
+    mats = [spd(d, 200 + d) for d in dims]
+    outs, info = ops.spd_inverse_batched([torch.from_numpy(m).cuda() for m in mats])
+    torch.cuda.synchronize()
+    assert info.cpu().tolist() == [0] * len(dims)
+    for m, o in zip(mats, outs):
+        check_inverse(m, o.cpu().numpy())
+
+
 @pytest.mark.parametrize('d', [10, 148, 2305])
 def test_single_inverse_free_function(d):
     from chainerkfac_amd.optimizers.cholesky_inverse import inverse
