@@ -54,6 +54,26 @@ def build_cnn(L, device, gen):
     return CNN()
 
 
+def build_cifar_cnn(L, device, gen):
+    """The CIFAR-shaped CNN of the benchmark's second configuration: three 3x3
+    convolutions (3->64->128->256, pad 1, bias) with ReLU and 2x2 max-pooling,
+    then a 4096->10 fully connected layer: A factors 28, 577, 1153, 4097."""
+    class CifarCNN(L.Chain):
+        def __init__(self):
+            super(CifarCNN, self).__init__()
+            self.conv1 = L.Convolution2D(3, 64, 3, 1, 1, device=device, generator=gen)
+            self.conv2 = L.Convolution2D(64, 128, 3, 1, 1, device=device, generator=gen)
+            self.conv3 = L.Convolution2D(128, 256, 3, 1, 1, device=device, generator=gen)
+            self.fc = L.Linear(4096, 10, device=device, generator=gen)
+
+        def __call__(self, x):
+            h = TF.max_pool2d(TF.relu(self.conv1(x)), 2)
+            h = TF.max_pool2d(TF.relu(self.conv2(h)), 2)
+            h = TF.max_pool2d(TF.relu(self.conv3(h)), 2)
+            return self.fc(h)
+    return CifarCNN()
+
+
 def copy_params(src, dst):
     for (n1, p1), (n2, p2) in zip(sorted(src.namedparams()), sorted(dst.namedparams())):
         assert n1 == n2
@@ -184,6 +204,49 @@ def test_cnn_with_batchnorm_two_steps():
     out = run_case(build_cnn, cnn_batches(2), lr=1e-2, momentum=0.9, cov_ema_decay=1.0, damping=1e-2,
                    stab_coeff=16.0)
     compare(*out, tol_param=2e-3, tol_kf=5e-3)
+
+
+def kfgrad_errors_vs_float64(A_damped, G_damped, gW, gb, kW, kb):
+    """Relative error of a float32 preconditioned gradient against the float64
+    product of the float64 inverses of the same (float32, damped) factors."""
+    grad = gW.reshape(gW.shape[0], -1).astype(np.float64)
+    if gb is not None:
+        grad = np.column_stack([grad, gb.astype(np.float64)])
+    kf = np.linalg.inv(G_damped.astype(np.float64)) @ grad @ np.linalg.inv(A_damped.astype(np.float64))
+    got = kW.reshape(kW.shape[0], -1)
+    if kb is not None:
+        got = np.column_stack([got, kb])
+    return rel(got, kf)
+
+
+def test_cifar_cnn_one_step_config2():
+    """Small CIFAR-shaped CNN, batch 128, input (128,3,32,32) ~ N(0,1), damping 1e-3:
+    one full optimizer step (factors 28/577/1153/4097 and 64/128/256/10).
+
+    The 4097x4097 factor of the last layer has rank 128 plus the damping (a
+    condition number near 1e6), so two float32 evaluations of G^-1 g A^-1 agree to
+    ~1e-3..1e-2 only; the bound there is the float64 result: the HIP path must be
+    no further from it than 4x the NumPy formula is."""
+    r = np.random.default_rng(2)
+    batches = [(r.standard_normal((128, 3, 32, 32)).astype(np.float32), r.integers(0, 10, 128).astype(np.int64))]
+    model, ref_model, opt, oracle = run_case(build_cifar_cnn, batches, lr=1e-3, momentum=0.9,
+                                             cov_ema_decay=0.99, damping=1e-3)
+    # (a bias starts at 0, so after one step it is the update itself: same bound as the kfgrads)
+    compare(model, ref_model, opt, oracle, tol_param=1e-2, tol_kf=1e-2)
+    assert [tuple(c.shape) for fb in opt.fblocks for c in fb.covs] == \
+        [(28, 28), (64, 64), (577, 577), (128, 128), (1153, 1153), (256, 256), (4097, 4097), (10, 10)]
+    ref_links = dict(ref_model.namedlinks())
+    for fb in opt.fblocks:
+        W, b = fb.link.W, fb.link.b
+        err_hip = kfgrad_errors_vs_float64(
+            fb.cov_emas[0].cpu().numpy(), fb.cov_emas[1].cpu().numpy(), W.grad.cpu().numpy(), b.grad.cpu().numpy(),
+            W.kfgrad.cpu().numpy(), b.kfgrad.cpu().numpy())
+        rl = ref_links[fb.linkname]
+        name = fb.linkname
+        err_ref = kfgrad_errors_vs_float64(
+            oracle.cov_emas[name][0], oracle.cov_emas[name][1], rl.W.grad.numpy(), rl.b.grad.numpy(),
+            oracle.kfgrads[(name, 'W')], oracle.kfgrads[(name, 'b')])
+        assert err_hip < max(4 * err_ref, 1e-3), (name, err_hip, err_ref)
 
 
 def test_accumulation_over_micro_batches():
