@@ -284,6 +284,86 @@ def run_gpu(args):
     return result, layers
 
 
+def write_per_layer(path, layers):
+    """Per-layer roofline table of the covariance kernels (markdown): every distinct
+    convolution / linear shape of the workload, its A and G factor timed alone on one
+    stream (HIP events inside the library around the SYRK launch, empty bracket
+    subtracted), against min(FP32 MFMA peak, arithmetic intensity x HBM peak)."""
+    import torch
+    from chainerkfac_amd import _lib, ops
+    from chainerkfac_amd import workloads as W
+    lib = _lib.load()
+    dev = torch.device('cuda:0')
+
+    def bracket_ms():
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(100)]
+        torch.cuda.synchronize()
+        for e0, e1 in pairs:
+            e0.record()
+            e1.record()
+        torch.cuda.synchronize()
+        return sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[50]
+
+    empty = bracket_ms()
+
+    def syrk_ms(fn, iters=10):
+        fn()
+        torch.cuda.synchronize()
+        _lib.check(lib.kfac_timing_enable(1))
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        n = ctypes.c_int64()
+        ms = ctypes.c_double()
+        _lib.check(lib.kfac_timing_read(0, ctypes.byref(n), ctypes.byref(ms)))
+        _lib.check(lib.kfac_timing_enable(0))
+        return max(ms.value / max(n.value, 1) - empty, 1e-6)
+
+    rows = []
+    seen = set()
+    for layer in layers:
+        if layer['kind'] == 'conv':
+            key = ('conv', layer['c_in'], layer['c_out'], layer['k'], layer['s'], layer['h'])
+        elif layer['kind'] == 'linear':
+            key = ('linear', layer['d_in'], layer['d_out'])
+        else:
+            continue
+        count = sum(1 for other in layers if other['kind'] == layer['kind'] and all(
+            other.get(f) == layer.get(f) for f in ('c_in', 'c_out', 'k', 's', 'h', 'd_in', 'd_out')))
+        if key in seen:
+            continue
+        seen.add(key)
+        dA, dG = W.factor_dims(layer)
+        M = W.cov_rows(layer, BATCH)
+        if layer['kind'] == 'conv':
+            ho = W.conv_out(layer['h'], layer['k'], layer['s'], layer['p'])
+            x = torch.randn(BATCH, layer['c_in'], layer['h'], layer['w'], device=dev)
+            gy = torch.randn(BATCH, layer['c_out'], ho, ho, device=dev)
+            ta = syrk_ms(lambda: ops.cov_conv_a(x, layer['k'], layer['s'], layer['p'], layer['bias'], 1.0 / BATCH))
+            tg = syrk_ms(lambda: ops.cov_conv_g(gy, 1.0))
+            desc = 'conv {}x{}/{} {}->{} @{}'.format(layer['k'], layer['k'], layer['s'], layer['c_in'], layer['c_out'],
+                                                   layer['h'])
+        else:
+            x = torch.randn(BATCH, layer['d_in'], device=dev)
+            gy = torch.randn(BATCH, layer['d_out'], device=dev)
+            ta = syrk_ms(lambda: ops.cov_linear(x, layer['bias'], 1.0 / BATCH))
+            tg = syrk_ms(lambda: ops.cov_linear(gy, False, float(BATCH)))
+            desc = 'linear {}->{}'.format(layer['d_in'], layer['d_out'])
+        in_a, in_g = x.numel() * 4.0, gy.numel() * 4.0
+        for fac, d, t, in_bytes in (('A', dA, ta, in_a), ('G', dG, tg, in_g)):
+            flop = float(M) * d * (d + 1)
+            ai = flop / (in_bytes + 4.0 * d * d)
+            cap = min(FP32_MFMA_PEAK_TFLOPS, ai * HBM_PEAK_GBPS / 1e3)
+            rows.append((desc, count, fac, d, M, flop / 1e9, t * 1e3, flop / t / 1e9, ai, cap, flop / t / 1e9 / cap))
+        del x, gy
+    with open(path, 'w') as f:
+        f.write('| layer (x count) | factor | d | rows M | GFLOP | SYRK kernel us | TFLOP/s | flop/B | roofline cap TFLOP/s '
+                '| fraction of cap |\n|---|---|---:|---:|---:|---:|---:|---:|---:|---:|\n')
+        for desc, count, fac, d, M, gf, us, tf, ai, cap, frac in rows:
+            f.write('| {} (x{}) | {} | {} | {} | {:.2f} | {:.1f} | {:.1f} | {:.0f} | {:.1f} | {:.2f} |\n'.format(
+                desc, count, fac, d, M, gf, us, tf, ai, cap, frac))
+
+
 def run_cpu_baseline(layers, budget_s=20.0):
     """The NumPy oracle (the restatement of the reference's --no_cuda arithmetic)
     on a bounded sample of the workload's layers, scaled to the whole step by
@@ -372,6 +452,9 @@ def main():
                          'rank-32 Woodbury form, which yields the same dense inverse)')
     ap.add_argument('--lanes', type=int, default=3,
                     help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
+    ap.add_argument('--per-layer', metavar='PATH', default=None,
+                    help='also time the covariance kernels of every distinct layer shape alone and write a '
+                         'markdown roofline table to PATH')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='first run one 256 MiB device-to-device elementwise copy (a kernel of known traffic, '
                          'the reference point for hardware byte counters collected under rocprofv3 --pmc)')
@@ -380,6 +463,8 @@ def main():
         sys.exit('bench.py measures the single-GPU K-FAC hot path: inter-GPU collectives are outside this '
                  'build, so --gpus must be 1 (got {})'.format(args.gpus))
     result, layers = run_gpu(args)
+    if args.per_layer:
+        write_per_layer(args.per_layer, layers)
     if not args.no_cpu:
         result['cpu_baseline'] = run_cpu_baseline(layers)
     print(json.dumps(result))
