@@ -52,6 +52,11 @@ _default_workspaces = {}
 _current_lane = None   # index of the lane whose work is being queued (None: the caller's stream)
 
 
+def current_lane():
+    """Index of the lane whose work is being queued, None on the caller's stream."""
+    return _current_lane
+
+
 def workspace(kind, nbytes, device):
     """Scratch buffer of ``kind`` for the lane being queued on (work on
     different lanes runs concurrently and must not share scratch memory)."""
