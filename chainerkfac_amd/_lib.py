@@ -45,6 +45,7 @@ PROTOTYPES = {
     'kfac_inverse_plan_create': (c_int, [c_int, c_i32p, c_vpp]),
     'kfac_inverse_plan_workspace_bytes': (c_sz, [c_vp]),
     'kfac_inverse_plan_destroy': (c_int, [c_vp]),
+    'kfac_inverse_plan_set_capture_origin': (c_int, [c_vp, c_int]),
     'kfac_spd_inverse_batched_f32': (c_int, [c_vp, c_vpp, c_vpp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_damp_plan_create': (c_int, [c_int, c_i32p, c_i32p, c_vpp]),
     'kfac_damp_plan_destroy': (c_int, [c_vp]),

@@ -536,6 +536,10 @@ struct kfac_inverse_plan {
   // The rest of a trailing update touches nothing the next group's sweep needs,
   // so it runs on a second stream beside that sweep.
   bool lookahead = true;
+  // Under stream capture the fork onto `side` is only safe from the stream the
+  // capture began on (a fork of a forked stream has crashed the runtime), which
+  // the library cannot find out by itself: the caller says so.
+  bool capture_origin = false;
   size_t rest_lds = 0;
   hipStream_t side = nullptr;
   std::vector<hipEvent_t> ev_main, ev_side;   // per step
@@ -779,6 +783,12 @@ extern "C" size_t kfac_inverse_plan_workspace_bytes(kfac_inverse_plan_t plan) {
   return plan->ws_floats * sizeof(float) + 256;
 }
 
+extern "C" int kfac_inverse_plan_set_capture_origin(kfac_inverse_plan_t plan, int is_origin) {
+  KFAC_REQUIRE(plan != nullptr, "plan is null");
+  plan->capture_origin = is_origin != 0;
+  return KFAC_OK;
+}
+
 extern "C" int kfac_inverse_plan_destroy(kfac_inverse_plan_t plan) {
   delete plan;
   return KFAC_OK;
@@ -796,6 +806,19 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     return kfac::fail(KFAC_ENOMEM, "inverse workspace too small: %zu < %zu bytes", ws_bytes,
                       kfac_inverse_plan_workspace_bytes(plan));
   hipStream_t s = kfac::as_stream(stream);
+  // The trailing updates fork onto the plan's own stream.  While `s` is being
+  // captured into a graph that is done only if the caller has declared `s` the
+  // capture's origin; otherwise everything stays on `s`, in program order.
+  bool lookahead = plan->lookahead;
+  if (lookahead && !plan->capture_origin) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
+      (void)hipGetLastError();   // e.g. the null stream beside a global-mode capture
+      lookahead = false;
+    } else if (cs != hipStreamCaptureStatusNone) {
+      lookahead = false;
+    }
+  }
   plan->in_sorted.resize(count);
   plan->out_sorted.resize(count);
   for (int i = 0; i < count; ++i) {
@@ -849,7 +872,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     if (deferred < 0) return KFAC_OK;
     const UpdateLaunch &r = plan->rest[deferred];
     hipStream_t st = s;
-    if (plan->lookahead) {
+    if (lookahead) {
       KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_main[deferred], 0));
       st = plan->side;
     }
@@ -858,7 +881,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       hipLaunchKernelGGL(update_kernel, dim3(r.count), dim3(THREADS), plan->rest_lds, st, tb,
                          r.task0, r.k0, r.k1);
     }
-    if (plan->lookahead) {
+    if (lookahead) {
       KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[deferred], plan->side));
       pending = deferred;
     }
@@ -873,9 +896,9 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     // The rest of the previous group itself only touches columns further right
     // and runs beside this group's sweep.
     const int two_back = k - 1 - plan->group;
-    if (plan->lookahead && k % plan->group == 0 && two_back >= 0 && plan->rest[two_back].count > 0)
+    if (lookahead && k % plan->group == 0 && two_back >= 0 && plan->rest[two_back].count > 0)
       KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[two_back], 0));
-    if (!plan->lookahead)
+    if (!lookahead)
       if (int rc2 = queue_rest()) return rc2;   // one stream: keep the program order
     {
       kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, s);
@@ -887,7 +910,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), kTileLdsBytes, s,
                          tb, k, na);
     if (plan->rest[k].count == 0) continue;
-    if (plan->lookahead) KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
+    if (lookahead) KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
     deferred = k;
   }
   if (int rc2 = queue_rest()) return rc2;

@@ -170,6 +170,11 @@ class InversePlan(object):
         if info is None:
             info = torch.empty(len(mats), dtype=torch.int32, device=dev)
         ws = _dev.workspace('inverse', self.workspace_bytes, dev)
+        # Under HIP-graph capture the plan may fork its trailing updates onto its
+        # own stream only from the stream the capture began on: torch's current
+        # stream when the call is not inside a lane (a lane is itself a fork).
+        origin = stream is None and _dev.current_lane() is None
+        _lib.check(_lib.load().kfac_inverse_plan_set_capture_origin(self._plan, int(origin)))
         _lib.check(_lib.load().kfac_spd_inverse_batched_f32(
             self._plan, _lib.ptr_array([m.data_ptr() for m in mats]),
             _lib.ptr_array([o.data_ptr() for o in outs]), info.data_ptr(), ws.data_ptr(),
@@ -177,22 +182,56 @@ class InversePlan(object):
         return outs, info
 
 
-_inverse_plans = {}
+class _PlanCache(object):
+    """Least-recently-used cache of plans.
+
+    A plan keeps its device-side pointer tables between calls and rewrites them
+    (stream synchronisation + blocking copy) when it is called with other
+    buffers.  Callers that pass persistent buffers -- the Fisher blocks do --
+    therefore get one plan per (shapes, buffers): equal-shaped layers do not
+    evict each other's tables, no call after the first touches the host-device
+    link, and a HIP graph captured over a call keeps replaying against tables
+    nobody rewrites.  Calls that let the wrapper allocate fresh outputs share
+    one plan per shape list instead (their pointers change every time)."""
+
+    def __init__(self, limit=1024):
+        from collections import OrderedDict
+        self._plans = OrderedDict()
+        self._limit = limit
+
+    def get(self, key, make):
+        plan = self._plans.get(key)
+        if plan is None:
+            while len(self._plans) >= self._limit:
+                self._plans.popitem(last=False)
+            plan = self._plans[key] = make()
+        else:
+            self._plans.move_to_end(key)
+        return plan
+
+    def __len__(self):
+        return len(self._plans)
 
 
-def inverse_plan(dims):
-    key = tuple(int(d) for d in dims)
-    plan = _inverse_plans.get(key)
-    if plan is None:
-        if len(_inverse_plans) > 64:
-            _inverse_plans.clear()
-        plan = _inverse_plans[key] = InversePlan(key)
-    return plan
+def _ptr_key(tensors):
+    return None if tensors is None else tuple(t.data_ptr() for t in tensors)
+
+
+_inverse_plans = _PlanCache()
+
+
+def inverse_plan(dims, bound_to=None):
+    """Plan for a list of matrix sizes; ``bound_to`` (any hashable, normally the
+    buffers' device pointers) gives callers with persistent buffers a plan of
+    their own."""
+    dims = tuple(int(d) for d in dims)
+    return _inverse_plans.get((dims, bound_to), lambda: InversePlan(dims))
 
 
 def spd_inverse_batched(mats, outs=None, info=None, stream=None):
     """Inverses of a list of SPD matrices (potrf + potri on the GPU)."""
-    return inverse_plan([m.shape[0] for m in mats]).run(mats, outs, info, stream)
+    bound = None if outs is None else (_ptr_key(mats), _ptr_key(outs))
+    return inverse_plan([m.shape[0] for m in mats], bound).run(mats, outs, info, stream)
 
 
 class BnLowrankPlan(object):
@@ -246,17 +285,14 @@ class BnLowrankPlan(object):
         return outs, info
 
 
-_bn_lowrank_plans = {}
+_bn_lowrank_plans = _PlanCache()
 
 
 def bn_lowrank_inverse_batched(Us, splits, d_gamma, d_beta, outs=None, info=None, stream=None):
     """(U^T U / n + diag(d_gamma | d_beta))^-1 for a list of (n, w) gradient matrices."""
     key = (Us[0].shape[0], tuple(U.shape[1] for U in Us), tuple(int(v) for v in splits))
-    plan = _bn_lowrank_plans.get(key)
-    if plan is None:
-        if len(_bn_lowrank_plans) > 64:
-            _bn_lowrank_plans.clear()
-        plan = _bn_lowrank_plans[key] = BnLowrankPlan(*key)
+    bound = None if outs is None else (_ptr_key(Us), _ptr_key(outs))
+    plan = _bn_lowrank_plans.get(key + (bound,), lambda: BnLowrankPlan(*key))
     return plan.run(Us, d_gamma, d_beta, outs, info, stream)
 
 
@@ -290,17 +326,14 @@ class DampPlan(object):
         return pi_out
 
 
-_damp_plans = {}
+_damp_plans = _PlanCache()
 
 
 def pi_damp_batched(As, Gs, rW, use_pi=True, pi_out=None, stream=None):
     """In-place trace-norm damping of (A, G) pairs; returns the device vector of pi."""
     key = (tuple(a.shape[0] for a in As), tuple(g.shape[0] for g in Gs))
-    plan = _damp_plans.get(key)
-    if plan is None:
-        if len(_damp_plans) > 64:
-            _damp_plans.clear()
-        plan = _damp_plans[key] = DampPlan(*key)
+    # the factors are damped in place, so their buffers identify the caller
+    plan = _damp_plans.get(key + (_ptr_key(As), _ptr_key(Gs)), lambda: DampPlan(*key))
     return plan.run(As, Gs, rW, use_pi, pi_out, stream)
 
 

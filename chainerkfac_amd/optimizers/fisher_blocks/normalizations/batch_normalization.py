@@ -20,6 +20,8 @@ class FisherBlockBatchNormalization(FisherBlock):
     def __init__(self, *args, **kwargs):
         self._F = None
         self._U = None
+        self._covs = None
+        self._own_factor = False
         self._ema_is_single_factor = False
         #: cleared by whoever replaces ``covs`` by something that is not this
         #: process's own single-batch factor (e.g. an average over ranks)
@@ -30,6 +32,20 @@ class FisherBlockBatchNormalization(FisherBlock):
     @property
     def funcclass(self):
         return links.BatchNormalizationFunction
+
+    # ``covs`` assigned by anyone but ``backward_preprocess`` (accumulation,
+    # an average over ranks, a caller's own factor) no longer is U^T U / n of
+    # the kept gradient matrix: forget U, so that the inverse is taken of the
+    # factor actually stored and not of the stale low-rank form.
+    @property
+    def covs(self):
+        return self._covs
+
+    @covs.setter
+    def covs(self, value):
+        self._covs = value
+        if not self._own_factor:
+            self._U = None
 
     @property
     def cov_forward(self):
@@ -61,7 +77,11 @@ class FisherBlockBatchNormalization(FisherBlock):
 
     def backward_preprocess(self, func, in_data, out_grad_data):
         self._F = self.compute_F(in_data, out_grad_data)
-        self.covs = [self._F]
+        self._own_factor = True
+        try:
+            self.covs = [self._F]
+        finally:
+            self._own_factor = False
 
     def compute_F(self, in_data, out_grad_data):
         x = in_data[0]
@@ -156,9 +176,19 @@ class FisherBlockBatchNormalization(FisherBlock):
             gamma.kfgrad = kg
         if beta is not None:
             beta.kfgrad = kb
-        if self.debug() and int(self.nan_flag.item()):
-            warnings.warn('Detected NaN in the kfgrads of the batch normalization layer; '
-                          '``grad`` was substituted for ``kfgrad``')
+        # The reference warns on the spot (batch_normalization.py:21-33), which
+        # costs a device->host read per block; here the flag stays on the device
+        # and KFAC.check_numerics() reads all of them together at the start of the
+        # next step.  ``link.debug`` asks for the immediate warning.
+        if self.debug():
+            self.warn_if_nan()
+
+    def warn_if_nan(self):
+        if self.nan_flag is not None and int(self.nan_flag.item()):
+            warnings.warn('Detected NaN in the kfgrads of the batch normalization layer {}; '
+                          '``grad`` was substituted for ``kfgrad``'.format(self.linkname))
+            return True
+        return False
 
     def extract_for_reduce_scatter_v(self):
         arrays = self.extract_attr_from_params('grad')

@@ -63,6 +63,15 @@ def fblock_constructor(sub_linkname, sub_link, **kwargs):
     return None
 
 
+def extract(blocks, indices, extractor):
+    """Per-rank lists of ``(array, triangular)`` in buffer order: for every rank
+    the arrays ``extractor(block)`` yields for the blocks that rank owns, blocks
+    in index order (reference kfac.py:456-464).  The result is what
+    ``_pack_arrays_to_buffer`` / ``_unpack_arrays_from_buffer`` consume."""
+    return [[array for index in local_indices for array in extractor(blocks[index])]
+            for local_indices in indices]
+
+
 class KFACHook(links.FunctionHook):
     """Routes each link-function call to the Fisher block that owns it.  The
     owner is found through the identity of the weight array (a dictionary
@@ -120,8 +129,15 @@ class KFACUpdateRule(object):
         self.t += 1
         if self.state is None:
             self.init_state(param)
-        if param._loss_scale is not None and getattr(param, 'kfgrad', None) is not None:
-            param.kfgrad /= param._loss_scale
+        # gradients of a scaled loss carry the scale (so do the preconditioned
+        # ones: G^-1 (s g) A^-1); both are divided back before the update, as
+        # Chainer's UpdateRule.update does for ``grad`` and the reference for
+        # ``kfgrad`` (kfac.py:72-78)
+        if param._loss_scale is not None:
+            if getattr(param, 'kfgrad', None) is not None:
+                param.kfgrad /= param._loss_scale
+            elif param.grad is not None:
+                param.grad /= param._loss_scale
         self.update_core(param)
 
     def update_core(self, param):
@@ -227,8 +243,50 @@ class KFAC(object):
             if param.grad is None:
                 param.grad = torch.zeros_like(param.data)
 
+    #: read the device-side failure flags of the previous step (NaN fallback of
+    #: the batch-norm blocks, non-positive pivots of the inversions) at the start
+    #: of every ``update`` and warn; one small device->host copy per step
+    numerics_check = True
+
+    def check_numerics(self):
+        """Warns about what the previous step's kernels flagged on the device:
+        batch-norm blocks whose preconditioned gradient held a NaN (the raw
+        gradient was used, reference batch_normalization.py:21-33) and factors
+        whose Cholesky factorisation met a non-positive pivot (the reference's
+        NumPy path raises there, its GPU path never looks).  Returns the names of
+        the affected links.  Must not be called while a HIP graph is captured."""
+        import warnings
+        import torch
+        flags, owners = [], []
+        for fb in self.fblocks:
+            nan_flag = getattr(fb, 'nan_flag', None)
+            if nan_flag is not None:
+                flags.append(nan_flag.reshape(-1))
+                owners.append((fb, 'nan'))
+            info = getattr(fb, 'inv_info', None)
+            if info is not None:
+                flags.append(info.reshape(-1))
+                owners.extend([(fb, 'pivot')] * info.numel())
+        if not flags:
+            return []
+        host = torch.cat(flags).cpu().tolist()
+        bad = []
+        for v, (fb, what) in zip(host, owners):
+            if not v:
+                continue
+            bad.append(fb.linkname)
+            if what == 'nan':
+                warnings.warn('Detected NaN in the kfgrads of the batch normalization layer {}; '
+                              '``grad`` was substituted for ``kfgrad``'.format(fb.linkname))
+            else:
+                warnings.warn('The damped factor of {} is not positive definite in float32 '
+                              '(non-positive Cholesky pivot); its inverse is not usable'.format(fb.linkname))
+        return bad
+
     # ---- one step -------------------------------------------------------
     def update(self, lossfun=None, *args, **kwargs):
+        if self.numerics_check and self.t > 0:
+            self.check_numerics()
         if lossfun is not None:
             for fblock in self.fblocks:
                 fblock.acc_state = (self.acc_iters, self.acc_count)
@@ -243,6 +301,10 @@ class KFAC(object):
                     (loss * self._loss_scale).backward()
                 else:
                     loss.backward()
+                # Chainer's backward(loss_scale=...) stamps the scale on every
+                # parameter that received a gradient; the update rule divides by it
+                for param in self.target.params():
+                    param._loss_scale = self._loss_scale
             del loss
         # the factor kernels of this pass ran on the side streams
         self._lanes.join()

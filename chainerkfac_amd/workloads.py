@@ -151,3 +151,57 @@ def flops(layers, batch):
         else:
             pre += 2 * dims[0] ** 2
     return dict(cov=cov, inverse=inv, precondition=pre)
+
+
+def build_resnet50_v1(device='cuda', generator=None, n_class=1000, bias=True):
+    """The network behind the ``resnet50_v1`` layer table as a callable chain of
+    ``chainerkfac_amd.links``: bottleneck topology of the reference's
+    examples/cifar10/models/resnet50.py:6-73 (1x1 -> 3x3 -> 1x1 with a batch
+    normalisation after every convolution, stride on the first 1x1, a projection
+    shortcut in the first bottleneck of every stage, no activation after the
+    sum) behind the ImageNet stem (7x7/2 convolution, 3x3/2 max-pooling), global
+    average pooling and an ``n_class``-way linear layer.  ``bias`` gives every
+    convolution a bias, as the benchmark configuration states."""
+    import torch.nn.functional as TF
+    from chainerkfac_amd import links as L
+
+    def conv(c_in, c_out, k, s, p):
+        return L.Convolution2D(c_in, c_out, k, s, p, nobias=not bias, device=device, generator=generator)
+
+    class Bottleneck(L.Chain):
+        def __init__(self, n_in, n_mid, n_out, stride, project):
+            super(Bottleneck, self).__init__()
+            self.conv1, self.bn1 = conv(n_in, n_mid, 1, stride, 0), L.BatchNormalization(n_mid, device=device)
+            self.conv2, self.bn2 = conv(n_mid, n_mid, 3, 1, 1), L.BatchNormalization(n_mid, device=device)
+            self.conv3, self.bn3 = conv(n_mid, n_out, 1, 1, 0), L.BatchNormalization(n_out, device=device)
+            if project:
+                self.conv4, self.bn4 = conv(n_in, n_out, 1, stride, 0), L.BatchNormalization(n_out, device=device)
+            self.project = project
+
+        def __call__(self, x):
+            h = TF.relu(self.bn1(self.conv1(x)))
+            h = TF.relu(self.bn2(self.conv2(h)))
+            h = self.bn3(self.conv3(h))
+            return h + (self.bn4(self.conv4(x)) if self.project else x)
+
+    class Net(L.Chain):
+        def __init__(self):
+            super(Net, self).__init__()
+            self.conv1, self.bn1 = conv(3, 64, 7, 2, 3), L.BatchNormalization(64, device=device)
+            n_in = 64
+            for si, (n_mid, n_out, blocks, stride) in enumerate(
+                    [(64, 256, 3, 1), (128, 512, 4, 2), (256, 1024, 6, 2), (512, 2048, 3, 2)]):
+                stage = L.ChainList(*[Bottleneck(n_in if b == 0 else n_out, n_mid, n_out,
+                                                 stride if b == 0 else 1, b == 0) for b in range(blocks)])
+                setattr(self, 'res{}'.format(si + 2), stage)
+                n_in = n_out
+            self.fc = L.Linear(2048, n_class, device=device, generator=generator)
+
+        def __call__(self, x):
+            h = TF.max_pool2d(TF.relu(self.bn1(self.conv1(x))), 3, 2, 1)
+            for name in ('res2', 'res3', 'res4', 'res5'):
+                for block in getattr(self, name):
+                    h = block(h)
+            return self.fc(h.mean(dim=(2, 3)))
+
+    return Net()

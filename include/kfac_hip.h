@@ -131,7 +131,7 @@ int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, int c,
                             int has_beta, float *U, void *ws, size_t ws_bytes,
                             void *stream);
 
-/* y_i = a*x_i + b*y_i over `count` arrays (host tables of device pointers).
+/* y = a*x + b*y over one pair of arrays of `nelems` floats.
  * Moving average of optimizers/fisher_block.py:162-163 (a = decay on the new
  * covariance, b = 1-decay) and the unfused accumulation of kfac.py:286-304. */
 int kfac_axpby_f32(const float *x, float *y, int64_t nelems, float a, float b,
@@ -151,6 +151,16 @@ int kfac_inverse_plan_create(int count, const int32_t *dims,
                              kfac_inverse_plan_t *plan_out);
 size_t kfac_inverse_plan_workspace_bytes(kfac_inverse_plan_t plan);
 int kfac_inverse_plan_destroy(kfac_inverse_plan_t plan);
+
+/* kfac_spd_inverse_batched_f32 runs part of its trailing updates on a stream
+ * of the plan's own, forked from and joined back into `stream` with events.
+ * While `stream` is being captured into a HIP graph that fork is only taken
+ * when the caller has declared, with is_origin != 0, that `stream` is the
+ * stream the capture began on; on any other capturing stream (one that itself
+ * was forked into the capture) the call keeps all launches on `stream`.  The
+ * results are the same either way.  No counterpart in the reference (which has
+ * no stream structure). */
+int kfac_inverse_plan_set_capture_origin(kfac_inverse_plan_t plan, int is_origin);
 
 /* out_i = in_i^-1 for SPD in_i (dims given at plan creation); the full
  * symmetric inverse is written.  in_i is read only.  info_dev[i] (device,

@@ -8,6 +8,12 @@ normalizations/batch_normalization.py:133-191), then the momentum rule
 (kfac.py:87-99).  State that the reference keeps across steps (cov_emas, the
 in-place damped diagonals of the NumPy path, momentum buffers, accumulators) is
 kept here the same way.
+
+Pinned by tests/test_oracle_step.py against an independent float64 restatement
+(torch unfold / explicit batch statistics, numpy.linalg.inv, an explicit
+Kronecker-product solve): one and three steps with the damped diagonal carried
+inside the moving average, decay 1, accumulation over two micro-batches, and a
+loss scale that must cancel.
 """
 import numpy as np
 
@@ -96,6 +102,10 @@ class OracleKFAC(object):
                 kf = {'W': kW, 'b': kb}
             for pname, p in r.params.items():
                 g = kf[pname]
+                # gradients of a scaled loss carry the scale; the update rule
+                # divides the preconditioned gradient back (kfac.py:72-78)
+                if self.loss_scale is not None:
+                    g = g / np.float32(self.loss_scale)
                 self.kfgrads[(r.name, pname)] = g
                 key = (r.name, pname)
                 if key not in self.v:

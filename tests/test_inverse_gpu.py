@@ -191,3 +191,44 @@ def test_bn_lowrank_rejects_bad_arguments():
     U = torch.zeros(4, 8, device='cuda')
     with pytest.raises(_lib.KfacHipError):
         ops.bn_lowrank_inverse_batched([U], [4], [0.0], [1e-3])        # non-positive damping
+
+
+def test_capture_on_a_forked_stream_keeps_the_inverse_on_that_stream():
+    """Captured into a HIP graph from a stream that is itself a fork of the
+    capture (a lane), the batched inverse must not fork again onto its own side
+    stream: the plan is told it is not on the capture's origin and keeps every
+    launch on the given stream.  The replayed results equal the eager ones bit for
+    bit, on every replay."""
+    from chainerkfac_amd import device, ops
+    dims = [700, 300, 129]           # 6 block columns: a plan with the look-ahead stream
+    mats = [torch.from_numpy(spd(d, 300 + d)).cuda() for d in dims]
+    eager, info_e = ops.spd_inverse_batched(mats)
+    torch.cuda.synchronize()
+    outs = [torch.zeros_like(m) for m in mats]
+    info = torch.zeros(len(dims), dtype=torch.int32, device='cuda')
+    lanes = device.Lanes(2)
+
+    def work():
+        lanes.run(lambda: ops.spd_inverse_batched(mats, outs=outs, info=info), mats)
+        lanes.join()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()                        # plans, tables and lane workspaces exist before the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for o, e in zip(outs, eager):
+        assert torch.equal(o, e)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        work()
+    for _ in range(3):
+        for o in outs:
+            o.zero_()                 # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert info.cpu().tolist() == [0, 0, 0]
+        for o, e in zip(outs, eager):
+            assert torch.equal(o, e)

@@ -198,12 +198,14 @@ def test_mlp_three_steps_moving_average_and_momentum():
     single-step tests is therefore relaxed to 5e-3 for the later steps."""
     out = run_case(build_mlp, mnist_batches(3, bs=32), lr=1e-2, momentum=0.9, cov_ema_decay=0.9, damping=1e-2)
     compare(*out, tol_param=2e-3, tol_kf=5e-3)
+    shadow_check(*out)
 
 
 def test_cnn_with_batchnorm_two_steps():
     out = run_case(build_cnn, cnn_batches(2), lr=1e-2, momentum=0.9, cov_ema_decay=1.0, damping=1e-2,
                    stab_coeff=16.0)
     compare(*out, tol_param=2e-3, tol_kf=5e-3)
+    shadow_check(*out)
 
 
 def kfgrad_errors_vs_float64(A_damped, G_damped, gW, gb, kW, kb):
@@ -217,6 +219,38 @@ def kfgrad_errors_vs_float64(A_damped, G_damped, gW, gb, kW, kb):
     if kb is not None:
         got = np.column_stack([got, kb])
     return rel(got, kf)
+
+
+def shadow_check(model, ref_model, opt, oracle, floor=1e-3):
+    """Second criterion for steps whose float32 results cannot agree to 1e-3 (factors that
+    are nearly singular before damping, inputs that already differ in the last bits after an
+    earlier step): on each side the preconditioned gradients are compared with the float64
+    product of the float64 inverses of that side's own damped factors and gradients.  The HIP
+    path must be no further from float64 than 4x what the NumPy formula of the reference is."""
+    ref_links = dict(ref_model.namedlinks())
+    for fb in opt.fblocks:
+        name = fb.linkname
+        rl = ref_links[name]
+        if hasattr(fb.link, 'W'):
+            W, b = fb.link.W, fb.link.b
+            err_hip = kfgrad_errors_vs_float64(
+                fb.cov_emas[0].cpu().numpy(), fb.cov_emas[1].cpu().numpy(), W.grad.cpu().numpy(),
+                None if b is None else b.grad.cpu().numpy(), W.kfgrad.cpu().numpy(),
+                None if b is None else b.kfgrad.cpu().numpy())
+            err_ref = kfgrad_errors_vs_float64(
+                oracle.cov_emas[name][0], oracle.cov_emas[name][1], rl.W.grad.numpy(),
+                None if rl.b is None else rl.b.grad.numpy(), oracle.kfgrads[(name, 'W')],
+                None if rl.b is None else oracle.kfgrads[(name, 'b')])
+        else:
+            def bn_err(F, g_gamma, g_beta, k_gamma, k_beta):
+                kf = np.linalg.inv(F.astype(np.float64)) @ np.concatenate([g_gamma, g_beta]).astype(np.float64)
+                return rel(np.concatenate([k_gamma, k_beta]), kf)
+            gm, bt = fb.link.gamma, fb.link.beta
+            err_hip = bn_err(fb.cov_emas[0].cpu().numpy(), gm.grad.cpu().numpy(), bt.grad.cpu().numpy(),
+                             gm.kfgrad.cpu().numpy(), bt.kfgrad.cpu().numpy())
+            err_ref = bn_err(oracle.cov_emas[name][0], rl.gamma.grad.numpy(), rl.beta.grad.numpy(),
+                             oracle.kfgrads[(name, 'gamma')], oracle.kfgrads[(name, 'beta')])
+        assert err_hip < max(4 * err_ref, floor), (name, err_hip, err_ref)
 
 
 def test_cifar_cnn_one_step_config2():
@@ -254,7 +288,93 @@ def test_accumulation_over_micro_batches():
     model, ref_model, opt, oracle = run_case(build_cnn, batches, lr=1e-2, momentum=0.0, cov_ema_decay=1.0,
                                              damping=1e-2, acc_iters=2)
     compare(model, ref_model, opt, oracle, tol_param=2e-3, tol_kf=5e-3)
+    shadow_check(model, ref_model, opt, oracle)
     assert opt.t == 2 and opt.acc_aware_iterations == 2 and opt.acc_count == 0
+
+
+def test_loss_scale_cancels_end_to_end():
+    """KFAC(loss_scale=128): the backward pass runs on 128 * loss, the factors undo the scale
+    through gy_scale and the update rule divides the preconditioned gradients back
+    (reference kfac.py:72-78), so the step is that of the unscaled loss: judged against the
+    oracle run WITHOUT a loss scale on the same model and batch."""
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import KFAC
+    hyper = dict(lr=1e-2, momentum=0.9, cov_ema_decay=1.0, damping=1e-2)
+    gen = torch.Generator(device='cpu').manual_seed(7)
+    ref_model = build_cnn(L, 'cpu', gen)
+    model = build_cnn(L, 'cuda', None)
+    copy_params(ref_model, model)
+    # a convolution without a Fisher block of its own would take the plain-gradient path;
+    # here every parameter has a block, so every update goes through kfgrad
+    opt = KFAC(loss_scale=128.0, **hyper).setup(model)
+    oracle = OracleKFAC(**hyper)
+
+    def lossfun(m, x, t):
+        return TF.cross_entropy(m(x), t)
+
+    for x, t in cnn_batches(2):
+        opt.update(lossfun, model, torch.from_numpy(x).cuda(), torch.from_numpy(t).cuda())
+        rec = Recorder(L, ref_model)
+        ref_model.cleargrads()
+        with rec.hook():
+            lossfun(ref_model, torch.from_numpy(x), torch.from_numpy(t)).backward()
+        oracle.step(rec.records())
+    torch.cuda.synchronize()
+    for p in model.params():
+        assert p._loss_scale == 128.0
+    by_name = {fb.linkname: fb for fb in opt.fblocks}
+    for name, emas in oracle.cov_emas.items():
+        for got, ref in zip(by_name[name].cov_emas, emas):
+            assert rel(got.cpu().numpy(), ref) < 1e-4, name
+    # kfgrads were divided by the scale in place; gradients still carry it
+    for (lname, pname), ref in oracle.kfgrads.items():
+        got = getattr(by_name[lname].link, pname).kfgrad.cpu().numpy()
+        assert rel(got, ref) < 5e-3, (lname, pname)
+    ref_params = dict(ref_model.namedparams())
+    for name, p in model.namedparams():
+        assert rel(p.grad.cpu().numpy(), 128.0 * ref_params[name].grad.numpy()) < 1e-4, name
+        assert rel(p.data.cpu().numpy(), ref_params[name].data.numpy()) < 2e-3, name
+
+
+def test_plain_gradient_path_divides_by_loss_scale():
+    """A parameter without a Fisher block is updated from ``grad`` (reference kfac.py:88); with
+    a loss scale that gradient is divided back first, as Chainer's UpdateRule.update does."""
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import KFAC
+
+    class Scale(L.Link):
+        def __init__(self):
+            super(Scale, self).__init__()
+            self.w = L.Parameter(torch.ones(5, device='cuda'))
+
+        def __call__(self, x):
+            return x * self.w.tensor
+
+    class Net(L.Chain):
+        def __init__(self):
+            super(Net, self).__init__()
+            self.fc = L.Linear(5, 3, device='cuda', generator=None)
+            self.scale = Scale()
+
+        def __call__(self, x):
+            return self.fc(self.scale(x))
+
+    torch.manual_seed(0)
+    x = torch.randn(4, 5, device='cuda')
+    t = torch.tensor([0, 1, 2, 1], device='cuda')
+    nets = []
+    for ls in (None, 64.0):
+        torch.manual_seed(1)
+        net = Net()
+        opt = KFAC(lr=0.1, momentum=0.0, damping=1e-2, cov_ema_decay=1.0, loss_scale=ls).setup(net)
+        assert [fb.linkname for fb in opt.fblocks] == ['/fc']
+        opt.update(lambda: TF.cross_entropy(net(x), t))
+        nets.append(net)
+    torch.cuda.synchronize()
+    a, b = nets
+    assert not torch.equal(a.scale.w.data, torch.ones(5, device='cuda'))
+    assert rel(b.scale.w.data.cpu().numpy(), a.scale.w.data.cpu().numpy()) < 1e-5
+    assert rel(b.fc.W.data.cpu().numpy(), a.fc.W.data.cpu().numpy()) < 1e-4
 
 
 def test_side_streams_do_not_change_results(monkeypatch):
@@ -343,3 +463,43 @@ def test_buffer_order_of_extract_helpers():
     assert [t for _, t in arrays] == [False, False, True]
     assert arrays[0][0] is bn.link.beta.grad and arrays[1][0] is bn.link.gamma.grad   # '/beta' < '/gamma'
     assert [a.shape for a, _ in conv.extract_for_all_gather_v('kfgrad')] == [conv.link.W.shape, conv.link.b.shape]
+
+
+def test_extract_builds_the_per_rank_lists_the_packer_consumes():
+    """``extract(blocks, indices, extractor)`` (reference kfac.py:456-464) defines the wire
+    order: per rank, the owned blocks in index order, each block's arrays in its own order.
+    Its output goes straight into the packer; unpacking into fresh arrays restores every
+    gradient and both triangles of every factor bit for bit, and a rank-filtered pack
+    fills exactly that rank's segment of the buffer."""
+    from chainerkfac_amd.communicators import ArrayPacker
+    from chainerkfac_amd.optimizers.kfac import extract
+    out = run_case(build_cnn, cnn_batches(1), damping=1e-2, cov_ema_decay=1.0)
+    opt = out[2]
+    n = len(opt.fblocks)
+    indices = [list(range(0, 2)), list(range(2, n))]      # two "ranks", contiguous runs of blocks
+    arrays = extract(opt.fblocks, indices, lambda b: b.extract_for_reduce_scatter_v())
+    assert len(arrays) == 2
+    flat = [a for fb in opt.fblocks for a in fb.extract_for_reduce_scatter_v()]
+    assert [id(a) for local in arrays for a, _ in local] == [id(a) for a, _ in flat]
+    assert [len(local) for local in arrays] == [sum(len(fb.extract_for_reduce_scatter_v()) for fb in opt.fblocks[:2]),
+                                                sum(len(fb.extract_for_reduce_scatter_v()) for fb in opt.fblocks[2:])]
+    packer = ArrayPacker()
+    nel = packer.get_nelems(arrays)
+    host = [[(a.cpu().numpy(), t) for a, t in local] for local in arrays]
+    assert nel == O.get_nelems(host)
+    buf = torch.zeros(nel, dtype=torch.float32, device='cuda')
+    packer._pack_arrays_to_buffer(arrays, buf)
+    ref = np.zeros(nel, np.float32)
+    O.pack(host, ref)
+    assert np.array_equal(buf.cpu().numpy(), ref)
+    back = [[(torch.full_like(a, float('nan')), t) for a, t in local] for local in arrays]
+    packer._unpack_arrays_from_buffer(back, buf)
+    for local, local_back in zip(arrays, back):
+        for (a, _), (b, _) in zip(local, local_back):
+            assert torch.equal(a, b)
+    # rank 1 only: the first rank's segment stays untouched
+    buf1 = torch.full_like(buf, -7.0)
+    packer._pack_arrays_to_buffer(arrays, buf1, target=1)
+    n0 = O.get_nelems([host[0]])
+    assert bool((buf1[:n0] == -7.0).all()) and np.array_equal(buf1[n0:].cpu().numpy(), ref[n0:])
+    assert extract(opt.fblocks, [[], [1]], lambda b: b.extract_for_all_gather_v('kfgrad'))[0] == []
