@@ -332,7 +332,9 @@ def test_loss_scale_cancels_end_to_end():
         assert rel(got, ref) < 5e-3, (lname, pname)
     ref_params = dict(ref_model.namedparams())
     for name, p in model.namedparams():
-        assert rel(p.grad.cpu().numpy(), 128.0 * ref_params[name].grad.numpy()) < 1e-4, name
+        # (the bias of conv1 feeds a batch normalisation: its gradient is zero up to rounding noise)
+        if name != '/conv1/b':
+            assert rel(p.grad.cpu().numpy(), 128.0 * ref_params[name].grad.numpy()) < 1e-4, name
         assert rel(p.data.cpu().numpy(), ref_params[name].data.numpy()) < 2e-3, name
 
 
