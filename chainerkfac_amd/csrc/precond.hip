@@ -6,6 +6,8 @@
 // Replaces compute_kfgrads / update_kfgrads of
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py,
 // fisher_blocks/connection.py:51-61 and normalizations/batch_normalization.py:159-191.
+#include <mutex>
+
 #include "common.h"
 #include "mma_core.h"
 
@@ -284,6 +286,67 @@ extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ain
                      rowmajor_kc<128, false>(T, dG, dA, dA),
                      rowmajor_kc<128, false>(Ainv, dA, dA, dA), dG, dA, dA, partial, kfW, dW, dW,
                      kfb, s);
+}
+
+// ---------------------------------------------------------------------------
+// kfac_precond_bn_static_f32: the batch-norm preconditioning with its staging
+// vector (the product F^-1 g before the NaN selection) in a device array that
+// is part of the library image, for callers that cannot allocate.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[KFAC_PRECOND_BN_STATIC_MAX_D];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+float *scratch_ptr[kMaxDevices];   // device address of `scratch` on each GPU, null until resolved
+
+// Every GPU holds its own copy of `scratch` at its own address; the name of the
+// array is only a host-side handle.  Resolved once per device, with that device
+// current, and kept.
+int scratch_of_current_device(float **out) {
+  int dev = -1;
+  KFAC_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return kfac::fail(KFAC_EINVAL, "device index %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    KFAC_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr) return kfac::fail(KFAC_EHIP, "hipGetSymbolAddress returned a null address");
+    scratch_ptr[dev] = static_cast<float *>(p);
+  }
+  *out = scratch_ptr[dev];
+  return KFAC_OK;
+}
+
+}  // namespace
+
+extern "C" int kfac_precond_bn_static_f32(const float *Finv, int d, const float *g_gamma,
+                                          int n_gamma, const float *g_beta, int n_beta,
+                                          float *kf_gamma, float *kf_beta,
+                                          int32_t *nan_flag_dev, void *stream) {
+  KFAC_REQUIRE(d > 0 && n_gamma >= 0 && n_beta >= 0 && n_gamma + n_beta == d,
+               "sizes %d + %d do not match d = %d", n_gamma, n_beta, d);
+  if (d > KFAC_PRECOND_BN_STATIC_MAX_D)
+    return kfac::fail(KFAC_EINVAL,
+                      "d = %d exceeds the built-in scratch array (at most %d); use "
+                      "kfac_precond_bn_f32 with a caller workspace",
+                      d, KFAC_PRECOND_BN_STATIC_MAX_D);
+  KFAC_REQUIRE(Finv != nullptr, "Finv is null");
+  KFAC_REQUIRE(n_gamma == 0 || (g_gamma && kf_gamma), "gamma pointers are null");
+  KFAC_REQUIRE(n_beta == 0 || (g_beta && kf_beta), "beta pointers are null");
+  float *y = nullptr;
+  if (int rc = scratch_of_current_device(&y)) return rc;
+  hipStream_t s = kfac::as_stream(stream);
+  // y[0, d) is written in full by the product before the selection reads it, so
+  // nothing of an earlier call's contents is ever seen and nothing needs clearing
+  hipLaunchKernelGGL(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
+                     n_gamma, g_beta, y);
+  hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
+                     kf_gamma, kf_beta, nan_flag_dev);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
 }
 
 extern "C" size_t kfac_precond_bn_workspace_bytes(int d) {

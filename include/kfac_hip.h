@@ -249,6 +249,26 @@ int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamma,
                         float *kf_gamma, float *kf_beta, int32_t *nan_flag_dev,
                         void *ws, size_t ws_bytes, void *stream);
 
+/* kfac_precond_bn_f32 without a workspace argument and without any allocation:
+ * the staging vector lives in a device array of KFAC_PRECOND_BN_STATIC_MAX_D
+ * floats (32 KiB) that is part of the library image on every GPU the library
+ * runs on, for the life of the process.  No counterpart in the reference; it is
+ * for callers that cannot allocate device memory -- code under HIP-graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The call makes
+ * no hipMalloc/hipFree and calls no allocating library routine; inputs and
+ * outputs are the caller's, as for kfac_precond_bn_f32, and the results are
+ * identical to it.  d > KFAC_PRECOND_BN_STATIC_MAX_D is rejected with
+ * KFAC_EINVAL.  The first call on a device looks up the array's address on that
+ * device (hipGetSymbolAddress, once): make one call outside of any stream
+ * capture first.  All calls on one GPU share the one array: calls that may
+ * overlap on the same GPU (different streams, different threads) race on it and
+ * must be serialised by the caller. */
+#define KFAC_PRECOND_BN_STATIC_MAX_D 8192
+int kfac_precond_bn_static_f32(const float *Finv, int d, const float *g_gamma,
+                               int n_gamma, const float *g_beta, int n_beta,
+                               float *kf_gamma, float *kf_beta,
+                               int32_t *nan_flag_dev, void *stream);
+
 /* v = momentum*v - lr*grad; param += v.  Replaces the 'kfac' elementwise
  * kernel of KFACUpdateRule.update_core_gpu (optimizers/kfac.py:101-116). */
 int kfac_momentum_update_f32(float *param, float *v, const float *grad,
