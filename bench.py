@@ -115,7 +115,7 @@ def run_gpu(args):
         for func, in_data, gy in work:
             hook.forward_postprocess(func, in_data)
             hook.backward_preprocess(func, in_data, gy)
-        opt._lanes.join()
+        opt.finish_covs()
 
     def inv_phase():
         opt.update_cov_emas(opt.fblocks)

@@ -38,6 +38,10 @@ PROTOTYPES = {
     'kfac_cov_linear_f32': (c_int, [c_vp, c_int, c_int, c_int, c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
     'kfac_cov_conv_a_f32': (c_int, [c_vp] + [c_int] * 11 + [c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
     'kfac_cov_conv_g_f32': (c_int, [c_vp, c_int, c_int, c_int, c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
+    'kfac_cov_group_create': (c_int, [c_int, c_vp, c_vpp]),
+    'kfac_cov_group_workspace_bytes': (c_sz, [c_vp]),
+    'kfac_cov_group_destroy': (c_int, [c_vp]),
+    'kfac_cov_group_run_f32': (c_int, [c_vp, c_vpp, c_vpp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_bn_workspace_bytes': (c_sz, [c_int, c_int]),
     'kfac_bn_grad_matrix_f32': (c_int, [c_vp, c_vp, c_int, c_int, c_int, c_f, c_f, c_int, c_int,
                                         c_vp, c_vp, c_sz, c_vp]),
@@ -110,6 +114,10 @@ def i64_array(values):
 
 def f64_array(values):
     return (ctypes.c_double * len(values))(*[float(v) for v in values])
+
+
+def f32_array(values):
+    return (ctypes.c_float * len(values))(*[float(v) for v in values])
 
 
 def ptr_array(values):

@@ -22,9 +22,14 @@
 // and the batch-norm block's grad^T grad.
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
 
 #include "common.h"
 #include "conv_halo.h"
+#include "conv_rows.h"
 #include "mma_core.h"
 
 namespace {
@@ -41,6 +46,15 @@ struct SyrkPlan {
 };
 
 constexpr int kFinishSplits = 8;
+
+// No plan uses more k-slices than this (every planner clamps to it, and the
+// workspace bound of kfac_cov_workspace_bytes is computed from it): about
+// kMaxWorkgroups workgroups per launch.
+constexpr long long kMaxWorkgroups = 3072;
+long long max_splits(int ntile) {
+  const long long m = kfac::ceil_div<long long>(kMaxWorkgroups, ntile);
+  return m < 1 ? 1 : m;
+}
 
 SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
   SyrkPlan p;
@@ -71,7 +85,7 @@ SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
     const long long slots = 512;
     double best = 0;
     long long best_ns = ns;
-    for (long long c = 1; c <= max_ns && c <= 4 * ns; ++c) {
+    for (long long c = 1; c <= max_ns && c <= 4 * ns && c <= max_splits(p.ntile); ++c) {
       const long long per = kfac::ceil_div(nk, c);
       const long long eff = kfac::ceil_div(nk, per);
       const long long rounds = kfac::ceil_div(p.ntile * eff, slots);
@@ -88,10 +102,56 @@ SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
     const long long forced = atoll(env);
     if (forced >= 1) ns = forced < nk ? forced : nk;
   }
+  if (ns > max_splits(p.ntile)) ns = max_splits(p.ntile);
   const long long per = kfac::ceil_div(nk, ns);
   p.nsplit = (int)kfac::ceil_div(nk, per);
   p.klen = per * panel_len;
   // partials are pre-reduced to at most kFinishSplits slots before finishing
+  p.nreduced = p.nsplit > kFinishSplits ? kFinishSplits : 0;
+  return p;
+}
+
+// Plan for the compile-time-geometry convolution kernel: 128-tiles, `steps`
+// reduction steps of `step_us` microseconds of matrix-core time each, `occ`
+// workgroups resident per CU.  The hardware deals workgroups to the 256 CUs as
+// slots free up, so a launch takes about ceil(workgroups / 256) workgroups' time
+// on the busiest CU; each workgroup also pays a fixed prologue / epilogue, each
+// extra slice a partial tile that is written and read back, and fewer
+// workgroups than CUs x occ leave matrix pipes without a second wave to hide
+// the staging phases.
+SyrkPlan plan_rows(int d, long long steps, double step_us, int occ) {
+  SyrkPlan p;
+  p.bm = 128;
+  p.tiles = kfac::ceil_div(d, p.bm);
+  p.ntile = p.tiles * (p.tiles + 1) / 2;
+  if (steps < 1) steps = 1;
+  const double fixed_us = 6.0, partial_us = 0.05, finish_us = 8.0;
+  long long best_c = 1;
+  double best = 0;
+  const long long cmax = std::min<long long>(steps, max_splits(p.ntile));
+  for (long long c = 1; c <= cmax; ++c) {
+    const long long per = kfac::ceil_div(steps, c);
+    const long long eff = kfac::ceil_div(steps, per);
+    if (eff != c) continue;
+    const long long wgs = (long long)p.ntile * eff;
+    const long long deep = kfac::ceil_div<long long>(wgs, 256);
+    double cost = (double)deep * ((double)per * step_us + fixed_us);
+    // measured: a CU with one resident workgroup runs its steps ~25 % slower than one with three
+    const double per_cu = std::min((double)occ, (double)wgs / 256.0);
+    if (per_cu < 3.0) cost *= 1.0 + 0.14 * (3.0 - per_cu);
+    if (eff > 1) cost += finish_us + partial_us * (double)wgs;
+    if (c == 1 || cost < best) {
+      best = cost;
+      best_c = c;
+    }
+  }
+  if (const char *env = getenv("KFAC_SYRK_SPLITS")) {   // tuning override
+    const long long forced = atoll(env);
+    if (forced >= 1) best_c = std::min(forced, cmax);
+  }
+  const long long per = kfac::ceil_div(steps, best_c);
+  p.nsplit = (int)kfac::ceil_div(steps, per);
+  p.klen = per;
   p.nreduced = p.nsplit > kFinishSplits ? kFinishSplits : 0;
   return p;
 }
@@ -243,10 +303,11 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
   float rs[WM];
 #pragma unroll
   for (int im = 0; im < WM; ++im) rs[im] = 0.f;
+  const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt);
   if (I == J)
-    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs);
+    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active);
   else
-    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
+    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active);
   const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
   float *mine = partial + split * slot;
   if (ones && I == J)
@@ -304,6 +365,50 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_conv_kernel(ConvGeom g, long 
     halo_mainloop<WM, NKK, true, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc, rs);
   else
     halo_mainloop<WM, NKK, false, MASK>(g, I * BM, J * BM, sbeg, send, smem, regA, regB, koff_tbl, acc, rs);
+  const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
+  float *mine = partial + split * slot;
+  if (ones && I == J)
+    write_rowsums<WM>(rs, I, dt, d, direct, count, alpha, beta, mine + (long long)ntile * (BM * BM), C);
+  if (direct) {
+    write_tile<WM>(acc, smem, I, J, dt, d, alpha, beta, C);
+    return;
+  }
+  float *out = mine + (long long)tile * (BM * BM);
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
+}
+
+// Convolution A factor through the compile-time row geometry of conv_rows.h;
+// `klen` counts reduction steps (RT output rows of a pair of samples each).
+template <class Cfg>
+__global__ __launch_bounds__(THREADS, 2) void syrk_rows_kernel(RowsGeom g, long long total_steps,
+                                                               long long klen, int ntile,
+                                                               int nsplit, int direct, int d,
+                                                               int ones, float count,
+                                                               float alpha, float beta,
+                                                               float *__restrict__ partial,
+                                                               float *__restrict__ C) {
+  constexpr int WM = Cfg::WM;
+  constexpr int BM = 64 * WM;
+  extern __shared__ float smem[];
+  const int dt = d - ones;   // rows of the tile grid
+  const int tiles = (dt + BM - 1) / BM;
+  int split, tile, I, J;
+  work_decode(blockIdx.x, ntile * nsplit, ntile, tiles, split, tile, I, J);
+  // padding columns, the planes of zeros and everything else not staged later
+  for (int e = threadIdx.x; e < Cfg::lds_floats(false); e += THREADS) smem[e] = 0.f;
+  __syncthreads();
+  const long long sbeg = (long long)split * klen;
+  long long send = sbeg + klen;
+  if (send > total_steps) send = total_steps;
+  floatx16 acc[WM][WM];
+  zero_acc<WM, WM>(acc);
+  float rs[WM];
+#pragma unroll
+  for (int im = 0; im < WM; ++im) rs[im] = 0.f;
+  if (I == J)
+    rows_mainloop<Cfg, true>(g, I * BM, J * BM, sbeg, send, smem, acc, rs);
+  else
+    rows_mainloop<Cfg, false>(g, I * BM, J * BM, sbeg, send, smem, acc, rs);
   const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
   float *mine = partial + split * slot;
   if (ones && I == J)
@@ -550,15 +655,18 @@ int run_conv_halo(const ConvGeom &g, int n, int d, int ones, float alpha, float 
       {syrk_conv_kernel<2, 25, false>, syrk_conv_kernel<2, 25, true>},
       {syrk_conv_kernel<2, 28, false>, syrk_conv_kernel<2, 28, true>},
       {syrk_conv_kernel<2, 32, false>, syrk_conv_kernel<2, 32, true>}};
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [] {
     for (int i = 0; i < 3; ++i)
-      for (int j = 0; j < 2; ++j)
-        KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kerns[i][j]),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           160 * 1024));
-    attr_set = true;
-  }
+      for (int j = 0; j < 2; ++j) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kerns[i][j]),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 160 * 1024);
+        if (e != hipSuccess) attr_rc = e;
+      }
+  });
+  KFAC_HIP_CHECK(attr_rc);
   float *partial = static_cast<float *>(ws);
   const int direct = p.nsplit == 1 ? 1 : 0;
   const dim3 grid(p.ntile * p.nsplit), block(THREADS);
@@ -571,6 +679,69 @@ int run_conv_halo(const ConvGeom &g, int n, int d, int ones, float alpha, float 
   KFAC_HIP_CHECK(hipGetLastError());
   if (direct) return KFAC_OK;
   return finish_partials(p, d, ones, count, alpha, beta, C, partial, stream);
+}
+
+// The compile-time-geometry kernel (conv_rows.h) for one of its instantiations.
+template <class Cfg>
+int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int ones, float alpha,
+                  float beta, float *C, void *ws, size_t ws_bytes, hipStream_t stream) {
+  RowsGeom g;
+  g.x = x;
+  g.n = n; g.C = c; g.H = h; g.W = w;
+  g.ho = ho;
+  g.rgroups = ho / Cfg::RT;
+  g.d_patch = c * Cfg::KK;
+  g.x_bytes = (unsigned)((long long)n * c * h * w * (long long)sizeof(float));
+  const long long total_steps = (long long)(n / 2) * g.rgroups;
+  const float count = (float)((long long)n * ho * Cfg::WS);
+  if (d - ones <= 320) return 1;   // small factors: 64-tiles of the general kernel
+  constexpr size_t lds = (size_t)Cfg::lds_floats(false) * sizeof(float);
+  constexpr int occ = (160 * 1024) / lds >= 3 ? 3 : (int)((160 * 1024) / lds);
+  const SyrkPlan p = plan_rows(d - ones, total_steps, Cfg::NK * Cfg::WM * Cfg::WM * 64 / 2400.0, occ);
+  if (int rc = check_ws(p, ws, ws_bytes)) return rc;
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [] {
+    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(syrk_rows_kernel<Cfg>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  });
+  KFAC_HIP_CHECK(attr_rc);
+  float *partial = static_cast<float *>(ws);
+  const int direct = p.nsplit == 1 ? 1 : 0;
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
+    hipLaunchKernelGGL((syrk_rows_kernel<Cfg>), dim3(p.ntile * p.nsplit), dim3(THREADS), lds, stream,
+                       g, total_steps, p.klen, p.ntile, p.nsplit, direct, d, ones, count, alpha, beta,
+                       partial, C);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  if (direct) return KFAC_OK;
+  return finish_partials(p, d, ones, count, alpha, beta, C, partial, stream);
+}
+
+// Picks the instantiation of the compile-time-geometry kernel that matches the
+// convolution; 1 when there is none (the caller then takes a general kernel).
+int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
+                  int pw, int ho, int wo, int d, int ones, float alpha, float beta, float *C,
+                  void *ws, size_t ws_bytes, hipStream_t stream) {
+  if (getenv("KFAC_CONV_ROWS_OFF")) return 1;   // tuning override: the general kernels only
+  if (n % 2 != 0 || kh != kw || sy != sx || ph != pw) return 1;
+  if ((long long)n * c * h * w * (long long)sizeof(float) >= (1ll << 31)) return 1;
+  const bool alt = getenv("KFAC_ROWS_ALT") != nullptr;
+#define KFAC_ROWS_CASE(K, S, P, WS, RT, PAD)                                                      \
+  if (kh == K && sy == S && ph == P && wo == WS && ho % RT == 0)                                  \
+    return run_conv_rows<RowsCfg<2, K, S, P, WS, RT, PAD>>(x, n, c, h, w, ho, d, ones, alpha,     \
+                                                           beta, C, ws, ws_bytes, stream);
+  if (alt) {
+    KFAC_ROWS_CASE(3, 1, 1, 56, 2, 4)
+    KFAC_ROWS_CASE(3, 1, 1, 28, 4, 3)
+  }
+  KFAC_ROWS_CASE(3, 1, 1, 56, 1, 0)
+  KFAC_ROWS_CASE(3, 1, 1, 28, 2, 1)
+  KFAC_ROWS_CASE(3, 1, 1, 14, 7, 3)
+  KFAC_ROWS_CASE(3, 1, 1, 7, 7, 9)
+#undef KFAC_ROWS_CASE
+  return 1;
 }
 
 bool kc_vec_ok(const float *base, long long sample_stride, long long row_stride, int L) {
@@ -631,14 +802,21 @@ LoaderIM<ROWS> make_im(const float *x, int c, int h, int w, int kh, int kw, int 
 
 extern "C" size_t kfac_cov_workspace_bytes(int d, int64_t rows) {
   if (d <= 0) return 0;
-  // upper bound over every reduction length (the convolution kernels count
-  // their panels differently): the split count never exceeds ceil(1536 / tiles)
+  // upper bound over every kernel and reduction length: no plan uses more than
+  // max_splits(tiles) k-slices (plus the slots of the pre-reduction), with 64- or
+  // 128-tiles, with or without a ones column (the tile grid then covers d - 1 rows)
   (void)rows;
-  size_t need = syrk_ws_floats(plan_syrk_panels(d, 1LL << 40, KT));
-  if (d > 1) {   // with a ones column the tile grid covers d - 1 rows
-    const size_t alt = syrk_ws_floats(plan_syrk_panels(d - 1, 1LL << 40, KT));
-    if (alt > need) need = alt;
-  }
+  size_t need = 0;
+  for (int dt = d > 1 ? d - 1 : d; dt <= d; ++dt)
+    for (int bm = 64; bm <= 128; bm *= 2) {
+      SyrkPlan p;
+      p.bm = bm;
+      p.tiles = kfac::ceil_div(dt, bm);
+      p.ntile = p.tiles * (p.tiles + 1) / 2;
+      p.nsplit = (int)max_splits(p.ntile);
+      p.nreduced = p.nsplit > kFinishSplits ? kFinishSplits : 0;
+      need = std::max(need, syrk_ws_floats(p));
+    }
   return need * sizeof(float);
 }
 
@@ -713,6 +891,11 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
     l64.px_stride = l128.px_stride = (unsigned)sx;
     return run_syrk(l64, l128, d, ones, K, alpha, beta, C, ws, ws_bytes, s);
   }
+  {
+    const int rc = try_conv_rows(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, d, ones, alpha, beta, C,
+                                 ws, ws_bytes, s);
+    if (rc <= 0) return rc;   // 1 = no instantiation for this shape
+  }
   ConvGeom geom;
   if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, &geom)) {
     const int rc = run_conv_halo(geom, n, d, ones, alpha, beta, C, ws, ws_bytes, s);
@@ -721,4 +904,368 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
   return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo),
                   make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo), d, ones, K, alpha,
                   beta, C, ws, ws_bytes, s);
+}
+
+// ---------------------------------------------------------------------------
+// Grouped launch: the factors of many small layers in a handful of launches.
+//
+// A network has dozens of factors whose SYRK is far too small to fill the GPU
+// (a few tiles, or a few hundred reduction panels): launched one by one each
+// costs a launch whose workgroups run two to six panels between a prologue and
+// an epilogue.  A group takes a list of such factors, cuts all of them into
+// (factor, tile, k-slice) tasks of about equal length (so a long reduction over
+// one tile and a short one over thousands of tiles end up in workgroups of
+// similar duration, ~100 panels where the work allows it) and runs the tasks of
+// all factors from one task table: one launch per loader kind, one for the
+// split-K finish.  All grouped factors use 64-tiles.
+// ---------------------------------------------------------------------------
+namespace {
+
+struct GroupItemStatic {
+  int d, ones, tiles, ntile, nsplit, direct;
+  long long K, klen;      // reduction length; per k-slice (a multiple of KT)
+  long long part_off;     // floats from the workspace base to this item's partial slots
+  float count;            // reduction length as a float: the corner entry of a ones column
+  int kind;               // KFAC_COV_LINEAR / KFAC_COV_SLAB
+  int vec;                // float4 loader
+  unsigned sample_stride, row_stride, L;   // slab: (sample, row, l) strides; l values per sample
+  unsigned line_len, line_stride, px_stride;
+  unsigned ld;            // linear: leading dimension
+  int rows_valid;
+};
+
+struct GroupItemDyn {
+  const float *in;
+  float *out;
+  float alpha, beta;
+};
+
+template <class Loader>
+struct GroupLoader;
+
+template <bool VEC>
+struct GroupLoader<LoaderKC<64, VEC>> {
+  static __device__ __forceinline__ LoaderKC<64, VEC> make(const GroupItemStatic &s, const float *in) {
+    LoaderKC<64, VEC> l;
+    l.base = in;
+    l.sample_stride = s.sample_stride;
+    l.row_stride = s.row_stride;
+    l.L = s.L;
+    l.rows_valid = s.rows_valid;
+    if constexpr (!VEC) {
+      l.line_len = s.line_len;
+      l.line_stride = s.line_stride;
+      l.px_stride = s.px_stride;
+    }
+    return l;
+  }
+};
+
+template <bool VEC>
+struct GroupLoader<LoaderKS<64, VEC>> {
+  static __device__ __forceinline__ LoaderKS<64, VEC> make(const GroupItemStatic &s, const float *in) {
+    LoaderKS<64, VEC> l;
+    l.base = in;
+    l.extra = nullptr;
+    l.ld = s.ld;
+    l.rows_valid = s.rows_valid;
+    l.has_extra = 0;
+    return l;
+  }
+};
+
+// task = (item, tile + ntile * k-slice)
+template <class Loader>
+__global__ __launch_bounds__(THREADS, 3) void syrk_group_kernel(const GroupItemStatic *__restrict__ st,
+                                                                const GroupItemDyn *__restrict__ dy,
+                                                                const int2 *__restrict__ tasks,
+                                                                float *__restrict__ ws) {
+  constexpr int WM = 1, BM = 64;
+  __shared__ float lds[2 * Panel<BM>::kFloats];
+  static_assert(2 * Panel<BM>::kFloats >= 64 * 65, "LDS too small for the epilogue transpose");
+  float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
+  const int2 task = tasks[blockIdx.x];
+  const GroupItemStatic s = st[task.x];
+  const GroupItemDyn v = dy[task.x];
+  const int split = task.y / s.ntile;
+  const int tile = task.y - split * s.ntile;
+  int I, J;
+  tri_decode(tile, I, J);
+  const int dt = s.d - s.ones;
+  Loader la = GroupLoader<Loader>::make(s, v.in), lb = la;
+  la.init(nullptr, I * BM);
+  lb.init(nullptr, J * BM);
+  const long long kbeg = (long long)split * s.klen;
+  long long kend = kbeg + s.klen;
+  if (kend > s.K) kend = s.K;
+  floatx16 acc[WM][WM];
+  zero_acc<WM, WM>(acc);
+  float rs[WM];
+  rs[0] = 0.f;
+  const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt);
+  if (I == J)
+    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active);
+  else
+    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active);
+  const long long slot = (long long)s.ntile * (BM * BM) + (long long)s.tiles * BM;
+  float *mine = ws + s.part_off + split * slot;
+  if (s.ones && I == J)
+    write_rowsums<WM>(rs, I, dt, s.d, s.direct, s.count, v.alpha, v.beta,
+                      mine + (long long)s.ntile * (BM * BM), v.out);
+  if (s.direct) {
+    write_tile<WM>(acc, lds, I, J, dt, s.d, v.alpha, v.beta, v.out);
+    return;
+  }
+  float *out = mine + (long long)tile * (BM * BM);
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float val) { out[r * BM + c] = val; });
+}
+
+// task = (item, 64 x 64 block of the lower triangle); sums the item's k-slices
+// in a fixed order and writes the block and its mirror image.
+__global__ __launch_bounds__(256) void finish_group_kernel(const GroupItemStatic *__restrict__ st,
+                                                           const GroupItemDyn *__restrict__ dy,
+                                                           const int2 *__restrict__ tasks,
+                                                           const float *__restrict__ ws) {
+  __shared__ float tile[64][65];
+  const int2 task = tasks[blockIdx.x];
+  const GroupItemStatic s = st[task.x];
+  const GroupItemDyn v = dy[task.x];
+  int si, sj;
+  tri_decode(task.y, si, sj);
+  const int dt = s.d - s.ones, d = s.d;
+  const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
+  const long long slot = (long long)s.ntile * 4096 + (long long)s.tiles * 64;
+  const float *p0 = ws + s.part_off + (long long)task.y * 4096;
+  float sum[16];
+#pragma unroll
+  for (int p = 0; p < 16; ++p) sum[p] = 0.f;
+  for (int k = 0; k < s.nsplit; ++k) {
+    const float *pk = p0 + k * slot;
+#pragma unroll
+    for (int p = 0; p < 16; ++p) sum[p] += pk[(lr0 + 4 * p) * 64 + lc];
+  }
+  float *C = v.out;
+  const float alpha = v.alpha, beta = v.beta;
+  if (s.ones && si == sj && threadIdx.x < 64) {
+    const int row = si * 64 + threadIdx.x;
+    const float *v0 = ws + s.part_off + (long long)s.ntile * 4096 + row;
+    float a = 0.f;
+    for (int k = 0; k < s.nsplit; ++k) a += v0[k * slot];
+    if (row < dt) {
+      float val = alpha * a;
+      if (beta != 0.f) val += beta * C[(long long)(d - 1) * d + row];
+      C[(long long)(d - 1) * d + row] = val;
+      C[(long long)row * d + d - 1] = val;
+    }
+    if (row == 0) {
+      float val = alpha * s.count;
+      if (beta != 0.f) val += beta * C[(long long)(d - 1) * d + d - 1];
+      C[(long long)(d - 1) * d + d - 1] = val;
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < 16; ++p) {
+    const int lr = lr0 + 4 * p;
+    const int r = si * 64 + lr, c = sj * 64 + lc;
+    float val = alpha * sum[p];
+    if (beta != 0.f && r < dt && c < dt) val += beta * C[(long long)r * d + c];
+    tile[lr][lc] = val;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < 16; ++p) {
+    const int lr = lr0 + 4 * p;
+    const int r = si * 64 + lr, c = sj * 64 + lc;
+    if (si == sj) {
+      if (r < dt && c < dt) C[(long long)r * d + c] = (lc <= lr) ? tile[lr][lc] : tile[lc][lr];
+    } else {
+      if (r < dt && c < dt) C[(long long)r * d + c] = tile[lr][lc];
+      const int mr = sj * 64 + lr, mc = si * 64 + lc;
+      if (mr < dt && mc < dt) C[(long long)mr * d + mc] = tile[lc][lr];
+    }
+  }
+}
+
+// Emits `natural` dealt so that each XCD (workgroup i of a launch runs on XCD
+// i % 8) receives one contiguous run of it.
+void deal_to_xcds(std::vector<int2> &table, const std::vector<int2> &natural) {
+  const size_t n = natural.size();
+  const size_t chunk = (n + kXcds - 1) / kXcds;
+  for (size_t p = 0; p < chunk; ++p)
+    for (size_t x = 0; x < (size_t)kXcds; ++x) {
+      const size_t i = x * chunk + p;
+      if (i < n) table.push_back(natural[i]);
+    }
+}
+
+constexpr int kGroupKinds = 4;   // slab float4, slab scalar, linear float4, linear scalar
+
+}  // namespace
+
+struct kfac_cov_group {
+  int count = 0;
+  std::vector<GroupItemStatic> items;
+  std::vector<GroupItemDyn> dyn;
+  size_t ws_floats = 0;
+  int task0[kGroupKinds] = {0, 0, 0, 0}, ntask[kGroupKinds] = {0, 0, 0, 0};
+  int ftask0 = 0, nftask = 0;
+  kfac::DevTable d_items, d_dyn, d_tasks;
+};
+
+extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac_cov_group_t *out) {
+  KFAC_REQUIRE(out != nullptr, "group_out is null");
+  *out = nullptr;
+  KFAC_REQUIRE(count >= 0 && (count == 0 || items), "bad item list");
+  auto *g = new (std::nothrow) kfac_cov_group;
+  if (!g) return kfac::fail(KFAC_ENOMEM, "out of host memory");
+  g->count = count;
+  g->items.resize(count);
+  g->dyn.resize(count);
+  std::vector<long long> nk(count);
+  double work = 0;   // tile-panels
+  for (int i = 0; i < count; ++i) {
+    const kfac_cov_item &it = items[i];
+    GroupItemStatic &s = g->items[i];
+    memset(&s, 0, sizeof(s));
+    auto bad = [&](const char *what) {
+      delete g;
+      return kfac::fail(KFAC_EINVAL, "item %d: %s", i, what);
+    };
+    if (it.kind != KFAC_COV_LINEAR && it.kind != KFAC_COV_SLAB) return bad("unknown kind");
+    if (it.n <= 0 || it.c <= 0) return bad("bad shape");
+    s.kind = it.kind;
+    s.ones = it.append_ones ? 1 : 0;
+    if (it.kind == KFAC_COV_LINEAR) {
+      // x (n, c) row-major
+      if ((long long)it.n * it.c >= 0x7fffffffLL) return bad("input too large");
+      s.K = it.n;
+      s.ld = (unsigned)it.c;
+      s.rows_valid = it.c;
+      s.vec = (it.aligned && it.c % 4 == 0) ? 1 : 0;
+    } else {
+      // (n, c, h, w) tensor; every sy-th line and sx-th pixel of it when subsampled
+      if (it.h <= 0 || it.w <= 0 || it.sy <= 0 || it.sx <= 0) return bad("bad shape");
+      if ((long long)it.n * it.c * it.h * it.w >= 0x7fffffffLL) return bad("input too large");
+      const int ho = (it.h - 1) / it.sy + 1, wo = (it.w - 1) / it.sx + 1;
+      const int hw = it.h * it.w;
+      s.K = (long long)it.n * ho * wo;
+      s.sample_stride = (unsigned)((long long)it.c * hw);
+      s.row_stride = (unsigned)hw;
+      s.L = (unsigned)(ho * wo);
+      s.rows_valid = it.c;
+      if (it.sy != 1 || it.sx != 1) {
+        s.line_len = (unsigned)wo;
+        s.line_stride = (unsigned)(it.sy * it.w);
+        s.px_stride = (unsigned)it.sx;
+        s.vec = 0;
+      } else {
+        s.px_stride = 1;
+        s.vec = (it.aligned && hw % 4 == 0) ? 1 : 0;
+      }
+    }
+    s.d = it.c + s.ones;
+    s.count = (float)s.K;
+    s.tiles = kfac::ceil_div(it.c, 64);
+    s.ntile = s.tiles * (s.tiles + 1) / 2;
+    nk[i] = kfac::ceil_div<long long>(s.K, KT);
+    work += (double)s.ntile * (double)nk[i];
+  }
+  // k-slices: workgroups of about equal length, ~2300 of them when the work allows
+  // it, none shorter than 8 panels (unless the whole reduction is) and at most 256 per factor
+  double per_wg = work / 2304.0;
+  if (per_wg < 8.0) per_wg = 8.0;
+  if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override: panels per workgroup
+    const double v = atof(env);
+    if (v >= 1.0) per_wg = v;
+  }
+  size_t off = 0;
+  std::vector<int2> natural[kGroupKinds], fin;
+  for (int i = 0; i < count; ++i) {
+    GroupItemStatic &s = g->items[i];
+    long long ns = (long long)((double)nk[i] / per_wg + 0.5);
+    if (ns < 1) ns = 1;
+    if (ns > 256) ns = 256;
+    if (ns > nk[i]) ns = nk[i];
+    const long long per = kfac::ceil_div(nk[i], ns);
+    s.nsplit = (int)kfac::ceil_div(nk[i], per);
+    s.klen = per * KT;
+    s.direct = s.nsplit == 1 ? 1 : 0;
+    s.part_off = (long long)off;
+    const size_t slot = (size_t)s.ntile * 4096 + (size_t)s.tiles * 64;
+    if (!s.direct) off += (size_t)s.nsplit * slot;
+    else if (s.ones) off += slot;   // the row sums of a direct item still pass through its slot
+    const int kind = (s.kind == KFAC_COV_SLAB ? 0 : 2) + (s.vec ? 0 : 1);
+    for (int w = 0; w < s.ntile * s.nsplit; ++w) natural[kind].push_back(make_int2(i, w));
+    if (!s.direct)
+      for (int b = 0; b < s.ntile; ++b) fin.push_back(make_int2(i, b));
+  }
+  g->ws_floats = off;
+  std::vector<int2> tasks;
+  for (int k = 0; k < kGroupKinds; ++k) {
+    g->task0[k] = (int)tasks.size();
+    g->ntask[k] = (int)natural[k].size();
+    deal_to_xcds(tasks, natural[k]);
+  }
+  g->ftask0 = (int)tasks.size();
+  g->nftask = (int)fin.size();
+  tasks.insert(tasks.end(), fin.begin(), fin.end());
+  if (tasks.empty()) tasks.push_back(make_int2(0, 0));
+  int rc = g->d_items.set(g->items.data(), sizeof(GroupItemStatic) * (size_t)count, nullptr);
+  if (rc == KFAC_OK) rc = g->d_tasks.set(tasks.data(), sizeof(int2) * tasks.size(), nullptr);
+  if (rc != KFAC_OK) {
+    delete g;
+    return rc;
+  }
+  *out = g;
+  return KFAC_OK;
+}
+
+extern "C" size_t kfac_cov_group_workspace_bytes(kfac_cov_group_t group) {
+  return group ? group->ws_floats * sizeof(float) + 256 : 0;
+}
+
+extern "C" int kfac_cov_group_destroy(kfac_cov_group_t group) {
+  delete group;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const *inputs,
+                                      float *const *outputs, const float *alpha,
+                                      const float *beta, void *ws, size_t ws_bytes, void *stream) {
+  KFAC_REQUIRE(group != nullptr, "group is null");
+  const int count = group->count;
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(inputs && outputs && alpha && beta, "null table");
+  if (ws == nullptr || ws_bytes < kfac_cov_group_workspace_bytes(group))
+    return kfac::fail(KFAC_ENOMEM, "covariance group workspace too small: %zu < %zu bytes", ws_bytes,
+                      kfac_cov_group_workspace_bytes(group));
+  for (int i = 0; i < count; ++i) {
+    KFAC_REQUIRE(inputs[i] && outputs[i], "item %d: null pointer", i);
+    KFAC_REQUIRE(!group->items[i].vec || reinterpret_cast<uintptr_t>(inputs[i]) % 16 == 0,
+                 "item %d was declared 16-byte aligned and is not", i);
+    group->dyn[i] = GroupItemDyn{inputs[i], outputs[i], alpha[i], beta[i]};
+  }
+  hipStream_t s = kfac::as_stream(stream);
+  if (int rc = group->d_dyn.set(group->dyn.data(), sizeof(GroupItemDyn) * (size_t)count, s)) return rc;
+  float *base = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
+  const GroupItemStatic *st = group->d_items.as<const GroupItemStatic>();
+  const GroupItemDyn *dy = group->d_dyn.as<const GroupItemDyn>();
+  const int2 *tasks = group->d_tasks.as<const int2>();
+  using Kern = void (*)(const GroupItemStatic *, const GroupItemDyn *, const int2 *, float *);
+  static const Kern kerns[kGroupKinds] = {
+      syrk_group_kernel<LoaderKC<64, true>>, syrk_group_kernel<LoaderKC<64, false>>,
+      syrk_group_kernel<LoaderKS<64, true>>, syrk_group_kernel<LoaderKS<64, false>>};
+  for (int k = 0; k < kGroupKinds; ++k) {
+    if (group->ntask[k] == 0) continue;
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
+    hipLaunchKernelGGL(kerns[k], dim3(group->ntask[k]), dim3(THREADS), 0, s, st, dy,
+                       tasks + group->task0[k], base);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  if (group->nftask > 0) {
+    hipLaunchKernelGGL(finish_group_kernel, dim3(group->nftask), dim3(256), 0, s, st, dy,
+                       tasks + group->ftask0, base);
+    KFAC_HIP_CHECK(hipGetLastError());
+  }
+  return KFAC_OK;
 }

@@ -86,7 +86,12 @@ __global__ __launch_bounds__(kThreads) void axpby_kernel(
     const float *__restrict__ x, float *__restrict__ y, long long n, float a, float b) {
   long long i = (long long)blockIdx.x * kThreads + threadIdx.x;
   const long long stride = (long long)gridDim.x * kThreads;
-  for (; i < n; i += stride) y[i] = a * x[i] + b * y[i];
+  // b == 0 overwrites: y is not read (it may be uninitialised memory holding NaN)
+  if (b == 0.f) {
+    for (; i < n; i += stride) y[i] = a * x[i];
+  } else {
+    for (; i < n; i += stride) y[i] = a * x[i] + b * y[i];
+  }
 }
 
 __global__ __launch_bounds__(kThreads) void add_diag_kernel(

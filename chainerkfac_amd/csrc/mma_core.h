@@ -392,10 +392,15 @@ __device__ __forceinline__ float fetch(const float *lds, int row, int k) {
 // With RS the lane also sums the A operand values it feeds to the matrix cores:
 // rs[im] ends as the sum over this lane's k-values (k = lane / 32 mod 2) of row
 // (wave_m * WM + im) * 32 + lane % 32, i.e. half of that row's sum.
+// A wave with `active` false stages panels like the others but feeds nothing to
+// the matrix cores (its block of the tile is not needed: above the diagonal of a
+// symmetric product, or past the end of the matrix); its accumulators stay as
+// they are.
 template <int WM, int WN, bool SAME, bool RS, class LA, class LB>
 __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int rowA0, int rowB0,
                                               long long kbeg, long long kend, float *ldsA,
-                                              float *ldsB, floatx16 (&acc)[WM][WN], float *rs) {
+                                              float *ldsB, floatx16 (&acc)[WM][WN], float *rs,
+                                              bool active = true) {
   constexpr int RA = 64 * WM, RB = 64 * WN;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -415,6 +420,7 @@ __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int ro
       la.load(ra, rowA0, k0 + KT, kend);
       if (!SAME) lb.load(rb, rowB0, k0 + KT, kend);
     }
+    if (active) {
 #pragma unroll
     for (int kk = 0; kk < KT / 2; ++kk) {
       float a[WM], b[WN];
@@ -438,6 +444,7 @@ __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int ro
         for (int in = 0; in < WN; ++in)
           acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
     }
+    }
     __syncthreads();
   }
 }
@@ -445,16 +452,28 @@ __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int ro
 template <int WM, int WN, bool SAME, class LA, class LB>
 __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, int rowB0,
                                          long long kbeg, long long kend, float *ldsA,
-                                         float *ldsB, floatx16 (&acc)[WM][WN]) {
-  mainloop_impl<WM, WN, SAME, false>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, nullptr);
+                                         float *ldsB, floatx16 (&acc)[WM][WN], bool active = true) {
+  mainloop_impl<WM, WN, SAME, false>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, nullptr,
+                                     active);
 }
 
 template <int WM, int WN, bool SAME, class LA, class LB>
 __device__ __forceinline__ void mainloop_rowsum(const LA &la, const LB &lb, int rowA0, int rowB0,
                                                 long long kbeg, long long kend, float *ldsA,
                                                 float *ldsB, floatx16 (&acc)[WM][WN],
-                                                float (&rs)[WM]) {
-  mainloop_impl<WM, WN, SAME, true>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, rs);
+                                                float (&rs)[WM], bool active = true) {
+  mainloop_impl<WM, WN, SAME, true>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, rs, active);
+}
+
+// Whether this wave's block of a symmetric product's tile (first rows row0A /
+// row0B, dt rows in all) is needed: it is not when it lies entirely above the
+// diagonal (the epilogues take those entries from the mirrored block) or past
+// the end of the matrix.
+template <int WM>
+__device__ __forceinline__ bool syrk_wave_active(int row0A, int row0B, int dt) {
+  const int wave = threadIdx.x >> 6;
+  const int ra = row0A + (wave >> 1) * WM * 32, rb = row0B + (wave & 1) * WM * 32;
+  return ra + WM * 32 > rb && ra < dt && rb < dt;
 }
 
 // Set every accumulator element of this lane to f(row, col), row / col relative
@@ -505,9 +524,12 @@ __device__ __forceinline__ void zero_acc(floatx16 (&acc)[WM][WN]) {
       for (int v = 0; v < 16; ++v) acc[im][in][v] = 0.f;
 }
 
-// Writes the finished tile: C[I,J] = alpha*acc + beta*C[I,J] and, for I != J,
-// the mirror C[J,I], 64x64 quadrant by quadrant through an LDS transpose so
-// that every global access is a contiguous row segment.
+// Writes the finished tile: C[I,J] = alpha*acc + beta*C[I,J] and its mirror
+// image C[J,I], 64x64 quadrant by quadrant through an LDS transpose so that
+// every global access is a contiguous row segment.  Only entries on or below
+// the diagonal of C are taken from the accumulators: a quadrant above the
+// diagonal of a diagonal tile is skipped (it is the mirror of the one below),
+// and a quadrant on the diagonal writes its upper triangle from its lower one.
 // Rows and columns below dt (the tiled part); d is the leading dimension of C.
 template <int WM>
 __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
@@ -518,6 +540,8 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
   const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
   for (int q = 0; q < WM * WM; ++q) {
     const int qm = q / WM, qn = q % WM;
+    if (I == J && qm < qn) continue;
+    const bool diag = I == J && qm == qn;
     __syncthreads();
     for_each_acc<WM, WM>(acc, [&](int r, int c, float v) {
       if (r / 64 == qm && c / 64 == qn) t[r % 64][c % 64] = v;
@@ -529,20 +553,24 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
       const int lr = lr0 + 4 * p;
       const int r = r0 + lr, c = c0 + lc;
       float v = alpha * t[lr][lc];
-      const bool ok = r < dt && c < dt;
+      const bool ok = r < dt && c < dt && (!diag || lc <= lr);
       if (ok) {
         if (beta != 0.f) v += beta * C[(long long)r * d + c];
         C[(long long)r * d + c] = v;
       }
-      if (beta != 0.f && I != J) t[lr][lc] = v;   // mirror gets the same value
+      if (beta != 0.f) t[lr][lc] = v;   // the mirror gets the same value
     }
-    if (I != J) {
-      if (beta != 0.f) __syncthreads();
+    if (beta != 0.f) __syncthreads();
 #pragma unroll 4
-      for (int p = 0; p < 16; ++p) {
-        const int lr = lr0 + 4 * p;
+    for (int p = 0; p < 16; ++p) {
+      const int lr = lr0 + 4 * p;
+      const float v = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
+      if (diag) {
+        const int r = r0 + lr, c = c0 + lc;     // upper triangle of the quadrant itself
+        if (lc > lr && r < dt && c < dt) C[(long long)r * d + c] = v;
+      } else {
         const int mr = c0 + lr, mc = r0 + lc;   // row of the mirrored quadrant = column here
-        if (mr < dt && mc < dt) C[(long long)mr * d + mc] = (beta != 0.f) ? t[lc][lr] : alpha * t[lc][lr];
+        if (mr < dt && mc < dt) C[(long long)mr * d + mc] = v;
       }
     }
   }

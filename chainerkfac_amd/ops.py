@@ -84,6 +84,107 @@ def cov_conv_g(gy, alpha, beta=0.0, out=None, stream=None):
     return out
 
 
+COV_LINEAR, COV_SLAB = 0, 1
+
+
+class _CovItem(ctypes.Structure):
+    _fields_ = [(name, ctypes.c_int32) for name in
+                ('kind', 'n', 'c', 'h', 'w', 'sy', 'sx', 'append_ones', 'aligned')]
+
+
+class CovGroup(object):
+    """The covariances of a fixed list of small layers as one grouped launch.
+    ``items``: tuples ``(kind, n, c, h, w, sy, sx, append_ones, aligned)``."""
+
+    def __init__(self, items):
+        self.items = tuple(tuple(int(v) for v in it) for it in items)
+        lib = _lib.load()
+        arr = (_CovItem * max(len(self.items), 1))()
+        for dst, it in zip(arr, self.items):
+            (dst.kind, dst.n, dst.c, dst.h, dst.w, dst.sy, dst.sx, dst.append_ones, dst.aligned) = it
+        plan = ctypes.c_void_p()
+        _lib.check(lib.kfac_cov_group_create(len(self.items), ctypes.cast(arr, ctypes.c_void_p),
+                                             ctypes.byref(plan)))
+        self._plan = plan
+        self.workspace_bytes = lib.kfac_cov_group_workspace_bytes(plan)
+
+    def __del__(self):
+        try:
+            plan, self._plan = self._plan, None
+            if plan is not None:
+                _lib._lib.kfac_cov_group_destroy(plan)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+    def run(self, inputs, outputs, alphas, betas, stream=None):
+        if len(inputs) != len(self.items) or len(outputs) != len(self.items):
+            raise ValueError('expected {} items'.format(len(self.items)))
+        if not self.items:
+            return outputs
+        for it, x, out in zip(self.items, inputs, outputs):
+            _dev.require_gpu_tensor(x, 'input')
+            _dev.require_gpu_tensor(out, 'out')
+            d = it[2] + it[7]
+            want = it[1] * it[2] * (it[3] * it[4] if it[0] == COV_SLAB else 1)
+            if x.numel() != want or tuple(out.shape) != (d, d):
+                raise ValueError('item {} does not match its tensors'.format(it))
+        ws = _dev.workspace('cov_group', self.workspace_bytes, inputs[0].device)
+        _lib.check(_lib.load().kfac_cov_group_run_f32(
+            self._plan, _lib.ptr_array([x.data_ptr() for x in inputs]),
+            _lib.ptr_array([o.data_ptr() for o in outputs]),
+            ctypes.cast(_lib.f32_array(alphas), ctypes.c_void_p),
+            ctypes.cast(_lib.f32_array(betas), ctypes.c_void_p),
+            ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
+        return outputs
+
+
+_cov_groups = None
+
+
+def cov_group(items):
+    """Cached ``CovGroup`` for a list of item descriptors."""
+    global _cov_groups
+    if _cov_groups is None:
+        _cov_groups = _PlanCache(32)
+    key = tuple(tuple(int(v) for v in it) for it in items)
+    return _cov_groups.get(key, lambda: CovGroup(key))
+
+
+class PendingCovs(object):
+    """Collects the factor computations of layers that are too small to fill
+    the GPU on their own; ``flush`` runs all of them as one grouped launch.
+    The tensors are kept alive until then."""
+
+    #: a factor is deferred when its SYRK has at most this many flops (rows * d * (d+1))
+    max_flops = 2.5e9
+
+    def __init__(self):
+        self.items, self.inputs, self.outputs, self.alphas, self.betas = [], [], [], [], []
+
+    def accepts(self, rows, d):
+        return float(rows) * d * (d + 1) <= self.max_flops
+
+    def add(self, kind, x, ones, out, alpha, beta, stride=1):
+        if kind == COV_LINEAR:
+            n, c = x.shape
+            h = w = 1
+        else:
+            n, c, h, w = x.shape
+        self.items.append((kind, n, c, h, w, stride, stride, int(bool(ones)), int(x.data_ptr() % 16 == 0)))
+        self.inputs.append(x)
+        self.outputs.append(out)
+        self.alphas.append(alpha)
+        self.betas.append(beta)
+
+    def flush(self, stream=None):
+        if not self.items:
+            return
+        try:
+            cov_group(self.items).run(self.inputs, self.outputs, self.alphas, self.betas, stream)
+        finally:
+            self.__init__()
+
+
 def bn_grad_matrix(x, gy, eps, gy_scale, has_gamma=True, has_beta=True, out=None, stream=None):
     """(n, 2C) matrix [sum_hw gy'*h | sum_hw gy'] of a batch-norm layer."""
     _dev.require_gpu_tensor(x, 'x')

@@ -75,6 +75,9 @@ class FisherBlock(object):
         self.diagonalize = False
         # (acc_iters, index of the current micro-batch); set by the optimizer
         self.acc_state = (1, 0)
+        #: ops.PendingCovs of the optimizer, or None: where the factors of small
+        #: layers wait for one grouped launch instead of being computed on the spot
+        self.pending_covs = None
         self._bufs = {}
 
     # ---- identity -------------------------------------------------------
@@ -145,6 +148,15 @@ class FisherBlock(object):
             return (self._buffer('acc_' + key, shape, device), scale / acc_iters,
                     0.0 if acc_index == 0 else 1.0)
         return self._buffer(key, shape, device), scale, 0.0
+
+    def _defer_cov(self, kind, x, ones, rows, out, alpha, beta, stride=1):
+        """Hands a factor to the grouped launch if there is one and the factor
+        is small; True when it did (``out`` is then filled at the flush)."""
+        pending = self.pending_covs
+        if pending is None or not pending.accepts(rows, out.shape[0]):
+            return False
+        pending.add(kind, x, ones, out, alpha, beta, stride)
+        return True
 
     # ---- moving average ---------------------------------------------------
     def update_cov_emas(self):

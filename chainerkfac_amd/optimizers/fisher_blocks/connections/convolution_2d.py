@@ -22,14 +22,20 @@ class FisherBlockConvolution2D(FisherBlockConnection):
         has_b = link.b is not None
         d = c * ksize * ksize + (1 if has_b else 0)
         out, alpha, beta = self._cov_target('A', (d, d), x.device, 1.0 / n)
+        if ksize == 1 and pad == 0:
+            # a 1x1 convolution's patch matrix is the (subsampled) NCHW tensor itself
+            ho, wo = (x.shape[2] - 1) // stride + 1, (x.shape[3] - 1) // stride + 1
+            if self._defer_cov(ops.COV_SLAB, x, has_b, n * ho * wo, out, alpha, beta, stride):
+                return out
         return ops.cov_conv_a(x, ksize, stride, pad, has_b, alpha, beta, out)
 
     def compute_G(self, in_data, out_grad_data):
         gy = out_grad_data[0]
         n, c, ho, wo = gy.shape
         scale = self.gy_scale(n) ** 2 / (n * ho * wo)
-        out, alpha, beta = self._cov_target('G', (c, c), gy.device, scale)
-        G = ops.cov_conv_g(gy, alpha, beta, out)
         if getattr(self.link, 'diag', False):
             raise NotImplementedError('link.diag (diagonal G) is not supported on the HIP path')
-        return G
+        out, alpha, beta = self._cov_target('G', (c, c), gy.device, scale)
+        if self._defer_cov(ops.COV_SLAB, gy, False, n * ho * wo, out, alpha, beta):
+            return out
+        return ops.cov_conv_g(gy, alpha, beta, out)

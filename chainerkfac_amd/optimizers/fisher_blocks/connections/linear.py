@@ -17,6 +17,8 @@ class FisherBlockLinear(FisherBlockConnection):
         has_b = self.link.b is not None
         d = d_in + (1 if has_b else 0)
         out, alpha, beta = self._cov_target('A', (d, d), x.device, 1.0 / n)
+        if self._defer_cov(ops.COV_LINEAR, x, has_b, n, out, alpha, beta):
+            return out
         return ops.cov_linear(x, has_b, alpha, beta, out)
 
     def compute_G(self, in_data, out_grad_data):
@@ -24,4 +26,6 @@ class FisherBlockLinear(FisherBlockConnection):
         n, d_out = gy.shape
         scale = self.gy_scale(n) ** 2 / n
         out, alpha, beta = self._cov_target('G', (d_out, d_out), gy.device, scale)
+        if self._defer_cov(ops.COV_LINEAR, gy, False, n, out, alpha, beta):
+            return out
         return ops.cov_linear(gy, False, alpha, beta, out)

@@ -99,6 +99,8 @@ class FisherBlockBatchNormalization(FisherBlock):
                                out=self._buffer('U', (n, width), x.device))
         self._U = U
         out, alpha, beta = self._cov_target('F', (width, width), x.device, 1.0 / n)
+        if self._defer_cov(ops.COV_LINEAR, U, False, n, out, alpha, beta):
+            return out
         return ops.cov_linear(U, False, alpha, beta, out)
 
     def update_cov_emas(self):

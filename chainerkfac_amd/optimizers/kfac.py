@@ -77,11 +77,13 @@ class KFACHook(links.FunctionHook):
     owner is found through the identity of the weight array (a dictionary
     lookup instead of the reference's scan over all blocks, kfac.py:38-48)."""
 
-    def __init__(self, fblocks, lanes=None):
+    def __init__(self, fblocks, lanes=None, pending=None):
         self.fblocks = fblocks
         self.lanes = lanes
+        self.pending = pending
         self._owner = {}
         for fb in fblocks:
+            fb.pending_covs = pending
             for p in fb.link.params():
                 self._owner[id(p.data)] = fb
 
@@ -161,6 +163,12 @@ class KFAC(object):
     #: dense Cholesky path for every block
     bn_lowrank_inverse = True
 
+    #: collect the factors of layers that are too small to fill the GPU (most
+    #: 1x1 convolutions' G or A, batch-norm and linear blocks) and compute them
+    #: with one grouped launch after the backward pass; False computes every
+    #: factor inside its hook call.  Read at ``setup``.
+    group_small_factors = True
+
     #: number of side streams the per-layer factor and preconditioning kernels
     #: are dealt onto (layers are independent of each other and most of their
     #: kernels are too small to fill the GPU alone); 0 keeps everything on the
@@ -222,8 +230,16 @@ class KFAC(object):
                 continue
             self.fblocks.append(fblock)
         self._lanes = _dev.Lanes(self.lanes)
-        self.kfhook = KFACHook(self.fblocks, self._lanes)
+        self._pending = ops.PendingCovs() if self.group_small_factors else None
+        self.kfhook = KFACHook(self.fblocks, self._lanes, self._pending)
         return self
+
+    def finish_covs(self):
+        """Joins the side streams the hooks queued factor kernels on and runs
+        the grouped launch of the factors that were deferred."""
+        self._lanes.join()
+        if self._pending is not None:
+            self._pending.flush()
 
     def create_update_rule(self):
         return KFACUpdateRule(self.hyperparam, adjust_momentum=self.adjust_momentum)
@@ -306,8 +322,8 @@ class KFAC(object):
                 for param in self.target.params():
                     param._loss_scale = self._loss_scale
             del loss
-        # the factor kernels of this pass ran on the side streams
-        self._lanes.join()
+        # the factor kernels of this pass ran on the side streams; the small ones are still to run
+        self.finish_covs()
 
         if self.acc_iters > 1:
             if self.accumulate():
@@ -377,7 +393,7 @@ class KFAC(object):
         self.precondition(fblocks)
 
     def update_cov_emas(self, fblocks):
-        self._lanes.join()   # factors computed by the hooks
+        self.finish_covs()   # factors computed by the hooks
         for fblock in fblocks:
             fblock.update_cov_emas()
 

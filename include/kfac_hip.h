@@ -118,6 +118,37 @@ int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, float alpha,
                         float beta, float *C, void *ws, size_t ws_bytes,
                         void *stream);
 
+/* The covariances of many (small) layers in a handful of launches.  A group is
+ * created once for a list of items -- each what one kfac_cov_linear_f32 or
+ * kfac_cov_conv_g_f32 / 1x1 kfac_cov_conv_a_f32 call would compute -- and run
+ * with that call's pointers and alpha / beta per item:
+ *   KFAC_COV_LINEAR  x (n, c) row-major: out = beta*out + alpha [x, 1]^T [x, 1]
+ *                    (linear.py:14-46, and the last step of the batch-norm
+ *                    factor, batch_normalization.py:121-131)
+ *   KFAC_COV_SLAB    the (n, c, h, w) tensor read as rows = channels, reduction
+ *                    over samples and pixels: the output-gradient factor of a
+ *                    convolution (convolution_2d.py:43-72) and, with
+ *                    append_ones, the input factor of a 1x1 convolution without
+ *                    padding (convolution_2d.py:19-41); sy / sx > 1 take every
+ *                    sy-th line and sx-th pixel (a strided 1x1 convolution).
+ * `aligned` states that the item's input pointer will be 16-byte aligned (it is
+ * then read with 16-byte loads where its strides allow).  The results are those
+ * of the single calls up to the order of the floating-point sums.  Replaces the
+ * per-layer loop over compute_A / compute_G / compute_F for layers too small to
+ * fill the GPU one at a time; no single call of the reference corresponds. */
+#define KFAC_COV_LINEAR 0
+#define KFAC_COV_SLAB 1
+typedef struct kfac_cov_item {
+  int32_t kind, n, c, h, w, sy, sx, append_ones, aligned;
+} kfac_cov_item;
+typedef struct kfac_cov_group *kfac_cov_group_t;
+int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac_cov_group_t *group_out);
+size_t kfac_cov_group_workspace_bytes(kfac_cov_group_t group);
+int kfac_cov_group_destroy(kfac_cov_group_t group);
+int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const *inputs,
+                           float *const *outputs, const float *alpha, const float *beta,
+                           void *ws, size_t ws_bytes, void *stream);
+
 /* Per-sample batch-norm gradient matrix U (n, 2C) = [sum_hw gy'*h | sum_hw gy']
  * with h the batch-normalised x (biased variance, eps inside the root) and
  * gy' = gy*gy_scale; hw = 1 for 2-D inputs.  Only the gamma half / beta half
@@ -131,7 +162,8 @@ int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, int c,
                             int has_beta, float *U, void *ws, size_t ws_bytes,
                             void *stream);
 
-/* y = a*x + b*y over one pair of arrays of `nelems` floats.
+/* y = a*x + b*y over one pair of arrays of `nelems` floats; with b == 0, y is
+ * overwritten without being read.
  * Moving average of optimizers/fisher_block.py:162-163 (a = decay on the new
  * covariance, b = 1-decay) and the unfused accumulation of kfac.py:286-304. */
 int kfac_axpby_f32(const float *x, float *y, int64_t nelems, float a, float b,

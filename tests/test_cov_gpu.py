@@ -70,6 +70,13 @@ CONV_CASES = [
     (1, 60, 20, 112, 3, 1, 1, True),    # rows wider than a step: two column segments
     (2, 12, 38, 38, 7, 2, 3, True),     # 7x7 stride 2, 19x19 outputs
     (3, 130, 9, 9, 3, 1, 0, True),      # no padding, 7x7 outputs, last panel past the channel count
+    # shapes that take the compile-time row-geometry kernel (3x3, pad 1, even batch, 56/28/14/7-wide outputs)
+    (2, 64, 56, 56, 3, 1, 1, True),     # one output row of a sample pair per step
+    (2, 40, 14, 14, 3, 1, 1, True),     # 361: seven rows per step, three tile rows with a ragged last one
+    (4, 37, 7, 7, 3, 1, 1, False),      # 333: channel count that ends inside a panel
+    (2, 150, 7, 7, 3, 1, 1, True),      # 1351: eleven tile rows, panels that start mid-channel
+    (6, 64, 14, 14, 3, 1, 1, True),     # three sample pairs
+    (2, 48, 28, 28, 3, 1, 1, True),     # 433
 ]
 
 
@@ -132,6 +139,77 @@ def test_accumulation_with_ones_column(shape):
     got = out.cpu().numpy()
     assert np.array_equal(got, got.T)
     assert abs(got[-1, -1] - acc[0][-1, -1]) <= 1e-6 * abs(acc[0][-1, -1])
+
+
+def test_grouped_launch_matches_the_single_calls():
+    """One grouped launch for a mixed list of small factors (convolution G, 1x1 convolution A
+    with and without a ones column, strided 1x1, odd pixel counts, linear layers, a batch-norm
+    gradient matrix; with and without accumulation onto an existing factor) against the
+    oracle, and against the single-call entry points."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(17)
+
+    def t(*shape):
+        return torch.from_numpy(r.standard_normal(shape).astype(np.float32)).cuda()
+
+    cases = [
+        # kind, input, ones, stride, alpha, beta
+        (ops.COV_SLAB, t(4, 64, 14, 14), False, 1, 0.25, 0.0),      # G, 64: one tile, float4 loads
+        (ops.COV_SLAB, t(4, 65, 14, 14), True, 1, 0.25, 0.0),       # 1x1 A with ones, 66: ragged second tile
+        (ops.COV_SLAB, t(2, 130, 7, 7), True, 1, 0.5, 0.0),         # 49 pixels: scalar loads
+        (ops.COV_SLAB, t(2, 96, 9, 7), True, 2, 0.5, 0.0),          # strided 1x1: every 2nd line / pixel
+        (ops.COV_SLAB, t(3, 200, 6, 6), False, 1, 1.0, 1.0),        # accumulates onto an existing factor
+        (ops.COV_SLAB, t(8, 32, 56, 56), False, 1, 0.125, 0.0),     # long reduction: several k-slices
+        (ops.COV_LINEAR, t(32, 256), False, 1, 1 / 32, 0.0),        # batch-norm gradient matrix
+        (ops.COV_LINEAR, t(16, 101), True, 1, 1 / 16, 1.0),         # linear A with ones, odd width
+        (ops.COV_LINEAR, t(128, 10), False, 1, 128.0, 0.0),         # linear G
+    ]
+    pending = ops.PendingCovs()
+    outs, refs, singles = [], [], []
+    for kind, x, ones, stride, alpha, beta in cases:
+        d = x.shape[1] + int(ones)
+        prev = t(d, d)
+        prev = (prev + prev.T).contiguous()
+        out = prev.clone()
+        xs = x.cpu().numpy()
+        if kind == ops.COV_SLAB:
+            sub = xs[:, :, ::stride, ::stride]
+            P = sub.transpose(0, 2, 3, 1).reshape(-1, xs.shape[1]).astype(np.float64)
+            single = ops.cov_conv_a(x, 1, stride, 0, ones, alpha, beta, prev.clone())
+        else:
+            P = xs.astype(np.float64)
+            single = ops.cov_linear(x, ones, alpha, beta, prev.clone())
+        if ones:
+            P = np.concatenate([P, np.ones((P.shape[0], 1))], axis=1)
+        refs.append(alpha * (P.T @ P) + beta * prev.cpu().numpy().astype(np.float64))
+        pending.add(kind, x, ones, out, alpha, beta, stride)
+        outs.append(out)
+        singles.append(single)
+    assert [o.shape[0] for o in outs] == [64, 66, 131, 97, 200, 32, 256, 102, 10]
+    pending.flush()
+    torch.cuda.synchronize()
+    assert pending.items == []
+    for out, ref, single in zip(outs, refs, singles):
+        got = out.cpu().numpy()
+        assert np.linalg.norm(got - ref) <= 1e-4 * np.linalg.norm(ref)
+        assert np.array_equal(got, got.T)
+        assert np.linalg.norm(got - single.cpu().numpy()) <= 1e-5 * np.linalg.norm(ref)
+    # the oracle's own functions on two of them
+    x = cases[1][1].cpu().numpy()
+    np.testing.assert_allclose(outs[1].cpu().numpy(), O.conv_A(x, 1, 1, 0, True) * (0.25 * 4), rtol=1e-4, atol=1e-4)
+    gy = cases[0][1].cpu().numpy()
+    np.testing.assert_allclose(outs[0].cpu().numpy(), O.conv_G(gy) * (0.25 * 14 * 14 / 4), rtol=1e-4, atol=1e-4)
+
+
+def test_grouped_launch_argument_checks():
+    from chainerkfac_amd import _lib, ops
+    with pytest.raises(_lib.KfacHipError):
+        ops.CovGroup([(7, 2, 3, 1, 1, 1, 1, 0, 1)])            # unknown kind
+    g = ops.CovGroup([(ops.COV_LINEAR, 4, 8, 1, 1, 1, 1, 0, 1)])
+    x = torch.zeros(4, 8, device='cuda')
+    with pytest.raises(ValueError):
+        g.run([x], [torch.zeros(9, 9, device='cuda')], [1.0], [0.0])
+    assert ops.CovGroup([]).run([], [], [], []) == []
 
 
 def test_workspace_too_small_is_reported():

@@ -28,6 +28,7 @@ def patch_cov64(x, k, s, p, bias):
 
 
 @pytest.mark.parametrize('c,hw,k,s,p', [(64, 56, 3, 1, 1),      # d = 577, 100 352 patches
+                                         (128, 28, 3, 1, 1),     # d = 1153
                                          (256, 14, 3, 1, 1),     # d = 2305
                                          (512, 7, 3, 1, 1),      # d = 4609
                                          (3, 224, 7, 2, 3),      # stem: d = 148, 401 408 patches
@@ -206,7 +207,7 @@ def test_resnet50d_accumulation_pack_inverse_precondition():
         for pname, p in model.namedparams():
             p.grad = torch.randn(p.shape, device=dev, generator=gen)
             ref_grads[pname] = ref_grads.get(pname, 0) + p.grad.double() / iters
-        opt._lanes.join()
+        opt.finish_covs()
         go_on = opt.accumulate()
         assert go_on == (it < iters - 1)
     # accumulated factors and gradients = means over the micro-batches

@@ -107,6 +107,10 @@ def test_axpby_and_momentum_update():
     x = r.standard_normal(100003).astype(np.float32); y = r.standard_normal(100003).astype(np.float32)
     got = ops.axpby(torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda(), 0.99, 0.01).cpu().numpy()
     np.testing.assert_allclose(got, np.float32(0.99) * x + np.float32(0.01) * y, rtol=1e-6, atol=1e-7)
+    # b == 0 overwrites without reading y (the accumulators start from uninitialised buffers)
+    ynan = torch.full((100003,), float('nan'), device='cuda')
+    got0 = ops.axpby(torch.from_numpy(x).cuda(), ynan, 0.5, 0.0).cpu().numpy()
+    assert np.array_equal(got0, np.float32(0.5) * x)
     p = r.standard_normal(1000).astype(np.float32); v = r.standard_normal(1000).astype(np.float32)
     g = r.standard_normal(1000).astype(np.float32)
     pd, vd = torch.from_numpy(p).cuda(), torch.from_numpy(v).cuda()
