@@ -77,13 +77,12 @@ template <class Cfg, bool SAME>
 __device__ __forceinline__ void rows_mainloop(const RowsGeom &g, int row0A, int row0B,
                                               long long sbeg, long long send, float *smem,
                                               floatx16 (&acc)[Cfg::WM][Cfg::WM],
-                                              float (&rs)[Cfg::WM]) {
+                                              float (&rs)[Cfg::WM], int wave) {
   constexpr int WM = Cfg::WM, KK = Cfg::KK, K = Cfg::K, S = Cfg::S, P = Cfg::P;
   constexpr int RIN = Cfg::RIN, WR = Cfg::WR, RSZ = Cfg::RSZ, REGION = Cfg::REGION;
   constexpr int PARTS = Cfg::PARTS, NK = Cfg::NK, CH = Cfg::CH, NCOL = Cfg::NCOL;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane & 31, lk = lane >> 5;
   const int HW = g.H * g.W;
@@ -175,7 +174,7 @@ __device__ __forceinline__ void rows_mainloop(const RowsGeom &g, int row0A, int 
 
   // a wave whose 64 x 64 block lies above the diagonal or past the end of the
   // factor stages like the others but leaves the matrix cores to them
-  const bool active = syrk_wave_active<WM>(row0A, row0B, g.d_patch);
+  const bool active = syrk_wave_active<WM>(row0A, row0B, g.d_patch, wave);
   if (sbeg < send) issue();
   for (long long s = sbeg; s < send; ++s) {
     stash();

@@ -119,9 +119,9 @@ SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
 // extra slice a partial tile that is written and read back, and fewer
 // workgroups than CUs x occ leave matrix pipes without a second wave to hide
 // the staging phases.
-SyrkPlan plan_rows(int d, long long steps, double step_us, int occ) {
+SyrkPlan plan_rows(int d, int bm, long long steps, double step_us, int occ) {
   SyrkPlan p;
-  p.bm = 128;
+  p.bm = bm;
   p.tiles = kfac::ceil_div(d, p.bm);
   p.ntile = p.tiles * (p.tiles + 1) / 2;
   if (steps < 1) steps = 1;
@@ -208,9 +208,10 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
 template <int WM>
 __device__ __forceinline__ void write_rowsums(float (&rs)[WM], int I, int dt, int d, int direct,
                                               float count, float alpha, float beta,
-                                              float *__restrict__ vec, float *__restrict__ C) {
+                                              float *__restrict__ vec, float *__restrict__ C,
+                                              int wave = threadIdx.x >> 6) {
   constexpr int BM = 64 * WM;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
 #pragma unroll
   for (int im = 0; im < WM; ++im) {
@@ -226,7 +227,7 @@ __device__ __forceinline__ void write_rowsums(float (&rs)[WM], int I, int dt, in
       C[(long long)row * d + d - 1] = v;
     }
   }
-  if (direct && I == 0 && threadIdx.x == 0) {
+  if (direct && I == 0 && wave == 0 && lane == 0) {
     float v = alpha * count;
     if (beta != 0.f) v += beta * C[(long long)(d - 1) * d + d - 1];
     C[(long long)(d - 1) * d + d - 1] = v;
@@ -303,21 +304,24 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_kernel(Loader ld, long long K
   float rs[WM];
 #pragma unroll
   for (int im = 0; im < WM; ++im) rs[im] = 0.f;
-  const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt);
+  const int wave = threadIdx.x >> 6;
+  const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt, wave);
   if (I == J)
-    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active);
+    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active,
+                                  wave);
   else
-    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active);
+    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active, wave);
   const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
   float *mine = partial + split * slot;
   if (ones && I == J)
-    write_rowsums<WM>(rs, I, dt, d, direct, (float)K, alpha, beta, mine + (long long)ntile * (BM * BM), C);
+    write_rowsums<WM>(rs, I, dt, d, direct, (float)K, alpha, beta, mine + (long long)ntile * (BM * BM), C,
+                      wave);
   if (direct) {
-    write_tile<WM>(acc, lds, I, J, dt, d, alpha, beta, C);
+    write_tile<WM>(acc, lds, I, J, dt, d, alpha, beta, C, wave);
     return;
   }
   float *out = mine + (long long)tile * (BM * BM);
-  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; }, wave);
 }
 
 // Convolution A factor through the LDS halo region (conv_halo.h); `klen` counts
@@ -405,20 +409,22 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_rows_kernel(RowsGeom g, long 
   float rs[WM];
 #pragma unroll
   for (int im = 0; im < WM; ++im) rs[im] = 0.f;
+  const int wave = threadIdx.x >> 6;
   if (I == J)
-    rows_mainloop<Cfg, true>(g, I * BM, J * BM, sbeg, send, smem, acc, rs);
+    rows_mainloop<Cfg, true>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave);
   else
-    rows_mainloop<Cfg, false>(g, I * BM, J * BM, sbeg, send, smem, acc, rs);
+    rows_mainloop<Cfg, false>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave);
   const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
   float *mine = partial + split * slot;
   if (ones && I == J)
-    write_rowsums<WM>(rs, I, dt, d, direct, count, alpha, beta, mine + (long long)ntile * (BM * BM), C);
+    write_rowsums<WM>(rs, I, dt, d, direct, count, alpha, beta, mine + (long long)ntile * (BM * BM), C,
+                      wave);
   if (direct) {
-    write_tile<WM>(acc, smem, I, J, dt, d, alpha, beta, C);
+    write_tile<WM>(acc, smem, I, J, dt, d, alpha, beta, C, wave);
     return;
   }
   float *out = mine + (long long)tile * (BM * BM);
-  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; }, wave);
 }
 
 // One workgroup per 64x64 sub-block (si >= sj) of C.  The number of slices is a
@@ -697,7 +703,7 @@ int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int
   if (d - ones <= 320) return 1;   // small factors: 64-tiles of the general kernel
   constexpr size_t lds = (size_t)Cfg::lds_floats(false) * sizeof(float);
   constexpr int occ = (160 * 1024) / lds >= 3 ? 3 : (int)((160 * 1024) / lds);
-  const SyrkPlan p = plan_rows(d - ones, total_steps, Cfg::NK * Cfg::WM * Cfg::WM * 64 / 2400.0, occ);
+  const SyrkPlan p = plan_rows(d - ones, 64 * Cfg::WM, total_steps, Cfg::NK * Cfg::WM * Cfg::WM * 64 / 2400.0, occ);
   if (int rc = check_ws(p, ws, ws_bytes)) return rc;
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
@@ -727,14 +733,22 @@ int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, in
   if (getenv("KFAC_CONV_ROWS_OFF")) return 1;   // tuning override: the general kernels only
   if (n % 2 != 0 || kh != kw || sy != sx || ph != pw) return 1;
   if ((long long)n * c * h * w * (long long)sizeof(float) >= (1ll << 31)) return 1;
-  const bool alt = getenv("KFAC_ROWS_ALT") != nullptr;
+  // 128-tiles feed the matrix cores with half the LDS traffic of 64-tiles, but a
+  // factor whose side is not a multiple of 128 pays for the padded part of its last
+  // tile row and every diagonal tile for its upper half: take 64-tiles when they
+  // save more than the ~15 % their main loop is slower by (576 rows: 45 tiles of
+  // 64 against 15 of 128, i.e. 45 against 60 units of matrix-core work).
+  const int dt = d - ones;
+  const long long t64 = kfac::ceil_div(dt, 64), t128 = kfac::ceil_div(dt, 128);
+  bool small_tiles = 1.15 * (double)(t64 * (t64 + 1) / 2) < 4.0 * (double)(t128 * (t128 + 1) / 2);
+  if (const char *env = getenv("KFAC_ROWS_WM")) small_tiles = atoi(env) == 1;   // tuning override
 #define KFAC_ROWS_CASE(K, S, P, WS, RT, PAD)                                                      \
-  if (kh == K && sy == S && ph == P && wo == WS && ho % RT == 0)                                  \
+  if (kh == K && sy == S && ph == P && wo == WS && ho % RT == 0) {                                \
+    if (small_tiles)                                                                              \
+      return run_conv_rows<RowsCfg<1, K, S, P, WS, RT, PAD>>(x, n, c, h, w, ho, d, ones, alpha,   \
+                                                             beta, C, ws, ws_bytes, stream);      \
     return run_conv_rows<RowsCfg<2, K, S, P, WS, RT, PAD>>(x, n, c, h, w, ho, d, ones, alpha,     \
-                                                           beta, C, ws, ws_bytes, stream);
-  if (alt) {
-    KFAC_ROWS_CASE(3, 1, 1, 56, 2, 4)
-    KFAC_ROWS_CASE(3, 1, 1, 28, 4, 3)
+                                                           beta, C, ws, ws_bytes, stream);        \
   }
   KFAC_ROWS_CASE(3, 1, 1, 56, 1, 0)
   KFAC_ROWS_CASE(3, 1, 1, 28, 2, 1)
@@ -922,7 +936,7 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
 namespace {
 
 struct GroupItemStatic {
-  int d, ones, tiles, ntile, nsplit, direct;
+  int d, ones, bm, tiles, ntile, nsplit, direct;
   long long K, klen;      // reduction length; per k-slice (a multiple of KT)
   long long part_off;     // floats from the workspace base to this item's partial slots
   float count;            // reduction length as a float: the corner entry of a ones column
@@ -943,10 +957,10 @@ struct GroupItemDyn {
 template <class Loader>
 struct GroupLoader;
 
-template <bool VEC>
-struct GroupLoader<LoaderKC<64, VEC>> {
-  static __device__ __forceinline__ LoaderKC<64, VEC> make(const GroupItemStatic &s, const float *in) {
-    LoaderKC<64, VEC> l;
+template <int ROWS, bool VEC>
+struct GroupLoader<LoaderKC<ROWS, VEC>> {
+  static __device__ __forceinline__ LoaderKC<ROWS, VEC> make(const GroupItemStatic &s, const float *in) {
+    LoaderKC<ROWS, VEC> l;
     l.base = in;
     l.sample_stride = s.sample_stride;
     l.row_stride = s.row_stride;
@@ -961,10 +975,10 @@ struct GroupLoader<LoaderKC<64, VEC>> {
   }
 };
 
-template <bool VEC>
-struct GroupLoader<LoaderKS<64, VEC>> {
-  static __device__ __forceinline__ LoaderKS<64, VEC> make(const GroupItemStatic &s, const float *in) {
-    LoaderKS<64, VEC> l;
+template <int ROWS, bool VEC>
+struct GroupLoader<LoaderKS<ROWS, VEC>> {
+  static __device__ __forceinline__ LoaderKS<ROWS, VEC> make(const GroupItemStatic &s, const float *in) {
+    LoaderKS<ROWS, VEC> l;
     l.base = in;
     l.extra = nullptr;
     l.ld = s.ld;
@@ -974,13 +988,13 @@ struct GroupLoader<LoaderKS<64, VEC>> {
   }
 };
 
-// task = (item, tile + ntile * k-slice)
-template <class Loader>
+// task = (item, tile + ntile * k-slice); WM = 1: items with 64-tiles, 2: 128-tiles
+template <int WM, class Loader>
 __global__ __launch_bounds__(THREADS, 3) void syrk_group_kernel(const GroupItemStatic *__restrict__ st,
                                                                 const GroupItemDyn *__restrict__ dy,
                                                                 const int2 *__restrict__ tasks,
                                                                 float *__restrict__ ws) {
-  constexpr int WM = 1, BM = 64;
+  constexpr int BM = 64 * WM;
   __shared__ float lds[2 * Panel<BM>::kFloats];
   static_assert(2 * Panel<BM>::kFloats >= 64 * 65, "LDS too small for the epilogue transpose");
   float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
@@ -1001,23 +1015,26 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_group_kernel(const GroupItemS
   floatx16 acc[WM][WM];
   zero_acc<WM, WM>(acc);
   float rs[WM];
-  rs[0] = 0.f;
-  const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt);
+#pragma unroll
+  for (int im = 0; im < WM; ++im) rs[im] = 0.f;
+  const int wave = threadIdx.x >> 6;
+  const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt, wave);
   if (I == J)
-    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active);
+    mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active,
+                                  wave);
   else
-    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active);
+    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active, wave);
   const long long slot = (long long)s.ntile * (BM * BM) + (long long)s.tiles * BM;
   float *mine = ws + s.part_off + split * slot;
   if (s.ones && I == J)
     write_rowsums<WM>(rs, I, dt, s.d, s.direct, s.count, v.alpha, v.beta,
-                      mine + (long long)s.ntile * (BM * BM), v.out);
+                      mine + (long long)s.ntile * (BM * BM), v.out, wave);
   if (s.direct) {
-    write_tile<WM>(acc, lds, I, J, dt, s.d, v.alpha, v.beta, v.out);
+    write_tile<WM>(acc, lds, I, J, dt, s.d, v.alpha, v.beta, v.out, wave);
     return;
   }
   float *out = mine + (long long)tile * (BM * BM);
-  for_each_acc<WM, WM>(acc, [&](int r, int c, float val) { out[r * BM + c] = val; });
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float val) { out[r * BM + c] = val; }, wave);
 }
 
 // task = (item, 64 x 64 block of the lower triangle); sums the item's k-slices
@@ -1034,21 +1051,26 @@ __global__ __launch_bounds__(256) void finish_group_kernel(const GroupItemStatic
   tri_decode(task.y, si, sj);
   const int dt = s.d - s.ones, d = s.d;
   const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
-  const long long slot = (long long)s.ntile * 4096 + (long long)s.tiles * 64;
-  const float *p0 = ws + s.part_off + (long long)task.y * 4096;
+  const int bm = s.bm, per = bm / 64;   // 64-blocks per tile side
+  const int I = si / per, J = sj / per;
+  const int t = I * (I + 1) / 2 + J;
+  const int r_in = (si - I * per) * 64, c_in = (sj - J * per) * 64;
+  const long long tile_stride = (long long)bm * bm;
+  const long long slot = (long long)s.ntile * tile_stride + (long long)s.tiles * bm;
+  const float *p0 = ws + s.part_off + (long long)t * tile_stride + (long long)r_in * bm + c_in;
   float sum[16];
 #pragma unroll
   for (int p = 0; p < 16; ++p) sum[p] = 0.f;
   for (int k = 0; k < s.nsplit; ++k) {
     const float *pk = p0 + k * slot;
 #pragma unroll
-    for (int p = 0; p < 16; ++p) sum[p] += pk[(lr0 + 4 * p) * 64 + lc];
+    for (int p = 0; p < 16; ++p) sum[p] += pk[(lr0 + 4 * p) * bm + lc];
   }
   float *C = v.out;
   const float alpha = v.alpha, beta = v.beta;
   if (s.ones && si == sj && threadIdx.x < 64) {
     const int row = si * 64 + threadIdx.x;
-    const float *v0 = ws + s.part_off + (long long)s.ntile * 4096 + row;
+    const float *v0 = ws + s.part_off + (long long)s.ntile * tile_stride + row;
     float a = 0.f;
     for (int k = 0; k < s.nsplit; ++k) a += v0[k * slot];
     if (row < dt) {
@@ -1098,7 +1120,7 @@ void deal_to_xcds(std::vector<int2> &table, const std::vector<int2> &natural) {
     }
 }
 
-constexpr int kGroupKinds = 4;   // slab float4, slab scalar, linear float4, linear scalar
+constexpr int kGroupKinds = 8;   // {64-tiles, 128-tiles} x {slab float4, slab scalar, linear float4, linear scalar}
 
 }  // namespace
 
@@ -1107,7 +1129,7 @@ struct kfac_cov_group {
   std::vector<GroupItemStatic> items;
   std::vector<GroupItemDyn> dyn;
   size_t ws_floats = 0;
-  int task0[kGroupKinds] = {0, 0, 0, 0}, ntask[kGroupKinds] = {0, 0, 0, 0};
+  int task0[kGroupKinds] = {}, ntask[kGroupKinds] = {};
   int ftask0 = 0, nftask = 0;
   kfac::DevTable d_items, d_dyn, d_tasks;
 };
@@ -1122,7 +1144,8 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
   g->items.resize(count);
   g->dyn.resize(count);
   std::vector<long long> nk(count);
-  double work = 0;   // tile-panels
+  std::vector<int> kind_of(count);
+  double work[kGroupKinds] = {};   // per launch, in panels of a 64-tile
   for (int i = 0; i < count; ++i) {
     const kfac_cov_item &it = items[i];
     GroupItemStatic &s = g->items[i];
@@ -1165,24 +1188,38 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     }
     s.d = it.c + s.ones;
     s.count = (float)s.K;
-    s.tiles = kfac::ceil_div(it.c, 64);
-    s.ntile = s.tiles * (s.tiles + 1) / 2;
     nk[i] = kfac::ceil_div<long long>(s.K, KT);
-    work += (double)s.ntile * (double)nk[i];
+    // 128-tiles feed the matrix cores with half the LDS and load instructions of
+    // 64-tiles and, in a grouped launch, need not be many to fill the GPU; 64-tiles for
+    // narrow factors (padding) and for short reductions over many tiles (all output
+    // traffic: smaller tiles spread the stores over more workgroups).
+    // KFAC_GROUP_BM64_MAX is a tuning override.
+    int bm64_max = 160;
+    if (const char *env = getenv("KFAC_GROUP_BM64_MAX")) bm64_max = atoi(env);
+    s.bm = (it.c <= bm64_max || nk[i] <= 4) ? 64 : 128;
+    s.tiles = kfac::ceil_div(it.c, s.bm);
+    s.ntile = s.tiles * (s.tiles + 1) / 2;
+    kind_of[i] = (s.bm == 64 ? 0 : 4) + (s.kind == KFAC_COV_SLAB ? 0 : 2) + (s.vec ? 0 : 1);
+    work[kind_of[i]] += (double)s.ntile * (double)nk[i] * (s.bm == 64 ? 1.0 : 4.0);
   }
-  // k-slices: workgroups of about equal length, ~2300 of them when the work allows
-  // it, none shorter than 8 panels (unless the whole reduction is) and at most 256 per factor
-  double per_wg = work / 2304.0;
-  if (per_wg < 8.0) per_wg = 8.0;
-  if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override: panels per workgroup
-    const double v = atof(env);
-    if (v >= 1.0) per_wg = v;
+  // k-slices: every launch (one per loader kind and tile size) is cut into workgroups
+  // of about equal length (a panel of a 128-tile counts four times a panel of a
+  // 64-tile), ~2300 of them when the work allows it, none shorter than 32 panel units
+  // (unless the whole reduction is) and at most 256 per factor
+  double per_wg[kGroupKinds];
+  for (int k = 0; k < kGroupKinds; ++k) {
+    per_wg[k] = work[k] / 2304.0;
+    if (per_wg[k] < 32.0) per_wg[k] = 32.0;
+    if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override: panel units per workgroup
+      const double v = atof(env);
+      if (v >= 1.0) per_wg[k] = v;
+    }
   }
   size_t off = 0;
   std::vector<int2> natural[kGroupKinds], fin;
   for (int i = 0; i < count; ++i) {
     GroupItemStatic &s = g->items[i];
-    long long ns = (long long)((double)nk[i] / per_wg + 0.5);
+    long long ns = (long long)((double)nk[i] * (s.bm == 64 ? 1.0 : 4.0) / per_wg[kind_of[i]] + 0.5);
     if (ns < 1) ns = 1;
     if (ns > 256) ns = 256;
     if (ns > nk[i]) ns = nk[i];
@@ -1191,13 +1228,13 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     s.klen = per * KT;
     s.direct = s.nsplit == 1 ? 1 : 0;
     s.part_off = (long long)off;
-    const size_t slot = (size_t)s.ntile * 4096 + (size_t)s.tiles * 64;
+    const size_t slot = (size_t)s.ntile * s.bm * s.bm + (size_t)s.tiles * s.bm;
     if (!s.direct) off += (size_t)s.nsplit * slot;
-    else if (s.ones) off += slot;   // the row sums of a direct item still pass through its slot
-    const int kind = (s.kind == KFAC_COV_SLAB ? 0 : 2) + (s.vec ? 0 : 1);
-    for (int w = 0; w < s.ntile * s.nsplit; ++w) natural[kind].push_back(make_int2(i, w));
-    if (!s.direct)
-      for (int b = 0; b < s.ntile; ++b) fin.push_back(make_int2(i, b));
+    for (int w = 0; w < s.ntile * s.nsplit; ++w) natural[kind_of[i]].push_back(make_int2(i, w));
+    if (!s.direct) {
+      const int sub = kfac::ceil_div(items[i].c, 64);
+      for (int b = 0; b < sub * (sub + 1) / 2; ++b) fin.push_back(make_int2(i, b));
+    }
   }
   g->ws_floats = off;
   std::vector<int2> tasks;
@@ -1253,8 +1290,10 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   const int2 *tasks = group->d_tasks.as<const int2>();
   using Kern = void (*)(const GroupItemStatic *, const GroupItemDyn *, const int2 *, float *);
   static const Kern kerns[kGroupKinds] = {
-      syrk_group_kernel<LoaderKC<64, true>>, syrk_group_kernel<LoaderKC<64, false>>,
-      syrk_group_kernel<LoaderKS<64, true>>, syrk_group_kernel<LoaderKS<64, false>>};
+      syrk_group_kernel<1, LoaderKC<64, true>>,   syrk_group_kernel<1, LoaderKC<64, false>>,
+      syrk_group_kernel<1, LoaderKS<64, true>>,   syrk_group_kernel<1, LoaderKS<64, false>>,
+      syrk_group_kernel<2, LoaderKC<128, true>>,  syrk_group_kernel<2, LoaderKC<128, false>>,
+      syrk_group_kernel<2, LoaderKS<128, true>>,  syrk_group_kernel<2, LoaderKS<128, false>>};
   for (int k = 0; k < kGroupKinds; ++k) {
     if (group->ntask[k] == 0) continue;
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);

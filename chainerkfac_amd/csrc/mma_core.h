@@ -400,10 +400,9 @@ template <int WM, int WN, bool SAME, bool RS, class LA, class LB>
 __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int rowA0, int rowB0,
                                               long long kbeg, long long kend, float *ldsA,
                                               float *ldsB, floatx16 (&acc)[WM][WN], float *rs,
-                                              bool active = true) {
+                                              bool active = true, int wave = threadIdx.x >> 6) {
   constexpr int RA = 64 * WM, RB = 64 * WN;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane & 31, lk = lane >> 5;
   typename LA::Regs ra;
@@ -452,17 +451,20 @@ __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int ro
 template <int WM, int WN, bool SAME, class LA, class LB>
 __device__ __forceinline__ void mainloop(const LA &la, const LB &lb, int rowA0, int rowB0,
                                          long long kbeg, long long kend, float *ldsA,
-                                         float *ldsB, floatx16 (&acc)[WM][WN], bool active = true) {
+                                         float *ldsB, floatx16 (&acc)[WM][WN], bool active = true,
+                                         int wave = threadIdx.x >> 6) {
   mainloop_impl<WM, WN, SAME, false>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, nullptr,
-                                     active);
+                                     active, wave);
 }
 
 template <int WM, int WN, bool SAME, class LA, class LB>
 __device__ __forceinline__ void mainloop_rowsum(const LA &la, const LB &lb, int rowA0, int rowB0,
                                                 long long kbeg, long long kend, float *ldsA,
                                                 float *ldsB, floatx16 (&acc)[WM][WN],
-                                                float (&rs)[WM], bool active = true) {
-  mainloop_impl<WM, WN, SAME, true>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, rs, active);
+                                                float (&rs)[WM], bool active = true,
+                                                int wave = threadIdx.x >> 6) {
+  mainloop_impl<WM, WN, SAME, true>(la, lb, rowA0, rowB0, kbeg, kend, ldsA, ldsB, acc, rs, active,
+                                    wave);
 }
 
 // Whether this wave's block of a symmetric product's tile (first rows row0A /
@@ -470,8 +472,8 @@ __device__ __forceinline__ void mainloop_rowsum(const LA &la, const LB &lb, int 
 // diagonal (the epilogues take those entries from the mirrored block) or past
 // the end of the matrix.
 template <int WM>
-__device__ __forceinline__ bool syrk_wave_active(int row0A, int row0B, int dt) {
-  const int wave = threadIdx.x >> 6;
+__device__ __forceinline__ bool syrk_wave_active(int row0A, int row0B, int dt,
+                                                 int wave = threadIdx.x >> 6) {
   const int ra = row0A + (wave >> 1) * WM * 32, rb = row0B + (wave & 1) * WM * 32;
   return ra + WM * 32 > rb && ra < dt && rb < dt;
 }
@@ -479,9 +481,8 @@ __device__ __forceinline__ bool syrk_wave_active(int row0A, int row0B, int dt) {
 // Set every accumulator element of this lane to f(row, col), row / col relative
 // to the workgroup tile.
 template <int WM, int WN, class F>
-__device__ __forceinline__ void fill_acc(floatx16 (&acc)[WM][WN], F f) {
+__device__ __forceinline__ void fill_acc(floatx16 (&acc)[WM][WN], F f, int wave = threadIdx.x >> 6) {
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 #pragma unroll
   for (int im = 0; im < WM; ++im)
@@ -498,9 +499,9 @@ __device__ __forceinline__ void fill_acc(floatx16 (&acc)[WM][WN], F f) {
 // Visit every accumulator element of this lane: f(row, col, value) with row /
 // col relative to the workgroup tile.
 template <int WM, int WN, class F>
-__device__ __forceinline__ void for_each_acc(floatx16 (&acc)[WM][WN], F f) {
+__device__ __forceinline__ void for_each_acc(floatx16 (&acc)[WM][WN], F f,
+                                             int wave = threadIdx.x >> 6) {
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 #pragma unroll
   for (int im = 0; im < WM; ++im)
@@ -534,7 +535,7 @@ __device__ __forceinline__ void zero_acc(floatx16 (&acc)[WM][WN]) {
 template <int WM>
 __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
                                            int dt, int d, float alpha, float beta,
-                                           float *__restrict__ C) {
+                                           float *__restrict__ C, int wave = threadIdx.x >> 6) {
   constexpr int BM = 64 * WM;
   float(*t)[65] = reinterpret_cast<float(*)[65]>(lds);
   const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
@@ -545,7 +546,7 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
     __syncthreads();
     for_each_acc<WM, WM>(acc, [&](int r, int c, float v) {
       if (r / 64 == qm && c / 64 == qn) t[r % 64][c % 64] = v;
-    });
+    }, wave);
     __syncthreads();
     const int r0 = I * BM + qm * 64, c0 = J * BM + qn * 64;
 #pragma unroll 4

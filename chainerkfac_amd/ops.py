@@ -155,8 +155,9 @@ class PendingCovs(object):
     the GPU on their own; ``flush`` runs all of them as one grouped launch.
     The tensors are kept alive until then."""
 
-    #: a factor is deferred when its SYRK has at most this many flops (rows * d * (d+1))
-    max_flops = 2.5e9
+    #: a factor is deferred when its SYRK has at most this many flops (rows * d * (d+1));
+    #: larger ones (the k x k convolutions of a deep network) fill the GPU on their own
+    max_flops = 8e9
 
     def __init__(self):
         self.items, self.inputs, self.outputs, self.alphas, self.betas = [], [], [], [], []

@@ -163,6 +163,9 @@ def test_grouped_launch_matches_the_single_calls():
         (ops.COV_LINEAR, t(32, 256), False, 1, 1 / 32, 0.0),        # batch-norm gradient matrix
         (ops.COV_LINEAR, t(16, 101), True, 1, 1 / 16, 1.0),         # linear A with ones, odd width
         (ops.COV_LINEAR, t(128, 10), False, 1, 128.0, 0.0),         # linear G
+        (ops.COV_SLAB, t(4, 600, 8, 8), False, 1, 0.25, 0.0),       # 128-tiles, float4 loads
+        (ops.COV_SLAB, t(6, 530, 7, 7), True, 1, 0.5, 1.0),         # 128-tiles, scalar loads, ones, accumulation
+        (ops.COV_LINEAR, t(200, 600), True, 1, 0.005, 0.0),         # 128-tiles, linear with ones
     ]
     pending = ops.PendingCovs()
     outs, refs, singles = [], [], []
@@ -185,7 +188,7 @@ def test_grouped_launch_matches_the_single_calls():
         pending.add(kind, x, ones, out, alpha, beta, stride)
         outs.append(out)
         singles.append(single)
-    assert [o.shape[0] for o in outs] == [64, 66, 131, 97, 200, 32, 256, 102, 10]
+    assert [o.shape[0] for o in outs] == [64, 66, 131, 97, 200, 32, 256, 102, 10, 600, 531, 601]
     pending.flush()
     torch.cuda.synchronize()
     assert pending.items == []
