@@ -838,7 +838,7 @@ extern "C" int kfac_cov_linear_f32(const float *x, int n, int d_in, int append_o
                                    float alpha, float beta, float *C, void *ws,
                                    size_t ws_bytes, void *stream) {
   KFAC_REQUIRE(n > 0 && d_in > 0, "bad shape n=%d d_in=%d", n, d_in);
-  KFAC_REQUIRE((long long)n * d_in < 0x7fffffffLL, "input too large");
+  KFAC_REQUIRE((long long)n * d_in < 0x40000000LL, "input too large");
   KFAC_REQUIRE(x && C, "null pointer");
   const int ones = append_ones ? 1 : 0;
   const int d = d_in + ones;
@@ -855,7 +855,7 @@ extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, floa
                                    float beta, float *C, void *ws, size_t ws_bytes,
                                    void *stream) {
   KFAC_REQUIRE(n > 0 && c > 0 && howo > 0, "bad shape n=%d c=%d howo=%d", n, c, howo);
-  KFAC_REQUIRE((long long)n * c * howo < 0x7fffffffLL, "input too large");
+  KFAC_REQUIRE((long long)n * c * howo < 0x40000000LL, "input too large");
   KFAC_REQUIRE(gy && C, "null pointer");
   const long long K = (long long)n * howo;
   if (kc_vec_ok(gy, (long long)c * howo, howo, howo))
@@ -880,7 +880,7 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
   const int wo = (w + 2 * pw - kw) / sx + 1;
   const long long dl = (long long)c * kh * kw + (append_ones ? 1 : 0);
   KFAC_REQUIRE(dl < 46340, "factor dimension %lld too large", dl);
-  KFAC_REQUIRE((long long)n * c * h * w < 0x7fffffffLL, "input too large");
+  KFAC_REQUIRE((long long)n * c * h * w < 0x40000000LL, "input too large");
   const int d = (int)dl;
   const int ones = append_ones ? 1 : 0;
   const long long K = (long long)n * ho * wo;
@@ -1160,7 +1160,7 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     s.ones = it.append_ones ? 1 : 0;
     if (it.kind == KFAC_COV_LINEAR) {
       // x (n, c) row-major
-      if ((long long)it.n * it.c >= 0x7fffffffLL) return bad("input too large");
+      if ((long long)it.n * it.c >= 0x40000000LL) return bad("input too large");
       s.K = it.n;
       s.ld = (unsigned)it.c;
       s.rows_valid = it.c;
@@ -1168,7 +1168,7 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     } else {
       // (n, c, h, w) tensor; every sy-th line and sx-th pixel of it when subsampled
       if (it.h <= 0 || it.w <= 0 || it.sy <= 0 || it.sx <= 0) return bad("bad shape");
-      if ((long long)it.n * it.c * it.h * it.w >= 0x7fffffffLL) return bad("input too large");
+      if ((long long)it.n * it.c * it.h * it.w >= 0x40000000LL) return bad("input too large");
       const int ho = (it.h - 1) / it.sy + 1, wo = (it.w - 1) / it.sx + 1;
       const int hw = it.h * it.w;
       s.K = (long long)it.n * ho * wo;

@@ -32,6 +32,20 @@ constexpr int KT = 32;        // k-values per LDS panel
 constexpr int THREADS = 256;  // 4 waves
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Loads from global memory at a wave-uniform base plus a 32-bit byte offset per
+// lane: the form of the load instruction that takes the base from scalar
+// registers, so that no 64-bit address is formed per lane and per load.  The
+// tensors read this way are smaller than 4 GiB (checked on the host).
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+#define KFAC_GLOBAL_AS __attribute__((address_space(1)))
+__device__ __forceinline__ float4 gload4(const float *base, unsigned byte_off) {
+  const floatx4 t = *(const KFAC_GLOBAL_AS floatx4 *)((const KFAC_GLOBAL_AS char *)base + byte_off);
+  return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ float gload1(const float *base, unsigned byte_off) {
+  return *(const KFAC_GLOBAL_AS float *)((const KFAC_GLOBAL_AS char *)base + byte_off);
+}
+
 template <int ROWS>
 struct Panel {
   static constexpr int kRowKStride = KT + 1;
@@ -48,7 +62,7 @@ struct Panel {
 // and apply validity masks when storing.  Nothing between load() and store()
 // touches the loaded registers, so the loads stay in flight while the matrix
 // cores work on the previous panel.  Offsets are 32-bit element offsets from
-// the tensor base (tensors hold fewer than 2^31 elements; checked on the host).
+// the tensor base (tensors hold fewer than 2^30 elements, 4 GiB; checked on the host).
 
 // ---------------------------------------------------------------------------
 // LoaderKC: element (row, kg) at base + (kg / L) * sample_stride
@@ -104,9 +118,8 @@ struct LoaderKC {
       const unsigned s = kc / L;
       koff = s * sample_stride + (kc - s * L);
     }
-    const float *p = base + koff;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) r.v[i] = *reinterpret_cast<const float4 *>(p + rowoff[i]);
+    for (int i = 0; i < NV; ++i) r.v[i] = gload4(base, (koff + rowoff[i]) * 4u);
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
@@ -182,7 +195,6 @@ struct LoaderKC<ROWS, false> {
       }
       koff = s * sample_stride + pix;
     }
-    const float *p = base + koff;
     // The row offsets are cheap to recompute and expensive to keep: hide the
     // row from the optimiser so that it does not hoist NR offsets per operand
     // out of the k loop (which spills under a 3-workgroup register budget).
@@ -192,7 +204,7 @@ struct LoaderKC<ROWS, false> {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       const unsigned off = off0 + (unsigned)(8 * i) * row_stride;
-      r.v[i] = p[off < last_off ? off : last_off];
+      r.v[i] = gload1(base, (koff + (off < last_off ? off : last_off)) * 4u);
     }
   }
 
@@ -248,7 +260,7 @@ struct LoaderKS {
         const long long kg = k0 + kk + KPP * i;
         const bool kok = full_k || kg < k_end;
         if (kok) r.kmask |= 1u << i;
-        r.v[i] = *reinterpret_cast<const float4 *>(base + (unsigned)(kok ? kg : 0) * ld + (unsigned)row);
+        r.v[i] = gload4(base, ((unsigned)(kok ? kg : 0) * ld + (unsigned)row) * 4u);
       }
     } else {
 #pragma unroll

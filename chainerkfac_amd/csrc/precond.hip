@@ -251,8 +251,8 @@ extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ain
   KFAC_REQUIRE((gradb == nullptr) == (kfb == nullptr), "gradb and kfb must both be given or both null");
   const int hb = gradb ? 1 : 0;
   KFAC_REQUIRE(dA - hb > 0, "dA too small");
-  KFAC_REQUIRE((long long)dG * dA < 0x7fffffffLL && (long long)dA * dA < 0x7fffffffLL &&
-                   (long long)dG * dG < 0x7fffffffLL,
+  KFAC_REQUIRE((long long)dG * dA < 0x40000000LL && (long long)dA * dA < 0x40000000LL &&
+                   (long long)dG * dG < 0x40000000LL,
                "factor too large");
   if (ws == nullptr || ws_bytes < kfac_precond_conn_workspace_bytes(dG, dA))
     return kfac::fail(KFAC_ENOMEM, "preconditioning workspace too small: %zu < %zu bytes",
