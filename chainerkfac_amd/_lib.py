@@ -61,6 +61,10 @@ PROTOTYPES = {
     'kfac_add_diag_f32': (c_int, [c_vp, c_int, c_int, c_d, c_d, c_vp]),
     'kfac_precond_conn_workspace_bytes': (c_sz, [c_int, c_int]),
     'kfac_precond_conn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    'kfac_precond_group_create': (c_int, [c_int, c_i32p, c_i32p, c_i32p, c_vpp]),
+    'kfac_precond_group_workspace_bytes': (c_sz, [c_vp]),
+    'kfac_precond_group_destroy': (c_int, [c_vp]),
+    'kfac_precond_group_run_f32': (c_int, [c_vp, c_vpp, c_vpp, c_vpp, c_vpp, c_vpp, c_vpp, c_vp, c_sz, c_vp]),
     'kfac_precond_bn_workspace_bytes': (c_sz, [c_int]),
     'kfac_precond_bn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_precond_bn_static_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp]),

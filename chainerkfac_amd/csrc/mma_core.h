@@ -36,7 +36,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // lane: the form of the load instruction that takes the base from scalar
 // registers, so that no 64-bit address is formed per lane and per load.  The
 // tensors read this way are smaller than 4 GiB (checked on the host).
-typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4), aligned(4)));
 #define KFAC_GLOBAL_AS __attribute__((address_space(1)))
 __device__ __forceinline__ float4 gload4(const float *base, unsigned byte_off) {
   const floatx4 t = *(const KFAC_GLOBAL_AS floatx4 *)((const KFAC_GLOBAL_AS char *)base + byte_off);
@@ -69,9 +69,14 @@ struct Panel {
 //                                     + row * row_stride + (kg % L)
 // rows >= rows_valid read as 0.
 // ---------------------------------------------------------------------------
-// VEC: float4 loads (strides and L multiples of 4, base 16-byte aligned); a
-// compile-time choice so that the common aligned case carries no scalar-path
-// code or registers.  The primary template is the float4 variant.
+// VEC: 16-byte loads of four consecutive k-values of a row; for tensors whose
+// rows start on 16-byte boundaries (base, row and sample strides multiples of 4
+// floats: misaligned 16-byte loads work but were measured slower than the
+// scalar variant below).  A quad that is cut by the end of the range, or that
+// runs from one sample into the next, is loaded element by element by the
+// lanes concerned, so the reduction length is free.  A compile-time choice so
+// that this common case carries no code or registers of the scalar variant.
+// The primary template is this one.
 template <int ROWS, bool VEC>
 struct LoaderKC {
   static_assert(VEC, "the scalar variant is the specialisation below");
@@ -107,19 +112,36 @@ struct LoaderKC {
 
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
     const unsigned kq = (threadIdx.x & 7) * 4;
-    const unsigned kg = (unsigned)k0 + kq;
+    const long long kgl = k0 + kq;
     const bool full_k = k0 + KT <= k_end;
     r.fast = full_rows && full_k;
-    const bool kok = full_k || (long long)kg + 3 < k_end;
-    r.kmask = kok ? 0xfu : 0u;
-    const unsigned kc = kok ? kg : 0u;
-    unsigned koff = kc;
+    const bool whole = full_k || kgl + 3 < k_end;
+    const long long left = k_end - kgl;   // valid k-values from kg on
+    r.kmask = whole ? 0xfu : (left > 0 ? (1u << (int)left) - 1u : 0u);
+    const unsigned kc = left > 0 ? (unsigned)kgl : 0u;
+    unsigned koff = kc, rem = kc;
     if (L < (unsigned)k_end) {  // more than one sample
       const unsigned s = kc / L;
-      koff = s * sample_stride + (kc - s * L);
+      rem = kc - s * L;
+      koff = s * sample_stride + rem;
     }
+    if (whole && rem + 3 < L) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) r.v[i] = gload4(base, (koff + rowoff[i]) * 4u);
+      for (int i = 0; i < NV; ++i) r.v[i] = gload4(base, (koff + rowoff[i]) * 4u);
+    } else {
+      // element by element: k-values past the range read k = 0 of the row (masked when
+      // stored), k-values past the end of the sample continue in the next sample
+      unsigned off[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool in = (r.kmask >> e) & 1u;
+        off[e] = in ? koff + e + (rem + e >= L ? sample_stride - L : 0u) : 0u;
+      }
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+        r.v[i] = make_float4(gload1(base, (off[0] + rowoff[i]) * 4u), gload1(base, (off[1] + rowoff[i]) * 4u),
+                             gload1(base, (off[2] + rowoff[i]) * 4u), gload1(base, (off[3] + rowoff[i]) * 4u));
+    }
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
@@ -150,9 +172,8 @@ struct LoaderKC {
   }
 };
 
-// Unaligned tensors (odd row strides such as d = 9C + 1): dword loads with the 32
-// lanes of a half-wave on 32 consecutive k-values of one row, so that every
-// load instruction reads whole 128-byte row segments whatever their alignment.
+// Scalar variant: dword loads with the 32 lanes of a half-wave on 32 consecutive
+// k-values of one row.  It is the one that can subsample (line_len > 0).
 template <int ROWS>
 struct LoaderKC<ROWS, false> {
   static constexpr bool kKRow = false;

@@ -6,7 +6,12 @@
 // Replaces compute_kfgrads / update_kfgrads of
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py,
 // fisher_blocks/connection.py:51-61 and normalizations/batch_normalization.py:159-191.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
+#include <new>
+#include <vector>
 
 #include "common.h"
 #include "mma_core.h"
@@ -28,9 +33,18 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(LA la_in, LB lb_in, in
   constexpr int BM = 64 * W;
   __shared__ float ldsA[Panel<BM>::kFloats];
   __shared__ float ldsB[Panel<BM>::kFloats];
-  const int tile = blockIdx.x % ntiles;
-  const int split = blockIdx.x / ntiles;
-  const int ti = tile / tiles_n, tj = tile % tiles_n;
+  // Workgroup i of a launch runs on XCD i % 8 (each XCD has its own L2): every XCD gets a
+  // contiguous run of the work list, which walks the tile rows of one tile column and
+  // k-slice first, so that the workgroups that read the same B panels share an L2.
+  const int total = (int)gridDim.x;
+  const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+  const int base = total / 8, rem = total % 8;
+  const int w = xcd * base + (xcd < rem ? xcd : rem) + idx;
+  const int tiles_m = ntiles / tiles_n;
+  const int split = w / ntiles;
+  const int q = w - split * ntiles;
+  const int tj = q / tiles_m, ti = q - tj * tiles_m;
+  const int tile = ti * tiles_n + tj;
   LA la = la_in;
   LB lb = lb_in;
   la.init(nullptr, ti * BM);
@@ -113,8 +127,10 @@ GemmPlan plan_gemm(int M, int N, int K) {
   return p;
 }
 
-bool kc_aligned(const float *base, int K, long long ld) {
-  return (ld % 4 == 0) && (K % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
+// 16-byte loads need rows that start on 16-byte boundaries (the reduction length
+// is free: the loader takes a quad cut by the end of the range element by element)
+bool kc_aligned(const float *base, long long ld) {
+  return (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(base) % 16 == 0);
 }
 
 bool ks_aligned(const float *base, long long ld) {
@@ -236,11 +252,16 @@ size_t align_floats(size_t n) { return (n + 63) & ~(size_t)63; }
 
 }  // namespace
 
+// Leading dimension of the intermediate product T = Ginv . grad: rows start on
+// 16-byte boundaries whatever dA is, so that the second product reads T with
+// 16-byte loads.
+int padded_ld(int dA) { return (dA + 3) & ~3; }
+
 extern "C" size_t kfac_precond_conn_workspace_bytes(int dG, int dA) {
   if (dG <= 0 || dA <= 0) return 0;
   const size_t p1 = plan_gemm(dG, dA, dG).partial_floats();
   const size_t p2 = plan_gemm(dG, dA, dA).partial_floats();
-  return (align_floats((size_t)dG * dA) + (p1 > p2 ? p1 : p2)) * sizeof(float) + 256;
+  return (align_floats((size_t)dG * padded_ld(dA)) + (p1 > p2 ? p1 : p2)) * sizeof(float) + 256;
 }
 
 extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ainv, int dA,
@@ -260,30 +281,32 @@ extern "C" int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ain
   hipStream_t s = kfac::as_stream(stream);
   float *T = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
   const int dW = dA - hb;
-  float *partial = T + align_floats((size_t)dG * dA);
+  const int ldT = padded_ld(dA);
+  float *partial = T + align_floats((size_t)dG * ldT);
   // T (dG x dA) = Ginv (dG x dG) . [gradW | gradb] (dG x dA); float4 loads when
   // both operands are aligned, scalar loads otherwise
   int rc;
-  if (kc_aligned(Ginv, dG, dG) && ks_aligned(gradW, dW))
+  if (kc_aligned(Ginv, dG) && ks_aligned(gradW, dW))
     rc = launch_gemm(rowmajor_kc<64, true>(Ginv, dG, dG, dG), colop_ks<64, true>(gradW, dW, dW, gradb),
                      rowmajor_kc<128, true>(Ginv, dG, dG, dG),
-                     colop_ks<128, true>(gradW, dW, dW, gradb), dG, dA, dG, partial, T, dA, dA,
+                     colop_ks<128, true>(gradW, dW, dW, gradb), dG, dA, dG, partial, T, ldT, dA,
                      nullptr, s);
   else
     rc = launch_gemm(rowmajor_kc<64, false>(Ginv, dG, dG, dG),
                      colop_ks<64, false>(gradW, dW, dW, gradb),
                      rowmajor_kc<128, false>(Ginv, dG, dG, dG),
-                     colop_ks<128, false>(gradW, dW, dW, gradb), dG, dA, dG, partial, T, dA, dA,
+                     colop_ks<128, false>(gradW, dW, dW, gradb), dG, dA, dG, partial, T, ldT, dA,
                      nullptr, s);
   if (rc != KFAC_OK) return rc;
-  // kf (dG x dA) = T . Ainv (symmetric: column j of Ainv is its row j)
-  if (kc_aligned(T, dA, dA) && kc_aligned(Ainv, dA, dA))
-    return launch_gemm(rowmajor_kc<64, true>(T, dG, dA, dA), rowmajor_kc<64, true>(Ainv, dA, dA, dA),
-                       rowmajor_kc<128, true>(T, dG, dA, dA),
+  // kf (dG x dA) = T . Ainv (symmetric: column j of Ainv is its row j); T is read with
+  // 16-byte loads, Ainv too when its rows are aligned (dA a multiple of 4)
+  if (kc_aligned(Ainv, dA))
+    return launch_gemm(rowmajor_kc<64, true>(T, dG, dA, ldT), rowmajor_kc<64, true>(Ainv, dA, dA, dA),
+                       rowmajor_kc<128, true>(T, dG, dA, ldT),
                        rowmajor_kc<128, true>(Ainv, dA, dA, dA), dG, dA, dA, partial, kfW, dW, dW,
                        kfb, s);
-  return launch_gemm(rowmajor_kc<64, false>(T, dG, dA, dA), rowmajor_kc<64, false>(Ainv, dA, dA, dA),
-                     rowmajor_kc<128, false>(T, dG, dA, dA),
+  return launch_gemm(rowmajor_kc<64, true>(T, dG, dA, ldT), rowmajor_kc<64, false>(Ainv, dA, dA, dA),
+                     rowmajor_kc<128, true>(T, dG, dA, ldT),
                      rowmajor_kc<128, false>(Ainv, dA, dA, dA), dG, dA, dA, partial, kfW, dW, dW,
                      kfb, s);
 }
@@ -371,5 +394,336 @@ extern "C" int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamm
   hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
                      kf_gamma, kf_beta, nan_flag_dev);
   KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Grouped launch: the preconditioning products of all connection layers of a
+// network.  Most layers' products are far too small to fill the GPU (a launch
+// each, two to four launches per layer with their split-K finishes): a group
+// cuts the first product of every layer into (layer, tile, k-slice) tasks of
+// about equal length and runs them from one task table, then the same for the
+// second product: a few launches per phase (one per tile size and loader kind)
+// for the whole network.
+// ---------------------------------------------------------------------------
+namespace {
+
+struct PreStatic {
+  int dG, dA, dW, hb, ldT, w;     // w: 1 = 64-tiles, 2 = 128-tiles
+  int tm, tn;
+  int nsplit[2];
+  long long klen[2];
+  long long t_off, part_off;      // floats from the workspace base: T, partial tiles
+};
+
+struct PreDyn {
+  const float *Ginv, *Ainv, *gradW, *gradb;
+  float *kfW, *kfb;
+};
+
+// task = (item, tile-and-slice index in the order (slice, tile column, tile row))
+template <int W, int PHASE, bool VA, bool VB>
+__global__ __launch_bounds__(THREADS, 2) void gemm_group_kernel(const PreStatic *__restrict__ st,
+                                                                const PreDyn *__restrict__ dy,
+                                                                const int2 *__restrict__ tasks,
+                                                                float *__restrict__ ws) {
+  constexpr int BM = 64 * W;
+  __shared__ float ldsA[Panel<BM>::kFloats];
+  __shared__ float ldsB[Panel<BM>::kFloats];
+  const int2 task = tasks[blockIdx.x];
+  const PreStatic s = st[task.x];
+  const PreDyn v = dy[task.x];
+  const int ntiles = s.tm * s.tn;
+  const int split = task.y / ntiles;
+  const int q = task.y - split * ntiles;
+  const int tj = q / s.tm, ti = q - tj * s.tm;
+  const int tile = ti * s.tn + tj;
+  float *T = ws + s.t_off;
+  float *partial = ws + s.part_off;
+  const int K = PHASE == 0 ? s.dG : s.dA;
+  const long long kbeg = (long long)split * s.klen[PHASE];
+  long long kend = kbeg + s.klen[PHASE];
+  if (kend > K) kend = K;
+  floatx16 acc[W][W];
+  zero_acc<W, W>(acc);
+  if (PHASE == 0) {
+    // T = Ginv . [gradW | gradb]
+    LoaderKC<BM, VA> la;
+    la.base = v.Ginv;
+    la.sample_stride = 0;
+    la.row_stride = (unsigned)s.dG;
+    la.L = (unsigned)s.dG;
+    la.rows_valid = s.dG;
+    LoaderKS<BM, VB> lb;
+    lb.base = v.gradW;
+    lb.extra = v.gradb;
+    lb.ld = (unsigned)s.dW;
+    lb.rows_valid = s.dW;
+    lb.has_extra = s.hb;
+    la.init(nullptr, ti * BM);
+    lb.init(nullptr, tj * BM);
+    mainloop<W, W, false>(la, lb, ti * BM, tj * BM, kbeg, kend, ldsA, ldsB, acc);
+  } else {
+    // kf = T . Ainv
+    LoaderKC<BM, VA> la;
+    la.base = T;
+    la.sample_stride = 0;
+    la.row_stride = (unsigned)s.ldT;
+    la.L = (unsigned)s.dA;
+    la.rows_valid = s.dG;
+    LoaderKC<BM, VB> lb;
+    lb.base = v.Ainv;
+    lb.sample_stride = 0;
+    lb.row_stride = (unsigned)s.dA;
+    lb.L = (unsigned)s.dA;
+    lb.rows_valid = s.dA;
+    la.init(nullptr, ti * BM);
+    lb.init(nullptr, tj * BM);
+    mainloop<W, W, false>(la, lb, ti * BM, tj * BM, kbeg, kend, ldsA, ldsB, acc);
+  }
+  if (s.nsplit[PHASE] > 1) {
+    float *out = partial + ((long long)split * ntiles + tile) * (BM * BM);
+    for_each_acc<W, W>(acc, [&](int r, int c, float val) { out[r * BM + c] = val; });
+    return;
+  }
+  const int M = s.dG, N = s.dA;
+  for_each_acc<W, W>(acc, [&](int r, int c, float val) {
+    const int i = ti * BM + r, j = tj * BM + c;
+    if (i < M && j < N) {
+      if (PHASE == 0)
+        T[(long long)i * s.ldT + j] = val;
+      else if (j < s.dW)
+        v.kfW[(long long)i * s.dW + j] = val;
+      else
+        v.kfb[i] = val;
+    }
+  });
+}
+
+// task = (item, block of 256 output elements): sums the item's k-slices
+template <int PHASE>
+__global__ __launch_bounds__(256) void gemm_group_finish_kernel(const PreStatic *__restrict__ st,
+                                                                const PreDyn *__restrict__ dy,
+                                                                const int2 *__restrict__ tasks,
+                                                                float *__restrict__ ws) {
+  const int2 task = tasks[blockIdx.x];
+  const PreStatic s = st[task.x];
+  const PreDyn v = dy[task.x];
+  const int M = s.dG, N = s.dA;
+  const long long idx = (long long)task.y * 256 + threadIdx.x;
+  if (idx >= (long long)M * N) return;
+  const int i = (int)(idx / N), j = (int)(idx - (long long)i * N);
+  const int bm = 64 * s.w;
+  const int ntiles = s.tm * s.tn;
+  const int tile = (i / bm) * s.tn + j / bm;
+  const float *p = ws + s.part_off + (long long)tile * bm * bm + (i % bm) * bm + (j % bm);
+  const long long stride = (long long)ntiles * bm * bm;
+  float sum = 0.f;
+  for (int k = 0; k < s.nsplit[PHASE]; ++k) sum += p[k * stride];
+  if (PHASE == 0)
+    (ws + s.t_off)[(long long)i * s.ldT + j] = sum;
+  else if (j < s.dW)
+    v.kfW[(long long)i * s.dW + j] = sum;
+  else
+    v.kfb[i] = sum;
+}
+
+void deal_tasks_to_xcds(std::vector<int2> &table, const std::vector<int2> &natural) {
+  const size_t n = natural.size();
+  const size_t chunk = (n + 7) / 8;
+  for (size_t p = 0; p < chunk; ++p)
+    for (size_t x = 0; x < 8; ++x) {
+      const size_t i = x * chunk + p;
+      if (i < n) table.push_back(natural[i]);
+    }
+}
+
+// launches of one phase: {64-tiles, 128-tiles} x {both operands with 16-byte loads,
+// A only (phase 2: T is always aligned), neither}
+constexpr int kPreKinds = 6;
+
+}  // namespace
+
+struct kfac_precond_group {
+  int count = 0;
+  std::vector<PreStatic> items;
+  std::vector<PreDyn> dyn;
+  std::vector<int> kind[2];         // per phase, per item
+  size_t ws_floats = 0;
+  int task0[2][kPreKinds] = {}, ntask[2][kPreKinds] = {};
+  int ftask0[2] = {0, 0}, nftask[2] = {0, 0};
+  kfac::DevTable d_items, d_dyn, d_tasks;
+};
+
+extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int32_t *dA,
+                                         const int32_t *has_bias, kfac_precond_group_t *out) {
+  KFAC_REQUIRE(out != nullptr, "group_out is null");
+  *out = nullptr;
+  KFAC_REQUIRE(count >= 0 && (count == 0 || (dG && dA && has_bias)), "bad item list");
+  auto *g = new (std::nothrow) kfac_precond_group;
+  if (!g) return kfac::fail(KFAC_ENOMEM, "out of host memory");
+  g->count = count;
+  g->items.resize(count);
+  g->dyn.resize(count);
+  g->kind[0].resize(count);
+  g->kind[1].resize(count);
+  double work[2][kPreKinds] = {};
+  std::vector<long long> nk[2];
+  nk[0].resize(count);
+  nk[1].resize(count);
+  size_t off = 0;
+  for (int i = 0; i < count; ++i) {
+    PreStatic &s = g->items[i];
+    memset(&s, 0, sizeof(s));
+    const int hb = has_bias[i] ? 1 : 0;
+    if (dG[i] <= 0 || dA[i] - hb <= 0 || (long long)dG[i] * dA[i] >= 0x40000000LL ||
+        (long long)dA[i] * dA[i] >= 0x40000000LL || (long long)dG[i] * dG[i] >= 0x40000000LL) {
+      delete g;
+      return kfac::fail(KFAC_EINVAL, "item %d: bad dimensions dG=%d dA=%d", i, dG[i], dA[i]);
+    }
+    s.dG = dG[i];
+    s.dA = dA[i];
+    s.hb = hb;
+    s.dW = dA[i] - hb;
+    s.ldT = padded_ld(dA[i]);
+    // 128-tiles unless they would be mostly padding
+    s.w = (s.dG >= 96 && s.dA >= 96) ? 2 : 1;
+    const int bm = 64 * s.w;
+    s.tm = kfac::ceil_div(s.dG, bm);
+    s.tn = kfac::ceil_div(s.dA, bm);
+    nk[0][i] = kfac::ceil_div(s.dG, KT);
+    nk[1][i] = kfac::ceil_div(s.dA, KT);
+    // loader kinds: 16-byte loads need aligned rows (the pointers are checked at run time)
+    const bool va0 = s.dG % 4 == 0, vb0 = s.dW % 4 == 0;
+    g->kind[0][i] = (s.w == 1 ? 0 : 3) + ((va0 && vb0) ? 0 : 2);
+    g->kind[1][i] = (s.w == 1 ? 0 : 3) + (s.dA % 4 == 0 ? 0 : 1);
+    for (int p = 0; p < 2; ++p)
+      work[p][g->kind[p][i]] += (double)s.tm * s.tn * (double)nk[p][i] * (s.w == 1 ? 1.0 : 4.0);
+    s.t_off = (long long)off;
+    off += align_floats((size_t)s.dG * s.ldT);
+  }
+  std::vector<int2> natural[2][kPreKinds], fin[2];
+  for (int p = 0; p < 2; ++p) {
+    double per_wg[kPreKinds];
+    for (int k = 0; k < kPreKinds; ++k) {
+      per_wg[k] = work[p][k] / 2304.0;
+      if (per_wg[k] < 32.0) per_wg[k] = 32.0;
+      if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override
+        const double val = atof(env);
+        if (val >= 1.0) per_wg[k] = val;
+      }
+    }
+    for (int i = 0; i < count; ++i) {
+      PreStatic &s = g->items[i];
+      long long ns = (long long)((double)nk[p][i] * (s.w == 1 ? 1.0 : 4.0) / per_wg[g->kind[p][i]] + 0.5);
+      if (ns < 1) ns = 1;
+      if (ns > 64) ns = 64;
+      if (ns > nk[p][i]) ns = nk[p][i];
+      const long long per = kfac::ceil_div(nk[p][i], ns);
+      s.nsplit[p] = (int)kfac::ceil_div(nk[p][i], per);
+      s.klen[p] = per * KT;
+      const int ntiles = s.tm * s.tn;
+      for (int w = 0; w < ntiles * s.nsplit[p]; ++w) natural[p][g->kind[p][i]].push_back(make_int2(i, w));
+      if (s.nsplit[p] > 1) {
+        const long long blocks = kfac::ceil_div<long long>((long long)s.dG * s.dA, 256);
+        for (long long b = 0; b < blocks; ++b) fin[p].push_back(make_int2(i, (int)b));
+      }
+    }
+  }
+  // partial tiles: one area per item, shared by the two phases
+  for (int i = 0; i < count; ++i) {
+    PreStatic &s = g->items[i];
+    const int bm = 64 * s.w;
+    const int ns = std::max(s.nsplit[0], s.nsplit[1]);
+    s.part_off = (long long)off;
+    if (ns > 1) off += (size_t)ns * s.tm * s.tn * bm * bm;
+  }
+  g->ws_floats = off;
+  std::vector<int2> tasks;
+  for (int p = 0; p < 2; ++p)
+    for (int k = 0; k < kPreKinds; ++k) {
+      g->task0[p][k] = (int)tasks.size();
+      g->ntask[p][k] = (int)natural[p][k].size();
+      deal_tasks_to_xcds(tasks, natural[p][k]);
+    }
+  for (int p = 0; p < 2; ++p) {
+    g->ftask0[p] = (int)tasks.size();
+    g->nftask[p] = (int)fin[p].size();
+    tasks.insert(tasks.end(), fin[p].begin(), fin[p].end());
+  }
+  if (tasks.empty()) tasks.push_back(make_int2(0, 0));
+  int rc = g->d_items.set(g->items.data(), sizeof(PreStatic) * (size_t)count, nullptr);
+  if (rc == KFAC_OK) rc = g->d_tasks.set(tasks.data(), sizeof(int2) * tasks.size(), nullptr);
+  if (rc != KFAC_OK) {
+    delete g;
+    return rc;
+  }
+  *out = g;
+  return KFAC_OK;
+}
+
+extern "C" size_t kfac_precond_group_workspace_bytes(kfac_precond_group_t group) {
+  return group ? group->ws_floats * sizeof(float) + 256 : 0;
+}
+
+extern "C" int kfac_precond_group_destroy(kfac_precond_group_t group) {
+  delete group;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_precond_group_run_f32(kfac_precond_group_t group, const float *const *Ginv,
+                                          const float *const *Ainv, const float *const *gradW,
+                                          const float *const *gradb, float *const *kfW,
+                                          float *const *kfb, void *ws, size_t ws_bytes,
+                                          void *stream) {
+  KFAC_REQUIRE(group != nullptr, "group is null");
+  const int count = group->count;
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(Ginv && Ainv && gradW && gradb && kfW && kfb, "null table");
+  if (ws == nullptr || ws_bytes < kfac_precond_group_workspace_bytes(group))
+    return kfac::fail(KFAC_ENOMEM, "preconditioning group workspace too small: %zu < %zu bytes",
+                      ws_bytes, kfac_precond_group_workspace_bytes(group));
+  auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  for (int i = 0; i < count; ++i) {
+    const PreStatic &s = group->items[i];
+    KFAC_REQUIRE(Ginv[i] && Ainv[i] && gradW[i] && kfW[i], "item %d: null pointer", i);
+    KFAC_REQUIRE((s.hb != 0) == (gradb[i] != nullptr) && (s.hb != 0) == (kfb[i] != nullptr),
+                 "item %d: bias pointers do not match the group's description", i);
+    // plans assume what torch allocations give; a misaligned view must use the single call
+    KFAC_REQUIRE(aligned16(Ginv[i]) && aligned16(Ainv[i]) && aligned16(gradW[i]),
+                 "item %d: factor and gradient pointers must be 16-byte aligned", i);
+    group->dyn[i] = PreDyn{Ginv[i], Ainv[i], gradW[i], gradb[i], kfW[i], kfb[i]};
+  }
+  hipStream_t s = kfac::as_stream(stream);
+  if (int rc = group->d_dyn.set(group->dyn.data(), sizeof(PreDyn) * (size_t)count, s)) return rc;
+  float *base = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
+  const PreStatic *st = group->d_items.as<const PreStatic>();
+  const PreDyn *dy = group->d_dyn.as<const PreDyn>();
+  const int2 *tasks = group->d_tasks.as<const int2>();
+  using Kern = void (*)(const PreStatic *, const PreDyn *, const int2 *, float *);
+  static const Kern kerns[2][kPreKinds] = {
+      {gemm_group_kernel<1, 0, true, true>, nullptr, gemm_group_kernel<1, 0, false, false>,
+       gemm_group_kernel<2, 0, true, true>, nullptr, gemm_group_kernel<2, 0, false, false>},
+      {gemm_group_kernel<1, 1, true, true>, gemm_group_kernel<1, 1, true, false>, nullptr,
+       gemm_group_kernel<2, 1, true, true>, gemm_group_kernel<2, 1, true, false>, nullptr}};
+  for (int p = 0; p < 2; ++p) {
+    for (int k = 0; k < kPreKinds; ++k) {
+      if (group->ntask[p][k] == 0) continue;
+      if (!kerns[p][k]) return kfac::fail(KFAC_EINVAL, "internal: no kernel for kind %d", k);
+      kfac::TimedLaunch timed(KFAC_TIMED_GEMM, s);
+      hipLaunchKernelGGL(kerns[p][k], dim3(group->ntask[p][k]), dim3(THREADS), 0, s, st, dy,
+                         tasks + group->task0[p][k], base);
+    }
+    KFAC_HIP_CHECK(hipGetLastError());
+    if (group->nftask[p] > 0) {
+      if (p == 0)
+        hipLaunchKernelGGL(gemm_group_finish_kernel<0>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
+                           tasks + group->ftask0[p], base);
+      else
+        hipLaunchKernelGGL(gemm_group_finish_kernel<1>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
+                           tasks + group->ftask0[p], base);
+      KFAC_HIP_CHECK(hipGetLastError());
+    }
+  }
   return KFAC_OK;
 }

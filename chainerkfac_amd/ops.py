@@ -465,6 +465,67 @@ def precond_conn(Ginv, Ainv, gradW, gradb=None, kfW=None, kfb=None, stream=None)
     return kfW, (kfb if has_b else None)
 
 
+class PrecondGroup(object):
+    """``precond_conn`` for a fixed list of layers ``(dG, dA, has_bias)`` as one grouped call."""
+
+    def __init__(self, shapes):
+        self.shapes = tuple((int(a), int(b), int(bool(c))) for a, b, c in shapes)
+        lib = _lib.load()
+        plan = ctypes.c_void_p()
+        _lib.check(lib.kfac_precond_group_create(
+            len(self.shapes), _lib.i32_array([s[0] for s in self.shapes]),
+            _lib.i32_array([s[1] for s in self.shapes]), _lib.i32_array([s[2] for s in self.shapes]),
+            ctypes.byref(plan)))
+        self._plan = plan
+        self.workspace_bytes = lib.kfac_precond_group_workspace_bytes(plan)
+
+    def __del__(self):
+        try:
+            plan, self._plan = self._plan, None
+            if plan is not None:
+                _lib._lib.kfac_precond_group_destroy(plan)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+    def run(self, Ginvs, Ainvs, gradWs, gradbs, kfWs, kfbs, stream=None):
+        n = len(self.shapes)
+        if not (len(Ginvs) == len(Ainvs) == len(gradWs) == len(gradbs) == len(kfWs) == len(kfbs) == n):
+            raise ValueError('expected {} layers'.format(n))
+        if n == 0:
+            return
+        for (dG, dA, hb), G, A, gW, gb, kW, kb in zip(self.shapes, Ginvs, Ainvs, gradWs, gradbs, kfWs, kfbs):
+            for t, nm in ((G, 'Ginv'), (A, 'Ainv'), (gW, 'gradW'), (kW, 'kfW')):
+                _dev.require_gpu_tensor(t, nm)
+            if tuple(G.shape) != (dG, dG) or tuple(A.shape) != (dA, dA) or gW.numel() != dG * (dA - hb) \
+                    or kW.numel() != gW.numel():
+                raise ValueError('layer ({}, {}, {}) does not match its tensors'.format(dG, dA, hb))
+            if bool(hb) != (gb is not None) or bool(hb) != (kb is not None):
+                raise ValueError('bias arrays do not match the group')
+            if hb:
+                _dev.require_gpu_tensor(gb, 'gradb')
+                _dev.require_gpu_tensor(kb, 'kfb')
+        ws = _dev.workspace('precond_group', self.workspace_bytes, Ginvs[0].device)
+        _lib.check(_lib.load().kfac_precond_group_run_f32(
+            self._plan, _lib.ptr_array([t.data_ptr() for t in Ginvs]),
+            _lib.ptr_array([t.data_ptr() for t in Ainvs]), _lib.ptr_array([t.data_ptr() for t in gradWs]),
+            _lib.ptr_array([_dev.ptr(t) for t in gradbs]), _lib.ptr_array([t.data_ptr() for t in kfWs]),
+            _lib.ptr_array([_dev.ptr(t) for t in kfbs]), ws.data_ptr(), ws.numel(),
+            _dev.stream_handle(stream)))
+
+
+_precond_groups = None
+
+
+def precond_group(shapes, bound_to=None):
+    """Cached ``PrecondGroup``; ``bound_to`` (the buffers' device pointers) gives callers
+    with persistent buffers a plan whose pointer table is never rewritten."""
+    global _precond_groups
+    if _precond_groups is None:
+        _precond_groups = _PlanCache(16)
+    key = tuple((int(a), int(b), int(bool(c))) for a, b, c in shapes)
+    return _precond_groups.get((key, bound_to), lambda: PrecondGroup(key))
+
+
 def precond_bn(Finv, g_gamma, g_beta, kf_gamma=None, kf_beta=None, nan_flag=None, stream=None):
     """Finv . [g_gamma ; g_beta] with the NaN fallback to the raw gradients."""
     _dev.require_gpu_tensor(Finv, 'Finv')

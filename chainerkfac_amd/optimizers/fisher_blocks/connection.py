@@ -80,17 +80,24 @@ class FisherBlockConnection(FisherBlock):
         setattr(self, 'diag_val_backward', (1 / pi) * rW)
         return [pi * (rW * np.ones(A.shape[0])), (1 / pi) * (rW * np.ones(G.shape[0]))]
 
-    def update_kfgrads(self):
+    def kfgrad_operands(self):
+        """``(G_inv, A_inv, gradW, gradb, kfW, kfb)`` of the preconditioning products, with
+        the output buffers this block keeps; publishes them as ``W.kfgrad`` / ``b.kfgrad``."""
         self.check_attr('invs')
         W = self.link.W
         b = self.link.b
         A_inv, G_inv = self.invs
         kfW = self._buffer('kfW', W.shape, W.data.device)
         kfb = None if b is None else self._buffer('kfb', b.shape, b.data.device)
-        ops.precond_conn(G_inv, A_inv, W.grad, None if b is None else b.grad, kfW, kfb)
         W.kfgrad = kfW
         if b is not None:
             b.kfgrad = kfb
+        gW = W.grad if W.grad.is_contiguous() else W.grad.contiguous()
+        gb = None if b is None else (b.grad if b.grad.is_contiguous() else b.grad.contiguous())
+        return G_inv, A_inv, gW, gb, kfW, kfb
+
+    def update_kfgrads(self):
+        ops.precond_conn(*self.kfgrad_operands())
 
     def compute_kfgrads(self, W, b, invs):
         """(G^-1 [dW | db]) A^-1 as one (c_out, dA) matrix, for callers that want

@@ -397,10 +397,25 @@ class KFAC(object):
         for fblock in fblocks:
             fblock.update_cov_emas()
 
+    #: run the preconditioning products of all connection blocks as one grouped call
+    #: (a few launches for the whole network); False calls every block's
+    #: ``update_kfgrads`` on its own
+    group_precondition = True
+
     def precondition(self, fblocks):
-        """``fblock.update_kfgrads()`` for every block, independent blocks side by side."""
+        """``fblock.update_kfgrads()`` for every block: the connection blocks' GEMMs as one
+        grouped call, the other blocks side by side on the lanes."""
+        conn = [fb for fb in fblocks if isinstance(fb, FB.FisherBlockConnection)] \
+            if self.group_precondition else []
+        grouped = set(id(fb) for fb in conn)
         for fblock in fblocks:
-            self._lanes.run(fblock.update_kfgrads)
+            if id(fblock) not in grouped:
+                self._lanes.run(fblock.update_kfgrads)
+        if conn:
+            operands = [fb.kfgrad_operands() for fb in conn]
+            shapes = [(o[0].shape[0], o[1].shape[0], o[3] is not None) for o in operands]
+            bound = tuple(0 if t is None else t.data_ptr() for o in operands for t in o)
+            ops.precond_group(shapes, bound).run(*[[o[i] for o in operands] for i in range(6)])
         self._lanes.join()
 
     def update_invs_batched(self, fblocks):

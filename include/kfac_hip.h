@@ -270,6 +270,25 @@ int kfac_precond_conn_f32(const float *Ginv, int dG, const float *Ainv, int dA,
                           const float *gradW, const float *gradb, float *kfW,
                           float *kfb, void *ws, size_t ws_bytes, void *stream);
 
+/* kfac_precond_conn_f32 for all connection layers of a network in a few
+ * launches: a group is created once for the layers' (dG, dA, has_bias) and run
+ * with one pointer per layer and operand (gradb[i] / kfb[i] NULL where the layer
+ * has no bias; all pointers 16-byte aligned).  The two products of every layer
+ * are cut into tasks of about equal length and run from task tables: first
+ * Ginv . [gradW | gradb] of all layers, then . Ainv of all layers.  Results as
+ * kfac_precond_conn_f32 up to the order of the floating-point sums.  Replaces
+ * the loop over fblock.update_kfgrads() (optimizers/kfac.py:306-310) for the
+ * connection blocks. */
+typedef struct kfac_precond_group *kfac_precond_group_t;
+int kfac_precond_group_create(int count, const int32_t *dG, const int32_t *dA,
+                              const int32_t *has_bias, kfac_precond_group_t *group_out);
+size_t kfac_precond_group_workspace_bytes(kfac_precond_group_t group);
+int kfac_precond_group_destroy(kfac_precond_group_t group);
+int kfac_precond_group_run_f32(kfac_precond_group_t group, const float *const *Ginv,
+                               const float *const *Ainv, const float *const *gradW,
+                               const float *const *gradb, float *const *kfW,
+                               float *const *kfb, void *ws, size_t ws_bytes, void *stream);
+
 /* kf = Finv . [g_gamma ; g_beta] split at n_gamma; if any element of kf is
  * NaN every output is the raw gradient instead and *nan_flag_dev (device
  * int32, may be NULL) is set to 1, else 0.  Either half may be absent

@@ -118,3 +118,36 @@ def test_axpby_and_momentum_update():
     O.momentum_update(p, v, g, 0.1, 0.9)
     np.testing.assert_allclose(vd.cpu().numpy(), v, rtol=1e-6, atol=1e-7)
     np.testing.assert_allclose(pd.cpu().numpy(), p, rtol=1e-6, atol=1e-7)
+
+
+def test_grouped_preconditioning_matches_the_single_calls():
+    """All layers' products in one grouped call: 64- and 128-tiles, with and without bias,
+    aligned and odd dimensions, several k-slices; against float64 and the single calls."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(23)
+
+    def spd(d):
+        X = r.standard_normal((2 * d, d)).astype(np.float32)
+        return torch.from_numpy((X.T @ X / (2 * d) + 0.1 * np.eye(d, dtype=np.float32)).astype(np.float32)).cuda()
+
+    shapes = [(64, 577, True), (10, 785, True), (256, 64, False), (130, 1153, True), (1000, 2049, True),
+              (96, 96, False), (7, 28, True), (512, 1024, False)]
+    ops_in = []
+    for dG, dA, hb in shapes:
+        gW = torch.from_numpy(r.standard_normal((dG, dA - int(hb))).astype(np.float32)).cuda()
+        gb = torch.from_numpy(r.standard_normal(dG).astype(np.float32)).cuda() if hb else None
+        ops_in.append((spd(dG), spd(dA), gW, gb, torch.full_like(gW, float('nan')),
+                       torch.full_like(gb, float('nan')) if hb else None))
+    group = ops.precond_group(shapes)
+    group.run(*[[o[i] for o in ops_in] for i in range(6)])
+    torch.cuda.synchronize()
+    for (dG, dA, hb), (G, A, gW, gb, kW, kb) in zip(shapes, ops_in):
+        grad = gW.double() if not hb else torch.cat([gW.double(), gb.double()[:, None]], dim=1)
+        ref = (G.double() @ grad @ A.double()).cpu().numpy()
+        got = kW.cpu().numpy() if not hb else np.column_stack([kW.cpu().numpy(), kb.cpu().numpy()])
+        assert rel(got, ref) < 1e-5, (dG, dA, hb)
+        sW, sb = ops.precond_conn(G, A, gW, gb)
+        single = sW.cpu().numpy() if not hb else np.column_stack([sW.cpu().numpy(), sb.cpu().numpy()])
+        assert rel(got, single) < 1e-5, (dG, dA, hb)
+    with pytest.raises(ValueError):
+        group.run(*[[o[i] for o in ops_in[:-1]] for i in range(6)])
