@@ -78,10 +78,21 @@ __device__ __forceinline__ float from_buf(__half v, int divisor) {
   return __half2float(__float2half_rn(__half2float(v) / __half2float(__int2half_rn(divisor))));
 }
 
+// Workgroup i of a launch runs on XCD i % 8, each XCD with an L2 of its own.
+// Every XCD takes one contiguous run of the unit list: neighbouring units touch
+// neighbouring memory (the cache lines at the seams of two tiles or chunks), and
+// a line that two workgroups each write half of is completed inside one L2
+// instead of being written back twice as partial lines.
+__device__ __forceinline__ int xcd_contiguous_unit(int total) {
+  const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+  const int base = total / 8, rem = total % 8;
+  return xcd * base + (xcd < rem ? xcd : rem) + idx;
+}
+
 template <class B>
 __global__ __launch_bounds__(kThreads) void pack_kernel(PackTables tb, B *__restrict__ buf,
                                                         int target) {
-  const int unit = blockIdx.x;
+  const int unit = xcd_contiguous_unit(gridDim.x);
   const int j = find_array(tb.pack_csum, tb.n, unit);
   if (target >= 0 && tb.rank[j] != target) return;
   const long long nel = tb.nel[j];
@@ -124,7 +135,7 @@ template <class B>
 __global__ __launch_bounds__(kThreads) void unpack_kernel(PackTables tb, const B *__restrict__ buf,
                                                           int target, int divisor) {
   __shared__ float tile[kTile][kTile + 1];
-  const int unit = blockIdx.x;
+  const int unit = xcd_contiguous_unit(gridDim.x);
   const int j = find_array(tb.unpack_csum, tb.n, unit);
   if (target >= 0 && tb.rank[j] != target) return;
   const int local = unit - tb.unpack_csum[j];
@@ -355,6 +366,58 @@ int run_unpack(kfac_pack_plan_t plan, const B *buf, int64_t buf_nelems, int targ
 }
 
 }  // namespace
+
+namespace {
+
+// Plain streaming copy, 16 bytes per lane and load, four loads in flight per
+// lane: the yardstick for the bandwidth-bound kernels of this file.
+__global__ __launch_bounds__(kThreads) void stream_copy_kernel(const float4 *__restrict__ src,
+                                                               float4 *__restrict__ dst,
+                                                               long long n4) {
+  const long long base = (long long)blockIdx.x * (kThreads * 4) + threadIdx.x;
+  float4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long long t = base + (long long)i * kThreads;
+    if (t < n4) v[i] = src[t];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long long t = base + (long long)i * kThreads;
+    if (t < n4) dst[t] = v[i];
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void stream_copy_tail_kernel(const float *__restrict__ src,
+                                                                    float *__restrict__ dst,
+                                                                    long long from, long long n) {
+  const long long t = from + threadIdx.x;
+  if (t < n) dst[t] = src[t];
+}
+
+}  // namespace
+
+extern "C" int kfac_stream_copy_f32(float *dst, const float *src, int64_t nelems, void *stream) {
+  KFAC_REQUIRE(nelems >= 0, "nelems < 0");
+  if (nelems == 0) return KFAC_OK;
+  KFAC_REQUIRE(dst && src, "null pointer");
+  KFAC_REQUIRE(((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) == 0,
+               "pointers must be 16-byte aligned");
+  hipStream_t s = kfac::as_stream(stream);
+  const long long n4 = nelems / 4;
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_COPY, s);
+    if (n4 > 0)
+      hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)kfac::ceil_div<long long>(n4, kThreads * 4)),
+                         dim3(kThreads), 0, s, reinterpret_cast<const float4 *>(src),
+                         reinterpret_cast<float4 *>(dst), n4);
+    if (n4 * 4 < nelems)
+      hipLaunchKernelGGL(stream_copy_tail_kernel, dim3(1), dim3(kThreads), 0, s, src, dst, n4 * 4,
+                         (long long)nelems);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
 
 extern "C" int kfac_pack_f32(kfac_pack_plan_t plan, float *buf, int64_t buf_nelems,
                              int target_rank, void *stream) {

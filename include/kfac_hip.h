@@ -339,7 +339,14 @@ int kfac_momentum_update_f32(float *param, float *v, const float *grad,
 #define KFAC_TIMED_GEMM 3       /* preconditioning GEMM kernel                */
 #define KFAC_TIMED_PACK 4       /* pack kernel                                */
 #define KFAC_TIMED_UNPACK 5     /* unpack kernel                              */
-#define KFAC_TIMED_FAMILIES 6
+#define KFAC_TIMED_COPY 6       /* kfac_stream_copy_f32                        */
+#define KFAC_TIMED_FAMILIES 7
+
+/* dst[i] = src[i] for nelems floats (16-byte aligned pointers): a plain
+ * streaming copy that moves 8 bytes per element, the yardstick that bench.py
+ * puts beside the pack / unpack bandwidth (what a copy kernel reaches on the
+ * same GPU in the same run).  No counterpart in the reference. */
+int kfac_stream_copy_f32(float *dst, const float *src, int64_t nelems, void *stream);
 
 int kfac_timing_enable(int on);
 int kfac_timing_read(int family, int64_t *launches, double *total_ms);
