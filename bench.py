@@ -1,27 +1,31 @@
 #!/usr/bin/env python
 """Benchmark of the K-FAC per-layer hot path on one MI355X.
 
-Workload (BASELINE.json configs[2]): ResNet-50 (bottleneck v1, 1000-way FC, all
-convs with bias) K-FAC step on one GPU's share, batch 32 at 224x224, fp32:
-for all 161 Kronecker factors, covariance (fused im2col SYRK) + pi-damped
+    python bench.py [--config c3] [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu]
+
+Headline workload (--config c3, the default): ResNet-50 (bottleneck v1, 1000-way
+FC, all convs with bias) K-FAC step on one GPU's share, batch 32 at 224x224,
+fp32: for all 161 Kronecker factors, covariance (fused im2col SYRK) + pi-damped
 Cholesky inverse + gradient preconditioning.  Per-layer activations, output
 gradients and parameter gradients are synthetic N(0,1) tensors of the real
 shapes (output gradients scaled by 1/(batch*sqrt(pixels)), the size a
 mean-reduced loss gives them, which keeps the rank-32 batch-norm factors
-positive definite in float32), resident in HBM before the timed region.  The step is driven through
-the drop-in host classes (FisherBlock*.forward_postprocess /
-backward_preprocess, KFAC.update_kfgrads).  The 53 batch-norm blocks, whose
-factor is the rank-32 matrix U^T U / 32 of this batch, are inverted through
-their Woodbury form (the same dense damped inverse as the Cholesky path, which
---dense-bn-inverse forces); the JSON states which path ran and reports the
-inverse rate both against the reference's 161 dense inversions and against
-the dense work actually executed.
+positive definite in float32), resident in HBM before the timed region.  The
+step is driven through the drop-in host classes (the function hook's
+forward_postprocess / backward_preprocess calls, KFAC.update_kfgrads).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu]
+The other configurations of the benchmark definition run the same way:
+  c1  MLP 784-1000-1000-10, batch 128, damping 1e-3 (6 factors)
+  c2  CIFAR-shaped CNN, batch 128, damping 1e-3 (8 factors, up to 4097^2)
+  c4  inverse only: 161 SPD matrices of ResNet-50's factor sizes (27^2 .. 4609^2)
+  c5  ResNet-50-D shapes, batch 32, acc_iters = 16: 16 micro-batches accumulated by
+      the covariance kernels, then triangular pack and unpack of all factors and
+      gradients, damped inverse, preconditioning
 
-prints ONE JSON line: ms per K-FAC step, per-phase TFLOP/s, the roofline of the
-dominant kernel family (covariance SYRK, timed live with HIP events inside the
-library) and the CPU baseline (the NumPy oracle on a bounded sample of layers).
+Prints ONE JSON line: ms per step (a step = one pass of the configuration's hot
+path), per-phase TFLOP/s, the roofline of the dominant kernel family (timed
+live with HIP events inside the library) and the CPU baseline (the NumPy oracle
+on a bounded sample of the same workload).
 """
 import argparse
 import ctypes
@@ -36,21 +40,43 @@ if ROOT not in sys.path:
 
 FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix peak
 HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E peak
-# HBM bytes per covariance SYRK launch (average over the 161 launches of a step):
-# hardware counters FETCH_SIZE and WRITE_SIZE collected with `rocprofv3 --pmc` on
-# this script (--no-graph --calibrate-copy), each scaled by what it reads for the
-# 256 MiB calibration copy; the counter summary is kept under profiles/.
-SYRK_HBM_BYTES_PER_LAUNCH = 41.4e6
+# HBM bytes per launch of the covariance SYRK family, written by
+# `bench.py --summarize-traffic` from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE)
+TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'syrk_hbm_traffic.json')
 BATCH = 32
 DAMPING = 2.5e-4
 STAB_COEFF = 16.0
+METRIC = 'ms per K-FAC step, ResNet-50 bs32/GPU; cov+inv TFLOP/s vs FP32 MFMA peak'
 
 
-def build_model(layers, device, gen):
+def configs():
+    from chainerkfac_amd import workloads as W
+    return {
+        'c1': dict(layers=W.mlp_mnist(), batch=128, damping=1e-3, decay=0.99, acc_iters=1,
+                   workload='MLP 784-1000-1000-10 (bias) K-FAC step, batch 128: 6 factors, '
+                            'cov + damped Cholesky inverse + precondition'),
+        'c2': dict(layers=W.cifar_cnn(), batch=128, damping=1e-3, decay=0.99, acc_iters=1,
+                   workload='CIFAR-shaped CNN (3 conv3x3 + FC 4096->10) K-FAC step, batch 128: 8 factors '
+                            'up to 4097^2, cov + damped Cholesky inverse + precondition'),
+        'c3': dict(layers=W.resnet50_v1(), batch=BATCH, damping=DAMPING, decay=1.0, acc_iters=1,
+                   workload='ResNet-50 v1 (bias, 1000-way) K-FAC step, batch 32 @224: 161 factors, '
+                            'cov + damped Cholesky inverse + precondition'),
+        'c4': dict(layers=None, batch=0, damping=1e-3, decay=1.0, acc_iters=1,
+                   workload='inverse only: 161 SPD fp32 matrices of ResNet-50 factor sizes (27^2 .. 4609^2), '
+                            'X^T X / n + 1e-3 I, damped Cholesky inverse of all of them'),
+        'c5': dict(layers=W.resnet50_d(), batch=BATCH, damping=DAMPING, decay=1.0, acc_iters=16,
+                   workload='ResNet-50-D shapes, batch 32, acc_iters 16: covariances of 16 micro-batches '
+                            'accumulated (167 factors), triangular pack + unpack of factors and gradients, '
+                            'damped inverse, precondition'),
+    }
+
+
+def build_model(layers, device, gen, batch=None):
     """Links with the layer table's shapes plus synthetic per-layer tensors."""
     import torch
     from chainerkfac_amd import links as L
     from chainerkfac_amd import workloads as W
+    batch = BATCH if batch is None else batch
     model = L.Chain()
     calls = []
     for i, layer in enumerate(layers):
@@ -59,20 +85,20 @@ def build_model(layers, device, gen):
             link = L.Convolution2D(layer['c_in'], layer['c_out'], layer['k'], layer['s'], layer['p'],
                                    nobias=not layer['bias'], device=device, generator=gen)
             ho = W.conv_out(layer['h'], layer['k'], layer['s'], layer['p'])
-            x = torch.randn(BATCH, layer['c_in'], layer['h'], layer['w'], device=device, generator=gen)
-            gy = torch.randn(BATCH, layer['c_out'], ho, ho, device=device, generator=gen) / (BATCH * ho)
+            x = torch.randn(batch, layer['c_in'], layer['h'], layer['w'], device=device, generator=gen)
+            gy = torch.randn(batch, layer['c_out'], ho, ho, device=device, generator=gen) / (batch * ho)
             func = L.Convolution2DFunction()
             in_data = (x, link.W.data) + ((link.b.data,) if layer['bias'] else ())
         elif layer['kind'] == 'linear':
             link = L.Linear(layer['d_in'], layer['d_out'], nobias=not layer['bias'], device=device, generator=gen)
-            x = torch.randn(BATCH, layer['d_in'], device=device, generator=gen)
-            gy = torch.randn(BATCH, layer['d_out'], device=device, generator=gen) / BATCH
+            x = torch.randn(batch, layer['d_in'], device=device, generator=gen)
+            gy = torch.randn(batch, layer['d_out'], device=device, generator=gen) / batch
             func = L.LinearFunction()
             in_data = (x, link.W.data) + ((link.b.data,) if layer['bias'] else ())
         else:
             link = L.BatchNormalization(layer['c'], device=device)
-            x = torch.randn(BATCH, layer['c'], layer['h'], layer['w'], device=device, generator=gen)
-            gy = torch.randn(BATCH, layer['c'], layer['h'], layer['w'], device=device, generator=gen) / (BATCH * layer['h'])
+            x = torch.randn(batch, layer['c'], layer['h'], layer['w'], device=device, generator=gen)
+            gy = torch.randn(batch, layer['c'], layer['h'], layer['w'], device=device, generator=gen) / (batch * layer['h'])
             func = L.BatchNormalizationFunction()
             in_data = (x, link.gamma.data, link.beta.data)
         setattr(model, name, link)
@@ -82,11 +108,135 @@ def build_model(layers, device, gen):
     return model, calls
 
 
-def run_gpu(args):
+def _events(n):
+    import torch
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def bracket_ms():
+    """What a pair of events adds to the launch it brackets (the time between an event and
+    the neighbouring kernel's edge): bracket nothing, many times, take the median."""
+    import torch
+    pairs = _events(200)
+    torch.cuda.synchronize()
+    for e0, e1 in pairs:
+        e0.record()
+        e1.record()
+    torch.cuda.synchronize()
+    return sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[len(pairs) // 2]
+
+
+def capture(fn):
+    """The launches of ``fn`` as one HIP graph (fixed sequence, fixed buffers): the host then
+    pays for a single launch per replay."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    return g.replay
+
+
+def timed_steps(run, steps):
+    """EXACTLY ``steps`` calls of ``run`` between two synchronisations: (mean ms over the
+    wall clock, median ms over per-call event pairs)."""
+    import torch
+    pairs = _events(steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e0, e1 in pairs:
+        e0.record()
+        run()
+        e1.record()
+    torch.cuda.synchronize()
+    mean = (time.perf_counter() - t0) * 1e3 / steps
+    each = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return mean, each[len(each) // 2]
+
+
+def timed(fn, reps=5):
+    import torch
+    pairs = _events(reps)
+    torch.cuda.synchronize()
+    for e0, e1 in pairs:
+        e0.record()
+        fn()
+        e1.record()
+    torch.cuda.synchronize()
+    return sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[reps // 2]
+
+
+def family_times(lib):
+    from chainerkfac_amd import _lib
+    fam = {}
+    for name, fid in (('syrk', 0), ('inv_update', 1), ('inv_lauum', 2), ('gemm', 3), ('pack', 4), ('unpack', 5),
+                      ('copy', 6)):
+        n = ctypes.c_int64()
+        ms = ctypes.c_double()
+        _lib.check(lib.kfac_timing_read(fid, ctypes.byref(n), ctypes.byref(ms)))
+        fam[name] = (n.value, ms.value)
+    return fam
+
+
+def read_traffic():
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+        return float(t['bytes_per_launch'])
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+def wire_format(arrays, dev, lib):
+    """Triangular pack / unpack of ``arrays`` (bandwidth-bound), beside a plain streaming copy
+    of the same number of bytes through the library's own copy kernel."""
+    import torch
+    from chainerkfac_amd import _lib
+    from chainerkfac_amd.communicators import ArrayPacker
+    packer = ArrayPacker()
+    nel = packer.get_nelems(arrays)
+    wire = torch.empty(nel, dtype=torch.float32, device=dev)
+    full = sum(a.numel() for a, _ in arrays[0])
+    packer._pack_arrays_to_buffer(arrays, wire)
+    packer._unpack_arrays_from_buffer(arrays, wire)
+    pack_ms = timed(lambda: packer._pack_arrays_to_buffer(arrays, wire), reps=11)
+    unpack_ms = timed(lambda: packer._unpack_arrays_from_buffer(arrays, wire), reps=11)
+    n_copy = (nel + full) // 2 // 4 * 4     # moves as many bytes as the unpack
+    src = torch.ones(n_copy, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+    copy_ms = timed(lambda: _lib.check(lib.kfac_stream_copy_f32(dst.data_ptr(), src.data_ptr(), n_copy, stream)),
+                    reps=11)
+    del src, dst
+    copy_gbps = 8.0 * n_copy / copy_ms / 1e6
+    out = {
+        'arrays': len(arrays[0]), 'triangular': sum(1 for _, t in arrays[0] if t),
+        'pack': {'ms': round(pack_ms, 4), 'GBps': round(8.0 * nel / pack_ms / 1e6, 1)},
+        'unpack': {'ms': round(unpack_ms, 4), 'GBps': round(4.0 * (nel + full) / unpack_ms / 1e6, 1)},
+        'stream_copy': {'ms': round(copy_ms, 4), 'GBps': round(copy_gbps, 1), 'bytes': 8 * n_copy},
+        'packed_MB': round(4.0 * nel / 1e6, 1), 'full_MB': round(4.0 * full / 1e6, 1),
+    }
+    for k in ('pack', 'unpack', 'stream_copy'):
+        out[k]['frac_of_hbm_peak'] = round(out[k]['GBps'] / HBM_PEAK_GBPS, 3)
+    for k in ('pack', 'unpack'):
+        out[k]['frac_of_stream_copy'] = round(out[k]['GBps'] / copy_gbps, 3)
+    return out, wire
+
+
+def run_step_config(args, name, cfg):
+    """c1, c2, c3, c5: cov (x acc_iters) [+ pack/unpack] + inverse + precondition."""
     import torch
     from chainerkfac_amd import _lib
     from chainerkfac_amd import workloads as W
     from chainerkfac_amd.optimizers import KFAC
+    from chainerkfac_amd.optimizers.kfac import extract
 
     lib = _lib.load()
     dev = torch.device('cuda:0')
@@ -99,10 +249,11 @@ def run_gpu(args):
         torch.add(src, 0.0, out=dst)   # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    layers = W.resnet50_v1()
-    flops = W.flops(layers, BATCH)
-    model, calls = build_model(layers, dev, gen)
-    opt = KFAC(damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0)
+    layers, batch, acc_iters = cfg['layers'], cfg['batch'], cfg['acc_iters']
+    flops = W.flops(layers, batch)
+    flops['cov'] *= acc_iters
+    model, calls = build_model(layers, dev, gen, batch)
+    opt = KFAC(damping=cfg['damping'], stab_coeff=STAB_COEFF, cov_ema_decay=cfg['decay'], acc_iters=acc_iters)
     opt.bn_lowrank_inverse = not args.dense_bn_inverse
     opt.lanes = args.lanes
     opt = opt.setup(model)
@@ -110,12 +261,32 @@ def run_gpu(args):
     assert len(opt.fblocks) == len(layers)
     hook = opt.kfhook
 
-    # the calls the function hooks make during forward/backward, then KFAC.update_kfgrads in its three parts
+    # the calls the function hooks make during forward/backward (per micro-batch), then
+    # KFAC.update_kfgrads in its three parts
     def cov_phase():
-        for func, in_data, gy in work:
-            hook.forward_postprocess(func, in_data)
-            hook.backward_preprocess(func, in_data, gy)
-        opt.finish_covs()
+        for it in range(acc_iters):
+            for fb in opt.fblocks:
+                fb.acc_state = (acc_iters, it)
+            for func, in_data, gy in work:
+                hook.forward_postprocess(func, in_data)
+                hook.backward_preprocess(func, in_data, gy)
+            opt.finish_covs()
+            if acc_iters > 1:
+                opt.accumulate_covs()
+
+    wire_state = {}
+
+    def wire_phase():
+        # what the communicator does with a rank's factors and gradients (configuration c5):
+        # pack into one flat buffer in the reference's order, unpack again
+        if 'arrays' not in wire_state:
+            from chainerkfac_amd.communicators import ArrayPacker
+            arrays = extract(opt.fblocks, [range(len(opt.fblocks))], lambda b: b.extract_for_reduce_scatter_v())
+            packer = ArrayPacker()
+            wire_state.update(arrays=arrays, packer=packer,
+                              buf=torch.empty(packer.get_nelems(arrays), dtype=torch.float32, device=dev))
+        wire_state['packer']._pack_arrays_to_buffer(wire_state['arrays'], wire_state['buf'])
+        wire_state['packer']._unpack_arrays_from_buffer(wire_state['arrays'], wire_state['buf'])
 
     def inv_phase():
         opt.update_cov_emas(opt.fblocks)
@@ -124,131 +295,77 @@ def run_gpu(args):
     def pre_phase():
         opt.precondition(opt.fblocks)
 
+    with_wire = name == 'c5'
+
     def step():
         cov_phase()
+        if with_wire:
+            wire_phase()
         inv_phase()
         pre_phase()
 
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
-
-    def capture(fn):
-        """The launches of ``fn`` as one HIP graph (fixed sequence, fixed buffers):
-        the host then pays for a single launch per replay."""
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            fn()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            fn()
-        g.replay()
-        torch.cuda.synchronize()
-        return g.replay
-
     run = step if args.no_graph else capture(step)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step, ms_median = timed_steps(run, args.steps)
 
     # per-phase split: each phase launched the same way as the step (its own graph), timed with events
-    def timed(fn, reps=3):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps
-
     phases = {'cov': cov_phase, 'inverse': inv_phase, 'precondition': pre_phase}
+    if with_wire:
+        phases['pack_unpack'] = wire_phase
     phase_ms = {k: timed(fn if args.no_graph else capture(fn)) for k, fn in phases.items()}
 
-    # wire format of the factors (outside the step: what a communicator would do with them): pack the
-    # lower triangles of all 161 factors into one buffer and unpack them again, HBM-bound
-    from chainerkfac_amd.communicators import ArrayPacker
-    packer = ArrayPacker()
-    arrays = [[(cov, True) for fb in opt.fblocks for cov in fb.covs]]
-    nel = packer.get_nelems(arrays)
-    wire = torch.empty(nel, dtype=torch.float32, device=dev)
-    full = sum(c.numel() for c, _ in arrays[0])
-    packer._pack_arrays_to_buffer(arrays, wire)
-    packer._unpack_arrays_from_buffer(arrays, wire)
-    pack_ms = timed(lambda: packer._pack_arrays_to_buffer(arrays, wire), reps=10)
-    unpack_ms = timed(lambda: packer._unpack_arrays_from_buffer(arrays, wire), reps=10)
-    wire_stats = {
-        'pack': {'ms': round(pack_ms, 4), 'GBps': round(8.0 * nel / pack_ms / 1e6, 1),
-                 'frac_of_hbm_peak': round(8.0 * nel / pack_ms / 1e6 / HBM_PEAK_GBPS, 3)},
-        'unpack': {'ms': round(unpack_ms, 4), 'GBps': round(4.0 * (nel + full) / unpack_ms / 1e6, 1),
-                   'frac_of_hbm_peak': round(4.0 * (nel + full) / unpack_ms / 1e6 / HBM_PEAK_GBPS, 3)},
-        'packed_MB': round(4.0 * nel / 1e6, 1), 'full_MB': round(4.0 * full / 1e6, 1),
-    }
+    # wire format of the factors (and, for c5, of the gradients too): outside the step for the
+    # configurations whose step has no communication
+    if with_wire:
+        arrays = wire_state['arrays']
+    else:
+        arrays = [[(cov, True) for fb in opt.fblocks for cov in fb.covs]]
+    wire_stats, _ = wire_format(arrays, dev, lib)
 
-    # dominant kernel family, timed launch by launch inside the library
-    # (one stream: with lanes, launches overlap and the time between a launch's events is shared with others)
+    # dominant kernel family, timed launch by launch inside the library (one stream: with lanes,
+    # launches overlap and the time between a launch's events is shared with others)
     opt._lanes.n = 0
     _lib.check(lib.kfac_timing_enable(1))
     step()
     torch.cuda.synchronize()
     opt._lanes.n = args.lanes
-    fam = {}
-    for name, fid in (('syrk', 0), ('inv_update', 1), ('inv_lauum', 2), ('gemm', 3)):
-        n = ctypes.c_int64()
-        ms = ctypes.c_double()
-        _lib.check(lib.kfac_timing_read(fid, ctypes.byref(n), ctypes.byref(ms)))
-        fam[name] = (n.value, ms.value)
+    fam = family_times(lib)
     _lib.check(lib.kfac_timing_enable(0))
-    info_bad = int((opt.inv_info != 0).sum().item())
+    info_bad = len(opt.check_numerics())
     lowrank = [fb for fb in opt.fblocks if getattr(fb, 'lowrank_inverse_args', lambda: None)() is not None] \
         if opt.bn_lowrank_inverse else []
-    info_bad += sum(int((fb.inv_info != 0).sum().item()) for fb in lowrank)
-    # d^3 of the factors that went through the dense Cholesky path (the reference inverts all 161 densely)
+    # d^3 of the factors that went through the dense Cholesky path (the reference inverts all of them densely)
     dense_inverse_flops = flops['inverse'] - sum(float(fb.cov_emas[0].shape[0]) ** 3 for fb in lowrank)
 
-    # What a pair of events adds to the launch it brackets (the time between an
-    # event and the neighbouring kernel's edge): bracket nothing, many times.
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(200)]
-    torch.cuda.synchronize()
-    for e0, e1 in pairs:
-        e0.record()
-        e1.record()
-    torch.cuda.synchronize()
-    bracket_ms = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[len(pairs) // 2]
-
+    empty = bracket_ms()
     syrk_n, syrk_raw_ms = fam['syrk']
-    syrk_ms = max(syrk_raw_ms - syrk_n * bracket_ms, 1e-9)
+    syrk_ms = max(syrk_raw_ms - syrk_n * empty, 1e-9)
     achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
     total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
     executed_flops = flops['cov'] + dense_inverse_flops + flops['precondition']
+    traffic = read_traffic() if name == 'c3' else None
     result = {
-        'metric': 'ms per K-FAC step, ResNet-50 bs32/GPU; cov+inv TFLOP/s vs FP32 MFMA peak',
+        'metric': METRIC,
         'value': round(ms_per_step, 4),
         'unit': 'ms/step',
         'n_gpus': 1,
         'steps': args.steps,
         'warmup': args.warmup,
         'ms_per_step': round(ms_per_step, 4),
+        'ms_per_step_median': round(ms_median, 4),
         'higher_is_better': False,
         'scaling': 'weak',
         'vs_baseline': None,
         'dtype': 'f32',
         'data': 'synthetic',
-        'config': {'workload': 'ResNet-50 v1 (bias, 1000-way) K-FAC step, batch 32 @224: 161 factors, '
-                               'cov + damped Cholesky inverse + precondition',
-                   'batch': BATCH, 'factors': len(W.all_factor_dims(layers)), 'damping': DAMPING,
-                   'hip_graph': not args.no_graph,
-            'lanes': args.lanes,
-                   'bn_inverse': 'woodbury rank-32 ({} blocks)'.format(len(lowrank)) if lowrank else 'dense'},
+        'config': {'workload': cfg['workload'], 'name': name, 'batch': batch,
+                   'factors': len(W.all_factor_dims(layers)), 'damping': cfg['damping'], 'acc_iters': acc_iters,
+                   'hip_graph': not args.no_graph, 'lanes': args.lanes,
+                   'bn_inverse': 'woodbury rank-{} ({} blocks)'.format(batch, len(lowrank)) if lowrank else 'dense'},
         # rates use the flops actually executed; the *_reference_work entries divide the work of the
-        # reference's algorithm (all 161 factors inverted densely) by the same times
+        # reference's algorithm (every factor inverted densely) by the same times
         'tflops': {
             'step': round(executed_flops / ms_per_step / 1e9, 2),
             'cov_inv': round((flops['cov'] + dense_inverse_flops) / ((phase_ms['cov'] + phase_ms['inverse'])) / 1e9, 2),
@@ -262,11 +379,11 @@ def run_gpu(args):
         'phase_ms': {k: round(v, 3) for k, v in phase_ms.items()},
         'gflop': dict({k: round(v / 1e9, 1) for k, v in flops.items()},
                       inverse_executed=round(dense_inverse_flops / 1e9, 1)),
-        'kernel_ms': {k: {'launches': n, 'total_ms': round(ms, 3)} for k, (n, ms) in fam.items()},
+        'kernel_ms': {k: {'launches': n, 'total_ms': round(ms - n * empty, 3)} for k, (n, ms) in fam.items() if n},
         'inverse_info_nonzero': info_bad,
         'wire_format': wire_stats,
         'roofline': {
-            'kernel': 'syrk_kernel (covariance, all loaders)',
+            'kernel': 'covariance SYRK family (syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
             'bound': 'mfma',
             'achieved': round(achieved, 2),
             'peak': FP32_MFMA_PEAK_TFLOPS,
@@ -275,13 +392,99 @@ def run_gpu(args):
             'launches': syrk_n,
             'avg_launch_ms': round(syrk_ms / max(syrk_n, 1), 4),
             'avg_launch_ms_with_event_bracket': round(syrk_raw_ms / max(syrk_n, 1), 4),
-            'event_bracket_ms': round(bracket_ms, 4),
-            'timed': 'launches on one stream (--lanes 0 for this pass), HIP events around each launch, empty bracket subtracted',
-            'traffic': SYRK_HBM_BYTES_PER_LAUNCH,
+            'event_bracket_ms': round(empty, 4),
+            'timed': 'launches on one stream (--lanes 0 for this pass), HIP events around each launch, '
+                     'empty bracket subtracted',
+            'traffic': traffic,
             'traffic_unit': 'bytes/launch',
         },
     }
-    return result, layers
+    if name == 'c3' and lowrank and not args.no_dense_field:
+        # the reference's algorithm inverts the batch-norm blocks densely as well: the same step with
+        # the Woodbury shortcut switched off, as a second figure
+        opt.bn_lowrank_inverse = False
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        run_dense = step if args.no_graph else capture(step)
+        dense_ms, dense_median = timed_steps(run_dense, max(args.steps // 2, 5))
+        inv_dense = timed(inv_phase if args.no_graph else capture(inv_phase))
+        result['dense_bn_inverse'] = {
+            'ms_per_step': round(dense_ms, 4), 'ms_per_step_median': round(dense_median, 4),
+            'inverse_ms': round(inv_dense, 3),
+            'inverse_tflops': round(flops['inverse'] / inv_dense / 1e9, 2),
+            'step_tflops': round(total_flops / dense_ms / 1e9, 2)}
+    return result
+
+
+def inverse_dims():
+    """The 161 factor sizes of ResNet-50 with the 3x3 no-bias stem of the reference's own model
+    file (27 instead of 148): the stated range 27^2 .. 4609^2."""
+    from chainerkfac_amd import workloads as W
+    dims = W.all_factor_dims(W.resnet50_v1())
+    dims[dims.index(148)] = 27
+    return dims
+
+
+def run_inverse_config(args, name, cfg):
+    """c4: damped Cholesky inverse of 161 SPD matrices."""
+    import torch
+    from chainerkfac_amd import _lib, ops
+    lib = _lib.load()
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(4)
+    dims = inverse_dims()
+    mats = []
+    for d in dims:
+        X = torch.randn(2 * d, d, device=dev, generator=gen)
+        mats.append(X.T @ X / (2 * d) + 1e-3 * torch.eye(d, device=dev))
+        del X
+    outs = [torch.empty_like(m) for m in mats]
+    info = torch.zeros(len(mats), dtype=torch.int32, device=dev)
+
+    def step():
+        ops.spd_inverse_batched(mats, outs=outs, info=info)
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    run = step if args.no_graph else capture(step)
+    ms_per_step, ms_median = timed_steps(run, args.steps)
+    _lib.check(lib.kfac_timing_enable(1))
+    step()
+    torch.cuda.synchronize()
+    fam = family_times(lib)
+    _lib.check(lib.kfac_timing_enable(0))
+    empty = bracket_ms()
+    worst = 0.0
+    seen = set()
+    for d, M, inv in zip(dims, mats, outs):
+        if d in seen:
+            continue
+        seen.add(d)
+        resid = float((M.double() @ inv.double() - torch.eye(d, device=dev, dtype=torch.float64)).norm()) / d ** 0.5
+        worst = max(worst, resid)
+    flop = float(sum(d ** 3 for d in dims))
+    achieved = flop / ms_per_step / 1e9
+    return {
+        'metric': METRIC, 'value': round(ms_per_step, 4), 'unit': 'ms/step', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4), 'ms_per_step_median': round(ms_median, 4),
+        'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': cfg['workload'], 'name': name, 'factors': len(dims), 'hip_graph': not args.no_graph},
+        'tflops': {'inverse': round(achieved, 2)},
+        'gflop': {'inverse': round(flop / 1e9, 1)},
+        'kernel_ms': {k: {'launches': n, 'total_ms': round(ms - n * empty, 3)} for k, (n, ms) in fam.items() if n},
+        'inverse_info_nonzero': int((info != 0).sum().item()),
+        'max_residual': worst,      # max over sizes of ||M M^-1 - I||_F / sqrt(d); the bound is 1e-3
+        'roofline': {
+            'kernel': 'batched inverse (copy_in, step, panel, update, lauum kernels)', 'bound': 'mfma',
+            'achieved': round(achieved, 2), 'peak': FP32_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
+            'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+            'timed': 'd^3 flop per matrix over the wall time of the whole batched call (its kernels overlap on two '
+                     'streams, so their durations do not add up)',
+            'traffic': None},
+    }, dims
 
 
 def write_per_layer(path, layers):
@@ -294,16 +497,6 @@ def write_per_layer(path, layers):
     from chainerkfac_amd import workloads as W
     lib = _lib.load()
     dev = torch.device('cuda:0')
-
-    def bracket_ms():
-        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(100)]
-        torch.cuda.synchronize()
-        for e0, e1 in pairs:
-            e0.record()
-            e1.record()
-        torch.cuda.synchronize()
-        return sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[50]
-
     empty = bracket_ms()
 
     def syrk_ms(fn, iters=10):
@@ -364,78 +557,145 @@ def write_per_layer(path, layers):
                 desc, count, fac, d, M, gf, us, tf, ai, cap, frac))
 
 
-def run_cpu_baseline(layers, budget_s=20.0):
-    """The NumPy oracle (the restatement of the reference's --no_cuda arithmetic)
-    on a bounded sample of the workload's layers, scaled to the whole step by
-    algorithmic FLOPs."""
+def _cpu_threads():
+    try:
+        from threadpoolctl import threadpool_info
+        return int(max([p.get('num_threads', 1) for p in threadpool_info()] or [1]))
+    except Exception:
+        return os.cpu_count()
+
+
+def _cpu_layer(O, rng, layer, batch, damping):
+    """One layer through the NumPy oracle (cov + damped inverse + precondition); seconds."""
+    import numpy as np
+    from chainerkfac_amd import workloads as W
+    if layer['kind'] == 'conv':
+        ho = W.conv_out(layer['h'], layer['k'], layer['s'], layer['p'])
+        x = rng.standard_normal((batch, layer['c_in'], layer['h'], layer['w']), dtype=np.float32)
+        gy = rng.standard_normal((batch, layer['c_out'], ho, ho), dtype=np.float32) / (batch * ho)
+        gW = rng.standard_normal((layer['c_out'], layer['c_in'], layer['k'], layer['k']), dtype=np.float32)
+        gb = rng.standard_normal(layer['c_out'], dtype=np.float32) if layer['bias'] else None
+        t0 = time.perf_counter()
+        A = O.conv_A(x, layer['k'], layer['s'], layer['p'], layer['bias'])
+        G = O.conv_G(gy)
+    elif layer['kind'] == 'linear':
+        x = rng.standard_normal((batch, layer['d_in']), dtype=np.float32)
+        gy = rng.standard_normal((batch, layer['d_out']), dtype=np.float32) / batch
+        gW = rng.standard_normal((layer['d_out'], layer['d_in']), dtype=np.float32)
+        gb = rng.standard_normal(layer['d_out'], dtype=np.float32) if layer['bias'] else None
+        t0 = time.perf_counter()
+        A = O.linear_A(x, layer['bias'])
+        G = O.linear_G(gy)
+    else:
+        x = rng.standard_normal((batch, layer['c'], layer['h'], layer['w']), dtype=np.float32)
+        gy = rng.standard_normal((batch, layer['c'], layer['h'], layer['w']), dtype=np.float32) / (batch * layer['h'])
+        gg = rng.standard_normal(layer['c'], dtype=np.float32)
+        gb = rng.standard_normal(layer['c'], dtype=np.float32)
+        t0 = time.perf_counter()
+        F = O.bn_F(x, gy, 2e-5)
+    if layer['kind'] == 'bn':
+        (dv,) = O.bn_diagvals(layer['c'], layer['c'], damping, STAB_COEFF)
+        (Finv,) = O.update_invs([F], [dv])
+        O.precondition_bn(Finv, gg, gb)
+    else:
+        dv, _ = O.connection_diagvals(A, G, damping)
+        Ainv, Ginv = O.update_invs([A, G], dv)
+        O.precondition_conn(Ainv, Ginv, gW, gb)
+    return time.perf_counter() - t0
+
+
+def run_cpu_baseline(name, cfg, budget_s=20.0):
+    """The NumPy oracle (the restatement of the reference's --no_cuda arithmetic) on a
+    bounded sample of the configuration's work, scaled to the whole step by algorithmic FLOPs."""
     import numpy as np
     from chainerkfac_amd import workloads as W
     from oracle import kfac_oracle as O
-    try:
-        from threadpoolctl import threadpool_info
-        threads = max([p.get('num_threads', 1) for p in threadpool_info()] or [1])
-    except Exception:
-        threads = os.cpu_count()
+    threads = _cpu_threads()
     rng = np.random.default_rng(3)
-    total = W.flops(layers, BATCH)
+    if name == 'c4':
+        dims = inverse_dims()
+        total_f = float(sum(d ** 3 for d in dims))
+        done_f, t_used, used = 0.0, 0.0, []
+        for d in sorted(set(dims)):
+            X = rng.standard_normal((2 * d, d), dtype=np.float32)
+            M = (X.T @ X / np.float32(2 * d) + np.float32(1e-3) * np.eye(d, dtype=np.float32)).astype(np.float32)
+            t0 = time.perf_counter()
+            O.inverse(M)
+            t_used += time.perf_counter() - t0
+            done_f += float(d) ** 3
+            used.append(d)
+            if t_used > budget_s:
+                break
+        return {'value': round(t_used * 1e3 * total_f / done_f, 1), 'unit': 'ms/step', 'cores': threads, 'kind': 'port',
+                'sample': 'NumPy oracle inverse (cholesky, inv, matmul) of one matrix of each size {} = {:.1f} of '
+                          '{:.1f} GFLOP in {:.1f} s, scaled by d^3'.format(used, done_f / 1e9, total_f / 1e9, t_used)}
+    layers, batch, acc_iters = cfg['layers'], cfg['batch'], cfg['acc_iters']
+    total = W.flops(layers, batch)
+    total['cov'] *= acc_iters
     total_f = sum(total.values())
-    # one bottleneck of every stage plus the FC (every kernel kind and every factor size class), in an
-    # order that puts the big stage-5 factors last, where the time budget cuts the sample off
-    sample = []
-    for prefix in ('res3/1/', 'res4/1/', 'fc', 'res2/1/', 'res5/1/', 'res4/2/', 'res5/2/', 'res3/2/'):
-        sample += [l for l in layers if l['name'].startswith(prefix) or l['name'] == prefix]
-    done_f = 0
-    names = []
-    t_used = 0.0
+    if name in ('c1', 'c2'):
+        sample = list(layers)                   # the whole step
+    else:
+        # one bottleneck of every stage plus the FC (every kernel kind and every factor size class), in an
+        # order that puts the big stage-5 factors last, where the time budget cuts the sample off
+        sample = []
+        for prefix in ('res3/1/', 'res4/1/', 'fc', 'res2/1/', 'res5/1/', 'res4/2/', 'res5/2/', 'res3/2/'):
+            sample += [l for l in layers if l['name'].startswith(prefix) or l['name'] == prefix]
+    done_f, t_used, names = 0.0, 0.0, []
     for layer in sample:
-        f = sum(W.flops([layer], BATCH).values())
-        t0 = time.perf_counter()
-        if layer['kind'] == 'conv':
-            ho = W.conv_out(layer['h'], layer['k'], layer['s'], layer['p'])
-            x = rng.standard_normal((BATCH, layer['c_in'], layer['h'], layer['w']), dtype=np.float32)
-            gy = rng.standard_normal((BATCH, layer['c_out'], ho, ho), dtype=np.float32) / (BATCH * ho)
-            gW = rng.standard_normal((layer['c_out'], layer['c_in'], layer['k'], layer['k']), dtype=np.float32)
-            gb = rng.standard_normal(layer['c_out'], dtype=np.float32) if layer['bias'] else None
-            t0 = time.perf_counter()
-            A = O.conv_A(x, layer['k'], layer['s'], layer['p'], layer['bias'])
-            G = O.conv_G(gy)
-        elif layer['kind'] == 'linear':
-            x = rng.standard_normal((BATCH, layer['d_in']), dtype=np.float32)
-            gy = rng.standard_normal((BATCH, layer['d_out']), dtype=np.float32) / BATCH
-            gW = rng.standard_normal((layer['d_out'], layer['d_in']), dtype=np.float32)
-            gb = rng.standard_normal(layer['d_out'], dtype=np.float32)
-            t0 = time.perf_counter()
-            A = O.linear_A(x, True)
-            G = O.linear_G(gy)
-        else:
-            x = rng.standard_normal((BATCH, layer['c'], layer['h'], layer['w']), dtype=np.float32)
-            gy = rng.standard_normal((BATCH, layer['c'], layer['h'], layer['w']), dtype=np.float32) / (BATCH * layer['h'])
-            gg = rng.standard_normal(layer['c'], dtype=np.float32)
-            gb = rng.standard_normal(layer['c'], dtype=np.float32)
-            t0 = time.perf_counter()
-            F = O.bn_F(x, gy, 2e-5)
-        if layer['kind'] == 'bn':
-            (dv,) = O.bn_diagvals(layer['c'], layer['c'], DAMPING, STAB_COEFF)
-            (Finv,) = O.update_invs([F], [dv])
-            O.precondition_bn(Finv, gg, gb)
-        else:
-            dv, _ = O.connection_diagvals(A, G, DAMPING)
-            Ainv, Ginv = O.update_invs([A, G], dv)
-            O.precondition_conn(Ainv, Ginv, gW, gb)
-        t_used += time.perf_counter() - t0
-        done_f += f
+        # (with accumulation the oracle repeats the covariance acc_iters times: one micro-batch is timed
+        # and counted, the scaling by FLOPs accounts for the rest)
+        t_used += _cpu_layer(O, rng, layer, batch, cfg['damping'])
+        done_f += sum(W.flops([layer], batch).values())
         names.append(layer['name'])
         if t_used > budget_s:
             break
-    est_ms = t_used * 1e3 * total_f / done_f
+    whole = len(names) == len(layers) and acc_iters == 1
     return {
-        'value': round(est_ms, 1),
-        'unit': 'ms/step',
-        'cores': int(threads),
-        'kind': 'port',
-        'sample': 'NumPy oracle (cov + damped inverse + precondition) on layers {} = {:.1f} of {:.1f} GFLOP '
-                  'in {:.1f} s, scaled by FLOPs'.format(','.join(names), done_f / 1e9, total_f / 1e9, t_used),
+        'value': round(t_used * 1e3 * (1.0 if whole else total_f / done_f), 1),
+        'unit': 'ms/step', 'cores': threads, 'kind': 'port',
+        'sample': ('NumPy oracle (cov + damped inverse + precondition), the whole step: {:.1f} s'.format(t_used)
+                   if whole else
+                   'NumPy oracle (cov + damped inverse + precondition) on layers {} = {:.1f} of {:.1f} GFLOP '
+                   'in {:.1f} s, scaled by FLOPs'.format(','.join(names), done_f / 1e9, total_f / 1e9, t_used)),
     }
+
+
+def summarize_traffic(fetch_dir, write_dir, out_path):
+    """Reads the per-dispatch FETCH_SIZE / WRITE_SIZE counters (KiB) that two
+    `rocprofv3 --pmc ... -- python3 bench.py --no-graph --lanes 0 --no-cpu --calibrate-copy --steps 1 --warmup 1`
+    runs wrote, scales each by what it reads for the 256 MiB calibration copy, and writes the
+    average HBM bytes per launch of the covariance SYRK family to ``out_path``."""
+    import csv
+    import glob
+
+    def load(d, counter):
+        rows = []
+        for f in glob.glob(os.path.join(d, '**', '*counter_collection.csv'), recursive=True):
+            for r in csv.DictReader(open(f)):
+                if r.get('Counter_Name') == counter:
+                    rows.append((r['Kernel_Name'], float(r['Counter_Value'])))
+        return rows
+
+    out = {}
+    total = 0.0
+    for d, counter, key in ((fetch_dir, 'FETCH_SIZE', 'fetch'), (write_dir, 'WRITE_SIZE', 'write')):
+        rows = load(d, counter)
+        syrk = [v for k, v in rows if 'syrk_' in k]
+        # the calibration copy is the largest elementwise launch of the run: 256 MiB each way
+        cal = [v for k, v in rows if 'elementwise_kernel' in k]
+        if not syrk or not cal:
+            raise SystemExit('no {} rows for the SYRK family or the calibration copy under {}'.format(counter, d))
+        scale = (256.0 * 1024.0) / max(cal)     # counter KiB -> true KiB
+        out[key + '_scale'] = round(scale, 4)
+        out[key + '_bytes_per_launch'] = sum(syrk) / len(syrk) * 1024.0 * scale
+        out['launches'] = len(syrk)
+        total += out[key + '_bytes_per_launch']
+    out['bytes_per_launch'] = total
+    with open(out_path, 'w') as f:
+        json.dump(out, f, indent=1)
+        f.write('\n')
+    print(json.dumps(out))
 
 
 def main():
@@ -443,13 +703,17 @@ def main():
     faulthandler.enable()   # a crash inside a native call still names the Python line it came from
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--config', default='c3', choices=['c1', 'c2', 'c3', 'c4', 'c5'],
+                    help='benchmark configuration (default: c3, the headline ResNet-50 batch-32 step)')
     ap.add_argument('--no-graph', action='store_true', help='launch every kernel from the host each step')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--dense-bn-inverse', action='store_true',
                     help='invert the batch-norm blocks with the dense Cholesky path as well (default: their '
                          'rank-32 Woodbury form, which yields the same dense inverse)')
+    ap.add_argument('--no-dense-field', action='store_true',
+                    help='skip the second measurement of c3 with all batch-norm blocks inverted densely')
     ap.add_argument('--lanes', type=int, default=3,
                     help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
     ap.add_argument('--per-layer', metavar='PATH', default=None,
@@ -458,15 +722,25 @@ def main():
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='first run one 256 MiB device-to-device elementwise copy (a kernel of known traffic, '
                          'the reference point for hardware byte counters collected under rocprofv3 --pmc)')
+    ap.add_argument('--summarize-traffic', nargs=2, metavar=('FETCH_DIR', 'WRITE_DIR'), default=None,
+                    help='no benchmark: turn the counter files of two rocprofv3 --pmc runs of this script into '
+                         'profiles/syrk_hbm_traffic.json (read back as roofline.traffic)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures the single-GPU K-FAC hot path: inter-GPU collectives are outside this '
                  'build, so --gpus must be 1 (got {})'.format(args.gpus))
-    result, layers = run_gpu(args)
-    if args.per_layer:
-        write_per_layer(args.per_layer, layers)
+    if args.summarize_traffic:
+        summarize_traffic(args.summarize_traffic[0], args.summarize_traffic[1], TRAFFIC_FILE)
+        return
+    cfg = configs()[args.config]
+    if args.config == 'c4':
+        result, _ = run_inverse_config(args, args.config, cfg)
+    else:
+        result = run_step_config(args, args.config, cfg)
+        if args.per_layer:
+            write_per_layer(args.per_layer, cfg['layers'])
     if not args.no_cpu:
-        result['cpu_baseline'] = run_cpu_baseline(layers)
+        result['cpu_baseline'] = run_cpu_baseline(args.config, cfg)
     print(json.dumps(result))
 
 

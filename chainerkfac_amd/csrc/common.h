@@ -47,10 +47,23 @@ class DevTable {
   ~DevTable() {
     if (dev_) (void)hipFree(dev_);
   }
+  bool matches(const void *host, size_t bytes) const {
+    return bytes == shadow_.size() && dev_ &&
+           (bytes == 0 || memcmp(host, shadow_.data(), bytes) == 0);
+  }
   int set(const void *host, size_t bytes, hipStream_t stream) {
-    if (bytes == shadow_.size() && dev_ &&
-        (bytes == 0 || memcmp(host, shadow_.data(), bytes) == 0))
-      return KFAC_OK;
+    if (matches(host, bytes)) return KFAC_OK;
+    // an upload waits for the stream and copies synchronously: impossible while the
+    // stream is being captured into a graph (and it would invalidate the capture)
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) != hipSuccess) {
+      (void)hipGetLastError();
+      cs = hipStreamCaptureStatusActive;
+    }
+    if (cs != hipStreamCaptureStatusNone)
+      return ::kfac::fail(KFAC_EINVAL,
+                          "a device table would have to be uploaded during stream capture: call once "
+                          "with the same arguments before capturing");
     KFAC_HIP_CHECK(hipStreamSynchronize(stream));
     if (bytes > capacity_) {
       if (dev_) KFAC_HIP_CHECK(hipFree(dev_));
@@ -73,6 +86,37 @@ class DevTable {
   void *dev_ = nullptr;
   size_t capacity_ = 0;
   std::vector<char> shadow_;
+};
+
+// A few device copies of a table whose contents alternate between a small number
+// of versions (e.g. the pointer / scale table of a grouped launch with beta = 0
+// on the first micro-batch and beta = 1 afterwards): a version that is resident
+// is used as it is, a new one replaces the least recently used copy.  A HIP
+// graph captured over a call keeps replaying against the copy it saw.
+class DevTableRing {
+ public:
+  static constexpr int kSlots = 4;
+  int set(const void *host, size_t bytes, hipStream_t stream, const void **dev_out) {
+    ++clock_;
+    int lru = 0;
+    for (int i = 0; i < kSlots; ++i) {
+      if (slots_[i].matches(host, bytes)) {
+        stamp_[i] = clock_;
+        *dev_out = slots_[i].as<const void>();
+        return KFAC_OK;
+      }
+      if (stamp_[i] < stamp_[lru]) lru = i;
+    }
+    if (int rc = slots_[lru].set(host, bytes, stream)) return rc;
+    stamp_[lru] = clock_;
+    *dev_out = slots_[lru].as<const void>();
+    return KFAC_OK;
+  }
+
+ private:
+  DevTable slots_[kSlots];
+  unsigned long long stamp_[kSlots] = {};
+  unsigned long long clock_ = 0;
 };
 
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }

@@ -1131,7 +1131,8 @@ struct kfac_cov_group {
   size_t ws_floats = 0;
   int task0[kGroupKinds] = {}, ntask[kGroupKinds] = {};
   int ftask0 = 0, nftask = 0;
-  kfac::DevTable d_items, d_dyn, d_tasks;
+  kfac::DevTable d_items, d_tasks;
+  kfac::DevTableRing d_dyn;
 };
 
 extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac_cov_group_t *out) {
@@ -1283,10 +1284,12 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
     group->dyn[i] = GroupItemDyn{inputs[i], outputs[i], alpha[i], beta[i]};
   }
   hipStream_t s = kfac::as_stream(stream);
-  if (int rc = group->d_dyn.set(group->dyn.data(), sizeof(GroupItemDyn) * (size_t)count, s)) return rc;
+  const void *dyn_dev = nullptr;
+  if (int rc = group->d_dyn.set(group->dyn.data(), sizeof(GroupItemDyn) * (size_t)count, s, &dyn_dev))
+    return rc;
   float *base = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
   const GroupItemStatic *st = group->d_items.as<const GroupItemStatic>();
-  const GroupItemDyn *dy = group->d_dyn.as<const GroupItemDyn>();
+  const GroupItemDyn *dy = static_cast<const GroupItemDyn *>(dyn_dev);
   const int2 *tasks = group->d_tasks.as<const int2>();
   using Kern = void (*)(const GroupItemStatic *, const GroupItemDyn *, const int2 *, float *);
   static const Kern kerns[kGroupKinds] = {

@@ -552,7 +552,8 @@ struct kfac_precond_group {
   size_t ws_floats = 0;
   int task0[2][kPreKinds] = {}, ntask[2][kPreKinds] = {};
   int ftask0[2] = {0, 0}, nftask[2] = {0, 0};
-  kfac::DevTable d_items, d_dyn, d_tasks;
+  kfac::DevTable d_items, d_tasks;
+  kfac::DevTableRing d_dyn;
 };
 
 extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int32_t *dA,
@@ -695,10 +696,11 @@ extern "C" int kfac_precond_group_run_f32(kfac_precond_group_t group, const floa
     group->dyn[i] = PreDyn{Ginv[i], Ainv[i], gradW[i], gradb[i], kfW[i], kfb[i]};
   }
   hipStream_t s = kfac::as_stream(stream);
-  if (int rc = group->d_dyn.set(group->dyn.data(), sizeof(PreDyn) * (size_t)count, s)) return rc;
+  const void *dyn_dev = nullptr;
+  if (int rc = group->d_dyn.set(group->dyn.data(), sizeof(PreDyn) * (size_t)count, s, &dyn_dev)) return rc;
   float *base = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
   const PreStatic *st = group->d_items.as<const PreStatic>();
-  const PreDyn *dy = group->d_dyn.as<const PreDyn>();
+  const PreDyn *dy = static_cast<const PreDyn *>(dyn_dev);
   const int2 *tasks = group->d_tasks.as<const int2>();
   using Kern = void (*)(const PreStatic *, const PreDyn *, const int2 *, float *);
   static const Kern kerns[2][kPreKinds] = {

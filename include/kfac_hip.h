@@ -135,7 +135,14 @@ int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, float alpha,
  * then read with 16-byte loads where its strides allow).  The results are those
  * of the single calls up to the order of the floating-point sums.  Replaces the
  * per-layer loop over compute_A / compute_G / compute_F for layers too small to
- * fill the GPU one at a time; no single call of the reference corresponds. */
+ * fill the GPU one at a time; no single call of the reference corresponds.
+ * The pointers and scales of a call travel to the GPU as a table; the group
+ * keeps the last four distinct tables resident, so calls that alternate between
+ * a few argument sets (beta = 0 on the first micro-batch, 1 afterwards) upload
+ * nothing.  Under stream capture only a resident table can be used (call once
+ * with the same arguments before capturing; KFAC_EINVAL otherwise), and a
+ * captured graph keeps reading the table it was captured with: do not push it
+ * out by running the same group with four other argument sets. */
 #define KFAC_COV_LINEAR 0
 #define KFAC_COV_SLAB 1
 typedef struct kfac_cov_item {

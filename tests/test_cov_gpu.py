@@ -204,6 +204,54 @@ def test_grouped_launch_matches_the_single_calls():
     np.testing.assert_allclose(outs[0].cpu().numpy(), O.conv_G(gy) * (0.25 * 14 * 14 / 4), rtol=1e-4, atol=1e-4)
 
 
+def test_grouped_launch_alternating_arguments_under_capture():
+    """Accumulation calls one group with beta = 0, then beta = 1: both argument tables stay
+    resident, so a graph can be captured over the pair after one eager pass, and every
+    replay gives the eager result.  An argument set that is not resident is refused inside a
+    capture instead of silently uploading."""
+    from chainerkfac_amd import _lib, ops
+    r = np.random.default_rng(23)
+    xs = [torch.from_numpy(r.standard_normal(s).astype(np.float32)).cuda()
+          for s in [(4, 64, 14, 14), (16, 101)]]
+    items = [(ops.COV_SLAB, 4, 64, 14, 14, 1, 1, 0, 1), (ops.COV_LINEAR, 16, 101, 1, 1, 1, 1, 1, 1)]
+    outs = [torch.empty(64, 64, device='cuda'), torch.empty(102, 102, device='cuda')]
+    group = ops.CovGroup(items)
+
+    def pair():
+        group.run(xs, outs, [0.5, 0.25], [0.0, 0.0])
+        group.run(xs, outs, [0.5, 0.25], [1.0, 1.0])
+
+    pair()
+    torch.cuda.synchronize()
+    want = [o.clone() for o in outs]
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            pair()
+    for _ in range(3):
+        for o in outs:
+            o.fill_(float('nan'))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, w in zip(outs, want):
+            assert torch.equal(o, w)
+    P = xs[1].cpu().numpy().astype(np.float64)
+    P = np.concatenate([P, np.ones((16, 1))], axis=1)
+    np.testing.assert_allclose(outs[1].cpu().numpy(), 0.5 * (P.T @ P), rtol=1e-4, atol=1e-4)
+    # a table the group has not seen cannot be uploaded while capturing
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph2, stream=side):
+            with pytest.raises(_lib.KfacHipError):
+                group.run(xs, outs, [0.125, 0.25], [0.0, 0.0])
+            group.run(xs, outs, [0.5, 0.25], [0.0, 0.0])
+    graph2.replay()
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(outs[1].cpu().numpy(), 0.25 * (P.T @ P), rtol=1e-4, atol=1e-4)
+
+
 def test_grouped_launch_argument_checks():
     from chainerkfac_amd import _lib, ops
     with pytest.raises(_lib.KfacHipError):
