@@ -243,10 +243,12 @@ def run_step_config(args, name, cfg):
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(3)
     if args.calibrate_copy:
+        from chainerkfac_amd import _lib
         src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
-        torch.add(src, 0.0, out=dst)   # reads 256 MiB, writes 256 MiB
+        # stream_copy_kernel: reads 256 MiB, writes 256 MiB
+        _lib.check(_lib.load().kfac_stream_copy_f32(dst.data_ptr(), src.data_ptr(), src.numel(), None))
         torch.cuda.synchronize()
         del src, dst
     layers, batch, acc_iters = cfg['layers'], cfg['batch'], cfg['acc_iters']
@@ -661,40 +663,206 @@ def run_cpu_baseline(name, cfg, budget_s=20.0):
     }
 
 
-def summarize_traffic(fetch_dir, write_dir, out_path):
-    """Reads the per-dispatch FETCH_SIZE / WRITE_SIZE counters (KiB) that two
-    `rocprofv3 --pmc ... -- python3 bench.py --no-graph --lanes 0 --no-cpu --calibrate-copy --steps 1 --warmup 1`
-    runs wrote, scales each by what it reads for the 256 MiB calibration copy, and writes the
-    average HBM bytes per launch of the covariance SYRK family to ``out_path``."""
+def _short_kernel_name(name):
+    for junk in ('void ', '(anonymous namespace)::', 'kfac::mma::', 'kfac::'):
+        name = name.replace(junk, '')
+    depth, out = 0, []
+    for ch in name:          # drop the argument list, keep the template arguments
+        if ch == '(' and depth == 0:
+            break
+        depth += ch == '<'
+        depth -= ch == '>'
+        out.append(ch)
+    name = ''.join(out)
+    return name if len(name) <= 90 else name[:87] + '...'
+
+
+def _csv_rows(directory, suffix):
     import csv
     import glob
+    for f in sorted(glob.glob(os.path.join(directory, '**', '*' + suffix), recursive=True)):
+        with open(f) as fh:
+            for r in csv.DictReader(fh):
+                yield r
 
+
+KERNEL_FAMILIES = (
+    ('covariance SYRK family', ('syrk_',)),
+    ('split-K finish of the covariances', ('finish_', 'reduce_kernel')),
+    ('inverse tile kernels', ('step_kernel', 'update_kernel', 'lauum_kernel', 'panel_kernel', 'copy_in', 'copy_out',
+                              'trtri', 'potrf', 'small_inverse')),
+    ('preconditioning GEMMs', ('gemm_',)),
+    ('batch-norm statistics', ('bn_',)),
+    ('pack / unpack / copy', ('pack_kernel', 'unpack_kernel', 'stream_copy')),
+)
+
+
+def _family_of(name):
+    for fam, keys in KERNEL_FAMILIES:
+        if any(k in name for k in keys):
+            return fam
+    return None
+
+
+def _own_kernel(name):
+    return not name.startswith('at::') and 'at::native' not in name and 'hiprand' not in name
+
+
+def summarize_kernel_trace(trace_dir, out_path, command):
+    """Markdown summary (per kernel and per kernel family) of the kernel trace a
+    `rocprofv3 --kernel-trace --stats` run of this script wrote under ``trace_dir``."""
+    agg = {}
+    for r in _csv_rows(trace_dir, 'kernel_trace.csv'):
+        name = _short_kernel_name(r['Kernel_Name'])
+        dur = int(r['End_Timestamp']) - int(r['Start_Timestamp'])
+        a = agg.setdefault(name, [0, 0, 1 << 62, 0])
+        a[0] += 1
+        a[1] += dur
+        a[2] = min(a[2], dur)
+        a[3] = max(a[3], dur)
+    if not agg:
+        raise SystemExit('no kernel_trace.csv under ' + trace_dir)
+    total = float(sum(a[1] for a in agg.values()))
+    lines = ['# Kernel time by kernel: ' + os.path.basename(out_path)[:-3].replace('_', ' '), '',
+             'Command (one MI355X, repository root; raw output stays outside the repository):', '', '```',
+             command, '```', '',
+             'All launches of the run are counted (warm-up, timed steps, the phase split and the pass that times '
+             'every launch with HIP events), so "launches" is a multiple of the per-step count.', '',
+             '| family | launches | total ms | avg us / launch | share of GPU time |', '|---|---:|---:|---:|---:|']
+    fam = {}
+    for name, a in agg.items():
+        f = _family_of(name)
+        if f:
+            t = fam.setdefault(f, [0, 0])
+            t[0] += a[0]
+            t[1] += a[1]
+    for f, _ in KERNEL_FAMILIES:
+        if f in fam:
+            n, t = fam[f]
+            lines.append('| {} | {} | {:.3f} | {:.1f} | {:.1f} % |'.format(f, n, t / 1e6, t / n / 1e3, 100 * t / total))
+    lines += ['', '| kernel | launches | total ms | avg us | min us | max us | share |', '|---|---:|---:|---:|---:|---:|---:|']
+    for name, a in sorted(agg.items(), key=lambda kv: -kv[1][1])[:40]:
+        if a[1] / total < 0.001:
+            break
+        lines.append('| `{}` | {} | {:.3f} | {:.1f} | {:.1f} | {:.1f} | {:.1f} % |'.format(
+            name, a[0], a[1] / 1e6, a[1] / a[0] / 1e3, a[2] / 1e3, a[3] / 1e3, 100 * a[1] / total))
+    with open(out_path, 'w') as f:
+        f.write('\n'.join(lines) + '\n')
+    print('\n'.join(lines[:22]))
+
+
+def summarize_mfma(pmc_dir, out_path, command):
+    """Matrix-pipe utilisation per kernel from a `rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES
+    GRBM_GUI_ACTIVE` run of this script.  SQ_VALU_MFMA_BUSY_CYCLES adds up, over the
+    chip's 1024 SIMDs, the cycles in which the SIMD's matrix pipe was busy;
+    GRBM_GUI_ACTIVE adds up the 8 XCDs' active cycles: busy fraction =
+    MFMA_BUSY / (GUI_ACTIVE / 8 * 1024)."""
+    disp = {}
+    for r in _csv_rows(pmc_dir, 'counter_collection.csv'):
+        d = disp.setdefault(r['Dispatch_Id'], {'name': _short_kernel_name(r['Kernel_Name'])})
+        d[r['Counter_Name']] = d.get(r['Counter_Name'], 0.0) + float(r['Counter_Value'])
+    agg = {}
+    for d in disp.values():
+        if 'SQ_VALU_MFMA_BUSY_CYCLES' not in d or 'GRBM_GUI_ACTIVE' not in d or not _own_kernel(d['name']):
+            continue
+        a = agg.setdefault(d['name'], [0, 0.0, 0.0])
+        a[0] += 1
+        a[1] += d['SQ_VALU_MFMA_BUSY_CYCLES']
+        a[2] += d['GRBM_GUI_ACTIVE']
+    if not agg:
+        raise SystemExit('no SQ_VALU_MFMA_BUSY_CYCLES / GRBM_GUI_ACTIVE rows under ' + pmc_dir)
+    lines = ['# FP32 matrix-pipe utilisation by kernel: ' + os.path.basename(out_path)[:-3].replace('_', ' '), '',
+             'Command (one MI355X, repository root; every kernel launched from the host on one stream so that each '
+             'dispatch has its own counter record):', '', '```', command, '```', '',
+             '`SQ_VALU_MFMA_BUSY_CYCLES` sums, over the 1024 SIMDs, the cycles in which a SIMD\'s matrix pipe was '
+             'busy; `GRBM_GUI_ACTIVE` sums the active cycles of the 8 XCDs.  busy = MFMA_BUSY / (GUI_ACTIVE / 8 x '
+             '1024): the share of all matrix-pipe cycles of the launch (ramp-up, tail and padding work included) '
+             'in which an MFMA was executing.  Only `v_mfma_f32_32x32x2_f32` is used, so busy x 157.3 TFLOP/s is '
+             'the rate of executed (padded) matrix work.', '',
+             '| family | launches | matrix pipe busy |', '|---|---:|---:|']
+    fam = {}
+    for name, a in agg.items():
+        f = _family_of(name)
+        if f:
+            t = fam.setdefault(f, [0, 0.0, 0.0])
+            for i in range(3):
+                t[i] += a[i]
+    for f, _ in KERNEL_FAMILIES:
+        if f in fam and fam[f][1] > 0:
+            n, busy, act = fam[f]
+            lines.append('| {} | {} | {:.1f} % |'.format(f, n, 100 * busy / (act / 8 * 1024)))
+    lines += ['', '| kernel | launches | active Mcycles / launch | matrix pipe busy |', '|---|---:|---:|---:|']
+    for name, a in sorted(agg.items(), key=lambda kv: -kv[1][2]):
+        if a[1] == 0:
+            continue
+        lines.append('| `{}` | {} | {:.3f} | {:.1f} % |'.format(name, a[0], a[2] / 8 / a[0] / 1e6,
+                                                              100 * a[1] / (a[2] / 8 * 1024)))
+    with open(out_path, 'w') as f:
+        f.write('\n'.join(lines) + '\n')
+    print('\n'.join(lines[12:40]))
+
+
+def summarize_traffic(fetch_dir, write_dir, out_path, command):
+    """Reads the per-dispatch FETCH_SIZE / WRITE_SIZE counters (KiB) of two
+    `rocprofv3 --pmc` runs of this script with --calibrate-copy, scales each by what it
+    reads for the 256 MiB calibration copy (stream_copy_kernel), and writes the average
+    HBM bytes per launch of the covariance SYRK family to ``out_path`` (JSON, read back as
+    roofline.traffic) and a per-kernel table next to it (markdown)."""
     def load(d, counter):
-        rows = []
-        for f in glob.glob(os.path.join(d, '**', '*counter_collection.csv'), recursive=True):
-            for r in csv.DictReader(open(f)):
-                if r.get('Counter_Name') == counter:
-                    rows.append((r['Kernel_Name'], float(r['Counter_Value'])))
-        return rows
+        rows = {}
+        for r in _csv_rows(d, 'counter_collection.csv'):
+            if r.get('Counter_Name') == counter:
+                key = (r['Dispatch_Id'], _short_kernel_name(r['Kernel_Name']))
+                rows[key] = rows.get(key, 0.0) + float(r['Counter_Value'])
+        return [(k[1], v) for k, v in sorted(rows.items(), key=lambda kv: int(kv[0][0]))]
 
     out = {}
     total = 0.0
+    per_kernel = {}
     for d, counter, key in ((fetch_dir, 'FETCH_SIZE', 'fetch'), (write_dir, 'WRITE_SIZE', 'write')):
         rows = load(d, counter)
         syrk = [v for k, v in rows if 'syrk_' in k]
-        # the calibration copy is the largest elementwise launch of the run: 256 MiB each way
-        cal = [v for k, v in rows if 'elementwise_kernel' in k]
+        cal = [v for k, v in rows if 'stream_copy_kernel' in k]
         if not syrk or not cal:
             raise SystemExit('no {} rows for the SYRK family or the calibration copy under {}'.format(counter, d))
-        scale = (256.0 * 1024.0) / max(cal)     # counter KiB -> true KiB
+        # the calibration copy is the run's first launch of the copy kernel
+        scale = (256.0 * 1024.0) / cal[0]       # counter KiB -> true KiB
+        out[key + '_counter_for_256MiB_copy'] = cal[0]
         out[key + '_scale'] = round(scale, 4)
         out[key + '_bytes_per_launch'] = sum(syrk) / len(syrk) * 1024.0 * scale
         out['launches'] = len(syrk)
         total += out[key + '_bytes_per_launch']
+        for k, v in rows:
+            if _own_kernel(k):
+                a = per_kernel.setdefault(k, {'fetch': [0, 0.0], 'write': [0, 0.0]})[key]
+                a[0] += 1
+                a[1] += v * scale
     out['bytes_per_launch'] = total
     with open(out_path, 'w') as f:
         json.dump(out, f, indent=1)
         f.write('\n')
+    lines = ['# HBM traffic per launch (hardware counters)', '',
+             'Two counter runs on one MI355X from the repository root (raw output stays outside the repository); '
+             'every kernel is launched from the host on one stream so that each dispatch has its own counter record, '
+             'and `--calibrate-copy` first runs `stream_copy_kernel` over 256 MiB (reads 256 MiB, writes 256 MiB):',
+             '', '```', command, '```', '',
+             'Calibration: for the 262144 KiB copy FETCH_SIZE reads {:.1f} and WRITE_SIZE reads {:.1f}, so the '
+             'counters are scaled by {:.3f} and {:.3f} to get KiB.'.format(
+                 out['fetch_counter_for_256MiB_copy'], out['write_counter_for_256MiB_copy'],
+                 out['fetch_scale'], out['write_scale']), '',
+             'Covariance SYRK family (`syrk_*`, {} launches in the run): **fetch {:.1f} MiB + write {:.1f} MiB = '
+             '{:.1f} MiB per launch** ({:.4g} bytes, the `roofline.traffic` of bench.py).'.format(
+                 out['launches'], out['fetch_bytes_per_launch'] / 2 ** 20, out['write_bytes_per_launch'] / 2 ** 20,
+                 total / 2 ** 20, total), '',
+             '| kernel | launches | fetch MiB/launch | write MiB/launch |', '|---|---:|---:|---:|']
+    def tot(v):
+        return v['fetch'][1] + v['write'][1]
+    for k, v in sorted(per_kernel.items(), key=lambda kv: -tot(kv[1]))[:24]:
+        n = max(v['fetch'][0], v['write'][0], 1)
+        lines.append('| `{}` | {} | {:.2f} | {:.2f} |'.format(k, n, v['fetch'][1] / n / 1024, v['write'][1] / n / 1024))
+    md = out_path[:-5] + '.md'
+    with open(md, 'w') as f:
+        f.write('\n'.join(lines) + '\n')
     print(json.dumps(out))
 
 
@@ -724,13 +892,26 @@ def main():
                          'the reference point for hardware byte counters collected under rocprofv3 --pmc)')
     ap.add_argument('--summarize-traffic', nargs=2, metavar=('FETCH_DIR', 'WRITE_DIR'), default=None,
                     help='no benchmark: turn the counter files of two rocprofv3 --pmc runs of this script into '
-                         'profiles/syrk_hbm_traffic.json (read back as roofline.traffic)')
+                         'profiles/syrk_hbm_traffic.json (read back as roofline.traffic) and a table beside it')
+    ap.add_argument('--summarize-trace', nargs=2, metavar=('TRACE_DIR', 'OUT_MD'), default=None,
+                    help='no benchmark: per-kernel / per-family table of a rocprofv3 --kernel-trace run')
+    ap.add_argument('--summarize-mfma', nargs=2, metavar=('PMC_DIR', 'OUT_MD'), default=None,
+                    help='no benchmark: matrix-pipe utilisation per kernel from a rocprofv3 --pmc '
+                         'SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE run')
+    ap.add_argument('--profiled-command', default='(not recorded)',
+                    help='the profiling command line, copied into the summary that --summarize-* writes')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures the single-GPU K-FAC hot path: inter-GPU collectives are outside this '
                  'build, so --gpus must be 1 (got {})'.format(args.gpus))
     if args.summarize_traffic:
-        summarize_traffic(args.summarize_traffic[0], args.summarize_traffic[1], TRAFFIC_FILE)
+        summarize_traffic(args.summarize_traffic[0], args.summarize_traffic[1], TRAFFIC_FILE, args.profiled_command)
+        return
+    if args.summarize_trace:
+        summarize_kernel_trace(args.summarize_trace[0], args.summarize_trace[1], args.profiled_command)
+        return
+    if args.summarize_mfma:
+        summarize_mfma(args.summarize_mfma[0], args.summarize_mfma[1], args.profiled_command)
         return
     cfg = configs()[args.config]
     if args.config == 'c4':

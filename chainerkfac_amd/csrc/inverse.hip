@@ -22,17 +22,19 @@
 // just before it is factored, K up to (kGroup-1)*NB), and after a group every
 // column to its right receives the whole group at once (K = kGroup*NB), which
 // reads and writes each trailing tile once per group instead of once per
-// column.  Per block column k, two dependent launches:
+// column.  Per block column k, three launches:
 //
-//   step(k)    one workgroup per matrix gives the diagonal tile the products it
+//   diag(k)    one workgroup per matrix gives the diagonal tile the products it
 //              is still owed, then does its Cholesky and U_kk = L_kk^-T inside
-//              LDS on 32x32 MFMA blocks; the other workgroups of the launch
-//              apply (*) to the rest of column k (inside a group: the group's
-//              earlier columns; on a group's first column: the previous group,
-//              for both columns of this group)
-//   panel(k)   M(x,k) = M(x,k) U_kk for x != k  (L(x,k) below, U(x,k) above)
+//              LDS on 32x32 MFMA blocks
+//   column(k)  beside diag(k), on a stream of its own: (*) for the rest of
+//              column k (inside a group: the group's earlier columns; on a
+//              group's first column: the previous group, for both columns of
+//              this group)
+//   panel(k)   after both: M(x,k) = M(x,k) U_kk for x != k  (L(x,k) below,
+//              U(x,k) above)
 //
-// and after a group's last column, on a second stream beside the next group's
+// and after a group's last column, on a further stream beside the next group's
 // sweep, rest(g): (*) for all tiles right of the next group.  A final launch
 // forms  out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T  (lauum) and writes the full
 // symmetric inverse.  Matrices of different sizes end their sweeps together (a
@@ -97,137 +99,188 @@ __device__ __forceinline__ float *tile_ptr(const InvTables &tb, int s, int I, in
   return tb.ws + tb.ws_off[s] + ((long long)I * tb.nt[s] + J) * (NB * NB);
 }
 
-// Operand loader of the shared main loop for a run of consecutive tiles of one
-// tile row: k-value k is column k % NB of tile k / NB.  A 128 x 32 panel is
-// 128 rows of 128 contiguous bytes inside one tile; no edge masks are needed
-// (the workspace is padded).
+// ---------------------------------------------------------------------------
+// The tile product  acc(128 x 128) += A(128 x K) B(128 x K)^T  of this file
+// ---------------------------------------------------------------------------
+// Operands are runs of consecutive workspace tiles (k-value k is column k % NB
+// of tile k / NB: 128 rows of 128 contiguous bytes per panel of KT k-values, no
+// edge masks, the workspace is padded) or one tile read as its transpose.
+//
+// Everything around the matrix instructions is kept off the vector ALU and
+// placed between them by hand: the products are short (K = 128 .. 512) and run
+// one or two workgroups per CU, so instructions that the compiler leaves in one
+// block (the LDS stores and the global loads of the next panels, 90 instructions
+// per pass with their address arithmetic) stall the matrix pipe with nothing
+// else to fill it.
+//   * global loads: wave-uniform base (scalar registers, advanced per pass) plus
+//     a per-lane 32-bit offset that never changes;
+//   * LDS: row-major panels with a row stride of KT + 4 floats, written and read
+//     16 bytes at a time.  v_mfma_f32_32x32x2_f32 takes two k-values per
+//     instruction, one from each half of the wave; which two does not matter as
+//     long as both operands agree, so the lanes of half h read the four k-values
+//     8g + 4h .. 8g + 4h + 3 of their row in one instruction and feed them to
+//     four consecutive MFMAs (k pairs {8g + j, 8g + 4 + j});
+//   * the LDS panels are double-buffered: one barrier per pass, and the stores
+//     and loads for the passes ahead are dealt out one per group of four MFMAs.
+// The global loads run PD passes ahead of the LDS stores (with less than two
+// passes of 64 k-values in flight, a third of the passes of a full GPU waited
+// 2-4 us for their operands, measured with time stamps).
 typedef float vfloat4 __attribute__((ext_vector_type(4)));   // register arrays of HIP's float4 struct can end up in scratch
 
-struct LoaderTile {
-  static constexpr bool kKRow = false;
-  struct Regs {
-    vfloat4 v[NB / 32];
-  };
-  const float *base;   // first tile of the run
-  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long) const {
-    const unsigned k = (unsigned)k0 + (threadIdx.x & 7) * 4;
-    const float *p = base + (size_t)(k / NB) * (NB * NB) + (k % NB) + (threadIdx.x >> 3) * NB;
-#pragma unroll
-    for (int i = 0; i < NB / 32; ++i) r.v[i] = *reinterpret_cast<const vfloat4 *>(p + 32 * i * NB);
-  }
-  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
-    const int kq = (threadIdx.x & 7) * 4;
-    const int rr = threadIdx.x >> 3;
-#pragma unroll
-    for (int i = 0; i < NB / 32; ++i) {
-      float *p = lds + (rr + 32 * i) * Panel<NB>::kRowKStride + kq;
-      p[0] = r.v[i].x;
-      p[1] = r.v[i].y;
-      p[2] = r.v[i].z;
-      p[3] = r.v[i].w;
-    }
-  }
-};
-
-// The same tile read as its transpose: operand row c, k-value q is element
-// (q, c).  Rows of the tile are contiguous in c, so the panel goes to LDS in the
-// k-major layout.
-struct LoaderTileT {
-  static constexpr bool kKRow = true;
-  struct Regs {
-    vfloat4 v[KT / 8];
-  };
-  const float *base;
-  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long) const {
-    const float *p = base + ((int)k0 + (threadIdx.x >> 5)) * NB + (threadIdx.x & 31) * 4;
-#pragma unroll
-    for (int i = 0; i < KT / 8; ++i) r.v[i] = *reinterpret_cast<const vfloat4 *>(p + 8 * i * NB);
-  }
-  __device__ __forceinline__ void store(const Regs &r, float *lds) const {
-    float *p = lds + (threadIdx.x >> 5) * Panel<NB>::kKRowStride + (threadIdx.x & 31) * 4;
-#pragma unroll
-    for (int i = 0; i < KT / 8; ++i)
-      *reinterpret_cast<vfloat4 *>(p + 8 * i * Panel<NB>::kKRowStride) = r.v[i];
-  }
-};
-
-// Main loop of the tile kernels: the shared loop with 64 k-values (two LDS
-// panels per operand) per pass instead of 32.  The products of this file are
-// short (K = 128 .. 512) and often one workgroup per CU, so what counts is how
-// many loads are in flight and how few barrier-to-barrier round trips a product
-// needs: K = 128 takes two passes instead of four.  K must be a multiple of 64.
-// lds: 4 panels (A0, A1, B0, B1) of Panel<NB>::kFloats.
-constexpr int kTileLdsFloats = 4 * Panel<NB>::kFloats;
+constexpr int RS = KT + 4;      // row stride of a row-major LDS panel (16-byte aligned rows; 8 lanes
+                                // of a 16-byte access then cover all 32 banks)
+constexpr int TS = NB + 4;      // k-row stride of a transposed LDS panel
+constexpr int PF = NB * RS;     // floats per LDS panel
+static_assert(KT * TS <= PF, "a transposed panel must fit the same buffer");
+constexpr int kTileLdsFloats = 4 * PF;   // A even / odd pass, B even / odd pass
 constexpr size_t kTileLdsBytes = kTileLdsFloats * sizeof(float);
 
-template <bool SAME, int D, class LA, class LB>
+// States that a pointer is the same in every lane, so that it is kept in scalar
+// registers (the compiler cannot always see this through the table lookups).
+__device__ __forceinline__ const float *wave_uniform(const float *p) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return reinterpret_cast<const float *>(((unsigned long long)hi << 32) | lo);
+}
+
+__device__ __forceinline__ vfloat4 gload16(const float *base, unsigned byte_off) {
+  return *(const KFAC_GLOBAL_AS vfloat4 *)((const KFAC_GLOBAL_AS char *)base + byte_off);
+}
+
+// k along the rows of a run of consecutive tiles
+struct OperandRows {
+  const float *base;   // first tile of the run
+  __device__ __forceinline__ static unsigned lane_offset() {
+    return (unsigned)(((threadIdx.x >> 3) * NB + (threadIdx.x & 7) * 4) * sizeof(float));
+  }
+  __device__ __forceinline__ void load(vfloat4 (&r)[4], unsigned off, int pass) const {
+    const int k = pass * KT;
+    const float *b = wave_uniform(base + (size_t)(k / NB) * (NB * NB) + (k % NB));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = gload16(b, off + i * (32 * NB * (unsigned)sizeof(float)));
+  }
+  __device__ __forceinline__ static void store1(const vfloat4 (&r)[4], int i, float *panel) {
+    float *p = panel + (threadIdx.x >> 3) * RS + (threadIdx.x & 7) * 4;
+    *reinterpret_cast<vfloat4 *>(p + 32 * i * RS) = r[i];
+  }
+  // the four k-values 8g + 4h .. + 3 of operand row `row`
+  __device__ __forceinline__ static vfloat4 fetch4(const float *panel, int row, int g, int h) {
+    return *reinterpret_cast<const vfloat4 *>(panel + row * RS + 8 * g + 4 * h);
+  }
+};
+
+// one tile read as its transpose: operand row c, k-value q is element (q, c)
+struct OperandCols {
+  const float *base;
+  __device__ __forceinline__ static unsigned lane_offset() {
+    return (unsigned)(((threadIdx.x >> 5) * NB + (threadIdx.x & 31) * 4) * sizeof(float));
+  }
+  __device__ __forceinline__ void load(vfloat4 (&r)[4], unsigned off, int pass) const {
+    const float *b = wave_uniform(base + pass * (KT * NB));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = gload16(b, off + i * (8 * NB * (unsigned)sizeof(float)));
+  }
+  __device__ __forceinline__ static void store1(const vfloat4 (&r)[4], int i, float *panel) {
+    float *p = panel + (threadIdx.x >> 5) * TS + (threadIdx.x & 31) * 4;
+    *reinterpret_cast<vfloat4 *>(p + 8 * i * TS) = r[i];
+  }
+  __device__ __forceinline__ static vfloat4 fetch4(const float *panel, int row, int g, int h) {
+    const float *p = panel + (8 * g + 4 * h) * TS + row;
+    vfloat4 v;
+    v.x = p[0];
+    v.y = p[TS];
+    v.z = p[2 * TS];
+    v.w = p[3 * TS];
+    return v;
+  }
+};
+
+// K must be a multiple of 4 * KT.  lds: kTileLdsFloats.  Ends with a barrier.
+template <bool SAME, int PD, class LA, class LB>
 __device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K, float *lds,
                                               floatx16 (&acc)[2][2]) {
-  constexpr int PF = Panel<NB>::kFloats;
-  // D: passes of 64 k-values held in registers ahead of the one in LDS.  With
-  // one, a third of the passes of a full GPU wait 2-4 us for their operands
-  // (measured with time stamps); two cover that where the registers allow it.
+  constexpr int UNROLL = PD % 2 == 0 ? PD : 2 * PD;   // register set and LDS buffer of a pass are static
   float *ldsA = lds, *ldsB = lds + 2 * PF;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane & 31, lk = lane >> 5;
-  typename LA::Regs ra[D][2];
-  typename LB::Regs rb[D][2];
+  const int P = K / KT;
+  const unsigned offA = LA::lane_offset(), offB = LB::lane_offset();
+  vfloat4 ra[PD][4];
+  vfloat4 rb[SAME ? 1 : PD][4];
 #pragma unroll
-  for (int d = 0; d < D; ++d) {
-    if (d * 2 * KT < K) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        la.load(ra[d][h], 0, d * 2 * KT + KT * h, K);
-        if (!SAME) lb.load(rb[d][h], 0, d * 2 * KT + KT * h, K);
-      }
+  for (int q = 0; q < PD; ++q) {
+    if (q < P) {
+      la.load(ra[q], offA, q);
+      if (!SAME) lb.load(rb[q], offB, q);
     }
   }
-  for (int kb = 0; kb < K; kb += D * 2 * KT) {
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const int k0 = kb + d * 2 * KT;
-      if (k0 < K) {
+  for (int i = 0; i < 4; ++i) {
+    LA::store1(ra[0], i, ldsA);
+    if (!SAME) LB::store1(rb[0], i, ldsB);
+  }
+  if (PD < P) {
+    la.load(ra[0], offA, PD);
+    if (!SAME) lb.load(rb[0], offB, PD);
+  }
+  __syncthreads();
+  for (int pb = 0; pb < P; pb += UNROLL) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        la.store(ra[d][h], ldsA + h * PF);
-        if (!SAME) lb.store(rb[d][h], ldsB + h * PF);
-      }
-      __syncthreads();
-      if (k0 + D * 2 * KT < K) {
+    for (int u = 0; u < UNROLL; ++u) {
+      const int p = pb + u;
+      if (UNROLL > 4 && p >= P) break;   // P is a multiple of 4
+      const float *pa = ldsA + (u & 1) * PF;
+      const float *pbuf = SAME ? pa : ldsB + (u & 1) * PF;
+      float *na = ldsA + ((u + 1) & 1) * PF, *nb = ldsB + ((u + 1) & 1) * PF;
+      const int r = (u + 1) % PD;            // register set of pass p + 1 (static once unrolled)
+      const bool ahead = p + 1 + PD < P;     // and its registers take pass p + 1 + PD
+      vfloat4 fa[2], fb[2];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          la.load(ra[d][h], 0, k0 + D * 2 * KT + KT * h, K);
-          if (!SAME) lb.load(rb[d][h], 0, k0 + D * 2 * KT + KT * h, K);
+      for (int im = 0; im < 2; ++im) fa[im] = LA::fetch4(pa, (wm * 2 + im) * 32 + lrow, 0, lk);
+#pragma unroll
+      for (int in = 0; in < 2; ++in)
+        fb[in] = SAME ? LA::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, 0, lk)
+                      : LB::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, 0, lk);
+#pragma unroll
+      for (int g = 0; g < KT / 8; ++g) {
+        vfloat4 ga[2], gb[2];
+        if (g + 1 < KT / 8) {
+#pragma unroll
+          for (int im = 0; im < 2; ++im) ga[im] = LA::fetch4(pa, (wm * 2 + im) * 32 + lrow, g + 1, lk);
+#pragma unroll
+          for (int in = 0; in < 2; ++in)
+            gb[in] = SAME ? LA::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, g + 1, lk)
+                          : LB::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, g + 1, lk);
         }
-      }
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const float *pa = ldsA + h * PF;
-        const float *pb = SAME ? pa : ldsB + h * PF;
-#pragma unroll
-        for (int kk = 0; kk < KT / 2; ++kk) {
-          float a[2], b[2];
-#pragma unroll
-          for (int im = 0; im < 2; ++im)
-            a[im] = fetch<NB, LA::kKRow>(pa, (wm * 2 + im) * 32 + lrow, 2 * kk + lk);
-#pragma unroll
-          for (int in = 0; in < 2; ++in) {
-            if (SAME)
-              b[in] = fetch<NB, LA::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
-            else
-              b[in] = fetch<NB, LB::kKRow>(pb, (wn * 2 + in) * 32 + lrow, 2 * kk + lk);
-          }
+        for (int j = 0; j < 4; ++j) {
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int im = 0; im < 2; ++im)
 #pragma unroll
             for (int in = 0; in < 2; ++in)
-              acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+              acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[im][j], fb[in][j], acc[im][in], 0, 0, 0);
+          // slot 4g + j of 16: one LDS store and one global load at most
+          // (the last pass stores what it holds as well, into the buffer nobody reads any more:
+          // cheaper than a branch per store)
+          const int slot = 4 * g + j;
+          if (slot >= 1 && slot < 5) LA::store1(ra[r], slot - 1, na);
+          if (!SAME && slot >= 5 && slot < 9) LB::store1(rb[SAME ? 0 : r], slot - 5, nb);
+        }
+        if (g == 1 && ahead) la.load(ra[r], offA, p + 1 + PD);       // after its stores (slots 1 .. 4)
+        if (!SAME && g == 2 && ahead) lb.load(rb[SAME ? 0 : r], offB, p + 1 + PD);   // slots 5 .. 8
+        if (g + 1 < KT / 8) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            fa[i] = ga[i];
+            fb[i] = gb[i];
+          }
         }
       }
       __syncthreads();
-      }
     }
   }
 }
@@ -303,8 +356,8 @@ __device__ __forceinline__ void diag_role(const InvTables &tb, int s, int k, int
   if (hi >= lo) {
     floatx16 acc[2][2];
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -tile[rr * NB + cc]; });
-    const LoaderTile la{tile_ptr(tb, s, k, lo)};
-    tile_mainloop<true, 1>(la, la, (hi - lo + 1) * NB, smem, acc);   // ends with a barrier
+    const OperandRows la{tile_ptr(tb, s, k, lo)};
+    tile_mainloop<true, 2>(la, la, (hi - lo + 1) * NB, smem, acc);   // ends with a barrier
     for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { S[rr * LS + cc] = -v; });
   } else {
     const int c4 = (threadIdx.x & 31) * 4, r0 = threadIdx.x >> 5;
@@ -406,7 +459,7 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int ste
   float *tile = tile_ptr(tb, s, x, k);
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
-  tile_mainloop<false, 1>(LoaderTile{tile}, LoaderTileT{tile_ptr(tb, s, k, k)}, NB, lds, acc);
+  tile_mainloop<false, 2>(OperandRows{tile}, OperandCols{tile_ptr(tb, s, k, k)}, NB, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { tile[rr * NB + cc] = v; });
 }
 
@@ -431,7 +484,7 @@ __device__ __forceinline__ void update_role(const InvTables &tb, int2 task, int 
     zero_acc<2, 2>(acc);
   else
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -C[rr * NB + cc]; });
-  const LoaderTile la{tile_ptr(tb, s, a, j_lo)}, lb{tile_ptr(tb, s, b, j_lo)};
+  const OperandRows la{tile_ptr(tb, s, a, j_lo)}, lb{tile_ptr(tb, s, b, j_lo)};
   if (a == b)
     tile_mainloop<true, D>(la, lb, K, lds, acc);
   else
@@ -448,35 +501,34 @@ __device__ __forceinline__ void local_range(const InvTables &tb, int s, int step
   k1 = step1 - shift;
 }
 
-// One launch per sweep step: workgroups [0, ndiag) factor the diagonal tile of
-// their matrix (after giving it the products of columns [step0, step1]), the
-// others apply the same columns to the tiles the next panel step reads.  The
-// diagonal workgroups come first in launch order, so the serial part starts at
-// once and the updates fill the rest of the GPU beside it.
-__global__ __launch_bounds__(THREADS, 2) void step_kernel(InvTables tb, int step, int ndiag,
-                                                          int task0, int step0, int step1) {
+// One workgroup per active matrix: the diagonal tile of sweep step `step`
+// (after it has received the products of columns [step0, step1]).  This is the
+// serial part of the sweep, and most of it is one wave's dependent chain of
+// vector instructions.  It runs at a third of its speed when its waves share
+// their SIMDs with those of a trailing update (measured: 20 us against 60-80 us
+// for the 128 x 128 factorisation), so the kernel asks for more LDS than fits
+// beside a workgroup of the trailing update (kDiagKernelLds): it waits for a CU
+// without one, at most the few microseconds until the next of them retires, and
+// keeps the following ones away from that CU while it runs.
+__global__ __launch_bounds__(THREADS, 2) void diag_kernel(InvTables tb, int step, int step0,
+                                                          int step1) {
   extern __shared__ float lds[];
-  if ((int)blockIdx.x < ndiag) {
-    const int s = blockIdx.x;
-    int k0, k1;
-    local_range(tb, s, step0, step1, k0, k1);
-    diag_role(tb, s, step - tb.shift[s], k0, k1, lds);
-  } else {
-    const int2 task = tb.tasks[task0 + blockIdx.x - ndiag];
-    int k0, k1;
-    local_range(tb, task.x, step0, step1, k0, k1);
-    update_role<1>(tb, task, k0, k1, lds);
-  }
+  const int s = blockIdx.x;
+  int k0, k1;
+  local_range(tb, s, step0, step1, k0, k1);
+  diag_role(tb, s, step - tb.shift[s], k0, k1, lds);
 }
 
-// The part of a trailing update that the next group's sweep does not read.
+// A list of tasks of (*): the column updates of a sweep step (the tiles the next
+// panel step reads; beside the diagonal kernel) or the part of a trailing update
+// that the next group's sweep does not read.
 __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0, int step0,
                                                             int step1) {
   extern __shared__ float lds[];
   const int2 task = tb.tasks[task0 + blockIdx.x];
   int k0, k1;
   local_range(tb, task.x, step0, step1, k0, k1);
-  update_role<1>(tb, task, k0, k1, lds);
+  update_role<2>(tb, task, k0, k1, lds);
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
@@ -490,26 +542,33 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int tas
   const int T = tb.nt[s];
   const int d = tb.dim[s];
   const int K = (T - I) * NB;
-  const LoaderTile la{tile_ptr(tb, s, I, I)}, lb{tile_ptr(tb, s, J, I)};
+  const OperandRows la{tile_ptr(tb, s, I, I)}, lb{tile_ptr(tb, s, J, I)};
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
   if (I == J)
-    tile_mainloop<true, 2>(la, lb, K, lds, acc);
+    tile_mainloop<true, 4>(la, lb, K, lds, acc);
   else
-    tile_mainloop<false, 2>(la, lb, K, lds, acc);
+    tile_mainloop<false, 4>(la, lb, K, lds, acc);
   // through an LDS transpose, so that the mirror is written in row segments too
   write_tile<2>(acc, lds, I, J, d, d, 1.f, 0.f, tb.out[s]);
 }
 
-// Dynamic LDS of the step kernel: the diagonal role's working tile and three
-// private blocks (at most three waves are busy in a pass of the triangular
-// inverse), 77 KB, so that two workgroups share a CU like the other tile kernels.
+// Dynamic LDS.  The trailing update ("rest") asks for 81 KB although it uses 74:
+// then one of its workgroups fits a CU, not two, and a column or panel workgroup
+// of the sweep (74 KB) always finds room beside it instead of queueing behind
+// the rest for a slot.  The diagonal kernel needs 77 KB (its working tile and
+// three private blocks: at most three waves are busy in a pass of the triangular
+// inverse) and asks for 80: two of its workgroups share a CU, but none shares
+// one with a workgroup of the rest.
 constexpr size_t kDiagLds = (size_t)(NB * LS + 3 * SB * PS) * sizeof(float);
-constexpr size_t kStepLds = kDiagLds > kTileLdsBytes ? kDiagLds : kTileLdsBytes;
-static_assert(2 * kStepLds <= 160 * 1024, "two step workgroups must fit a CU");
 constexpr size_t kRestLdsBytes = 81 * 1024;
-static_assert(2 * kRestLdsBytes > 160 * 1024 && kRestLdsBytes + kStepLds <= 160 * 1024,
-              "one rest workgroup per CU, with room for a step workgroup");
+constexpr size_t kDiagKernelLds = 80 * 1024;
+static_assert(kDiagLds <= kDiagKernelLds && kTileLdsBytes <= kDiagKernelLds, "diagonal role's LDS");
+static_assert(2 * kDiagKernelLds <= 160 * 1024 && kDiagKernelLds + kRestLdsBytes > 160 * 1024 &&
+                  kDiagKernelLds + kTileLdsBytes <= 160 * 1024,
+              "a diagonal workgroup shares a CU with another or with a column workgroup, not with the rest");
+static_assert(2 * kRestLdsBytes > 160 * 1024 && kRestLdsBytes + kTileLdsBytes <= 160 * 1024,
+              "one rest workgroup per CU, with room for a column or panel workgroup");
 
 }  // namespace
 
@@ -542,11 +601,15 @@ struct kfac_inverse_plan {
   bool capture_origin = false;
   size_t rest_lds = 0;
   hipStream_t side = nullptr;
-  std::vector<hipEvent_t> ev_main, ev_side;   // per step
+  // The column updates of a step are independent of its diagonal tiles: they run
+  // on a third stream beside the diagonal kernel.
+  hipStream_t col = nullptr;
+  std::vector<hipEvent_t> ev_main, ev_side, ev_fork, ev_col;   // per step
   ~kfac_inverse_plan() {
-    for (hipEvent_t e : ev_main) (void)hipEventDestroy(e);
-    for (hipEvent_t e : ev_side) (void)hipEventDestroy(e);
+    for (auto *v : {&ev_main, &ev_side, &ev_fork, &ev_col})
+      for (hipEvent_t e : *v) (void)hipEventDestroy(e);
     if (side) (void)hipStreamDestroy(side);
+    if (col) (void)hipStreamDestroy(col);
   }
   int total_tiles = 0;
   int lauum_task0 = 0, lauum_count = 0;
@@ -758,14 +821,14 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_panel, panel_cs.data(), sizeof(int) * (count + 1));
   up(p->d_tasks, tasks.data(), sizeof(int2) * tasks.size());
   if (rc == KFAC_OK && p->lookahead && p->max_t > p->group) {
-    bool ok = hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess;
-    for (int g = 0; ok && g < p->max_t; ++g) {
-      hipEvent_t a = nullptr, b = nullptr;
-      ok = hipEventCreateWithFlags(&a, hipEventDisableTiming) == hipSuccess;
-      if (ok) p->ev_main.push_back(a);
-      ok = ok && hipEventCreateWithFlags(&b, hipEventDisableTiming) == hipSuccess;
-      if (ok && b) p->ev_side.push_back(b);
-    }
+    bool ok = hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess &&
+              hipStreamCreateWithFlags(&p->col, hipStreamNonBlocking) == hipSuccess;
+    for (int g = 0; ok && g < p->max_t; ++g)
+      for (auto *v : {&p->ev_main, &p->ev_side, &p->ev_fork, &p->ev_col}) {
+        hipEvent_t e = nullptr;
+        ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
+        if (ok) v->push_back(e);
+      }
     if (!ok) rc = kfac::fail(KFAC_EHIP, "cannot create the look-ahead stream or its events");
   } else {
     p->lookahead = false;
@@ -834,9 +897,9 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   rc = plan->d_out.set(plan->out_sorted.data(), sizeof(void *) * count, s);
   if (rc != KFAC_OK) return rc;
   if (!plan->attr_set) {
-    KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(step_kernel),
+    KFAC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(diag_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kStepLds));
+                                       (int)kDiagKernelLds));
     for (const void *f : {reinterpret_cast<const void *>(panel_kernel),
                           reinterpret_cast<const void *>(lauum_kernel)})
       KFAC_HIP_CHECK(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -900,10 +963,22 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[two_back], 0));
     if (!lookahead)
       if (int rc2 = queue_rest()) return rc2;   // one stream: keep the program order
-    {
-      kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, s);
-      hipLaunchKernelGGL(step_kernel, dim3(na + w.count), dim3(THREADS), kStepLds, s, tb, k, na,
-                         w.task0, w.k0, w.k1);
+    // the diagonal tiles on `s`, the column updates beside them
+    hipStream_t cs = s;
+    if (lookahead && w.count > 0) {
+      KFAC_HIP_CHECK(hipEventRecord(plan->ev_fork[k], s));
+      KFAC_HIP_CHECK(hipStreamWaitEvent(plan->col, plan->ev_fork[k], 0));
+      cs = plan->col;
+    }
+    hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(THREADS), kDiagKernelLds, s, tb, k, w.k0, w.k1);
+    if (w.count > 0) {
+      kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, cs);
+      hipLaunchKernelGGL(update_kernel, dim3(w.count), dim3(THREADS), kTileLdsBytes, cs, tb, w.task0,
+                         w.k0, w.k1);
+    }
+    if (cs != s) {
+      KFAC_HIP_CHECK(hipEventRecord(plan->ev_col[k], cs));
+      KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_col[k], 0));
     }
     if (int rc2 = queue_rest()) return rc2;
     if (plan->panel_total[k] > 0)
