@@ -60,17 +60,29 @@ constexpr int SB = 32;
 constexpr int LS = NB + 1;  // LDS row stride of the diagonal-tile kernel
 constexpr int PS = SB + 1;  // row stride of a wave's private 32x32 block
 
+// One tile product, resolved on the host when the plan is built: a workgroup
+// reads its record (one scalar load) and can issue its operand loads at once,
+// instead of walking the per-matrix tables first (three dependent round trips
+// of 1-2 us each on a busy GPU, on the critical path of every launch of the
+// sweep).  Offsets are float offsets into the workspace.
+struct TileTask {
+  long long c_off;   // tile that is updated / written; lauum: the slot of the matrix
+  long long a_off;   // first tile of the A operand's run
+  long long b_off;   // first tile of the B operand's run; diagonal task: caller index | dimension << 32
+  int K;             // reduction length; 0: nothing to do (diagonal task: no products owed)
+  int flags;         // update: kFirst | kSame; diagonal task: block column k; lauum: I | J << 16
+};
+constexpr int kFirst = 1;   // the accumulators start from zero (first product of an upper tile)
+constexpr int kSame = 2;    // both operands are the same run
+
 struct InvTables {
   const float *const *in;    // [count] sorted slot -> input matrix
   float *const *out;         // [count]
-  const int *orig;           // [count] slot -> caller index
   const int *dim;            // [count]
   const int *nt;             // [count] tiles per side
-  const int *shift;          // [count] sweep step at which the matrix starts
   const long long *ws_off;   // [count] float offset of the padded matrix
-  const int *tile_cs;        // [count+1] cumulative lower-tile counts
-  const int *panel_cs;       // [count+1] cumulative (nt-1)
-  const int2 *tasks;         // update tasks of all launches: {slot, a | b << 16}
+  const int *tile_cs;        // [count+1] cumulative lower-tile counts (copy-in)
+  const TileTask *tasks;     // the tile tasks of all launches
   float *ws;                 // padded matrices
   int *info;
 };
@@ -340,24 +352,24 @@ __device__ __forceinline__ void wave_visit(const floatx16 &acc, F f) {
   for (int v = 0; v < 16; ++v) f(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), lane & 31, acc[v]);
 }
 
-// Diagonal tile (k,k) of matrix s: first the products it is still owed,
-//   C(k,k) -= sum_{j = lo .. hi} M(k,j) M(k,j)^T        (nothing when hi < lo),
+// Diagonal tile (k,k) of a matrix: first the products it is still owed,
+//   C(k,k) -= sum_{j = lo .. hi} M(k,j) M(k,j)^T        (nothing when K = 0),
 // through the shared main loop (the other tiles of the column receive theirs
 // from the update workgroups of the same launch), then the factorisation.
-__device__ __forceinline__ void diag_role(const InvTables &tb, int s, int k, int lo, int hi,
-                                          float *smem) {
+__device__ __forceinline__ void diag_role(const InvTables &tb, const TileTask &t, float *smem) {
   float *S = smem;                      // NB x LS working tile
   float *scratch = smem + NB * LS;      // 3 waves x SB x PS
-  const int d = tb.dim[s];
+  const int d = (int)(t.b_off >> 32);
+  const int k = t.flags;
   constexpr int ld = NB;
-  float *tile = tile_ptr(tb, s, k, k);
+  float *tile = tb.ws + t.c_off;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  if (hi >= lo) {
+  if (t.K > 0) {
     floatx16 acc[2][2];
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -tile[rr * NB + cc]; });
-    const OperandRows la{tile_ptr(tb, s, k, lo)};
-    tile_mainloop<true, 2>(la, la, (hi - lo + 1) * NB, smem, acc);   // ends with a barrier
+    const OperandRows la{tb.ws + t.a_off};
+    tile_mainloop<true, 2>(la, la, t.K, smem, acc);   // ends with a barrier
     for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { S[rr * LS + cc] = -v; });
   } else {
     const int c4 = (threadIdx.x & 31) * 4, r0 = threadIdx.x >> 5;
@@ -381,7 +393,7 @@ __device__ __forceinline__ void diag_role(const InvTables &tb, int s, int k, int
     if (wave == 0) {
       const int bad = kfac::chol_inv_32<LS>(S, jb * SB);
       if (lane == 0) {
-        int *pinfo = &tb.info[tb.orig[s]];
+        int *pinfo = &tb.info[(int)(t.b_off & 0xffffffffLL)];
         if (k == 0 && jb == 0) *pinfo = 0;
         const int col = k * NB + jb * SB + bad - 1;
         if (bad && col < d && *pinfo == 0) *pinfo = col + 1;
@@ -450,55 +462,36 @@ __device__ __forceinline__ void diag_role(const InvTables &tb, int s, int k, int
 // ---------------------------------------------------------------------------
 // M(x,k) = M(x,k) W^T = M(x,k) U_kk in place for every x != k; the operand
 // W^T is the diagonal tile itself, read transposed.
-__global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int step, int nactive) {
+__global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int task0) {
   extern __shared__ float lds[];
-  const int s = find_slot(tb.panel_cs, nactive, blockIdx.x);
-  const int k = step - tb.shift[s];
-  const int local = blockIdx.x - tb.panel_cs[s];
-  const int x = local < k ? local : local + 1;
-  float *tile = tile_ptr(tb, s, x, k);
+  const TileTask t = tb.tasks[task0 + blockIdx.x];
+  float *tile = tb.ws + t.c_off;
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
-  tile_mainloop<false, 2>(OperandRows{tile}, OperandCols{tile_ptr(tb, s, k, k)}, NB, lds, acc);
+  tile_mainloop<false, 2>(OperandRows{tile}, OperandCols{tb.ws + t.b_off}, NB, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { tile[rr * NB + cc] = v; });
 }
 
-// One task of (*): tile (a,b) of matrix `slot`, products over the block
-// columns [k0, k1] clipped to the tile's own range.  The accumulators start
-// from -C, so the tile is read while the first operand panels are in flight and
-// the epilogue is a plain store.  An upper tile whose row lies inside [k0, k1]
-// receives its first product here and is overwritten (it holds stale data).
+// One task of (*): tile (a,b) of a matrix, products over the block columns of
+// the launch clipped to the tile's own range (resolved in the task record).  The
+// accumulators start from -C, so the tile is read while the first operand panels
+// are in flight and the epilogue is a plain store.  An upper tile whose row lies
+// inside the source columns receives its first product here and is overwritten
+// (it holds stale data): kFirst.
 template <int D>
-__device__ __forceinline__ void update_role(const InvTables &tb, int2 task, int k0, int k1,
-                                            float *lds) {
-  const int s = task.x;
-  const int a = task.y & 0xffff, b = task.y >> 16;
-  const bool upper = a < b;
-  const int j_lo = upper && a > k0 ? a : k0;
-  const int j_hi = upper && b - 1 < k1 ? b - 1 : k1;
-  const int K = (j_hi - j_lo + 1) * NB;
-  const bool first = upper && a >= k0;
-  float *C = tile_ptr(tb, s, a, b);
+__device__ __forceinline__ void update_role(const InvTables &tb, const TileTask &t, float *lds) {
+  float *C = tb.ws + t.c_off;
   floatx16 acc[2][2];
-  if (first)
+  if (t.flags & kFirst)
     zero_acc<2, 2>(acc);
   else
     fill_acc<2, 2>(acc, [&](int rr, int cc) { return -C[rr * NB + cc]; });
-  const OperandRows la{tile_ptr(tb, s, a, j_lo)}, lb{tile_ptr(tb, s, b, j_lo)};
-  if (a == b)
-    tile_mainloop<true, D>(la, lb, K, lds, acc);
+  const OperandRows la{tb.ws + t.a_off}, lb{tb.ws + t.b_off};
+  if (t.flags & kSame)
+    tile_mainloop<true, D>(la, lb, t.K, lds, acc);
   else
-    tile_mainloop<false, D>(la, lb, K, lds, acc);
+    tile_mainloop<false, D>(la, lb, t.K, lds, acc);
   for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[rr * NB + cc] = -v; });
-}
-
-// The group's block columns [step0, step1] in matrix s's own numbering (a
-// matrix that starts inside the group has a shorter first group).
-__device__ __forceinline__ void local_range(const InvTables &tb, int s, int step0, int step1,
-                                            int &k0, int &k1) {
-  const int shift = tb.shift[s];
-  k0 = step0 > shift ? step0 - shift : 0;
-  k1 = step1 - shift;
 }
 
 // One workgroup per active matrix: the diagonal tile of sweep step `step`
@@ -510,47 +503,40 @@ __device__ __forceinline__ void local_range(const InvTables &tb, int s, int step
 // beside a workgroup of the trailing update (kDiagKernelLds): it waits for a CU
 // without one, at most the few microseconds until the next of them retires, and
 // keeps the following ones away from that CU while it runs.
-__global__ __launch_bounds__(THREADS, 2) void diag_kernel(InvTables tb, int step, int step0,
-                                                          int step1) {
+__global__ __launch_bounds__(THREADS, 2) void diag_kernel(InvTables tb, int task0) {
   extern __shared__ float lds[];
-  const int s = blockIdx.x;
-  int k0, k1;
-  local_range(tb, s, step0, step1, k0, k1);
-  diag_role(tb, s, step - tb.shift[s], k0, k1, lds);
+  const TileTask t = tb.tasks[task0 + blockIdx.x];
+  diag_role(tb, t, lds);
 }
 
 // A list of tasks of (*): the column updates of a sweep step (the tiles the next
 // panel step reads; beside the diagonal kernel) or the part of a trailing update
 // that the next group's sweep does not read.
-__global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0, int step0,
-                                                            int step1) {
+__global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int task0) {
   extern __shared__ float lds[];
-  const int2 task = tb.tasks[task0 + blockIdx.x];
-  int k0, k1;
-  local_range(tb, task.x, step0, step1, k0, k1);
-  update_role<2>(tb, task, k0, k1, lds);
+  const TileTask t = tb.tasks[task0 + blockIdx.x];
+  update_role<2>(tb, t, lds);
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
 // One task per tile; the table deals whole tile rows to XCDs (see the plan).
 __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int task0) {
   extern __shared__ float lds[];
-  const int2 task = tb.tasks[task0 + blockIdx.x];
-  const int s = task.x;
-  if (s < 0) return;   // padding of an XCD's shorter list
-  const int I = task.y & 0xffff, J = task.y >> 16;
-  const int T = tb.nt[s];
+  const TileTask t = tb.tasks[task0 + blockIdx.x];
+  if (t.K == 0) return;   // padding of an XCD's shorter list
+  const int s = (int)t.c_off;
+  const int I = t.flags & 0xffff, J = t.flags >> 16;
   const int d = tb.dim[s];
-  const int K = (T - I) * NB;
-  const OperandRows la{tile_ptr(tb, s, I, I)}, lb{tile_ptr(tb, s, J, I)};
+  float *out = tb.out[s];
+  const OperandRows la{tb.ws + t.a_off}, lb{tb.ws + t.b_off};
   floatx16 acc[2][2];
   zero_acc<2, 2>(acc);
   if (I == J)
-    tile_mainloop<true, 4>(la, lb, K, lds, acc);
+    tile_mainloop<true, 4>(la, lb, t.K, lds, acc);
   else
-    tile_mainloop<false, 4>(la, lb, K, lds, acc);
+    tile_mainloop<false, 4>(la, lb, t.K, lds, acc);
   // through an LDS transpose, so that the mirror is written in row segments too
-  write_tile<2>(acc, lds, I, J, d, d, 1.f, 0.f, tb.out[s]);
+  write_tile<2>(acc, lds, I, J, d, d, 1.f, 0.f, out);
 }
 
 // Dynamic LDS.  The trailing update ("rest") asks for 81 KB although it uses 74:
@@ -585,6 +571,7 @@ struct kfac_inverse_plan {
   std::vector<int> nt;             // per slot
   std::vector<int> nactive;        // per step
   std::vector<int> panel_total;    // per step
+  std::vector<int> diag_task0, panel_task0;   // per step: first record of the launch
   // per step: the update tasks that share the launch with the diagonal tiles:
   // inside a group the left-looking update of column k, on a group's first
   // column the previous group's trailing update of this group's columns
@@ -615,7 +602,7 @@ struct kfac_inverse_plan {
   int lauum_task0 = 0, lauum_count = 0;
   size_t ws_floats = 0;            // padded matrices
   std::vector<const void *> in_sorted, out_sorted;
-  kfac::DevTable d_in, d_out, d_orig, d_dim, d_nt, d_shift, d_off, d_tile, d_panel, d_tasks;
+  kfac::DevTable d_in, d_out, d_dim, d_nt, d_off, d_tile, d_tasks;
   bool attr_set = false;
 };
 
@@ -624,10 +611,11 @@ namespace {
 // Workgroup i of a launch runs on XCD i % 8.  Deal the tasks out so that each
 // XCD receives one contiguous run of the natural order (neighbouring tasks
 // share operand row slabs, which then stay in that XCD's L2).
-void append_tasks(std::vector<int2> &table, const std::vector<int2> &natural) {
+template <class T>
+void append_tasks(std::vector<T> &table, const std::vector<T> &natural) {
   const size_t n = natural.size();
   const size_t chunk = (n + 7) / 8;
-  std::vector<int2> dealt;
+  std::vector<T> dealt;
   dealt.reserve(n);
   // position p of XCD x holds natural[x * chunk + p]; emit in launch order
   // (p major, x minor) and skip the holes of a ragged last chunk
@@ -676,7 +664,8 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   p->ws_floats = total;
   p->total_tiles = tile_cs[count];
   p->max_t = count ? p->nt[0] : 0;
-  std::vector<int2> tasks, natural;
+  std::vector<TileTask> tasks;
+  std::vector<int2> natural;
   p->with_diag.resize(p->max_t);
   p->rest.resize(p->max_t);
   if (const char *e = getenv("KFAC_INVERSE_LOOKAHEAD")) p->lookahead = atoi(e) != 0;
@@ -701,6 +690,31 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   if (const char *e = getenv("KFAC_INVERSE_ALIGN")) align = std::min(100, std::max(0, atoi(e)));
   std::vector<int> shift(count);
   for (int s = 0; s < count; ++s) shift[s] = (p->max_t - p->nt[s]) * align / 100;
+  auto tile_off = [&](int s, int I, int J) {
+    return off[s] + ((long long)I * p->nt[s] + J) * (long long)(NB * NB);
+  };
+  // tile (a,b) of a matrix receives the products of the sweep steps [step0, step1]: those of
+  // them that are block columns of this matrix (one that starts inside the range has fewer)
+  // and lie inside the tile's own range
+  auto resolve = [&](const std::vector<int2> &list, int step0, int step1) {
+    std::vector<TileTask> out;
+    out.reserve(list.size());
+    for (const int2 &t : list) {
+      const int s = t.x, a = t.y & 0xffff, b = t.y >> 16;
+      const int k0 = step0 > shift[s] ? step0 - shift[s] : 0, k1 = step1 - shift[s];
+      const bool upper = a < b;
+      const int j_lo = upper && a > k0 ? a : k0;
+      const int j_hi = upper && b - 1 < k1 ? b - 1 : k1;
+      TileTask r;
+      r.c_off = tile_off(s, a, b);
+      r.a_off = tile_off(s, a, j_lo);
+      r.b_off = tile_off(s, b, j_lo);
+      r.K = (j_hi - j_lo + 1) * NB;
+      r.flags = (upper && a >= k0 ? kFirst : 0) | (a == b ? kSame : 0);
+      out.push_back(r);
+    }
+    return out;
+  };
   // Tiles right of the source group [s0, s1] (sweep steps) that receive its
   // products: the columns of the following group when `next`, otherwise
   // everything right of those.  The upper tiles whose row lies inside the source
@@ -755,8 +769,39 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     }
     w.task0 = (int)tasks.size();
     w.count = (int)(natural.size() + tail.size());
-    append_tasks(tasks, natural);
-    append_tasks(tasks, tail);
+    append_tasks(tasks, resolve(natural, w.k0, w.k1));
+    append_tasks(tasks, resolve(tail, w.k0, w.k1));
+    // the diagonal tiles of the step, which take the same columns' products themselves
+    p->diag_task0.push_back((int)tasks.size());
+    for (int s = 0; s < na; ++s) {
+      const int k = g - shift[s];
+      const int k0 = w.k0 > shift[s] ? w.k0 - shift[s] : 0, k1 = w.k1 - shift[s];
+      TileTask r;
+      r.c_off = tile_off(s, k, k);
+      r.a_off = tile_off(s, k, k0);
+      r.b_off = (long long)p->order[s] | ((long long)dim[s] << 32);
+      r.K = k1 >= k0 ? (k1 - k0 + 1) * NB : 0;
+      r.flags = k;
+      tasks.push_back(r);
+    }
+    // and the panel step: every other tile of block column k times U_kk
+    p->panel_task0.push_back((int)tasks.size());
+    {
+      std::vector<TileTask> panel;
+      for (int s = 0; s < na; ++s) {
+        const int k = g - shift[s];
+        for (int x = 0; x < p->nt[s]; ++x) {
+          if (x == k) continue;
+          TileTask r;
+          r.c_off = r.a_off = tile_off(s, x, k);
+          r.b_off = tile_off(s, k, k);
+          r.K = NB;
+          r.flags = 0;
+          panel.push_back(r);
+        }
+      }
+      tasks.insert(tasks.end(), panel.begin(), panel.end());
+    }
     if (g == g1 && g1 + 1 < p->max_t) {
       natural.clear();
       tail.clear();
@@ -766,8 +811,8 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
       u.count = (int)(natural.size() + tail.size());
       u.k0 = g0;
       u.k1 = g1;
-      append_tasks(tasks, natural);
-      append_tasks(tasks, tail);
+      append_tasks(tasks, resolve(natural, u.k0, u.k1));
+      append_tasks(tasks, resolve(tail, u.k0, u.k1));
     }
   }
   // Final products out(I,J) = sum_k U(I,k) U(J,k)^T: the I + 1 tiles of tile row I
@@ -791,35 +836,40 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
       mine[x].push_back(r);
       load[x] += r.cost;
     }
-    std::vector<int2> list[8];
+    std::vector<TileTask> list[8];
     size_t longest = 0;
     for (int x = 0; x < 8; ++x) {
       std::stable_sort(mine[x].begin(), mine[x].end(), [&](const Row &a, const Row &b) {
         return p->nt[a.s] - a.I > p->nt[b.s] - b.I;
       });
       for (const Row &r : mine[x])
-        for (int J = 0; J <= r.I; ++J) list[x].push_back(pack(r.s, r.I, J));
+        for (int J = 0; J <= r.I; ++J) {
+          TileTask t;
+          t.c_off = r.s;
+          t.a_off = tile_off(r.s, r.I, r.I);
+          t.b_off = tile_off(r.s, J, r.I);
+          t.K = (p->nt[r.s] - r.I) * NB;
+          t.flags = r.I | (J << 16);
+          list[x].push_back(t);
+        }
       longest = std::max(longest, list[x].size());
     }
     p->lauum_task0 = (int)tasks.size();
     for (size_t i = 0; i < longest; ++i)
       for (int x = 0; x < 8; ++x)
-        tasks.push_back(i < list[x].size() ? list[x][i] : make_int2(-1, 0));
+        tasks.push_back(i < list[x].size() ? list[x][i] : TileTask{0, 0, 0, 0, 0});
     p->lauum_count = (int)(longest * 8);
   }
-  if (tasks.empty()) tasks.push_back(make_int2(0, 0));
+  if (tasks.empty()) tasks.push_back(TileTask{0, 0, 0, 0, 0});
   int rc = KFAC_OK;
   auto up = [&](kfac::DevTable &t, const void *h, size_t b) {
     if (rc == KFAC_OK) rc = t.set(h, b, nullptr);
   };
-  up(p->d_orig, p->order.data(), sizeof(int) * count);
   up(p->d_dim, dim.data(), sizeof(int) * count);
   up(p->d_nt, p->nt.data(), sizeof(int) * count);
-  up(p->d_shift, shift.data(), sizeof(int) * count);
   up(p->d_off, off.data(), sizeof(long long) * count);
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
-  up(p->d_panel, panel_cs.data(), sizeof(int) * (count + 1));
-  up(p->d_tasks, tasks.data(), sizeof(int2) * tasks.size());
+  up(p->d_tasks, tasks.data(), sizeof(TileTask) * tasks.size());
   if (rc == KFAC_OK && p->lookahead && p->max_t > p->group) {
     bool ok = hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess &&
               hipStreamCreateWithFlags(&p->col, hipStreamNonBlocking) == hipSuccess;
@@ -911,14 +961,11 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   InvTables tb;
   tb.in = plan->d_in.as<const float *const>();
   tb.out = plan->d_out.as<float *const>();
-  tb.orig = plan->d_orig.as<const int>();
   tb.dim = plan->d_dim.as<const int>();
   tb.nt = plan->d_nt.as<const int>();
-  tb.shift = plan->d_shift.as<const int>();
   tb.ws_off = plan->d_off.as<const long long>();
   tb.tile_cs = plan->d_tile.as<const int>();
-  tb.panel_cs = plan->d_panel.as<const int>();
-  tb.tasks = plan->d_tasks.as<const int2>();
+  tb.tasks = plan->d_tasks.as<const TileTask>();
   uintptr_t base = (reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255;
   tb.ws = reinterpret_cast<float *>(base);
   tb.info = info_dev;
@@ -942,7 +989,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     {
       kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
       hipLaunchKernelGGL(update_kernel, dim3(r.count), dim3(THREADS), plan->rest_lds, st, tb,
-                         r.task0, r.k0, r.k1);
+                         r.task0);
     }
     if (lookahead) {
       KFAC_HIP_CHECK(hipEventRecord(plan->ev_side[deferred], plan->side));
@@ -970,11 +1017,11 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       KFAC_HIP_CHECK(hipStreamWaitEvent(plan->col, plan->ev_fork[k], 0));
       cs = plan->col;
     }
-    hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(THREADS), kDiagKernelLds, s, tb, k, w.k0, w.k1);
+    hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(THREADS), kDiagKernelLds, s, tb,
+                       plan->diag_task0[k]);
     if (w.count > 0) {
       kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, cs);
-      hipLaunchKernelGGL(update_kernel, dim3(w.count), dim3(THREADS), kTileLdsBytes, cs, tb, w.task0,
-                         w.k0, w.k1);
+      hipLaunchKernelGGL(update_kernel, dim3(w.count), dim3(THREADS), kTileLdsBytes, cs, tb, w.task0);
     }
     if (cs != s) {
       KFAC_HIP_CHECK(hipEventRecord(plan->ev_col[k], cs));
@@ -983,7 +1030,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     if (int rc2 = queue_rest()) return rc2;
     if (plan->panel_total[k] > 0)
       hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), kTileLdsBytes, s,
-                         tb, k, na);
+                         tb, plan->panel_task0[k]);
     if (plan->rest[k].count == 0) continue;
     if (lookahead) KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
     deferred = k;

@@ -50,6 +50,16 @@ def compute_pi(lcov, rcov, pi_type=PI_TYPE_TRACENORM):
     return 1.0
 
 
+def as_float32(t):
+    """float16 activations and gradients enter the factor and preconditioning kernels as
+    float32, like the reference's cast before its GEMMs (linear.py:22-23, 38-39,
+    convolution_2d.py:35-37, 57-66, batch_normalization.py:122-129)."""
+    import torch
+    if t is not None and t.dtype == torch.float16:
+        return t.float()
+    return t
+
+
 class FisherBlock(object):
 
     def __init__(self, linkname, link, cov_ema_decay, damping,

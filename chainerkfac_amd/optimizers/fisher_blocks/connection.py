@@ -3,6 +3,7 @@ factors A (inputs) and G (output gradients).  Counterpart of the reference's
 chainerkfac/optimizers/fisher_blocks/connection.py."""
 from chainerkfac_amd import ops
 from chainerkfac_amd.optimizers.fisher_block import FisherBlock
+from chainerkfac_amd.optimizers.fisher_block import as_float32
 from chainerkfac_amd.optimizers.fisher_block import PI_TYPE_TRACENORM
 
 
@@ -92,12 +93,22 @@ class FisherBlockConnection(FisherBlock):
         W.kfgrad = kfW
         if b is not None:
             b.kfgrad = kfb
-        gW = W.grad if W.grad.is_contiguous() else W.grad.contiguous()
-        gb = None if b is None else (b.grad if b.grad.is_contiguous() else b.grad.contiguous())
+        gW = as_float32(W.grad)
+        gW = gW if gW.is_contiguous() else gW.contiguous()
+        gb = None if b is None else as_float32(b.grad)
+        gb = None if gb is None else (gb if gb.is_contiguous() else gb.contiguous())
         return G_inv, A_inv, gW, gb, kfW, kfb
+
+    def finish_kfgrads(self):
+        """After the products: ``kfgrad`` in the gradient's own type when that is
+        float16 (reference linear.py:55-61, convolution_2d.py:84-90)."""
+        for param in (self.link.W, self.link.b):
+            if param is not None and param.kfgrad is not None and param.kfgrad.dtype != param.grad.dtype:
+                param.kfgrad = param.kfgrad.to(param.grad.dtype)
 
     def update_kfgrads(self):
         ops.precond_conn(*self.kfgrad_operands())
+        self.finish_kfgrads()
 
     def compute_kfgrads(self, W, b, invs):
         """(G^-1 [dW | db]) A^-1 as one (c_out, dA) matrix, for callers that want

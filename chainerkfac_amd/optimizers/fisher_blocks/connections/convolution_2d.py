@@ -5,6 +5,7 @@ the SYRK kernel.  Counterpart of
 chainerkfac/optimizers/fisher_blocks/connections/convolution_2d.py."""
 from chainerkfac_amd import links
 from chainerkfac_amd import ops
+from chainerkfac_amd.optimizers.fisher_block import as_float32
 from chainerkfac_amd.optimizers.fisher_blocks.connection import FisherBlockConnection
 
 
@@ -15,7 +16,7 @@ class FisherBlockConvolution2D(FisherBlockConnection):
         return links.Convolution2DFunction
 
     def compute_A(self, in_data):
-        x = in_data[0]
+        x = as_float32(in_data[0])
         link = self.link
         ksize, stride, pad = link.ksize, link.stride[0], link.pad[0]
         n, c = x.shape[0], x.shape[1]
@@ -30,7 +31,7 @@ class FisherBlockConvolution2D(FisherBlockConnection):
         return ops.cov_conv_a(x, ksize, stride, pad, has_b, alpha, beta, out)
 
     def compute_G(self, in_data, out_grad_data):
-        gy = out_grad_data[0]
+        gy = as_float32(out_grad_data[0])
         n, c, ho, wo = gy.shape
         scale = self.gy_scale(n) ** 2 / (n * ho * wo)
         if getattr(self.link, 'diag', False):

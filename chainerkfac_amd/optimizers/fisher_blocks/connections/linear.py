@@ -2,6 +2,7 @@
 Counterpart of chainerkfac/optimizers/fisher_blocks/connections/linear.py."""
 from chainerkfac_amd import links
 from chainerkfac_amd import ops
+from chainerkfac_amd.optimizers.fisher_block import as_float32
 from chainerkfac_amd.optimizers.fisher_blocks.connection import FisherBlockConnection
 
 
@@ -12,7 +13,7 @@ class FisherBlockLinear(FisherBlockConnection):
         return links.LinearFunction
 
     def compute_A(self, in_data):
-        x = in_data[0]
+        x = as_float32(in_data[0])
         n, d_in = x.shape
         has_b = self.link.b is not None
         d = d_in + (1 if has_b else 0)
@@ -22,7 +23,7 @@ class FisherBlockLinear(FisherBlockConnection):
         return ops.cov_linear(x, has_b, alpha, beta, out)
 
     def compute_G(self, in_data, out_grad_data):
-        gy = out_grad_data[0]
+        gy = as_float32(out_grad_data[0])
         n, d_out = gy.shape
         scale = self.gy_scale(n) ** 2 / n
         out, alpha, beta = self._cov_target('G', (d_out, d_out), gy.device, scale)

@@ -6,6 +6,7 @@ import warnings
 from chainerkfac_amd import links
 from chainerkfac_amd import ops
 from chainerkfac_amd.optimizers.fisher_block import FisherBlock
+from chainerkfac_amd.optimizers.fisher_block import as_float32
 
 
 def _same_array(a, b):
@@ -84,8 +85,8 @@ class FisherBlockBatchNormalization(FisherBlock):
             self._own_factor = False
 
     def compute_F(self, in_data, out_grad_data):
-        x = in_data[0]
-        gy = out_grad_data[0]
+        x = as_float32(in_data[0])
+        gy = as_float32(out_grad_data[0])
         if x.ndim not in (2, 4):
             raise RuntimeError('len(x.shape) must be 2 or 4, not {}.'.format(x.ndim))
         n = x.shape[0]
@@ -165,8 +166,8 @@ class FisherBlockBatchNormalization(FisherBlock):
     def update_kfgrads(self):
         self.check_attr('invs')
         gamma, beta = self.link.gamma, self.link.beta
-        g = None if gamma is None else gamma.grad
-        b = None if beta is None else beta.grad
+        g = None if gamma is None else as_float32(gamma.grad)
+        b = None if beta is None else as_float32(beta.grad)
         kg = None if gamma is None else self._buffer('kf_gamma', gamma.shape, gamma.data.device)
         kb = None if beta is None else self._buffer('kf_beta', beta.shape, beta.data.device)
         if self.nan_flag is None:
@@ -174,10 +175,11 @@ class FisherBlockBatchNormalization(FisherBlock):
             self.nan_flag = torch.zeros(1, dtype=torch.int32, device=self.invs[0].device)
         # NaN anywhere in F^-1 grad makes the kernel hand back the raw gradients
         ops.precond_bn(self.invs[0], g, b, kg, kb, self.nan_flag)
+        # kfgrad in the gradient's own type (reference batch_normalization.py:185-193)
         if gamma is not None:
-            gamma.kfgrad = kg
+            gamma.kfgrad = kg if gamma.grad.dtype == kg.dtype else kg.to(gamma.grad.dtype)
         if beta is not None:
-            beta.kfgrad = kb
+            beta.kfgrad = kb if beta.grad.dtype == kb.dtype else kb.to(beta.grad.dtype)
         # The reference warns on the spot (batch_normalization.py:21-33), which
         # costs a device->host read per block; here the flag stays on the device
         # and KFAC.check_numerics() reads all of them together at the start of the

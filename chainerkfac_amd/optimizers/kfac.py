@@ -120,10 +120,19 @@ class KFACUpdateRule(object):
         self.state = None
         self.t = 0
         self.enabled = True
+        self._use_fp32_update = False
+        self._fp32_param = None
+
+    def use_fp32_update(self, flag=True):
+        """Keep a float32 master copy of a float16 parameter and update that
+        (Chainer's UpdateRule.use_fp32_update; reference kfac.py:64-85)."""
+        self._use_fp32_update = flag
 
     def init_state(self, param):
         import torch
-        self.state = {'v': torch.zeros_like(param.data)}
+        # the momentum kernel works in float32: a float16 parameter always gets a float32
+        # velocity and master copy (what the reference does under use_fp32_update)
+        self.state = {'v': torch.zeros(param.data.shape, dtype=torch.float32, device=param.data.device)}
 
     def update(self, param):
         if not self.enabled:
@@ -135,6 +144,20 @@ class KFACUpdateRule(object):
         # ones: G^-1 (s g) A^-1); both are divided back before the update, as
         # Chainer's UpdateRule.update does for ``grad`` and the reference for
         # ``kfgrad`` (kfac.py:72-78)
+        import torch
+        if param.data.dtype == torch.float16:
+            # float32 master copy and float32 gradient (reference kfac.py:64-72, 80-85)
+            if self._fp32_param is None:
+                self._fp32_param = param.data.float()
+            grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
+            if grad is None:
+                return
+            grad = grad.float()
+            if param._loss_scale is not None:
+                grad = grad / param._loss_scale
+            self.update_core(param, self._fp32_param, grad)
+            param.data.copy_(self._fp32_param)
+            return
         if param._loss_scale is not None:
             if getattr(param, 'kfgrad', None) is not None:
                 param.kfgrad /= param._loss_scale
@@ -142,8 +165,9 @@ class KFACUpdateRule(object):
                 param.grad /= param._loss_scale
         self.update_core(param)
 
-    def update_core(self, param):
-        grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
+    def update_core(self, param, data=None, grad=None):
+        if grad is None:
+            grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
         if grad is None:
             return
         lr = self.hyperparam.lr
@@ -151,7 +175,8 @@ class KFACUpdateRule(object):
         momentum = self.hyperparam.momentum
         if self.adjust_momentum and lr < lr_pre:
             momentum *= lr / lr_pre
-        ops.momentum_update(param.data, self.state['v'], grad.contiguous(), lr, momentum)
+        ops.momentum_update(param.data if data is None else data, self.state['v'], grad.contiguous(), lr,
+                            momentum)
 
     update_core_gpu = update_core
 
@@ -240,6 +265,14 @@ class KFAC(object):
         self._lanes.join()
         if self._pending is not None:
             self._pending.flush()
+
+    def use_fp32_update(self, flag=True):
+        """Chainer's Optimizer.use_fp32_update: float32 master copies for float16
+        parameters (this implementation always keeps them; the flag is recorded)."""
+        self._use_fp32_update = flag
+        for param in self.target.params():
+            if param.update_rule is not None:
+                param.update_rule.use_fp32_update(flag)
 
     def create_update_rule(self):
         return KFACUpdateRule(self.hyperparam, adjust_momentum=self.adjust_momentum)
@@ -416,6 +449,8 @@ class KFAC(object):
             shapes = [(o[0].shape[0], o[1].shape[0], o[3] is not None) for o in operands]
             bound = tuple(0 if t is None else t.data_ptr() for o in operands for t in o)
             ops.precond_group(shapes, bound).run(*[[o[i] for o in operands] for i in range(6)])
+            for fb in conn:
+                fb.finish_kfgrads()
         self._lanes.join()
 
     def update_invs_batched(self, fblocks):

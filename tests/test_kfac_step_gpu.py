@@ -505,3 +505,88 @@ def test_extract_builds_the_per_rank_lists_the_packer_consumes():
     n0 = O.get_nelems([host[0]])
     assert bool((buf1[:n0] == -7.0).all()) and np.array_equal(buf1[n0:].cpu().numpy(), ref[n0:])
     assert extract(opt.fblocks, [[], [1]], lambda b: b.extract_for_all_gather_v('kfgrad'))[0] == []
+
+
+def test_float16_activations_and_gradients_are_cast_up():
+    """float16 activations / output gradients give the factors of their float32 values, and a
+    float16 gradient is preconditioned in float32 and handed back as float16 (reference
+    linear.py:22-23, 38-39, 55-61; convolution_2d.py:35-37, 57-66; batch_normalization.py:122-129)."""
+    from chainerkfac_amd import links
+    from chainerkfac_amd.optimizers import fisher_blocks as FB
+    g = torch.Generator(device='cuda').manual_seed(5)
+
+    def rnd(*shape):
+        return torch.randn(*shape, device='cuda', generator=g)
+
+    kw = dict(cov_ema_decay=1.0, damping=1e-2)
+    lin = links.Linear(24, 12, generator=g)
+    fb = FB.FisherBlockLinear('/l', lin, **kw)
+    x16, gy16 = rnd(16, 24).half(), rnd(16, 12).half()
+    a16 = fb.compute_A((x16, lin.W.data, lin.b.data)).clone()
+    a32 = fb.compute_A((x16.float(), lin.W.data, lin.b.data)).clone()
+    g16 = fb.compute_G((x16,), (gy16,)).clone()
+    g32 = fb.compute_G((x16,), (gy16.float(),)).clone()
+    assert torch.equal(a16, a32) and torch.equal(g16, g32)
+
+    conv = links.Convolution2D(6, 8, 3, pad=1, generator=g)
+    fc = FB.FisherBlockConvolution2D('/c', conv, **kw)
+    xc, gc = rnd(4, 6, 8, 8).half(), rnd(4, 8, 8, 8).half()
+    assert torch.equal(fc.compute_A((xc, conv.W.data, conv.b.data)).clone(),
+                       fc.compute_A((xc.float(), conv.W.data, conv.b.data)).clone())
+    assert torch.equal(fc.compute_G((xc,), (gc,)).clone(), fc.compute_G((xc,), (gc.float(),)).clone())
+
+    bn = links.BatchNormalization(8)
+    fbn = FB.FisherBlockBatchNormalization('/bn', bn, **kw)
+    xb, gb = rnd(4, 8, 5, 5).half(), rnd(4, 8, 5, 5).half()
+    f16 = fbn.compute_F((xb, bn.gamma.data, bn.beta.data), (gb,)).clone()
+    f32 = fbn.compute_F((xb.float(), bn.gamma.data, bn.beta.data), (gb.float(),)).clone()
+    assert torch.equal(f16, f32)
+
+    # preconditioning of float16 gradients: float32 products of the cast gradients, float16 result
+    fb.forward_postprocess(None, (x16, lin.W.data, lin.b.data))
+    fb.backward_preprocess(None, (x16,), (gy16,))
+    fb.update_cov_emas()
+    fb.update_invs()
+    gw, gbias = rnd(12, 24).half(), rnd(12).half()
+
+    class Half(object):
+        def __init__(self, p, grad):
+            self.p, self.grad, self.kfgrad = p, grad, None
+            self.shape, self.data = p.shape, p.data
+
+    lin.W, lin.b = Half(lin.W, gw), Half(lin.b, gbias)
+    fb.update_kfgrads()
+    assert lin.W.kfgrad.dtype == torch.float16 and lin.b.kfgrad.dtype == torch.float16
+    A_inv, G_inv = [m.double() for m in fb.invs]
+    full = G_inv @ torch.cat([gw.double(), gbias.double()[:, None]], dim=1) @ A_inv
+    got = torch.cat([lin.W.kfgrad.double(), lin.b.kfgrad.double()[:, None]], dim=1)
+    assert (got - full).norm() <= 2e-3 * full.norm()
+
+
+def test_float16_parameter_is_updated_through_a_float32_master_copy():
+    """reference kfac.py:64-85: the update runs on a float32 copy; the float16 parameter follows."""
+    from chainerkfac_amd.optimizers.kfac import KFACUpdateRule, Hyperparameter
+
+    class P(object):
+        pass
+
+    g = torch.Generator(device='cuda').manual_seed(6)
+    p = P()
+    p.data = torch.randn(257, device='cuda', generator=g).half()
+    p.grad = None
+    p._loss_scale = 8.0
+    hp = Hyperparameter()
+    hp.lr, hp.lr_pre, hp.momentum = 0.01, 0.01, 0.9
+    rule = KFACUpdateRule(hp)
+    master = p.data.double()
+    v = torch.zeros_like(master)
+    for _ in range(3):
+        p.kfgrad = (torch.randn(257, device='cuda', generator=g) * 8.0).half()
+        kf = p.kfgrad.double() / 8.0
+        rule.update(p)
+        v = 0.9 * v - 0.01 * kf
+        master = master + v
+        assert p.data.dtype == torch.float16
+        # the float16 parameter is the rounded master copy, not an accumulation of rounded steps
+        assert torch.equal(p.data, rule._fp32_param.half())
+        assert (rule._fp32_param.double() - master).abs().max() <= 1e-5
