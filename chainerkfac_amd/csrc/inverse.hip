@@ -160,6 +160,49 @@ __device__ __forceinline__ vfloat4 gload16(const float *base, unsigned byte_off)
   return *(const KFAC_GLOBAL_AS vfloat4 *)((const KFAC_GLOBAL_AS char *)base + byte_off);
 }
 
+__device__ __forceinline__ void gstore1(float *base, unsigned byte_off, float v) {
+  *(KFAC_GLOBAL_AS float *)((KFAC_GLOBAL_AS char *)base + byte_off) = v;
+}
+
+// The accumulators <-> a row-major NB x NB tile at a wave-uniform address, as
+// scalar base + one lane offset per group of eight elements + immediates (no
+// 64-bit address per element).
+__device__ __forceinline__ unsigned acc_lane_offset() {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row0 = (wave >> 1) * 64 + 4 * (lane >> 5), col0 = (wave & 1) * 64 + (lane & 31);
+  return (unsigned)((row0 * NB + col0) * sizeof(float));
+}
+// acc = -C
+__device__ __forceinline__ void load_neg_tile(const float *C, floatx16 (&acc)[2][2]) {
+  const unsigned lane_off = acc_lane_offset();
+#pragma unroll
+  for (int im = 0; im < 2; ++im)
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const unsigned o = lane_off + (unsigned)((im * 32 + 8 * vq) * NB * sizeof(float));
+#pragma unroll
+      for (int vr = 0; vr < 4; ++vr)
+#pragma unroll
+        for (int in = 0; in < 2; ++in)
+          acc[im][in][vq * 4 + vr] = -gload1(C, o + (unsigned)((vr * NB + in * 32) * sizeof(float)));
+    }
+}
+// C = -acc
+__device__ __forceinline__ void store_neg_tile(float *C, const floatx16 (&acc)[2][2]) {
+  const unsigned lane_off = acc_lane_offset();
+#pragma unroll
+  for (int im = 0; im < 2; ++im)
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const unsigned o = lane_off + (unsigned)((im * 32 + 8 * vq) * NB * sizeof(float));
+#pragma unroll
+      for (int vr = 0; vr < 4; ++vr)
+#pragma unroll
+        for (int in = 0; in < 2; ++in)
+          gstore1(C, o + (unsigned)((vr * NB + in * 32) * sizeof(float)), -acc[im][in][vq * 4 + vr]);
+    }
+}
+
 // k along the rows of a run of consecutive tiles
 struct OperandRows {
   const float *base;   // first tile of the run
@@ -208,16 +251,69 @@ struct OperandCols {
   }
 };
 
+// One pass of KT k-values from the LDS panels `pa` / `pb` (both `pa` when SAME),
+// ending with a barrier.  Beside the MFMAs it writes the register set `ra` /
+// `rb` (the pass after this one) to the panels `na` / `nb`, then calls
+// `refill_a()` / `refill_b()`, which load that register set again.
+template <bool SAME, class LA, class LB, class FA, class FB>
+__device__ __forceinline__ void tile_pass(const float *pa, const float *pb, float *na, float *nb,
+                                          vfloat4 (&ra)[4], vfloat4 (&rb)[4],
+                                          floatx16 (&acc)[2][2], FA refill_a, FB refill_b) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane & 31, lk = lane >> 5;
+  vfloat4 fa[2], fb[2];
+#pragma unroll
+  for (int im = 0; im < 2; ++im) fa[im] = LA::fetch4(pa, (wm * 2 + im) * 32 + lrow, 0, lk);
+#pragma unroll
+  for (int in = 0; in < 2; ++in)
+    fb[in] = SAME ? LA::fetch4(pa, (wn * 2 + in) * 32 + lrow, 0, lk)
+                  : LB::fetch4(pb, (wn * 2 + in) * 32 + lrow, 0, lk);
+#pragma unroll
+  for (int g = 0; g < KT / 8; ++g) {
+    vfloat4 ga[2], gb[2];
+    if (g + 1 < KT / 8) {
+#pragma unroll
+      for (int im = 0; im < 2; ++im) ga[im] = LA::fetch4(pa, (wm * 2 + im) * 32 + lrow, g + 1, lk);
+#pragma unroll
+      for (int in = 0; in < 2; ++in)
+        gb[in] = SAME ? LA::fetch4(pa, (wn * 2 + in) * 32 + lrow, g + 1, lk)
+                      : LB::fetch4(pb, (wn * 2 + in) * 32 + lrow, g + 1, lk);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int im = 0; im < 2; ++im)
+#pragma unroll
+        for (int in = 0; in < 2; ++in)
+          acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[im][j], fb[in][j], acc[im][in], 0, 0, 0);
+      // slot 4g + j of 16: one LDS store at most (the last pass of a product stores what it
+      // holds as well, into the buffer nobody reads any more: cheaper than a branch per store)
+      const int slot = 4 * g + j;
+      if (slot >= 1 && slot < 5) LA::store1(ra, slot - 1, na);
+      if (!SAME && slot >= 5 && slot < 9) LB::store1(rb, slot - 5, nb);
+    }
+    if (g == 1) refill_a();               // after its stores (slots 1 .. 4)
+    if (!SAME && g == 2) refill_b();      // slots 5 .. 8
+    if (g + 1 < KT / 8) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = ga[i];
+        fb[i] = gb[i];
+      }
+    }
+  }
+  __syncthreads();
+}
+
 // K must be a multiple of 4 * KT.  lds: kTileLdsFloats.  Ends with a barrier.
 template <bool SAME, int PD, class LA, class LB>
 __device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K, float *lds,
                                               floatx16 (&acc)[2][2]) {
   constexpr int UNROLL = PD % 2 == 0 ? PD : 2 * PD;   // register set and LDS buffer of a pass are static
   float *ldsA = lds, *ldsB = lds + 2 * PF;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int lrow = lane & 31, lk = lane >> 5;
   const int P = K / KT;
   const unsigned offA = LA::lane_offset(), offB = LB::lane_offset();
   vfloat4 ra[PD][4];
@@ -244,55 +340,13 @@ __device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K,
     for (int u = 0; u < UNROLL; ++u) {
       const int p = pb + u;
       if (UNROLL > 4 && p >= P) break;   // P is a multiple of 4
-      const float *pa = ldsA + (u & 1) * PF;
-      const float *pbuf = SAME ? pa : ldsB + (u & 1) * PF;
-      float *na = ldsA + ((u + 1) & 1) * PF, *nb = ldsB + ((u + 1) & 1) * PF;
       const int r = (u + 1) % PD;            // register set of pass p + 1 (static once unrolled)
-      const bool ahead = p + 1 + PD < P;     // and its registers take pass p + 1 + PD
-      vfloat4 fa[2], fb[2];
-#pragma unroll
-      for (int im = 0; im < 2; ++im) fa[im] = LA::fetch4(pa, (wm * 2 + im) * 32 + lrow, 0, lk);
-#pragma unroll
-      for (int in = 0; in < 2; ++in)
-        fb[in] = SAME ? LA::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, 0, lk)
-                      : LB::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, 0, lk);
-#pragma unroll
-      for (int g = 0; g < KT / 8; ++g) {
-        vfloat4 ga[2], gb[2];
-        if (g + 1 < KT / 8) {
-#pragma unroll
-          for (int im = 0; im < 2; ++im) ga[im] = LA::fetch4(pa, (wm * 2 + im) * 32 + lrow, g + 1, lk);
-#pragma unroll
-          for (int in = 0; in < 2; ++in)
-            gb[in] = SAME ? LA::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, g + 1, lk)
-                          : LB::fetch4(pbuf, (wn * 2 + in) * 32 + lrow, g + 1, lk);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int im = 0; im < 2; ++im)
-#pragma unroll
-            for (int in = 0; in < 2; ++in)
-              acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[im][j], fb[in][j], acc[im][in], 0, 0, 0);
-          // slot 4g + j of 16: one LDS store and one global load at most
-          // (the last pass stores what it holds as well, into the buffer nobody reads any more:
-          // cheaper than a branch per store)
-          const int slot = 4 * g + j;
-          if (slot >= 1 && slot < 5) LA::store1(ra[r], slot - 1, na);
-          if (!SAME && slot >= 5 && slot < 9) LB::store1(rb[SAME ? 0 : r], slot - 5, nb);
-        }
-        if (g == 1 && ahead) la.load(ra[r], offA, p + 1 + PD);       // after its stores (slots 1 .. 4)
-        if (!SAME && g == 2 && ahead) lb.load(rb[SAME ? 0 : r], offB, p + 1 + PD);   // slots 5 .. 8
-        if (g + 1 < KT / 8) {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            fa[i] = ga[i];
-            fb[i] = gb[i];
-          }
-        }
-      }
-      __syncthreads();
+      const bool ahead = p + 1 + PD < P;     // which then takes pass p + 1 + PD
+      tile_pass<SAME, LA, LB>(
+          ldsA + (u & 1) * PF, ldsB + (u & 1) * PF, ldsA + ((u + 1) & 1) * PF, ldsB + ((u + 1) & 1) * PF,
+          ra[r], rb[SAME ? 0 : r], acc,
+          [&]() { if (ahead) la.load(ra[r], offA, p + 1 + PD); },
+          [&]() { if (ahead) lb.load(rb[SAME ? 0 : r], offB, p + 1 + PD); });
     }
   }
 }
@@ -480,18 +534,18 @@ __global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int tas
 // (it holds stale data): kFirst.
 template <int D>
 __device__ __forceinline__ void update_role(const InvTables &tb, const TileTask &t, float *lds) {
-  float *C = tb.ws + t.c_off;
+  float *C = const_cast<float *>(wave_uniform(tb.ws + t.c_off));
   floatx16 acc[2][2];
   if (t.flags & kFirst)
     zero_acc<2, 2>(acc);
   else
-    fill_acc<2, 2>(acc, [&](int rr, int cc) { return -C[rr * NB + cc]; });
+    load_neg_tile(C, acc);
   const OperandRows la{tb.ws + t.a_off}, lb{tb.ws + t.b_off};
   if (t.flags & kSame)
     tile_mainloop<true, D>(la, lb, t.K, lds, acc);
   else
     tile_mainloop<false, D>(la, lb, t.K, lds, acc);
-  for_each_acc<2, 2>(acc, [&](int rr, int cc, float v) { C[rr * NB + cc] = -v; });
+  store_neg_tile(C, acc);
 }
 
 // One workgroup per active matrix: the diagonal tile of sweep step `step`
