@@ -552,6 +552,17 @@ def write_per_layer(path, layers):
             rows.append((desc, count, fac, d, M, flop / 1e9, t * 1e3, flop / t / 1e9, ai, cap, flop / t / 1e9 / cap))
         del x, gy
     with open(path, 'w') as f:
+        f.write('# Covariance kernels layer by layer (every distinct convolution / linear shape of the workload)\n\n'
+                'Command (one MI355X, repository root):\n\n```\npython3 bench.py --config c3 --no-cpu --no-dense-field '
+                '--steps 5 --per-layer {}\n```\n\n'
+                'Each factor is computed alone, by the single-factor entry point, on one stream; "SYRK kernel us" is '
+                'the duration of its SYRK launch (HIP events inside the library around the launch, 10 repetitions, the '
+                '{:.1f} us an empty event bracket measures subtracted); the kernels that sum split-K partial tiles are '
+                'not in it. In a K-FAC step the small factors (at most 8 GFLOP: most 1x1 convolutions, linear and '
+                'batch-norm layers) do not run alone but in a handful of grouped launches, so their rows here show the '
+                'latency floor of a single launch, not their cost in the step. GFLOP = M d (d+1); flop/B = that over '
+                'the bytes of the input tensor read once plus the factor written once; roofline cap = min(157.3 '
+                'TFLOP/s FP32 MFMA, flop/B x 8 TB/s).\n\n'.format(path, empty * 1e3))
         f.write('| layer (x count) | factor | d | rows M | GFLOP | SYRK kernel us | TFLOP/s | flop/B | roofline cap TFLOP/s '
                 '| fraction of cap |\n|---|---|---:|---:|---:|---:|---:|---:|---:|---:|\n')
         for desc, count, fac, d, M, gf, us, tf, ai, cap, frac in rows:
@@ -689,7 +700,7 @@ def _csv_rows(directory, suffix):
 KERNEL_FAMILIES = (
     ('covariance SYRK family', ('syrk_',)),
     ('split-K finish of the covariances', ('finish_', 'reduce_kernel')),
-    ('inverse tile kernels', ('step_kernel', 'update_kernel', 'lauum_kernel', 'panel_kernel', 'copy_in', 'copy_out',
+    ('inverse tile kernels', ('diag_kernel', 'update_kernel', 'lauum_kernel', 'panel_kernel', 'copy_in', 'copy_out',
                               'trtri', 'potrf', 'small_inverse')),
     ('preconditioning GEMMs', ('gemm_',)),
     ('batch-norm statistics', ('bn_',)),

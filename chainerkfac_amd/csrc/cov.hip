@@ -1037,6 +1037,103 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_group_kernel(const GroupItemS
   for_each_acc<WM, WM>(acc, [&](int r, int c, float val) { out[r * BM + c] = val; }, wave);
 }
 
+// Macro-tile variant for 128-tile slab items with several k-slices: a workgroup
+// of four teams (4 x 256 threads) computes the 2 x 2 tiles (2 MI + a, 2 MJ + b)
+// of one k-slice from four operand panels staged once.  Tiles that share an
+// operand panel only share it in L2 when they run within a microsecond of each
+// other (an XCD's workgroups stream 3 MB through its 4 MB L2 per panel step), and
+// as separate workgroups they do not: the grouped launch of 128-tiles fetched
+// its inputs 2.2 - 2.5 times (hardware counters).  Here team t stages panel t
+// (rows 2 MI, 2 MI + 1, 2 MJ, 2 MJ + 1; a macro-tile on the diagonal has only the
+// first two) with the same loader code as a 256-thread workgroup, and team
+// (a, b) multiplies tile (2 MI + a, 2 MJ + b) out of panels a and 2 + b.  Every
+// barrier is reached by all 1024 threads: a team without a tile or a panel (above
+// the diagonal, past a ragged end) skips the work, never the barrier.
+// task = (item, macro-tile + nmacro * k-slice); partial tiles go to the same
+// slots as syrk_group_kernel's, so the finish launch is shared.
+constexpr int kMacroThreads = 4 * THREADS;
+constexpr size_t kMacroLdsBytes = 4 * Panel<128>::kFloats * sizeof(float);
+
+template <class Loader>
+__global__ __launch_bounds__(kMacroThreads, 1) void syrk_macro_kernel(
+    const GroupItemStatic *__restrict__ st, const GroupItemDyn *__restrict__ dy,
+    const int2 *__restrict__ tasks, float *__restrict__ ws) {
+  constexpr int BM = 128, WM = 2;
+  constexpr int PF = Panel<BM>::kFloats;
+  extern __shared__ float lds[];
+  const int team = threadIdx.x >> 8;
+  const int ta = team >> 1, tb = team & 1;
+  const int wave = (threadIdx.x >> 6) & 3;
+  const int lane = threadIdx.x & 63;
+  const int2 task = tasks[blockIdx.x];
+  const GroupItemStatic s = st[task.x];
+  const GroupItemDyn v = dy[task.x];
+  const int mtiles = (s.tiles + 1) / 2;
+  const int nmacro = mtiles * (mtiles + 1) / 2;
+  const int split = task.y / nmacro;
+  int MI, MJ;
+  tri_decode(task.y - split * nmacro, MI, MJ);
+  const bool on_diag = MI == MJ;
+  const int I = 2 * MI + ta, J = 2 * MJ + tb;
+  const int dt = s.d - s.ones;
+  // this team's tile and this team's panel
+  const bool has_tile = I < s.tiles && J <= I;
+  const int prow = (team < 2 ? 2 * MI : 2 * MJ) + (team & 1);
+  const bool stages = prow < s.tiles && !(on_diag && team >= 2);
+  float *mine_panel = lds + team * PF;
+  const float *pa = lds + ta * PF;
+  const float *pb = lds + (on_diag ? tb : 2 + tb) * PF;
+  Loader ld = GroupLoader<Loader>::make(s, v.in);
+  ld.init(nullptr, stages ? prow * BM : 0);
+  const long long kbeg = (long long)split * s.klen;
+  long long kend = kbeg + s.klen;
+  if (kend > s.K) kend = s.K;
+  floatx16 acc[WM][WM];
+  zero_acc<WM, WM>(acc);
+  float rs[WM] = {0.f, 0.f};
+  const bool active = has_tile && syrk_wave_active<WM>(I * BM, J * BM, dt, wave);
+  const bool sums = active && I == J;   // diagonal tile: also the row sums (the ones column)
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane & 31, lk = lane >> 5;
+  typename Loader::Regs r;
+  if (stages && kbeg < kend) ld.load(r, prow * BM, kbeg, kend);
+  for (long long k0 = kbeg; k0 < kend; k0 += KT) {
+    if (stages) ld.store(r, mine_panel);
+    __syncthreads();
+    if (stages && k0 + KT < kend) ld.load(r, prow * BM, k0 + KT, kend);
+    if (active) {
+#pragma unroll
+      for (int kk = 0; kk < KT / 2; ++kk) {
+        float a[WM], b[WM];
+#pragma unroll
+        for (int im = 0; im < WM; ++im)
+          a[im] = fetch<BM, Loader::kKRow>(pa, (wm * WM + im) * 32 + lrow, 2 * kk + lk);
+        if (sums) {
+#pragma unroll
+          for (int im = 0; im < WM; ++im) rs[im] += a[im];
+        }
+#pragma unroll
+        for (int in = 0; in < WM; ++in)
+          b[in] = fetch<BM, Loader::kKRow>(pb, (wn * WM + in) * 32 + lrow, 2 * kk + lk);
+#pragma unroll
+        for (int im = 0; im < WM; ++im)
+#pragma unroll
+          for (int in = 0; in < WM; ++in)
+            acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  if (!has_tile) return;
+  const long long slot = (long long)s.ntile * (BM * BM) + (long long)s.tiles * BM;
+  float *mine = ws + s.part_off + split * slot;
+  if (s.ones && I == J)
+    write_rowsums<WM>(rs, I, dt, s.d, 0, s.count, v.alpha, v.beta, mine + (long long)s.ntile * (BM * BM),
+                      v.out, wave);
+  float *out = mine + (long long)(I * (I + 1) / 2 + J) * (BM * BM);
+  for_each_acc<WM, WM>(acc, [&](int rr, int cc, float val) { out[rr * BM + cc] = val; }, wave);
+}
+
 // task = (item, 64 x 64 block of the lower triangle); sums the item's k-slices
 // in a fixed order and writes the block and its mirror image.
 __global__ __launch_bounds__(256) void finish_group_kernel(const GroupItemStatic *__restrict__ st,
@@ -1120,7 +1217,10 @@ void deal_to_xcds(std::vector<int2> &table, const std::vector<int2> &natural) {
     }
 }
 
-constexpr int kGroupKinds = 8;   // {64-tiles, 128-tiles} x {slab float4, slab scalar, linear float4, linear scalar}
+// {64-tiles, 128-tiles} x {slab float4, slab scalar, linear float4, linear scalar},
+// then the macro-tile launches {slab float4, slab scalar}
+constexpr int kGroupKinds = 10;
+constexpr int kMacroKind0 = 8;
 
 }  // namespace
 
@@ -1201,7 +1301,19 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     s.tiles = kfac::ceil_div(it.c, s.bm);
     s.ntile = s.tiles * (s.tiles + 1) / 2;
     kind_of[i] = (s.bm == 64 ? 0 : 4) + (s.kind == KFAC_COV_SLAB ? 0 : 2) + (s.vec ? 0 : 1);
-    work[kind_of[i]] += (double)s.ntile * (double)nk[i] * (s.bm == 64 ? 1.0 : 4.0);
+    // slabs of several 128-tiles with a reduction long enough to cut into slices: macro-tiles
+    // (KFAC_GROUP_MACRO=0 switches them off, for comparisons)
+    static const bool macro_on = [] {
+      const char *env = getenv("KFAC_GROUP_MACRO");
+      return !(env && atoi(env) == 0);
+    }();
+    if (macro_on && s.bm == 128 && s.kind == KFAC_COV_SLAB && s.tiles >= 2 && nk[i] >= 16) {
+      kind_of[i] = kMacroKind0 + (s.vec ? 0 : 1);
+      const int mt = (s.tiles + 1) / 2;
+      work[kind_of[i]] += (double)(mt * (mt + 1) / 2) * (double)nk[i];
+    } else {
+      work[kind_of[i]] += (double)s.ntile * (double)nk[i] * (s.bm == 64 ? 1.0 : 4.0);
+    }
   }
   // k-slices: every launch (one per loader kind and tile size) is cut into workgroups
   // of about equal length (a panel of a 128-tile counts four times a panel of a
@@ -1216,22 +1328,33 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
       if (v >= 1.0) per_wg[k] = v;
     }
   }
+  // a macro-tile workgroup has a CU to itself: ~6 rounds of 256 (measured: fewer, longer
+  // workgroups balance worse, more gain nothing), at least 8 panels each
+  // (work counted in panels per macro-tile; KFAC_GROUP_MACRO_TASKS is a tuning override)
+  for (int k = kMacroKind0; k < kGroupKinds; ++k) {
+    double ntasks = 1536.0;
+    if (const char *env = getenv("KFAC_GROUP_MACRO_TASKS")) ntasks = std::max(1.0, atof(env));
+    per_wg[k] = std::max(8.0, work[k] / ntasks);
+  }
   size_t off = 0;
   std::vector<int2> natural[kGroupKinds], fin;
   for (int i = 0; i < count; ++i) {
     GroupItemStatic &s = g->items[i];
-    long long ns = (long long)((double)nk[i] * (s.bm == 64 ? 1.0 : 4.0) / per_wg[kind_of[i]] + 0.5);
+    const bool macro = kind_of[i] >= kMacroKind0;
+    long long ns = (long long)((double)nk[i] * (macro ? 1.0 : s.bm == 64 ? 1.0 : 4.0) / per_wg[kind_of[i]] + 0.5);
     if (ns < 1) ns = 1;
     if (ns > 256) ns = 256;
     if (ns > nk[i]) ns = nk[i];
     const long long per = kfac::ceil_div(nk[i], ns);
     s.nsplit = (int)kfac::ceil_div(nk[i], per);
     s.klen = per * KT;
-    s.direct = s.nsplit == 1 ? 1 : 0;
+    s.direct = (s.nsplit == 1 && !macro) ? 1 : 0;   // the macro-tile kernel always writes partial tiles
     s.part_off = (long long)off;
     const size_t slot = (size_t)s.ntile * s.bm * s.bm + (size_t)s.tiles * s.bm;
     if (!s.direct) off += (size_t)s.nsplit * slot;
-    for (int w = 0; w < s.ntile * s.nsplit; ++w) natural[kind_of[i]].push_back(make_int2(i, w));
+    const int mt = (s.tiles + 1) / 2;
+    const int per_slice = macro ? mt * (mt + 1) / 2 : s.ntile;
+    for (int w = 0; w < per_slice * s.nsplit; ++w) natural[kind_of[i]].push_back(make_int2(i, w));
     if (!s.direct) {
       const int sub = kfac::ceil_div(items[i].c, 64);
       for (int b = 0; b < sub * (sub + 1) / 2; ++b) fin.push_back(make_int2(i, b));
@@ -1292,16 +1415,35 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   const GroupItemDyn *dy = static_cast<const GroupItemDyn *>(dyn_dev);
   const int2 *tasks = group->d_tasks.as<const int2>();
   using Kern = void (*)(const GroupItemStatic *, const GroupItemDyn *, const int2 *, float *);
-  static const Kern kerns[kGroupKinds] = {
+  static const Kern kerns[kMacroKind0] = {
       syrk_group_kernel<1, LoaderKC<64, true>>,   syrk_group_kernel<1, LoaderKC<64, false>>,
       syrk_group_kernel<1, LoaderKS<64, true>>,   syrk_group_kernel<1, LoaderKS<64, false>>,
       syrk_group_kernel<2, LoaderKC<128, true>>,  syrk_group_kernel<2, LoaderKC<128, false>>,
       syrk_group_kernel<2, LoaderKS<128, true>>,  syrk_group_kernel<2, LoaderKS<128, false>>};
-  for (int k = 0; k < kGroupKinds; ++k) {
+  for (int k = 0; k < kMacroKind0; ++k) {
     if (group->ntask[k] == 0) continue;
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
     hipLaunchKernelGGL(kerns[k], dim3(group->ntask[k]), dim3(THREADS), 0, s, st, dy,
                        tasks + group->task0[k], base);
+  }
+  static const Kern macro_kerns[2] = {syrk_macro_kernel<LoaderKC<128, true>>,
+                                      syrk_macro_kernel<LoaderKC<128, false>>};
+  static std::once_flag macro_attr;
+  static hipError_t macro_attr_rc = hipSuccess;
+  std::call_once(macro_attr, [&] {
+    for (Kern f : macro_kerns) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(f),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               (int)kMacroLdsBytes);
+      if (e != hipSuccess) macro_attr_rc = e;
+    }
+  });
+  KFAC_HIP_CHECK(macro_attr_rc);
+  for (int k = kMacroKind0; k < kGroupKinds; ++k) {
+    if (group->ntask[k] == 0) continue;
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
+    hipLaunchKernelGGL(macro_kerns[k - kMacroKind0], dim3(group->ntask[k]), dim3(kMacroThreads),
+                       kMacroLdsBytes, s, st, dy, tasks + group->task0[k], base);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (group->nftask > 0) {

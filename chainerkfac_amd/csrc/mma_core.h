@@ -46,6 +46,11 @@ __device__ __forceinline__ float gload1(const float *base, unsigned byte_off) {
   return *(const KFAC_GLOBAL_AS float *)((const KFAC_GLOBAL_AS char *)base + byte_off);
 }
 
+// Thread index inside a team of THREADS threads.  The workgroups of this engine
+// have THREADS threads, except those of the macro-tile covariance kernel, whose
+// four teams each stage and multiply like one such workgroup.
+__device__ __forceinline__ int team_tid() { return (int)(threadIdx.x & (THREADS - 1)); }
+
 template <int ROWS>
 struct Panel {
   static constexpr int kRowKStride = KT + 1;
@@ -98,7 +103,7 @@ struct LoaderKC {
   bool full_rows;
 
   __device__ __forceinline__ void init(float *, int row0) {
-    const int rr = threadIdx.x >> 3;
+    const int rr = team_tid() >> 3;
     rowvalid = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -111,7 +116,7 @@ struct LoaderKC {
   }
 
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
-    const unsigned kq = (threadIdx.x & 7) * 4;
+    const unsigned kq = (team_tid() & 7) * 4;
     const long long kgl = k0 + kq;
     const bool full_k = k0 + KT <= k_end;
     r.fast = full_rows && full_k;
@@ -145,8 +150,8 @@ struct LoaderKC {
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
-    const int kq = (threadIdx.x & 7) * 4;
-    const int rr = threadIdx.x >> 3;
+    const int kq = (team_tid() & 7) * 4;
+    const int rr = team_tid() >> 3;
     if (r.fast) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
@@ -198,12 +203,12 @@ struct LoaderKC<ROWS, false> {
   unsigned last_off;
 
   __device__ __forceinline__ void init(float *, int row0) {
-    first_row = row0 + (threadIdx.x >> 5);
+    first_row = row0 + (team_tid() >> 5);
     last_off = (unsigned)(rows_valid > 0 ? rows_valid - 1 : 0) * row_stride;
   }
 
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
-    const long long kg = k0 + (threadIdx.x & 31);
+    const long long kg = k0 + (team_tid() & 31);
     r.kvalid = kg < k_end;
     const unsigned kc = r.kvalid ? (unsigned)kg : 0u;
     unsigned koff = kc;
@@ -230,7 +235,7 @@ struct LoaderKC<ROWS, false> {
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
-    float *p = lds + (threadIdx.x >> 5) * Panel<ROWS>::kRowKStride + (threadIdx.x & 31);
+    float *p = lds + (team_tid() >> 5) * Panel<ROWS>::kRowKStride + (team_tid() & 31);
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       const int row = first_row + 8 * i;
@@ -265,13 +270,13 @@ struct LoaderKS {
   bool full_rows;
 
   __device__ __forceinline__ void init(float *, int row0) {
-    row = row0 + (threadIdx.x % RQ) * 4;
+    row = row0 + (team_tid() % RQ) * 4;
     quad_ok = VEC && row + 3 < rows_valid;
     full_rows = VEC && row0 + ROWS <= rows_valid;
   }
 
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
-    const int kk = threadIdx.x / RQ;
+    const int kk = team_tid() / RQ;
     const bool full_k = k0 + KT <= k_end;
     r.fast = full_rows && full_k;
     r.kmask = 0;
@@ -304,8 +309,8 @@ struct LoaderKS {
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
-    const int rq = (threadIdx.x % RQ) * 4;
-    const int kk = threadIdx.x / RQ;
+    const int rq = (team_tid() % RQ) * 4;
+    const int kk = team_tid() / RQ;
     if (r.fast) {
 #pragma unroll
       for (int i = 0; i < NV; ++i)
@@ -354,7 +359,7 @@ struct LoaderIM {
   // Build the per-row table for panel rows [row0, row0 + ROWS).
   __device__ __forceinline__ void init(float *lds_table, int row0) {
     table = reinterpret_cast<int2 *>(lds_table);
-    for (int t = threadIdx.x; t < ROWS; t += THREADS) {
+    for (int t = team_tid(); t < ROWS; t += THREADS) {
       const int row = row0 + t;
       int2 e;
       if (row < d_patch) {
@@ -373,8 +378,8 @@ struct LoaderIM {
   }
 
   __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
-    const int k = threadIdx.x & 31;
-    const int rr = threadIdx.x >> 5;
+    const int k = team_tid() & 31;
+    const int rr = team_tid() >> 5;
     const long long kg = k0 + k;
     const bool kok = kg < k_end;
     const unsigned kc = kok ? (unsigned)kg : 0u;
@@ -399,8 +404,8 @@ struct LoaderIM {
   }
 
   __device__ __forceinline__ void store(const Regs &r, float *lds) const {
-    const int k = threadIdx.x & 31;
-    const int rr = threadIdx.x >> 5;
+    const int k = team_tid() & 31;
+    const int rr = team_tid() >> 5;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
       lds[(rr + 8 * i) * Panel<ROWS>::kRowKStride + k] = ((r.use >> i) & 1u) ? r.v[i] : 0.f;

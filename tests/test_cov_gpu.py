@@ -204,6 +204,51 @@ def test_grouped_launch_matches_the_single_calls():
     np.testing.assert_allclose(outs[0].cpu().numpy(), O.conv_G(gy) * (0.25 * 14 * 14 / 4), rtol=1e-4, atol=1e-4)
 
 
+def test_grouped_launch_macro_tiles():
+    """Slabs of several 128-tiles with a long reduction take the macro-tile kernel (four teams
+    per workgroup, 2 x 2 tiles from four panels staged once): an even and an odd number of
+    tiles, a ragged last tile, 16-byte and scalar loads, a ones column, accumulation; against
+    float64 and the single-call entry point."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(29)
+
+    def t(*shape):
+        return torch.from_numpy(r.standard_normal(shape).astype(np.float32)).cuda()
+
+    cases = [
+        # input, ones, stride, alpha, beta
+        (t(8, 256, 28, 28), False, 1, 1.0 / 8, 0.0),     # 2 tiles: one macro-tile on the diagonal
+        (t(4, 384, 28, 28), True, 1, 0.25, 0.0),         # 3 tiles: ragged last macro row, ones column
+        (t(6, 500, 20, 20), True, 1, 0.5, 1.0),          # 4 tiles, ragged last tile, accumulation
+        (t(8, 272, 15, 15), True, 1, 0.125, 0.0),        # 225 pixels: scalar loads
+        (t(4, 300, 30, 30), False, 2, 0.25, 0.0),        # strided 1x1: scalar loads, 3 tiles
+        (t(2, 1024, 16, 16), False, 1, 0.5, 0.0),        # 8 tiles: 10 macro-tiles per slice
+    ]
+    pending = ops.PendingCovs()
+    outs, refs, singles = [], [], []
+    for x, ones, stride, alpha, beta in cases:
+        d = x.shape[1] + int(ones)
+        prev = t(d, d)
+        prev = (prev + prev.T).contiguous()
+        out = prev.clone()
+        sub = x.cpu().numpy()[:, :, ::stride, ::stride]
+        P = sub.transpose(0, 2, 3, 1).reshape(-1, x.shape[1]).astype(np.float64)
+        if ones:
+            P = np.concatenate([P, np.ones((P.shape[0], 1))], axis=1)
+        refs.append(alpha * (P.T @ P) + beta * prev.cpu().numpy().astype(np.float64))
+        singles.append(ops.cov_conv_a(x, 1, stride, 0, ones, alpha, beta, prev.clone()))
+        pending.add(ops.COV_SLAB, x, ones, out, alpha, beta, stride)
+        outs.append(out)
+    pending.flush()
+    torch.cuda.synchronize()
+    for out, ref, single in zip(outs, refs, singles):
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all()
+        assert np.linalg.norm(got - ref) <= 1e-4 * np.linalg.norm(ref)
+        assert np.array_equal(got, got.T)
+        assert np.linalg.norm(got - single.cpu().numpy()) <= 1e-5 * np.linalg.norm(ref)
+
+
 def test_grouped_launch_alternating_arguments_under_capture():
     """Accumulation calls one group with beta = 0, then beta = 1: both argument tables stay
     resident, so a graph can be captured over the pair after one eager pass, and every
