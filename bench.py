@@ -364,7 +364,7 @@ def run_step_config(args, name, cfg):
         'data': 'synthetic',
         'config': {'workload': cfg['workload'], 'name': name, 'batch': batch,
                    'factors': len(W.all_factor_dims(layers)), 'damping': cfg['damping'], 'acc_iters': acc_iters,
-                   'hip_graph': not args.no_graph, 'lanes': args.lanes,
+                   'hip_graph': not args.no_graph, 'lanes': args.lanes, 'macro_tiles': bool(args.macro_tiles),
                    'bn_inverse': 'woodbury rank-{} ({} blocks)'.format(batch, len(lowrank)) if lowrank else 'dense'},
         # rates use the flops actually executed; the *_reference_work entries divide the work of the
         # reference's algorithm (every factor inverted densely) by the same times
@@ -895,6 +895,9 @@ def main():
                     help='skip the second measurement of c3 with all batch-norm blocks inverted densely')
     ap.add_argument('--lanes', type=int, default=3,
                     help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
+    ap.add_argument('--macro-tiles', action='store_true',
+                    help='grouped covariance launches use the macro-tile kernel for slabs of several 128-tiles '
+                         '(KFAC_GROUP_MACRO=1: less HBM traffic, about 1 %% slower)')
     ap.add_argument('--per-layer', metavar='PATH', default=None,
                     help='also time the covariance kernels of every distinct layer shape alone and write a '
                          'markdown roofline table to PATH')
@@ -924,6 +927,8 @@ def main():
     if args.summarize_mfma:
         summarize_mfma(args.summarize_mfma[0], args.summarize_mfma[1], args.profiled_command)
         return
+    if args.macro_tiles:
+        os.environ['KFAC_GROUP_MACRO'] = '1'
     cfg = configs()[args.config]
     if args.config == 'c4':
         result, _ = run_inverse_config(args, args.config, cfg)

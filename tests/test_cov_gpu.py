@@ -204,12 +204,14 @@ def test_grouped_launch_matches_the_single_calls():
     np.testing.assert_allclose(outs[0].cpu().numpy(), O.conv_G(gy) * (0.25 * 14 * 14 / 4), rtol=1e-4, atol=1e-4)
 
 
-def test_grouped_launch_macro_tiles():
-    """Slabs of several 128-tiles with a long reduction take the macro-tile kernel (four teams
+def test_grouped_launch_macro_tiles(monkeypatch):
+    """With KFAC_GROUP_MACRO=1 (read when a group is created), slabs of several 128-tiles with
+    a long reduction take the macro-tile kernel (four teams
     per workgroup, 2 x 2 tiles from four panels staged once): an even and an odd number of
     tiles, a ragged last tile, 16-byte and scalar loads, a ones column, accumulation; against
     float64 and the single-call entry point."""
     from chainerkfac_amd import ops
+    monkeypatch.setenv('KFAC_GROUP_MACRO', '1')
     r = np.random.default_rng(29)
 
     def t(*shape):
