@@ -59,6 +59,9 @@ PROTOTYPES = {
     'kfac_bn_lowrank_plan_destroy': (c_int, [c_vp]),
     'kfac_bn_lowrank_inverse_batched_f32': (c_int, [c_vp, c_vpp, c_vpp, c_dp, c_dp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_add_diag_f32': (c_int, [c_vp, c_int, c_int, c_d, c_d, c_vp]),
+    'kfac_diag_batch_create': (c_int, [c_vp]),
+    'kfac_diag_batch_destroy': (c_int, [c_vp]),
+    'kfac_add_diag_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     'kfac_precond_conn_workspace_bytes': (c_sz, [c_int, c_int]),
     'kfac_precond_conn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_precond_group_create': (c_int, [c_int, c_i32p, c_i32p, c_i32p, c_vpp]),

@@ -1,5 +1,8 @@
 // Small bandwidth-bound helpers of the K-FAC step: axpby (moving average and
 // unfused accumulation), diagonal damping and the momentum update rule.
+#include <new>
+#include <vector>
+
 #include "common.h"
 
 namespace kfac {
@@ -103,6 +106,22 @@ __global__ __launch_bounds__(kThreads) void add_diag_kernel(
   }
 }
 
+struct DiagItem {
+  float *M;
+  int d, split;
+  double v0, v1;
+};
+
+// blockIdx.y = matrix, blockIdx.x = chunk of its diagonal
+__global__ __launch_bounds__(kThreads) void add_diag_batched_kernel(const DiagItem *__restrict__ items) {
+  const DiagItem it = items[blockIdx.y];
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < it.d) {
+    const long long at = (long long)i * it.d + i;
+    it.M[at] = (float)((double)it.M[at] + (i < it.split ? it.v0 : it.v1));
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void momentum_kernel(
     float *__restrict__ p, float *__restrict__ v, const float *__restrict__ g,
     long long n, float lr, float momentum) {
@@ -141,6 +160,48 @@ extern "C" int kfac_add_diag_f32(float *M, int d, int split, double v0, double v
   KFAC_REQUIRE(M != nullptr, "M is null");
   hipLaunchKernelGGL(add_diag_kernel, dim3(kfac::ceil_div(d, kThreads)), dim3(kThreads),
                      0, kfac::as_stream(stream), M, d, split, v0, v1);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+struct kfac_diag_batch {
+  std::vector<DiagItem> host;
+  kfac::DevTableRing table;
+};
+
+extern "C" int kfac_diag_batch_create(kfac_diag_batch_t *out) {
+  KFAC_REQUIRE(out != nullptr, "batch_out is null");
+  *out = new (std::nothrow) kfac_diag_batch;
+  if (!*out) return kfac::fail(KFAC_ENOMEM, "out of host memory");
+  return KFAC_OK;
+}
+
+extern "C" int kfac_diag_batch_destroy(kfac_diag_batch_t batch) {
+  delete batch;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_add_diag_batched_f32(kfac_diag_batch_t batch, int count, float *const *mats,
+                                         const int32_t *dims, const int32_t *splits,
+                                         const double *v0, const double *v1, void *stream) {
+  KFAC_REQUIRE(batch != nullptr, "batch is null");
+  KFAC_REQUIRE(count >= 0, "count < 0");
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(mats && dims && splits && v0 && v1, "null table");
+  KFAC_REQUIRE(count <= 65535, "more than 65535 matrices");
+  batch->host.resize(count);
+  int max_d = 0;
+  for (int i = 0; i < count; ++i) {
+    KFAC_REQUIRE(dims[i] >= 0 && (dims[i] == 0 || mats[i]), "matrix %d: bad dimension or null pointer", i);
+    batch->host[i] = DiagItem{mats[i], dims[i], splits[i], v0[i], v1[i]};
+    max_d = dims[i] > max_d ? dims[i] : max_d;
+  }
+  if (max_d == 0) return KFAC_OK;
+  hipStream_t s = kfac::as_stream(stream);
+  const void *dev = nullptr;
+  if (int rc = batch->table.set(batch->host.data(), sizeof(DiagItem) * (size_t)count, s, &dev)) return rc;
+  hipLaunchKernelGGL(add_diag_batched_kernel, dim3(kfac::ceil_div(max_d, kThreads), count), dim3(kThreads),
+                     0, s, static_cast<const DiagItem *>(dev));
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }

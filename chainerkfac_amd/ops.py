@@ -233,6 +233,50 @@ def add_diag(M, v0, v1=None, split=None, stream=None):
     return M
 
 
+class _DiagBatch(object):
+    def __init__(self):
+        h = ctypes.c_void_p()
+        _lib.check(_lib.load().kfac_diag_batch_create(ctypes.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        try:
+            h, self._h = self._h, None
+            if h is not None:
+                _lib._lib.kfac_diag_batch_destroy(h)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+
+_diag_batches = None
+
+
+def add_diag_batched(mats, v0s, v1s=None, splits=None, stream=None):
+    """``add_diag`` for a list of square matrices in one launch: diag(M_i)[j] += v0s[i] for
+    j < splits[i] else v1s[i]."""
+    global _diag_batches
+    if not mats:
+        return mats
+    dims = []
+    for M in mats:
+        _dev.require_gpu_tensor(M, 'M')
+        if M.ndim != 2 or M.shape[0] != M.shape[1]:
+            raise ValueError('M must be square')
+        dims.append(M.shape[0])
+    if v1s is None:
+        v1s, splits = v0s, dims
+    if not (len(v0s) == len(v1s) == len(splits) == len(mats)):
+        raise ValueError('one value pair and one split per matrix')
+    if _diag_batches is None:
+        _diag_batches = _PlanCache(16)
+    ptrs = tuple(M.data_ptr() for M in mats)
+    batch = _diag_batches.get(ptrs, _DiagBatch)
+    _lib.check(_lib.load().kfac_add_diag_batched_f32(
+        batch._h, len(mats), _lib.ptr_array(ptrs), _lib.i32_array(dims), _lib.i32_array(splits),
+        _lib.f64_array(v0s), _lib.f64_array(v1s), _dev.stream_handle(stream)))
+    return mats
+
+
 class InversePlan(object):
     """Schedule for inverting a fixed list of SPD matrix sizes together."""
 

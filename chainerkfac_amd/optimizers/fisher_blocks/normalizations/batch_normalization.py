@@ -153,15 +153,20 @@ class FisherBlockBatchNormalization(FisherBlock):
             return [d_beta * np.ones(beta.size)]
         return [np.hstack((d_gamma * np.ones(gamma.size), d_beta * np.ones(beta.size)))]
 
-    def damp(self):
+    def damp_args(self):
+        """``(F, v0, v1, split)``: the damping adds v0 to the first ``split`` diagonal
+        entries of F and v1 to the others."""
         d_gamma, d_beta = self._diag_pair()
         F = self.cov_emas[0]
         if d_beta is None:
-            ops.add_diag(F, d_gamma)
-        elif d_gamma is None:
-            ops.add_diag(F, d_beta)
-        else:
-            ops.add_diag(F, d_gamma, d_beta, split=self.link.gamma.size)
+            return F, d_gamma, d_gamma, F.shape[0]
+        if d_gamma is None:
+            return F, d_beta, d_beta, F.shape[0]
+        return F, d_gamma, d_beta, self.link.gamma.size
+
+    def damp(self):
+        F, v0, v1, split = self.damp_args()
+        ops.add_diag(F, v0, v1, split=split)
 
     def update_kfgrads(self):
         self.check_attr('invs')

@@ -472,8 +472,17 @@ class KFAC(object):
             else:
                 for fb in conn:
                     fb.damp()
+        # the other blocks' damping in one launch where they can say what it adds
+        batched = [fb for fb in other if hasattr(fb, 'damp_args')]
+        if len(batched) > 1:
+            args = [fb.damp_args() for fb in batched]
+            ops.add_diag_batched([a[0] for a in args], [a[1] for a in args], [a[2] for a in args],
+                                 [a[3] for a in args])
+        else:
+            batched = []
         for fb in other:
-            fb.damp()
+            if fb not in batched:
+                fb.damp()
         # batch-norm blocks whose factor is this step's rank-n matrix U^T U / n:
         # Woodbury inverse (the same dense result, an n x n Cholesky each)
         lowrank = []

@@ -261,6 +261,18 @@ int kfac_bn_lowrank_inverse_batched_f32(kfac_bn_lowrank_plan_t plan,
 int kfac_add_diag_f32(float *M, int d, int split, double v0, double v1,
                       void *stream);
 
+/* The same for `count` matrices in one launch (the damping of all batch-norm
+ * blocks of a network: the loop of update_invs, fisher_block.py:165-179, over
+ * normalizations/batch_normalization.py:133-157).  The batch object keeps the
+ * argument table on the device; the last four distinct tables stay resident
+ * (under stream capture only a resident table can be used). */
+typedef struct kfac_diag_batch *kfac_diag_batch_t;
+int kfac_diag_batch_create(kfac_diag_batch_t *batch_out);
+int kfac_diag_batch_destroy(kfac_diag_batch_t batch);
+int kfac_add_diag_batched_f32(kfac_diag_batch_t batch, int count, float *const *mats,
+                              const int32_t *dims, const int32_t *splits, const double *v0,
+                              const double *v1, void *stream);
+
 /* ------------------------------------------------------------------------
  * (3) Preconditioning
  * --------------------------------------------------------------------- */

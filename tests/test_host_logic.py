@@ -13,7 +13,7 @@ def test_lanes_disabled_runs_inline():
     lanes.join()   # nothing to wait for
 
 
-def test_resnet50_workload_matches_the_survey_totals():
+def test_resnet50_workload_totals():
     from chainerkfac_amd import workloads as W
     layers = W.resnet50_v1()
     dims = W.all_factor_dims(layers)

@@ -152,6 +152,37 @@ def test_add_diag_batch_norm_halves():
 
 
 @pytest.mark.gpu
+def test_add_diag_batched_matches_the_single_calls():
+    """One launch for the damping of many blocks (ragged sizes, gamma+beta, one half only):
+    bit-identical to the oracle's in-place damping and to a second call with other values."""
+    from chainerkfac_amd import ops
+    sizes = [(10, 6), (1, 1), (300, 150), (64, 64), (513, 0)]
+    mats, refs, v0s, v1s, splits = [], [], [], [], []
+    for i, (d, split) in enumerate(sizes):
+        F = spd(d, 20 + i)
+        (dv,) = O.bn_diagvals(max(split, 1), max(d - split, 1), damping=2.5e-4 * (i + 1), stab_coeff=16.0, l2_beta=0.5)
+        v0, v1 = float(dv[0]), float(dv[-1])
+        ref = F.copy()
+        diag = np.where(np.arange(d) < split, v0, v1)
+        O.damp_inplace(ref, diag)
+        mats.append(torch.from_numpy(F).cuda())
+        refs.append(ref)
+        v0s.append(v0)
+        v1s.append(v1)
+        splits.append(split)
+    ops.add_diag_batched(mats, v0s, v1s, splits)
+    for M, ref in zip(mats, refs):
+        assert np.array_equal(M.cpu().numpy(), ref)
+    # the same matrices again with other values: the argument table is replaced
+    ops.add_diag_batched(mats, [1.0] * len(mats))
+    for M, ref in zip(mats, refs):
+        want = ref.copy()
+        O.damp_inplace(want, np.ones(ref.shape[0]))
+        assert np.array_equal(M.cpu().numpy(), want)
+    assert ops.add_diag_batched([], []) == []
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize('n', [32, 7, 1])
 def test_bn_lowrank_inverse_matches_dense_oracle(n):
     """(U^T U / n + D)^-1 by the Woodbury identity against the dense float64 inverse and the
