@@ -79,6 +79,10 @@ struct InvTables {
   const float *const *in;    // [count] sorted slot -> input matrix
   float *const *out;         // [count]
   const int *dim;            // [count]
+  const int *core;           // [count] rows of the tiled part: dim, or dim - 1 for a bordered matrix
+  const int *orig;           // [count] sorted slot -> caller index
+  const long long *vec_off;  // [count] bordered matrix: float offset of its vectors a | y | w (core floats
+                             // each) and the scalars alpha, S, 1/S behind them; -1 otherwise
   const int *nt;             // [count] tiles per side
   const long long *ws_off;   // [count] float offset of the padded matrix
   const int *tile_cs;        // [count+1] cumulative lower-tile counts (copy-in)
@@ -358,7 +362,7 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
   const int s = find_slot(tb.tile_cs, count, blockIdx.x);
   int I, J;
   tri_decode(blockIdx.x - tb.tile_cs[s], I, J);
-  const int d = tb.dim[s];
+  const int d = tb.dim[s], dc = tb.core[s];
   const float *__restrict__ src = tb.in[s];
   float *__restrict__ dst = tile_ptr(tb, s, I, J);
   const int c4 = (threadIdx.x & 31) * 4;
@@ -373,10 +377,17 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
     for (int e = 0; e < 4; ++e) {
       const int ce = c + e;
       float x = (r == ce) ? 1.f : 0.f;
-      if (r < d && ce < d) x = src[(long long)r * d + ce];
+      if (r < dc && ce < dc) x = src[(long long)r * d + ce];
       v[e] = x;
     }
     *reinterpret_cast<float4 *>(dst + rl * NB + c4) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+  // a bordered matrix: its last column and corner go beside the tiles
+  const long long vo = tb.vec_off[s];
+  if (vo >= 0 && I == J) {
+    float *vec = tb.ws + vo;
+    if (threadIdx.x < NB) vec[I * NB + threadIdx.x] = src[(long long)(I * NB + threadIdx.x) * d + d - 1];
+    if (I == 0 && threadIdx.x == 0) vec[3 * (long long)dc] = src[(long long)(d - 1) * d + d - 1];   // scal[0]
   }
 }
 
@@ -572,6 +583,141 @@ __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int ta
   update_role<2>(tb, t, lds);
 }
 
+// ---------------------------------------------------------------------------
+// Bordered matrices.  The Kronecker factor of a layer with a bias has d = 9C + 1
+// or C + 1 rows: one more than a multiple of the tile size for every
+// power-of-two C, which as a tiled matrix pays a whole extra tile row and column
+// (4609 -> 37 tiles instead of 36; 11 % of the tile products of ResNet-50's
+// factors).  Such a matrix M = [A a; a^T alpha] is inverted from its leading
+// block instead, which the sweep above factors as A^-1 = U U^T:
+//     y = U^T a,  S = alpha - y^T y  (the last pivot of M's Cholesky, squared),
+//     w = U y = A^-1 a,
+//     M^-1 = [A^-1 + w w^T / S, -w / S; -w^T / S, 1 / S].
+// y and w are two tile-wise matrix-vector products (HBM-bound, the U tiles read
+// once each); the rank-1 term is added to the accumulators of the final product.
+// ---------------------------------------------------------------------------
+
+// Both products are cut into chunks of kBorderChunk tiles along the summed index, one
+// workgroup each, whose partial vectors are added in a fixed order afterwards.
+constexpr int kBorderChunk = 6;
+
+// vectors of a bordered matrix in the workspace: a | y | w | scalars (64) | partial vectors
+struct BorderVecs {
+  float *a, *y, *w, *scal, *part;
+  int dc;
+};
+__device__ __forceinline__ BorderVecs border_vecs(const InvTables &tb, int s) {
+  BorderVecs v;
+  v.dc = tb.core[s];
+  v.a = tb.ws + tb.vec_off[s];
+  v.y = v.a + v.dc;
+  v.w = v.y + v.dc;
+  v.scal = v.w + v.dc;
+  v.part = v.scal + 64;
+  return v;
+}
+
+// partial y_k = sum_{i in chunk, i <= k} U(i,k)^T a_i; task = (matrix, k | chunk << 16)
+__global__ __launch_bounds__(256) void border_y_kernel(InvTables tb, const int2 *__restrict__ tasks) {
+  __shared__ float as[NB];
+  __shared__ float part[8][NB];
+  const int s = tasks[blockIdx.x].x;
+  const int k = tasks[blockIdx.x].y & 0xffff, ch = tasks[blockIdx.x].y >> 16;
+  const BorderVecs v = border_vecs(tb, s);
+  const int c4 = (threadIdx.x & 31) * 4, rg = threadIdx.x >> 5;   // 4 columns, rows rg*16 .. +15
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int i_end = min((ch + 1) * kBorderChunk, k + 1);
+  for (int i = ch * kBorderChunk; i < i_end; ++i) {
+    __syncthreads();
+    if (threadIdx.x < NB) as[threadIdx.x] = v.a[i * NB + threadIdx.x];
+    __syncthreads();
+    const float *U = tile_ptr(tb, s, i, k) + (rg * 16) * NB + c4;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float4 u = *reinterpret_cast<const float4 *>(U + r * NB);
+      const float av = as[rg * 16 + r];
+      acc.x += u.x * av;
+      acc.y += u.y * av;
+      acc.z += u.z * av;
+      acc.w += u.w * av;
+    }
+  }
+  *reinterpret_cast<float4 *>(&part[rg][c4]) = acc;
+  __syncthreads();
+  if (threadIdx.x < NB) {
+    float t = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) t += part[g][threadIdx.x];
+    v.part[(long long)ch * v.dc + k * NB + threadIdx.x] = t;
+  }
+}
+
+// y = sum of its partial vectors; S = alpha - y^T y in float64; info = d when S is not positive
+__global__ __launch_bounds__(256) void border_s_kernel(InvTables tb, const int *__restrict__ slots) {
+  __shared__ double red[256];
+  const int s = slots[blockIdx.x];
+  const BorderVecs v = border_vecs(tb, s);
+  double sum = 0.0;
+  for (int j = threadIdx.x; j < v.dc; j += 256) {
+    const int nch = (j / NB) / kBorderChunk + 1;   // chunks with i <= k
+    float t = 0.f;
+    for (int ch = 0; ch < nch; ++ch) t += v.part[(long long)ch * v.dc + j];
+    v.y[j] = t;
+    sum += (double)t * (double)t;
+  }
+  red[threadIdx.x] = sum;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const double S = (double)v.scal[0] - red[0];
+    v.scal[1] = (float)S;
+    v.scal[2] = (float)(1.0 / S);
+    int *pinfo = &tb.info[tb.orig[s]];
+    if (!(S > 0.0) && *pinfo == 0) *pinfo = tb.dim[s];
+  }
+}
+
+// partial w_i = sum_{k in chunk, k >= i} U(i,k) y_k; task = (matrix, i | chunk << 16); two threads per row
+__global__ __launch_bounds__(256) void border_w_kernel(InvTables tb, const int2 *__restrict__ tasks) {
+  __shared__ float ys[NB];
+  const int s = tasks[blockIdx.x].x;
+  const int i = tasks[blockIdx.x].y & 0xffff, ch = tasks[blockIdx.x].y >> 16;
+  const BorderVecs v = border_vecs(tb, s);
+  const int T = tb.nt[s];
+  const int r = threadIdx.x >> 1, half = threadIdx.x & 1;
+  float acc = 0.f;
+  const int k_end = min((ch + 1) * kBorderChunk, T);
+  for (int k = max(i, ch * kBorderChunk); k < k_end; ++k) {
+    __syncthreads();
+    if (threadIdx.x < NB) ys[threadIdx.x] = v.y[k * NB + threadIdx.x];
+    __syncthreads();
+    const float4 *U = reinterpret_cast<const float4 *>(tile_ptr(tb, s, i, k) + r * NB + half * (NB / 2));
+#pragma unroll
+    for (int q = 0; q < NB / 8; ++q) {
+      const float4 u = U[q];
+      const float *yv = ys + half * (NB / 2) + 4 * q;
+      acc += u.x * yv[0] + u.y * yv[1] + u.z * yv[2] + u.w * yv[3];
+    }
+  }
+  acc += __shfl_xor(acc, 1, 64);
+  if (half == 0) v.part[(long long)ch * v.dc + i * NB + r] = acc;
+}
+
+// w = sum of its partial vectors
+__global__ __launch_bounds__(256) void border_wsum_kernel(InvTables tb, const int *__restrict__ slots) {
+  const int s = slots[blockIdx.x];
+  const BorderVecs v = border_vecs(tb, s);
+  const int nch_all = (tb.nt[s] - 1) / kBorderChunk + 1;
+  for (int j = threadIdx.x; j < v.dc; j += 256) {
+    float t = 0.f;
+    for (int ch = (j / NB) / kBorderChunk; ch < nch_all; ++ch) t += v.part[(long long)ch * v.dc + j];
+    v.w[j] = t;
+  }
+}
+
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
 // One task per tile; the table deals whole tile rows to XCDs (see the plan).
 __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int task0) {
@@ -580,7 +726,8 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int tas
   if (t.K == 0) return;   // padding of an XCD's shorter list
   const int s = (int)t.c_off;
   const int I = t.flags & 0xffff, J = t.flags >> 16;
-  const int d = tb.dim[s];
+  const int d = tb.dim[s], dc = tb.core[s];
+  const long long vo = tb.vec_off[s];
   float *out = tb.out[s];
   const OperandRows la{tb.ws + t.a_off}, lb{tb.ws + t.b_off};
   floatx16 acc[2][2];
@@ -589,8 +736,31 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int tas
     tile_mainloop<true, 4>(la, lb, t.K, lds, acc);
   else
     tile_mainloop<false, 4>(la, lb, t.K, lds, acc);
+  if (vo >= 0) {
+    // bordered matrix: + w w^T / S on the leading block, -w / S in the last row and column
+    const BorderVecs bv = border_vecs(tb, s);
+    const float sigma = bv.scal[2];
+    const float *wi = bv.w + I * NB, *wj = bv.w + J * NB;
+#pragma unroll
+    for (int im = 0; im < 2; ++im)
+#pragma unroll
+      for (int in = 0; in < 2; ++in)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+          const int row = ((wave >> 1) * 2 + im) * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          const int col = ((wave & 1) * 2 + in) * 32 + (lane & 31);
+          acc[im][in][v] += sigma * wi[row] * wj[col];
+        }
+    if (I == J && threadIdx.x < NB) {
+      const float b = -sigma * wi[threadIdx.x];
+      out[(long long)(d - 1) * d + I * NB + threadIdx.x] = b;
+      out[(long long)(I * NB + threadIdx.x) * d + d - 1] = b;
+      if (I == 0 && threadIdx.x == 0) out[(long long)(d - 1) * d + d - 1] = sigma;
+    }
+  }
   // through an LDS transpose, so that the mirror is written in row segments too
-  write_tile<2>(acc, lds, I, J, d, d, 1.f, 0.f, out);
+  write_tile<2>(acc, lds, I, J, dc, d, 1.f, 0.f, out);
 }
 
 // Dynamic LDS.  The trailing update ("rest") asks for 81 KB although it uses 74:
@@ -654,6 +824,8 @@ struct kfac_inverse_plan {
   }
   int total_tiles = 0;
   int lauum_task0 = 0, lauum_count = 0;
+  int nborder = 0, nborder_y = 0, nborder_w = 0;   // bordered matrices; tasks of their two products
+  kfac::DevTable d_core, d_orig, d_vec, d_border_slots, d_border_tiles, d_border_w_tiles;
   size_t ws_floats = 0;            // padded matrices
   std::vector<const void *> in_sorted, out_sorted;
   kfac::DevTable d_in, d_out, d_dim, d_nt, d_off, d_tile, d_tasks;
@@ -706,15 +878,39 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   std::vector<long long> off(count);
   p->nt.resize(count);
   size_t total = 0;
+  // matrices of 128 m + 1 rows are inverted from their leading 128 m x 128 m block
+  // (KFAC_INVERSE_BORDER=0 tiles them whole, for comparisons)
+  bool border_on = true;
+  if (const char *e = getenv("KFAC_INVERSE_BORDER")) border_on = atoi(e) != 0;
+  std::vector<int> core(count);
+  std::vector<long long> vec_off(count, -1);
+  std::vector<int> border_slots;
+  std::vector<int2> border_tiles, border_w_tiles;
   for (int s = 0; s < count; ++s) {
     dim[s] = dims[p->order[s]];
-    const int T = kfac::ceil_div(dim[s], NB);
+    core[s] = (border_on && dim[s] > NB && dim[s] % NB == 1) ? dim[s] - 1 : dim[s];
+    const int T = kfac::ceil_div(core[s], NB);
     p->nt[s] = T;
     off[s] = (long long)total;
     total += (size_t)T * NB * T * NB;
     tile_cs[s + 1] = tile_cs[s] + T * (T + 1) / 2;
     panel_cs[s + 1] = panel_cs[s] + (T - 1);
   }
+  for (int s = 0; s < count; ++s) {
+    if (core[s] == dim[s]) continue;
+    vec_off[s] = (long long)total;
+    const int nch = (p->nt[s] - 1) / kBorderChunk + 1;
+    total += (size_t)(3 + nch) * core[s] + 64;
+    border_slots.push_back(s);
+    // y: chunks of tile rows i <= k; w: chunks of tile columns k >= i
+    for (int k = 0; k < p->nt[s]; ++k)
+      for (int ch = 0; ch * kBorderChunk <= k; ++ch) border_tiles.push_back(make_int2(s, k | (ch << 16)));
+    for (int i = 0; i < p->nt[s]; ++i)
+      for (int ch = i / kBorderChunk; ch < nch; ++ch) border_w_tiles.push_back(make_int2(s, i | (ch << 16)));
+  }
+  p->nborder = (int)border_slots.size();
+  p->nborder_y = (int)border_tiles.size();
+  p->nborder_w = (int)border_w_tiles.size();
   p->ws_floats = total;
   p->total_tiles = tile_cs[count];
   p->max_t = count ? p->nt[0] : 0;
@@ -833,7 +1029,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
       TileTask r;
       r.c_off = tile_off(s, k, k);
       r.a_off = tile_off(s, k, k0);
-      r.b_off = (long long)p->order[s] | ((long long)dim[s] << 32);
+      r.b_off = (long long)p->order[s] | ((long long)core[s] << 32);
       r.K = k1 >= k0 ? (k1 - k0 + 1) * NB : 0;
       r.flags = k;
       tasks.push_back(r);
@@ -920,6 +1116,14 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     if (rc == KFAC_OK) rc = t.set(h, b, nullptr);
   };
   up(p->d_dim, dim.data(), sizeof(int) * count);
+  up(p->d_core, core.data(), sizeof(int) * count);
+  up(p->d_orig, p->order.data(), sizeof(int) * count);
+  up(p->d_vec, vec_off.data(), sizeof(long long) * count);
+  if (p->nborder > 0) {
+    up(p->d_border_slots, border_slots.data(), sizeof(int) * border_slots.size());
+    up(p->d_border_tiles, border_tiles.data(), sizeof(int2) * border_tiles.size());
+    up(p->d_border_w_tiles, border_w_tiles.data(), sizeof(int2) * border_w_tiles.size());
+  }
   up(p->d_nt, p->nt.data(), sizeof(int) * count);
   up(p->d_off, off.data(), sizeof(long long) * count);
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
@@ -1016,6 +1220,9 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.in = plan->d_in.as<const float *const>();
   tb.out = plan->d_out.as<float *const>();
   tb.dim = plan->d_dim.as<const int>();
+  tb.core = plan->d_core.as<const int>();
+  tb.orig = plan->d_orig.as<const int>();
+  tb.vec_off = plan->d_vec.as<const long long>();
   tb.nt = plan->d_nt.as<const int>();
   tb.ws_off = plan->d_off.as<const long long>();
   tb.tile_cs = plan->d_tile.as<const int>();
@@ -1092,6 +1299,16 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   if (int rc2 = queue_rest()) return rc2;
   if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
   KFAC_HIP_CHECK(hipGetLastError());
+  if (plan->nborder > 0) {
+    const int *slots = plan->d_border_slots.as<const int>();
+    hipLaunchKernelGGL(border_y_kernel, dim3(plan->nborder_y), dim3(256), 0, s, tb,
+                       plan->d_border_tiles.as<const int2>());
+    hipLaunchKernelGGL(border_s_kernel, dim3(plan->nborder), dim3(256), 0, s, tb, slots);
+    hipLaunchKernelGGL(border_w_kernel, dim3(plan->nborder_w), dim3(256), 0, s, tb,
+                       plan->d_border_w_tiles.as<const int2>());
+    hipLaunchKernelGGL(border_wsum_kernel, dim3(plan->nborder), dim3(256), 0, s, tb, slots);
+    KFAC_HIP_CHECK(hipGetLastError());
+  }
   {
     kfac::TimedLaunch timed(KFAC_TIMED_INV_LAUUM, s);
     hipLaunchKernelGGL(lauum_kernel, dim3(plan->lauum_count), dim3(THREADS), kTileLdsBytes, s, tb,

@@ -104,6 +104,40 @@ def test_non_spd_and_nan_are_flagged_per_matrix():
         O.inverse(bad)
 
 
+def test_bordered_matrices(monkeypatch):
+    """Matrices of 128 m + 1 rows (a layer with a bias) are inverted from their leading
+    block plus a border; the result equals the whole-matrix path (KFAC_INVERSE_BORDER=0) to
+    rounding, a non-positive last pivot is reported as info = d, and sizes around the rule
+    (128 m, 128 m + 2, 129) take their own paths."""
+    from chainerkfac_amd import ops
+    dims = [129, 257, 513, 641, 130, 256, 258, 1153]
+    mats = [spd(d, 300 + d) for d in dims]
+    dev = [torch.from_numpy(m).cuda() for m in mats]
+    outs, info = ops.spd_inverse_batched(dev)
+    torch.cuda.synchronize()
+    assert info.cpu().tolist() == [0] * len(dims)
+    for m, o in zip(mats, outs):
+        check_inverse(m, o.cpu().numpy())
+    # the same through the whole-matrix path (a plan reads the switch when it is created)
+    monkeypatch.setenv('KFAC_INVERSE_BORDER', '0')
+    whole, info = ops.spd_inverse_batched(dev + [torch.from_numpy(spd(3, 1)).cuda()])
+    for m, o, w in zip(mats, outs, whole):
+        ref64 = np.linalg.inv(m.astype(np.float64))
+        assert np.linalg.norm(o.cpu().numpy() - w.cpu().numpy()) <= 2e-4 * np.linalg.norm(ref64)
+    monkeypatch.delenv('KFAC_INVERSE_BORDER')
+    # last pivot not positive: SPD leading block, corner too small
+    bad = spd(257, 9).astype(np.float64)
+    a = bad[:256, 256]
+    bad[256, 256] = a @ np.linalg.solve(bad[:256, :256], a) * 0.5
+    early = spd(385, 10)
+    early[100, 100] = -1.0
+    outs, info = ops.spd_inverse_batched([torch.from_numpy(bad.astype(np.float32)).cuda(),
+                                          torch.from_numpy(early).cuda(),
+                                          torch.from_numpy(spd(257, 11)).cuda()])
+    assert info.cpu().tolist() == [257, 101, 0]
+    check_inverse(spd(257, 11), outs[2].cpu().numpy())
+
+
 def test_repeated_calls_reuse_plan_and_workspace():
     from chainerkfac_amd import ops
     mats = [torch.from_numpy(spd(d, d)).cuda() for d in (300, 50)]
