@@ -75,6 +75,7 @@ struct TileTask {
 constexpr int kFirst = 1;   // the accumulators start from zero (first product of an upper tile)
 constexpr int kSame = 2;    // both operands are the same run
 
+struct BorderTask;
 struct InvTables {
   const float *const *in;    // [count] sorted slot -> input matrix
   float *const *out;         // [count]
@@ -87,6 +88,7 @@ struct InvTables {
   const long long *ws_off;   // [count] float offset of the padded matrix
   const int *tile_cs;        // [count+1] cumulative lower-tile counts (copy-in)
   const TileTask *tasks;     // the tile tasks of all launches
+  const BorderTask *btasks;  // the vector tasks of the bordered matrices
   float *ws;                 // padded matrices
   int *info;
 };
@@ -523,12 +525,172 @@ __device__ __forceinline__ void diag_role(const InvTables &tb, const TileTask &t
 }
 
 // ---------------------------------------------------------------------------
+// Bordered matrices.  The Kronecker factor of a layer with a bias has d = 9C + 1
+// or C + 1 rows: one more than a multiple of the tile size for every
+// power-of-two C, which as a tiled matrix pays a whole extra tile row and column
+// (4609 -> 37 tiles instead of 36; 11 % of the tile products of ResNet-50's
+// factors).  Such a matrix M = [A a; a^T alpha] keeps its last row out of the
+// tiles: the sweep factors the leading block A = L L^T, and the last row of M's
+// Cholesky factor, l = L^-1 a, follows it as a vector, by the same block forward
+// substitution that a tile row would go through,
+//     l_k = U_kk^T (a_k - sum_{j<k} L(k,j) l_j),
+// as do the last column of the triangular inverse and the last pivot,
+//     w = U l = A^-1 a  (w_i = sum_{k >= i} U(i,k) l_k),   S = alpha - l^T l,
+//     M^-1 = [A^-1 + w w^T / S, -w / S; -w^T / S, 1 / S].
+// These are tile-by-vector products, a few workgroups per step that ride in the
+// launches of the sweep: beside the diagonal tiles of step k the partial sums of
+// sum_{j<k} L(k,j) l_j (chunks of kBorderChunk tiles) and w += U(.,k-1) l_{k-1},
+// beside the panel step l_k itself.  (Forming l = U^T a from the finished inverse
+// instead loses a factor of cond(L) in accuracy against the substitution.)  The
+// rank-1 term is added to the accumulators of the final product.
+// ---------------------------------------------------------------------------
+constexpr int kBorderChunk = 6;
+constexpr int kBorderSum = 0;     // part[j] = sum_{c in chunk j} L(i,c) l_c          (i = k, j = chunk)
+constexpr int kBorderSolve = 1;   // l_i = U_ii^T (a_i - sum of the partial vectors)
+constexpr int kBorderW = 2;       // w_i (+)= U(i,j) l_j, the first term (j = i) overwrites
+constexpr int kBorderPivot = 3;   // S = alpha - l^T l in float64, 1 / S, info
+struct BorderTask {
+  int s, kind, i, j;
+};
+constexpr int kBorderLdsFloats = NB + NB * 33;
+
+// vectors of a bordered matrix in the workspace: a | l | w | scalars (64) | partial vectors
+struct BorderVecs {
+  float *a, *y, *w, *scal, *part;
+  int dc;
+};
+__device__ __forceinline__ BorderVecs border_vecs(const InvTables &tb, int s) {
+  BorderVecs v;
+  v.dc = tb.core[s];
+  v.a = tb.ws + tb.vec_off[s];
+  v.y = v.a + v.dc;
+  v.w = v.y + v.dc;
+  v.scal = v.w + v.dc;
+  v.part = v.scal + 64;
+  return v;
+}
+
+// p[r] += sum_{c in the thread's 4 columns} M[rg * 16 + r][c] x[c] for one NB x NB tile; x in LDS
+__device__ __forceinline__ void border_rows_acc(const float *tile, const float *xs, float (&p)[16]) {
+  const int c4 = (threadIdx.x & 31) * 4, rg = threadIdx.x >> 5;
+  const float4 x = *reinterpret_cast<const float4 *>(xs + c4);
+  const float *m = tile + (rg * 16) * NB + c4;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float4 u = *reinterpret_cast<const float4 *>(m + r * NB);
+    p[r] += u.x * x.x + u.y * x.y + u.z * x.z + u.w * x.w;
+  }
+}
+// the row sums of p over the 32 threads of a row group, in a fixed order; valid in threads < NB
+__device__ __forceinline__ float border_rows_reduce(const float (&p)[16], float *red) {
+  const int q = threadIdx.x & 31, rg = threadIdx.x >> 5;
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[(rg * 16 + r) * 33 + q] = p[r];
+  __syncthreads();
+  float t = 0.f;
+  if (threadIdx.x < NB) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) t += red[threadIdx.x * 33 + i];
+  }
+  return t;
+}
+
+__device__ __forceinline__ void border_role(const InvTables &tb, const BorderTask t, float *lds) {
+  float *xs = lds;         // NB floats
+  float *red = lds + NB;   // NB x 33
+  const BorderVecs v = border_vecs(tb, t.s);
+  if (t.kind == kBorderSum) {
+    float p[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) p[r] = 0.f;
+    const int j_end = min((t.j + 1) * kBorderChunk, t.i);
+    for (int j = t.j * kBorderChunk; j < j_end; ++j) {
+      __syncthreads();
+      if (threadIdx.x < NB) xs[threadIdx.x] = v.y[j * NB + threadIdx.x];
+      __syncthreads();
+      border_rows_acc(tile_ptr(tb, t.s, t.i, j), xs, p);
+    }
+    const float sum = border_rows_reduce(p, red);
+    if (threadIdx.x < NB) v.part[t.j * NB + threadIdx.x] = sum;
+  } else if (t.kind == kBorderSolve) {
+    if (threadIdx.x < NB) {
+      float x = v.a[t.i * NB + threadIdx.x];
+      const int nch = (t.i + kBorderChunk - 1) / kBorderChunk;
+      for (int ch = 0; ch < nch; ++ch) x -= v.part[ch * NB + threadIdx.x];
+      xs[threadIdx.x] = x;
+    }
+    __syncthreads();
+    // l_k[c] = sum_r U_kk[r][c] x[r]
+    const int c4 = (threadIdx.x & 31) * 4, rg = threadIdx.x >> 5;
+    const float *U = tile_ptr(tb, t.s, t.i, t.i) + (rg * 16) * NB + c4;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float4 u = *reinterpret_cast<const float4 *>(U + r * NB);
+      const float xv = xs[rg * 16 + r];
+      acc.x += u.x * xv;
+      acc.y += u.y * xv;
+      acc.z += u.z * xv;
+      acc.w += u.w * xv;
+    }
+    *reinterpret_cast<float4 *>(red + rg * NB + c4) = acc;
+    __syncthreads();
+    if (threadIdx.x < NB) {
+      float l = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) l += red[g * NB + threadIdx.x];
+      v.y[t.i * NB + threadIdx.x] = l;
+    }
+  } else if (t.kind == kBorderW) {
+    float p[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) p[r] = 0.f;
+    if (threadIdx.x < NB) xs[threadIdx.x] = v.y[t.j * NB + threadIdx.x];
+    __syncthreads();
+    border_rows_acc(tile_ptr(tb, t.s, t.i, t.j), xs, p);
+    const float sum = border_rows_reduce(p, red);
+    if (threadIdx.x < NB) {
+      float *w = v.w + t.i * NB + threadIdx.x;
+      *w = t.j == t.i ? sum : *w + sum;
+    }
+  } else {
+    double *dred = reinterpret_cast<double *>(lds);
+    double sum = 0.0;
+    for (int j = threadIdx.x; j < v.dc; j += THREADS) sum += (double)v.y[j] * (double)v.y[j];
+    dred[threadIdx.x] = sum;
+    __syncthreads();
+    for (int w = THREADS / 2; w > 0; w >>= 1) {
+      if ((int)threadIdx.x < w) dred[threadIdx.x] += dred[threadIdx.x + w];
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+      const double S = (double)v.scal[0] - dred[0];
+      v.scal[1] = (float)S;
+      v.scal[2] = (float)(1.0 / S);
+      int *pinfo = &tb.info[tb.orig[t.s]];
+      if (!(S > 0.0) && *pinfo == 0) *pinfo = tb.dim[t.s];
+    }
+  }
+}
+
+// the border tasks that follow the last step of the sweep
+__global__ __launch_bounds__(THREADS) void border_kernel(InvTables tb, int btask0) {
+  __shared__ __align__(16) float lds[kBorderLdsFloats];
+  border_role(tb, tb.btasks[btask0 + blockIdx.x], lds);
+}
+
+// ---------------------------------------------------------------------------
 // panel and update: 128x128x128 tile products through the shared main loop
 // ---------------------------------------------------------------------------
 // M(x,k) = M(x,k) W^T = M(x,k) U_kk in place for every x != k; the operand
 // W^T is the diagonal tile itself, read transposed.
-__global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int task0) {
+__global__ __launch_bounds__(THREADS, 2) void panel_kernel(InvTables tb, int task0, int ntask, int btask0) {
   extern __shared__ float lds[];
+  if ((int)blockIdx.x >= ntask) {   // bordered matrices: l_k of this step
+    border_role(tb, tb.btasks[btask0 + blockIdx.x - ntask], lds);
+    return;
+  }
   const TileTask t = tb.tasks[task0 + blockIdx.x];
   float *tile = tb.ws + t.c_off;
   floatx16 acc[2][2];
@@ -568,8 +730,12 @@ __device__ __forceinline__ void update_role(const InvTables &tb, const TileTask 
 // beside a workgroup of the trailing update (kDiagKernelLds): it waits for a CU
 // without one, at most the few microseconds until the next of them retires, and
 // keeps the following ones away from that CU while it runs.
-__global__ __launch_bounds__(THREADS, 2) void diag_kernel(InvTables tb, int task0) {
+__global__ __launch_bounds__(THREADS, 2) void diag_kernel(InvTables tb, int task0, int ntask, int btask0) {
   extern __shared__ float lds[];
+  if ((int)blockIdx.x >= ntask) {   // bordered matrices: the vector work this step can start with
+    border_role(tb, tb.btasks[btask0 + blockIdx.x - ntask], lds);
+    return;
+  }
   const TileTask t = tb.tasks[task0 + blockIdx.x];
   diag_role(tb, t, lds);
 }
@@ -581,141 +747,6 @@ __global__ __launch_bounds__(THREADS, 2) void update_kernel(InvTables tb, int ta
   extern __shared__ float lds[];
   const TileTask t = tb.tasks[task0 + blockIdx.x];
   update_role<2>(tb, t, lds);
-}
-
-// ---------------------------------------------------------------------------
-// Bordered matrices.  The Kronecker factor of a layer with a bias has d = 9C + 1
-// or C + 1 rows: one more than a multiple of the tile size for every
-// power-of-two C, which as a tiled matrix pays a whole extra tile row and column
-// (4609 -> 37 tiles instead of 36; 11 % of the tile products of ResNet-50's
-// factors).  Such a matrix M = [A a; a^T alpha] is inverted from its leading
-// block instead, which the sweep above factors as A^-1 = U U^T:
-//     y = U^T a,  S = alpha - y^T y  (the last pivot of M's Cholesky, squared),
-//     w = U y = A^-1 a,
-//     M^-1 = [A^-1 + w w^T / S, -w / S; -w^T / S, 1 / S].
-// y and w are two tile-wise matrix-vector products (HBM-bound, the U tiles read
-// once each); the rank-1 term is added to the accumulators of the final product.
-// ---------------------------------------------------------------------------
-
-// Both products are cut into chunks of kBorderChunk tiles along the summed index, one
-// workgroup each, whose partial vectors are added in a fixed order afterwards.
-constexpr int kBorderChunk = 6;
-
-// vectors of a bordered matrix in the workspace: a | y | w | scalars (64) | partial vectors
-struct BorderVecs {
-  float *a, *y, *w, *scal, *part;
-  int dc;
-};
-__device__ __forceinline__ BorderVecs border_vecs(const InvTables &tb, int s) {
-  BorderVecs v;
-  v.dc = tb.core[s];
-  v.a = tb.ws + tb.vec_off[s];
-  v.y = v.a + v.dc;
-  v.w = v.y + v.dc;
-  v.scal = v.w + v.dc;
-  v.part = v.scal + 64;
-  return v;
-}
-
-// partial y_k = sum_{i in chunk, i <= k} U(i,k)^T a_i; task = (matrix, k | chunk << 16)
-__global__ __launch_bounds__(256) void border_y_kernel(InvTables tb, const int2 *__restrict__ tasks) {
-  __shared__ float as[NB];
-  __shared__ float part[8][NB];
-  const int s = tasks[blockIdx.x].x;
-  const int k = tasks[blockIdx.x].y & 0xffff, ch = tasks[blockIdx.x].y >> 16;
-  const BorderVecs v = border_vecs(tb, s);
-  const int c4 = (threadIdx.x & 31) * 4, rg = threadIdx.x >> 5;   // 4 columns, rows rg*16 .. +15
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  const int i_end = min((ch + 1) * kBorderChunk, k + 1);
-  for (int i = ch * kBorderChunk; i < i_end; ++i) {
-    __syncthreads();
-    if (threadIdx.x < NB) as[threadIdx.x] = v.a[i * NB + threadIdx.x];
-    __syncthreads();
-    const float *U = tile_ptr(tb, s, i, k) + (rg * 16) * NB + c4;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float4 u = *reinterpret_cast<const float4 *>(U + r * NB);
-      const float av = as[rg * 16 + r];
-      acc.x += u.x * av;
-      acc.y += u.y * av;
-      acc.z += u.z * av;
-      acc.w += u.w * av;
-    }
-  }
-  *reinterpret_cast<float4 *>(&part[rg][c4]) = acc;
-  __syncthreads();
-  if (threadIdx.x < NB) {
-    float t = 0.f;
-#pragma unroll
-    for (int g = 0; g < 8; ++g) t += part[g][threadIdx.x];
-    v.part[(long long)ch * v.dc + k * NB + threadIdx.x] = t;
-  }
-}
-
-// y = sum of its partial vectors; S = alpha - y^T y in float64; info = d when S is not positive
-__global__ __launch_bounds__(256) void border_s_kernel(InvTables tb, const int *__restrict__ slots) {
-  __shared__ double red[256];
-  const int s = slots[blockIdx.x];
-  const BorderVecs v = border_vecs(tb, s);
-  double sum = 0.0;
-  for (int j = threadIdx.x; j < v.dc; j += 256) {
-    const int nch = (j / NB) / kBorderChunk + 1;   // chunks with i <= k
-    float t = 0.f;
-    for (int ch = 0; ch < nch; ++ch) t += v.part[(long long)ch * v.dc + j];
-    v.y[j] = t;
-    sum += (double)t * (double)t;
-  }
-  red[threadIdx.x] = sum;
-  __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
-    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    const double S = (double)v.scal[0] - red[0];
-    v.scal[1] = (float)S;
-    v.scal[2] = (float)(1.0 / S);
-    int *pinfo = &tb.info[tb.orig[s]];
-    if (!(S > 0.0) && *pinfo == 0) *pinfo = tb.dim[s];
-  }
-}
-
-// partial w_i = sum_{k in chunk, k >= i} U(i,k) y_k; task = (matrix, i | chunk << 16); two threads per row
-__global__ __launch_bounds__(256) void border_w_kernel(InvTables tb, const int2 *__restrict__ tasks) {
-  __shared__ float ys[NB];
-  const int s = tasks[blockIdx.x].x;
-  const int i = tasks[blockIdx.x].y & 0xffff, ch = tasks[blockIdx.x].y >> 16;
-  const BorderVecs v = border_vecs(tb, s);
-  const int T = tb.nt[s];
-  const int r = threadIdx.x >> 1, half = threadIdx.x & 1;
-  float acc = 0.f;
-  const int k_end = min((ch + 1) * kBorderChunk, T);
-  for (int k = max(i, ch * kBorderChunk); k < k_end; ++k) {
-    __syncthreads();
-    if (threadIdx.x < NB) ys[threadIdx.x] = v.y[k * NB + threadIdx.x];
-    __syncthreads();
-    const float4 *U = reinterpret_cast<const float4 *>(tile_ptr(tb, s, i, k) + r * NB + half * (NB / 2));
-#pragma unroll
-    for (int q = 0; q < NB / 8; ++q) {
-      const float4 u = U[q];
-      const float *yv = ys + half * (NB / 2) + 4 * q;
-      acc += u.x * yv[0] + u.y * yv[1] + u.z * yv[2] + u.w * yv[3];
-    }
-  }
-  acc += __shfl_xor(acc, 1, 64);
-  if (half == 0) v.part[(long long)ch * v.dc + i * NB + r] = acc;
-}
-
-// w = sum of its partial vectors
-__global__ __launch_bounds__(256) void border_wsum_kernel(InvTables tb, const int *__restrict__ slots) {
-  const int s = slots[blockIdx.x];
-  const BorderVecs v = border_vecs(tb, s);
-  const int nch_all = (tb.nt[s] - 1) / kBorderChunk + 1;
-  for (int j = threadIdx.x; j < v.dc; j += 256) {
-    float t = 0.f;
-    for (int ch = (j / NB) / kBorderChunk; ch < nch_all; ++ch) t += v.part[(long long)ch * v.dc + j];
-    v.w[j] = t;
-  }
 }
 
 // out(i,j) = sum_{k >= i} U(i,k) U(j,k)^T for i >= j, written with its mirror.
@@ -824,8 +855,12 @@ struct kfac_inverse_plan {
   }
   int total_tiles = 0;
   int lauum_task0 = 0, lauum_count = 0;
-  int nborder = 0, nborder_y = 0, nborder_w = 0;   // bordered matrices; tasks of their two products
-  kfac::DevTable d_core, d_orig, d_vec, d_border_slots, d_border_tiles, d_border_w_tiles;
+  // bordered matrices: their vector tasks per step (beside the diagonal tiles, beside the
+  // panel step) and after the sweep
+  int nborder = 0;
+  std::vector<int> bdiag_task0, bdiag_count, bpanel_task0, bpanel_count;
+  int bfinal_task0 = 0, bfinal_count = 0;
+  kfac::DevTable d_core, d_orig, d_vec, d_btasks;
   size_t ws_floats = 0;            // padded matrices
   std::vector<const void *> in_sorted, out_sorted;
   kfac::DevTable d_in, d_out, d_dim, d_nt, d_off, d_tile, d_tasks;
@@ -885,7 +920,6 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   std::vector<int> core(count);
   std::vector<long long> vec_off(count, -1);
   std::vector<int> border_slots;
-  std::vector<int2> border_tiles, border_w_tiles;
   for (int s = 0; s < count; ++s) {
     dim[s] = dims[p->order[s]];
     core[s] = (border_on && dim[s] > NB && dim[s] % NB == 1) ? dim[s] - 1 : dim[s];
@@ -900,17 +934,10 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     if (core[s] == dim[s]) continue;
     vec_off[s] = (long long)total;
     const int nch = (p->nt[s] - 1) / kBorderChunk + 1;
-    total += (size_t)(3 + nch) * core[s] + 64;
+    total += (size_t)3 * core[s] + 64 + (size_t)nch * NB;
     border_slots.push_back(s);
-    // y: chunks of tile rows i <= k; w: chunks of tile columns k >= i
-    for (int k = 0; k < p->nt[s]; ++k)
-      for (int ch = 0; ch * kBorderChunk <= k; ++ch) border_tiles.push_back(make_int2(s, k | (ch << 16)));
-    for (int i = 0; i < p->nt[s]; ++i)
-      for (int ch = i / kBorderChunk; ch < nch; ++ch) border_w_tiles.push_back(make_int2(s, i | (ch << 16)));
   }
   p->nborder = (int)border_slots.size();
-  p->nborder_y = (int)border_tiles.size();
-  p->nborder_w = (int)border_w_tiles.size();
   p->ws_floats = total;
   p->total_tiles = tile_cs[count];
   p->max_t = count ? p->nt[0] : 0;
@@ -940,6 +967,37 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   if (const char *e = getenv("KFAC_INVERSE_ALIGN")) align = std::min(100, std::max(0, atoi(e)));
   std::vector<int> shift(count);
   for (int s = 0; s < count; ++s) shift[s] = (p->max_t - p->nt[s]) * align / 100;
+  std::vector<BorderTask> btasks;
+  // step g, bordered matrix s at its block column k = g - shift: beside the diagonal tiles the
+  // chunks of sum_{j<k} L(k,j) l_j and w_i (+)= U(i,k-1) l_{k-1} (k = nt: only the latter);
+  // beside the panel step l_k
+  for (int g = 0; g <= p->max_t; ++g) {
+    const int first = (int)btasks.size();
+    for (int s : border_slots) {
+      const int k = g - shift[s], T = p->nt[s];
+      if (k < 1 || k > T) continue;
+      if (k < T)
+        for (int ch = 0; ch * kBorderChunk < k; ++ch) btasks.push_back(BorderTask{s, kBorderSum, k, ch});
+      for (int i = 0; i < k; ++i) btasks.push_back(BorderTask{s, kBorderW, i, k - 1});
+    }
+    if (g < p->max_t) {
+      p->bdiag_task0.push_back(first);
+      p->bdiag_count.push_back((int)btasks.size() - first);
+      const int pfirst = (int)btasks.size();
+      for (int s : border_slots) {
+        const int k = g - shift[s];
+        if (k >= 0 && k < p->nt[s]) btasks.push_back(BorderTask{s, kBorderSolve, k, 0});
+      }
+      p->bpanel_task0.push_back(pfirst);
+      p->bpanel_count.push_back((int)btasks.size() - pfirst);
+    } else {
+      // after the sweep: the last terms of w and the pivots
+      for (int s : border_slots) btasks.push_back(BorderTask{s, kBorderPivot, 0, 0});
+      p->bfinal_task0 = first;
+      p->bfinal_count = (int)btasks.size() - first;
+    }
+  }
+  if (btasks.empty()) btasks.push_back(BorderTask{0, 0, 0, 0});
   auto tile_off = [&](int s, int I, int J) {
     return off[s] + ((long long)I * p->nt[s] + J) * (long long)(NB * NB);
   };
@@ -1119,11 +1177,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_core, core.data(), sizeof(int) * count);
   up(p->d_orig, p->order.data(), sizeof(int) * count);
   up(p->d_vec, vec_off.data(), sizeof(long long) * count);
-  if (p->nborder > 0) {
-    up(p->d_border_slots, border_slots.data(), sizeof(int) * border_slots.size());
-    up(p->d_border_tiles, border_tiles.data(), sizeof(int2) * border_tiles.size());
-    up(p->d_border_w_tiles, border_w_tiles.data(), sizeof(int2) * border_w_tiles.size());
-  }
+  up(p->d_btasks, btasks.data(), sizeof(BorderTask) * btasks.size());
   up(p->d_nt, p->nt.data(), sizeof(int) * count);
   up(p->d_off, off.data(), sizeof(long long) * count);
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
@@ -1227,6 +1281,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.ws_off = plan->d_off.as<const long long>();
   tb.tile_cs = plan->d_tile.as<const int>();
   tb.tasks = plan->d_tasks.as<const TileTask>();
+  tb.btasks = plan->d_btasks.as<const BorderTask>();
   uintptr_t base = (reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255;
   tb.ws = reinterpret_cast<float *>(base);
   tb.info = info_dev;
@@ -1278,8 +1333,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       KFAC_HIP_CHECK(hipStreamWaitEvent(plan->col, plan->ev_fork[k], 0));
       cs = plan->col;
     }
-    hipLaunchKernelGGL(diag_kernel, dim3(na), dim3(THREADS), kDiagKernelLds, s, tb,
-                       plan->diag_task0[k]);
+    hipLaunchKernelGGL(diag_kernel, dim3(na + plan->bdiag_count[k]), dim3(THREADS), kDiagKernelLds, s, tb,
+                       plan->diag_task0[k], na, plan->bdiag_task0[k]);
     if (w.count > 0) {
       kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, cs);
       hipLaunchKernelGGL(update_kernel, dim3(w.count), dim3(THREADS), kTileLdsBytes, cs, tb, w.task0);
@@ -1289,9 +1344,10 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_col[k], 0));
     }
     if (int rc2 = queue_rest()) return rc2;
-    if (plan->panel_total[k] > 0)
-      hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k]), dim3(THREADS), kTileLdsBytes, s,
-                         tb, plan->panel_task0[k]);
+    if (plan->panel_total[k] + plan->bpanel_count[k] > 0)
+      hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k] + plan->bpanel_count[k]), dim3(THREADS),
+                         kTileLdsBytes, s, tb, plan->panel_task0[k], plan->panel_total[k],
+                         plan->bpanel_task0[k]);
     if (plan->rest[k].count == 0) continue;
     if (lookahead) KFAC_HIP_CHECK(hipEventRecord(plan->ev_main[k], s));
     deferred = k;
@@ -1299,14 +1355,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   if (int rc2 = queue_rest()) return rc2;
   if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
   KFAC_HIP_CHECK(hipGetLastError());
-  if (plan->nborder > 0) {
-    const int *slots = plan->d_border_slots.as<const int>();
-    hipLaunchKernelGGL(border_y_kernel, dim3(plan->nborder_y), dim3(256), 0, s, tb,
-                       plan->d_border_tiles.as<const int2>());
-    hipLaunchKernelGGL(border_s_kernel, dim3(plan->nborder), dim3(256), 0, s, tb, slots);
-    hipLaunchKernelGGL(border_w_kernel, dim3(plan->nborder_w), dim3(256), 0, s, tb,
-                       plan->d_border_w_tiles.as<const int2>());
-    hipLaunchKernelGGL(border_wsum_kernel, dim3(plan->nborder), dim3(256), 0, s, tb, slots);
+  if (plan->bfinal_count > 0) {
+    hipLaunchKernelGGL(border_kernel, dim3(plan->bfinal_count), dim3(THREADS), 0, s, tb, plan->bfinal_task0);
     KFAC_HIP_CHECK(hipGetLastError());
   }
   {
