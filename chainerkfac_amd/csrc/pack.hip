@@ -6,19 +6,32 @@
 // takes n(n+1)/2 slots, slot r(r+1)/2 + c holding M[r, c] for c <= r; any
 // other array is copied flat.
 //
-// Both kernels are bandwidth bound.  Work is cut into units that a workgroup
-// finds with one wave-uniform binary search over a small cumulative table
-// (the reference searches once per *element*):
-//   pack    unit = 4096 consecutive packed slots of one array.  Packed slots
-//           are walked linearly, so stores are fully coalesced and loads are
-//           contiguous along each matrix row; the upper triangle is never
-//           touched.
+// Both kernels are bandwidth bound and move 16 bytes per lane and access, at
+// float granularity (neither the packed rows nor the rows of an odd-sized matrix
+// start on 16-byte boundaries).  Work is cut into units; a per-unit owner table
+// tells a workgroup its array with one load (the reference searches once per
+// *element*):
+//   pack    unit = 512 aligned quads of buffer slots (2048 slots) of one array, a
+//           thread fills two of them: packed slots are walked linearly, so stores
+//           are aligned and fully coalesced and loads are contiguous along each
+//           matrix row; the upper triangle is never touched.  Units are dealt
+//           round-robin to the XCDs, stores are streaming (non-temporal) stores.
 //   unpack  unit = one 64x64 tile (I >= J) of a triangular array: the tile's
 //           row segments are read once from the buffer, written to M[I, J]
 //           directly and to M[J, I] through an LDS transpose, so every global
-//           access is a contiguous 256-byte run per wave.  Flat arrays use
-//           4096-element chunks.
+//           access is a contiguous 256-byte run per 16 lanes.  Flat arrays use
+//           4096-element chunks.  Units of matrices whose rows start on cache
+//           lines (sides that are multiples of 32) are dealt round-robin too; of
+//           the others every XCD takes a contiguous run, so that a line two
+//           neighbouring tiles each write a part of is completed inside one L2.
+// Measured on an MI355X (ResNet-50-D factor list, 0.53 GB packed): pack 5.7 TB/s,
+// unpack 5.5 TB/s; a kernel that only reads n and writes 2 n bytes (unpack's mix)
+// reaches 6.0 TB/s, a plain copy 6.2 - 6.6 TB/s.  What did not help: streaming
+// loads (slower for unpack), streaming stores in unpack (rows that are not
+// line-aligned then never merge in L2), more than two quads per thread.
 #include <hip/hip_fp16.h>
+
+#include <algorithm>
 
 #include "common.h"
 
@@ -26,8 +39,10 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kChunk = 4096;           // packed slots per pack unit
-constexpr int kPerThread = kChunk / kThreads;
 constexpr int kTile = 64;              // unpack tile side
+constexpr int kPackU = 2;              // quads of buffer slots per thread of the pack kernel
+constexpr int kUnpackThreads = 512;    // threads of an unpack workgroup (two passes over a tile)
+constexpr int kPackQuads = kThreads * kPackU;
 
 struct PackTables {
   const float *const *ptrs;   // [n] array base pointers
@@ -37,30 +52,19 @@ struct PackTables {
   const long long *buf_off;   // [n] first slot in the buffer
   const int *pack_csum;       // [n+1] cumulative pack units
   const int *unpack_csum;     // [n+1] cumulative unpack units
+  const int *pack_owner;      // [pack units] array of each unit (one load instead of a search)
+  const int2 *unpack_sched;   // [unpack workgroups] {unit, array}; unit < 0: nothing to do
   int n;
 };
 
-// Index j with csum[j] <= unit < csum[j+1]; `unit` is wave-uniform so the
-// search runs on the scalar unit.
-__device__ __forceinline__ int find_array(const int *__restrict__ csum, int n,
-                                          int unit) {
-  int lo = 0, hi = n - 1;
-  while (lo < hi) {
-    int mid = (lo + hi + 1) >> 1;
-    if (csum[mid] <= unit)
-      lo = mid;
-    else
-      hi = mid - 1;
-  }
-  return lo;
-}
-
-// Row of packed slot t: the largest r with r(r+1)/2 <= t.
-__device__ __forceinline__ int tri_row(long long t) {
-  long long r = (long long)((sqrt(8.0 * (double)t + 1.0) - 1.0) * 0.5);
-  while (r * (r + 1) / 2 > t) --r;
-  while ((r + 1) * (r + 2) / 2 <= t) ++r;
-  return (int)r;
+// Row of packed slot t: the largest r with r(r+1)/2 <= t.  t < 2^30 (a triangle of
+// side <= 46340), so 32-bit arithmetic holds every r(r+1)/2 that is compared; the
+// float estimate is off by one at most and the two loops correct it.
+__device__ __forceinline__ int tri_row(unsigned t) {
+  int r = (int)((__builtin_sqrtf(8.f * (float)t + 1.f) - 1.f) * 0.5f);
+  while ((unsigned)r * (unsigned)(r + 1) / 2u > t) --r;
+  while ((unsigned)(r + 1) * (unsigned)(r + 2) / 2u <= t) ++r;
+  return r;
 }
 
 // Element type of the packed buffer: float, or __half for the float16 wire
@@ -78,65 +82,140 @@ __device__ __forceinline__ float from_buf(__half v, int divisor) {
   return __half2float(__float2half_rn(__half2float(v) / __half2float(__int2half_rn(divisor))));
 }
 
-// Workgroup i of a launch runs on XCD i % 8, each XCD with an L2 of its own.
-// Every XCD takes one contiguous run of the unit list: neighbouring units touch
-// neighbouring memory (the cache lines at the seams of two tiles or chunks), and
-// a line that two workgroups each write half of is completed inside one L2
-// instead of being written back twice as partial lines.
-__device__ __forceinline__ int xcd_contiguous_unit(int total) {
-  const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
-  const int base = total / 8, rem = total % 8;
-  return xcd * base + (xcd < rem ? xcd : rem) + idx;
+// Four consecutive buffer slots as one access.
+typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));   // 16-byte load at any float address
+typedef float floatx4a __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_quad(float *p, const float (&v)[4]) {
+  floatx4a o;
+  o.x = v[0];
+  o.y = v[1];
+  o.z = v[2];
+  o.w = v[3];
+  // streamed: the buffer is next read by another kernel (or the network), not by this one
+  __builtin_nontemporal_store(o, reinterpret_cast<floatx4a *>(p));
+}
+__device__ __forceinline__ floatx4u load_quad(const float *p) {
+  return *reinterpret_cast<const floatx4u *>(p);
+}
+__device__ __forceinline__ void store_quad(__half *p, const float (&v)[4]) {
+  __half2 lo = __halves2half2(__float2half_rn(v[0]), __float2half_rn(v[1]));
+  __half2 hi = __halves2half2(__float2half_rn(v[2]), __float2half_rn(v[3]));
+  uint2 u;
+  u.x = *reinterpret_cast<unsigned *>(&lo);
+  u.y = *reinterpret_cast<unsigned *>(&hi);
+  *reinterpret_cast<uint2 *>(p) = u;
 }
 
-template <class B>
+// pack: a thread fills one aligned quad of buffer slots (slots 4q .. 4q + 3 of the
+// whole buffer, so that the store is one aligned 16-byte access whatever the
+// array's offset in the buffer) from four consecutive elements of a matrix row
+// (one 16-byte load; a quad that runs over the end of a row, or that the array
+// only partly owns at its first or last slot, goes element by element).  U quads
+// per thread, 256 U quads per unit.
+template <class B, int U>
 __global__ __launch_bounds__(kThreads) void pack_kernel(PackTables tb, B *__restrict__ buf,
                                                         int target) {
-  const int unit = xcd_contiguous_unit(gridDim.x);
-  const int j = find_array(tb.pack_csum, tb.n, unit);
+  const int unit = blockIdx.x;
+  const int j = tb.pack_owner[unit];
   if (target >= 0 && tb.rank[j] != target) return;
   const long long nel = tb.nel[j];
-  const long long t0 = (long long)(unit - tb.pack_csum[j]) * kChunk + threadIdx.x;
+  const long long off = tb.buf_off[j];
   const float *__restrict__ src = tb.ptrs[j];
-  B *__restrict__ dst = buf + tb.buf_off[j];
   const int d = tb.tri[j];
-  float val[kPerThread];
-  if (d > 0) {
-    int r = 0, c = 0;
-    if (t0 < nel) {
-      r = tri_row(t0);
-      c = (int)(t0 - (long long)r * (r + 1) / 2);
-    }
+  const long long q0 = (long long)(unit - tb.pack_csum[j]) * (kThreads * U) + threadIdx.x;
+  float val[U][4];
+  long long t[U];
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const long long t = t0 + (long long)i * kThreads;
-      val[i] = (t < nel) ? src[(long long)r * d + c] : 0.f;
-      c += kThreads;
-      while (c > r) {
-        c -= r + 1;
-        ++r;
+  for (int i = 0; i < U; ++i) {
+    // first slot of the quad relative to the array: -3 .. nel - 1
+    t[i] = ((off >> 2) + q0 + (long long)i * kThreads) * 4 - off;
+    const long long tq = t[i];
+    if (tq >= nel) continue;
+    if (d > 0) {
+      const unsigned tc = tq > 0 ? (unsigned)tq : 0u;
+      int r = tri_row(tc);
+      int c = (int)(tc - (unsigned)r * (unsigned)(r + 1) / 2u);
+      if (tq >= 0 && tq + 3 < nel && c + 3 <= r) {
+        const floatx4u v = load_quad(src + (long long)r * d + c);
+        val[i][0] = v.x;
+        val[i][1] = v.y;
+        val[i][2] = v.z;
+        val[i][3] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const long long te = tq + e;
+          val[i][e] = 0.f;
+          if (te >= 0 && te < nel) {
+            val[i][e] = src[(long long)r * d + c];
+            if (++c > r) {
+              c = 0;
+              ++r;
+            }
+          }
+        }
+      }
+    } else if (tq >= 0 && tq + 3 < nel) {
+      const floatx4u v = load_quad(src + tq);
+      val[i][0] = v.x;
+      val[i][1] = v.y;
+      val[i][2] = v.z;
+      val[i][3] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const long long te = tq + e;
+        val[i][e] = (te >= 0 && te < nel) ? src[te] : 0.f;
       }
     }
-  } else {
-#pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const long long t = t0 + (long long)i * kThreads;
-      val[i] = (t < nel) ? src[t] : 0.f;
-    }
   }
+  B *__restrict__ dst = buf + off;
 #pragma unroll
-  for (int i = 0; i < kPerThread; ++i) {
-    const long long t = t0 + (long long)i * kThreads;
-    if (t < nel) to_buf(val[i], dst[t]);
+  for (int i = 0; i < U; ++i) {
+    const long long tq = t[i];
+    if (tq >= nel) continue;
+    if (tq >= 0 && tq + 3 < nel) {
+      store_quad(dst + tq, val[i]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (tq + e >= 0 && tq + e < nel) to_buf(val[i][e], dst[tq + e]);
+    }
   }
 }
 
-template <class B>
-__global__ __launch_bounds__(kThreads) void unpack_kernel(PackTables tb, const B *__restrict__ buf,
-                                                          int target, int divisor) {
+// Four consecutive buffer elements, scaled: one 16-byte load for a float buffer.
+__device__ __forceinline__ void load_scaled4(const float *p, int divisor, float (&o)[4]) {
+  const floatx4u v = load_quad(p);
+  o[0] = from_buf(v.x, divisor);
+  o[1] = from_buf(v.y, divisor);
+  o[2] = from_buf(v.z, divisor);
+  o[3] = from_buf(v.w, divisor);
+}
+__device__ __forceinline__ void load_scaled4(const __half *p, int divisor, float (&o)[4]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = from_buf(p[e], divisor);
+}
+// Four consecutive floats of an array at any float address, as one 16-byte store.
+__device__ __forceinline__ void store_row4(float *p, const float (&v)[4]) {
+  floatx4u o;
+  o.x = v[0];
+  o.y = v[1];
+  o.z = v[2];
+  o.w = v[3];
+  *reinterpret_cast<floatx4u *>(p) = o;
+}
+
+// unpack: a thread moves four consecutive elements of a row at a time (16-byte
+// accesses at float granularity: neither the packed rows nor the rows of an
+// odd-sized matrix start on 16-byte boundaries).
+template <class B, int TH>
+__global__ __launch_bounds__(TH) void unpack_kernel(PackTables tb, const B *__restrict__ buf,
+                                                    int target, int divisor) {
   __shared__ float tile[kTile][kTile + 1];
-  const int unit = xcd_contiguous_unit(gridDim.x);
-  const int j = find_array(tb.unpack_csum, tb.n, unit);
+  const int2 sched = tb.unpack_sched[blockIdx.x];
+  const int unit = sched.x, j = sched.y;
+  if (unit < 0) return;
   if (target >= 0 && tb.rank[j] != target) return;
   const int local = unit - tb.unpack_csum[j];
   float *__restrict__ dst = const_cast<float *>(tb.ptrs[j]);
@@ -144,41 +223,59 @@ __global__ __launch_bounds__(kThreads) void unpack_kernel(PackTables tb, const B
   const int d = tb.tri[j];
   if (d == 0) {
     const long long nel = tb.nel[j];
-    const long long t0 = (long long)local * kChunk + threadIdx.x;
-    B val[kPerThread];
+    const long long t0 = (long long)local * kChunk + 4 * threadIdx.x;
+    constexpr int kQuads = kChunk / (4 * TH);   // per thread
+    float val[kQuads][4];
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const long long t = t0 + (long long)i * kThreads;
-      if (t < nel) val[i] = src[t];
+    for (int i = 0; i < kQuads; ++i) {
+      const long long t = t0 + (long long)i * (4 * TH);
+      if (t + 3 < nel) {
+        load_scaled4(src + t, divisor, val[i]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (t + e < nel) val[i][e] = from_buf(src[t + e], divisor);
+      }
     }
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const long long t = t0 + (long long)i * kThreads;
-      if (t < nel) dst[t] = from_buf(val[i], divisor);
+    for (int i = 0; i < kQuads; ++i) {
+      const long long t = t0 + (long long)i * (4 * TH);
+      if (t + 3 < nel) {
+        store_row4(dst + t, val[i]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (t + e < nel) dst[t + e] = val[i][e];
+      }
     }
     return;
   }
   // tile (I, J), I >= J, from the unit index in row-major lower order
-  const int I = tri_row(local);
+  const int I = tri_row((unsigned)local);
   const int J = local - I * (I + 1) / 2;
-  const int lc = threadIdx.x % kTile;   // column inside the tile
-  const int lr0 = threadIdx.x / kTile;  // 0..3
-  constexpr int kRowsPerPass = kThreads / kTile;
+  const int lc = (threadIdx.x % (kTile / 4)) * 4;   // first of the thread's four columns
+  const int lr0 = threadIdx.x / (kTile / 4);        // 0..15
+  constexpr int kRowsPerPass = TH / (kTile / 4);
   constexpr int kPasses = kTile / kRowsPerPass;
-  B val[kPasses];
-  bool have[kPasses];
+  float val[kPasses][4];
 #pragma unroll
   for (int p = 0; p < kPasses; ++p) {
     const int lr = lr0 + p * kRowsPerPass;
     const int r = I * kTile + lr;
     const int c = J * kTile + lc;
-    have[p] = r < d && c <= r;
-    if (have[p]) val[p] = src[(long long)r * (r + 1) / 2 + c];
+    const long long row0 = (long long)r * (r + 1) / 2;
+    if (r < d && c + 3 <= r) {
+      load_scaled4(src + row0 + c, divisor, val[p]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) val[p][e] = (r < d && c + e <= r) ? from_buf(src[row0 + c + e], divisor) : 0.f;
+    }
   }
 #pragma unroll
   for (int p = 0; p < kPasses; ++p) {
     const int lr = lr0 + p * kRowsPerPass;
-    tile[lr][lc] = have[p] ? from_buf(val[p], divisor) : 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) tile[lr][lc + e] = val[p][e];
   }
   __syncthreads();
   if (I == J) {
@@ -187,8 +284,16 @@ __global__ __launch_bounds__(kThreads) void unpack_kernel(PackTables tb, const B
       const int lr = lr0 + p * kRowsPerPass;
       const int r = I * kTile + lr;
       const int c = J * kTile + lc;
-      if (r < d && c < d)
-        dst[(long long)r * d + c] = (lc <= lr) ? tile[lr][lc] : tile[lc][lr];
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (lc + e <= lr) ? tile[lr][lc + e] : tile[lc + e][lr];
+      if (r < d && c + 3 < d) {
+        store_row4(dst + (long long)r * d + c, o);
+      } else if (r < d) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (c + e < d) dst[(long long)r * d + c + e] = o[e];
+      }
     }
   } else {
 #pragma unroll
@@ -196,11 +301,20 @@ __global__ __launch_bounds__(kThreads) void unpack_kernel(PackTables tb, const B
       const int lr = lr0 + p * kRowsPerPass;
       const int r = I * kTile + lr;
       const int c = J * kTile + lc;
-      if (r < d) dst[(long long)r * d + c] = tile[lr][lc];  // c < r < d
-      // mirrored tile (J, I): row J*64 + lr, column I*64 + lc
+      if (r < d) store_row4(dst + (long long)r * d + c, val[p]);   // c + 3 < I * 64 <= r < d
+      // mirrored tile (J, I): row J*64 + lr (< I*64 < d), columns I*64 + lc ..
       const int mr = J * kTile + lr;
       const int mc = I * kTile + lc;
-      if (mc < d) dst[(long long)mr * d + mc] = tile[lc][lr];  // mr < I*64 < d
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = tile[lc + e][lr];
+      if (mc + 3 < d) {
+        store_row4(dst + (long long)mr * d + mc, o);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (mc + e < d) dst[(long long)mr * d + mc + e] = o[e];
+      }
     }
   }
 }
@@ -212,8 +326,9 @@ struct kfac_pack_plan {
   long long total_packed = 0;
   int pack_units = 0;
   int unpack_units = 0;
+  int unpack_blocks = 0;   // workgroups of an unpack launch (>= unpack_units, see the schedule)
   std::vector<const void *> ptrs;
-  kfac::DevTable d_ptrs, d_tri, d_rank, d_nel, d_off, d_pcs, d_ucs;
+  kfac::DevTable d_ptrs, d_tri, d_rank, d_nel, d_off, d_pcs, d_ucs, d_pown, d_uown;
   PackTables tables() const {
     PackTables t;
     t.ptrs = d_ptrs.as<const float *const>();
@@ -223,6 +338,8 @@ struct kfac_pack_plan {
     t.buf_off = d_off.as<const long long>();
     t.pack_csum = d_pcs.as<const int>();
     t.unpack_csum = d_ucs.as<const int>();
+    t.pack_owner = d_pown.as<const int>();
+    t.unpack_sched = d_uown.as<const int2>();
     t.n = n;
     return t;
   }
@@ -264,6 +381,7 @@ extern "C" int kfac_pack_plan_create(int n_arrays, const void *const *ptrs,
   for (int i = 0; i < n_arrays; ++i) {
     const long long t = triangle_size[i];
     KFAC_REQUIRE(sizes[i] >= 0 && t >= 0, "array %d: negative size", i);
+    KFAC_REQUIRE(t <= 46340, "array %d: triangle side %lld exceeds 46340", i, t);
     KFAC_REQUIRE(sizes[i] == 0 || ptrs[i] != nullptr, "array %d: null pointer", i);
     long long packed;
     if (t > 0) {
@@ -276,7 +394,9 @@ extern "C" int kfac_pack_plan_create(int n_arrays, const void *const *ptrs,
       packed = sizes[i];
       uunits += kfac::ceil_div<long long>(packed, kChunk);
     }
-    punits += kfac::ceil_div<long long>(packed, kChunk);
+    // pack: units of kPackQuads aligned quads of buffer slots
+    if (packed > 0)
+      punits += kfac::ceil_div<long long>(kfac::ceil_div<long long>(total + packed, 4) - total / 4, kPackQuads);
     KFAC_REQUIRE(punits < 0x7fffffffLL && uunits < 0x7fffffffLL, "too many work units");
     tri[i] = (int)t;
     rank[i] = rank_of[i];
@@ -305,6 +425,36 @@ extern "C" int kfac_pack_plan_create(int n_arrays, const void *const *ptrs,
   up(p->d_off, off.data(), sizeof(long long) * n_arrays);
   up(p->d_pcs, pcs.data(), sizeof(int) * (n_arrays + 1));
   up(p->d_ucs, ucs.data(), sizeof(int) * (n_arrays + 1));
+  std::vector<int> pown((size_t)punits + 1, 0);
+  for (int i = 0; i < n_arrays; ++i) std::fill(pown.begin() + pcs[i], pown.begin() + pcs[i + 1], i);
+  up(p->d_pown, pown.data(), sizeof(int) * pown.size());
+  // The unpack schedule: workgroup b (which runs on XCD b % 8, each XCD with an L2
+  // of its own) takes entry b / 8 of its XCD's queue.  The tiles of matrices whose rows do not start on cache lines
+  // (side not a multiple of 32) go to the queues as eight contiguous runs; all
+  // other units are dealt round-robin behind them.
+  {
+    std::vector<int2> queue[8];
+    std::vector<int2> ragged, even;
+    for (int i = 0; i < n_arrays; ++i)
+      for (int u = ucs[i]; u < ucs[i + 1]; ++u)
+        (tri[i] > 0 && tri[i] % 32 != 0 ? ragged : even).push_back(make_int2(u, i));
+    const size_t chunk = (ragged.size() + 7) / 8;
+    for (size_t k = 0; k < ragged.size(); ++k) queue[k / (chunk ? chunk : 1)].push_back(ragged[k]);
+    for (size_t k = 0; k < even.size(); ++k) {
+      // to the shortest queue, first the one whose turn it is
+      size_t best = k % 8;
+      for (size_t x = 0; x < 8; ++x)
+        if (queue[x].size() + 1 < queue[best].size()) best = x;
+      queue[best].push_back(even[k]);
+    }
+    size_t longest = 0;
+    for (auto &q : queue) longest = std::max(longest, q.size());
+    std::vector<int2> sched(std::max<size_t>(longest * 8, 1), make_int2(-1, 0));
+    for (size_t x = 0; x < 8; ++x)
+      for (size_t k = 0; k < queue[x].size(); ++k) sched[k * 8 + x] = queue[x][k];
+    p->unpack_blocks = (int)(longest * 8);
+    up(p->d_uown, sched.data(), sizeof(int2) * sched.size());
+  }
   if (rc != KFAC_OK) {
     delete p;
     return rc;
@@ -341,8 +491,10 @@ int run_pack(kfac_pack_plan_t plan, B *buf, int64_t buf_nelems, int target_rank,
                plan->total_packed);
   if (plan->pack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
+  KFAC_REQUIRE(reinterpret_cast<uintptr_t>(buf) % (4 * sizeof(B)) == 0,
+               "the buffer must be aligned to four of its elements (%zu bytes)", 4 * sizeof(B));
   kfac::TimedLaunch timed(KFAC_TIMED_PACK, kfac::as_stream(stream));
-  hipLaunchKernelGGL(pack_kernel<B>, dim3(plan->pack_units), dim3(kThreads), 0,
+  hipLaunchKernelGGL((pack_kernel<B, kPackU>), dim3(plan->pack_units), dim3(kThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -359,7 +511,7 @@ int run_unpack(kfac_pack_plan_t plan, const B *buf, int64_t buf_nelems, int targ
   if (plan->unpack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
   kfac::TimedLaunch timed(KFAC_TIMED_UNPACK, kfac::as_stream(stream));
-  hipLaunchKernelGGL(unpack_kernel<B>, dim3(plan->unpack_units), dim3(kThreads), 0,
+  hipLaunchKernelGGL((unpack_kernel<B, kUnpackThreads>), dim3(plan->unpack_blocks), dim3(kUnpackThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank, divisor);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -369,23 +521,16 @@ int run_unpack(kfac_pack_plan_t plan, const B *buf, int64_t buf_nelems, int targ
 
 namespace {
 
-// Plain streaming copy, 16 bytes per lane and load, four loads in flight per
-// lane: the yardstick for the bandwidth-bound kernels of this file.
-__global__ __launch_bounds__(kThreads) void stream_copy_kernel(const float4 *__restrict__ src,
-                                                               float4 *__restrict__ dst,
+// Plain streaming copy, the yardstick for the bandwidth-bound kernels of this
+// file: one 16-byte streaming load and store per lane, 4 KB per workgroup (the
+// fastest of the structures measured on an MI355X: 6.6 TB/s; two, four or eight
+// accesses per lane, grid-stride loops and per-XCD contiguous ranges reach 4.3 -
+// 6.3 TB/s, hipMemcpyAsync 5.3 TB/s).
+__global__ __launch_bounds__(kThreads) void stream_copy_kernel(const floatx4a *__restrict__ src,
+                                                               floatx4a *__restrict__ dst,
                                                                long long n4) {
-  const long long base = (long long)blockIdx.x * (kThreads * 4) + threadIdx.x;
-  float4 v[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const long long t = base + (long long)i * kThreads;
-    if (t < n4) v[i] = src[t];
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const long long t = base + (long long)i * kThreads;
-    if (t < n4) dst[t] = v[i];
-  }
+  const long long t = (long long)blockIdx.x * kThreads + threadIdx.x;
+  if (t < n4) __builtin_nontemporal_store(__builtin_nontemporal_load(src + t), dst + t);
 }
 
 __global__ __launch_bounds__(kThreads) void stream_copy_tail_kernel(const float *__restrict__ src,
@@ -408,9 +553,9 @@ extern "C" int kfac_stream_copy_f32(float *dst, const float *src, int64_t nelems
   {
     kfac::TimedLaunch timed(KFAC_TIMED_COPY, s);
     if (n4 > 0)
-      hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)kfac::ceil_div<long long>(n4, kThreads * 4)),
-                         dim3(kThreads), 0, s, reinterpret_cast<const float4 *>(src),
-                         reinterpret_cast<float4 *>(dst), n4);
+      hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)kfac::ceil_div<long long>(n4, kThreads)),
+                         dim3(kThreads), 0, s, reinterpret_cast<const floatx4a *>(src),
+                         reinterpret_cast<floatx4a *>(dst), n4);
     if (n4 * 4 < nelems)
       hipLaunchKernelGGL(stream_copy_tail_kernel, dim3(1), dim3(kThreads), 0, s, src, dst, n4 * 4,
                          (long long)nelems);

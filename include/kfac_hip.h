@@ -64,7 +64,9 @@ int kfac_pack_plan_destroy(kfac_pack_plan_t plan);
 
 /* buf[off_j + r(r+1)/2 + c] = M_j[r, c] for c <= r (triangular arrays), flat
  * copy otherwise; arrays whose rank differs from target_rank are skipped when
- * target_rank >= 0.  Replaces cupy_batched_pack_arrays and its launch
+ * target_rank >= 0.  buf must be 16-byte aligned (8-byte for the float16
+ * variant): the kernel stores aligned quads of buffer slots.  Triangle sides up
+ * to 46340.  Replaces cupy_batched_pack_arrays and its launch
  * (pure_nccl_communicator.py:300-377, :110-127). */
 int kfac_pack_f32(kfac_pack_plan_t plan, float *buf, int64_t buf_nelems,
                   int target_rank, void *stream);
