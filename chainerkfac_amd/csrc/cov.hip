@@ -21,6 +21,7 @@
 // chainerkfac/optimizers/fisher_blocks/connections/{linear,convolution_2d}.py
 // and the batch-norm block's grad^T grad.
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -205,18 +206,19 @@ __device__ __forceinline__ void tri_decode(int t, int &I, int &J) {
 // direct: C[d-1, row] = C[row, d-1] = alpha * sum + beta * C[d-1, row], and the
 // first tile also writes the corner alpha * count + beta * C[d-1, d-1];
 // otherwise the sums go to the k-slice's row-sum slot.
+// rowmask: bit im set = row block im of this wave is its to write.
 template <int WM>
 __device__ __forceinline__ void write_rowsums(float (&rs)[WM], int I, int dt, int d, int direct,
                                               float count, float alpha, float beta,
                                               float *__restrict__ vec, float *__restrict__ C,
-                                              int wave = threadIdx.x >> 6) {
+                                              int wave = threadIdx.x >> 6, unsigned rowmask = 0xffffffffu) {
   constexpr int BM = 64 * WM;
   const int lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
 #pragma unroll
   for (int im = 0; im < WM; ++im) {
     const float tot = rs[im] + __shfl_xor(rs[im], 32, 64);
-    if (wn != 0 || lane >= 32) continue;
+    if (wn != 0 || lane >= 32 || !((rowmask >> im) & 1u)) continue;
     const int row = I * BM + (wm * WM + im) * 32 + lane;
     if (!direct) {
       vec[row] = tot;
@@ -227,7 +229,7 @@ __device__ __forceinline__ void write_rowsums(float (&rs)[WM], int I, int dt, in
       C[(long long)row * d + d - 1] = v;
     }
   }
-  if (direct && I == 0 && wave == 0 && lane == 0) {
+  if (direct && I == 0 && wave == 0 && (rowmask & 1u) && lane == 0) {
     float v = alpha * count;
     if (beta != 0.f) v += beta * C[(long long)(d - 1) * d + d - 1];
     C[(long long)(d - 1) * d + d - 1] = v;
@@ -999,6 +1001,7 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_group_kernel(const GroupItemS
   static_assert(2 * Panel<BM>::kFloats >= 64 * 65, "LDS too small for the epilogue transpose");
   float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
   const int2 task = tasks[blockIdx.x];
+  if (task.x < 0) return;   // padding of a shorter XCD run
   const GroupItemStatic s = st[task.x];
   const GroupItemDyn v = dy[task.x];
   const int split = task.y / s.ntile;
@@ -1017,24 +1020,41 @@ __global__ __launch_bounds__(THREADS, 3) void syrk_group_kernel(const GroupItemS
   float rs[WM];
 #pragma unroll
   for (int im = 0; im < WM; ++im) rs[im] = 0.f;
-  const int wave = threadIdx.x >> 6;
+  int wave = threadIdx.x >> 6;
   const bool active = syrk_wave_active<WM>(I * BM, J * BM, dt, wave);
-  if (I == J)
+  unsigned store = 0xfu, rowmask = 0x3u;
+  if (I != J) {
+    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active, wave);
+  } else if (WM == 2 && (I + 1) * BM <= dt) {
+    // a whole diagonal 128-tile: all four waves share its ten blocks
+    const DiagRole role = diag_tile_role(wave);
+    wave = role.role;
+    store = role.compute == 0xdu ? 0xfu : role.store;
+    rowmask = role.compute == 0xdu ? 0x3u : (role.compute == 0x3u ? 0x1u : 0x2u);
+    if (role.compute == 0xdu)
+      mainloop_impl<WM, WM, true, true, Loader, Loader, 0xdu>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB,
+                                                             acc, rs, true, wave);
+    else if (role.compute == 0x3u)
+      mainloop_impl<WM, WM, true, true, Loader, Loader, 0x3u>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB,
+                                                             acc, rs, true, wave);
+    else
+      mainloop_impl<WM, WM, true, true, Loader, Loader, 0xcu>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB,
+                                                             acc, rs, true, wave);
+  } else {
     mainloop_rowsum<WM, WM, true>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, rs, active,
                                   wave);
-  else
-    mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc, active, wave);
+  }
   const long long slot = (long long)s.ntile * (BM * BM) + (long long)s.tiles * BM;
   float *mine = ws + s.part_off + split * slot;
   if (s.ones && I == J)
     write_rowsums<WM>(rs, I, dt, s.d, s.direct, s.count, v.alpha, v.beta,
-                      mine + (long long)s.ntile * (BM * BM), v.out, wave);
+                      mine + (long long)s.ntile * (BM * BM), v.out, wave, rowmask);
   if (s.direct) {
-    write_tile<WM>(acc, lds, I, J, dt, s.d, v.alpha, v.beta, v.out, wave);
+    write_tile<WM>(acc, lds, I, J, dt, s.d, v.alpha, v.beta, v.out, wave, store);
     return;
   }
   float *out = mine + (long long)tile * (BM * BM);
-  for_each_acc<WM, WM>(acc, [&](int r, int c, float val) { out[r * BM + c] = val; }, wave);
+  for_each_acc_masked<WM, WM>(acc, store, [&](int r, int c, float val) { out[r * BM + c] = val; }, wave);
 }
 
 // Macro-tile variant for 128-tile slab items with several k-slices: a workgroup
@@ -1066,6 +1086,7 @@ __global__ __launch_bounds__(kMacroThreads, 1) void syrk_macro_kernel(
   const int wave = (threadIdx.x >> 6) & 3;
   const int lane = threadIdx.x & 63;
   const int2 task = tasks[blockIdx.x];
+  if (task.x < 0) return;   // padding of a shorter XCD run
   const GroupItemStatic s = st[task.x];
   const GroupItemDyn v = dy[task.x];
   const int mtiles = (s.tiles + 1) / 2;
@@ -1206,15 +1227,31 @@ __global__ __launch_bounds__(256) void finish_group_kernel(const GroupItemStatic
 }
 
 // Emits `natural` dealt so that each XCD (workgroup i of a launch runs on XCD
-// i % 8) receives one contiguous run of it.
-void deal_to_xcds(std::vector<int2> &table, const std::vector<int2> &natural) {
+// i % 8) receives one contiguous run of it, the runs cut at equal shares of the
+// total weight (the time a task takes: its reduction length, three quarters of it
+// for a whole diagonal 128-tile); shorter runs are padded with empty tasks (item
+// -1).  Measured on ResNet-50's grouped launch of 128-tiles before this: runs of
+// equal task counts left the XCDs with 21 400 .. 25 500 panel steps of work, and the
+// launch lasted as long as the slowest of them.
+void deal_to_xcds(std::vector<int2> &table, const std::vector<int2> &natural,
+                  const std::vector<double> &weight) {
   const size_t n = natural.size();
-  const size_t chunk = (n + kXcds - 1) / kXcds;
-  for (size_t p = 0; p < chunk; ++p)
-    for (size_t x = 0; x < (size_t)kXcds; ++x) {
-      const size_t i = x * chunk + p;
-      if (i < n) table.push_back(natural[i]);
-    }
+  double total = 0.0;
+  for (double w : weight) total += w;
+  std::vector<int2> queue[kXcds];
+  double cum = 0.0;
+  for (size_t i = 0; i < n; ++i) {
+    // the run in which the middle of the task falls
+    int x = total > 0.0 ? (int)((cum + 0.5 * weight[i]) * kXcds / total) : 0;
+    if (x >= kXcds) x = kXcds - 1;
+    queue[x].push_back(natural[i]);
+    cum += weight[i];
+  }
+  size_t longest = 0;
+  for (const auto &q : queue) longest = std::max(longest, q.size());
+  for (size_t p = 0; p < longest; ++p)
+    for (size_t x = 0; x < (size_t)kXcds; ++x)
+      table.push_back(p < queue[x].size() ? queue[x][p] : make_int2(-1, 0));
 }
 
 // {64-tiles, 128-tiles} x {slab float4, slab scalar, linear float4, linear scalar},
@@ -1340,6 +1377,7 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
   }
   size_t off = 0;
   std::vector<int2> natural[kGroupKinds], fin;
+  std::vector<double> weight[kGroupKinds];
   for (int i = 0; i < count; ++i) {
     GroupItemStatic &s = g->items[i];
     const bool macro = kind_of[i] >= kMacroKind0;
@@ -1356,7 +1394,21 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     if (!s.direct) off += (size_t)s.nsplit * slot;
     const int mt = (s.tiles + 1) / 2;
     const int per_slice = macro ? mt * (mt + 1) / 2 : s.ntile;
-    for (int w = 0; w < per_slice * s.nsplit; ++w) natural[kind_of[i]].push_back(make_int2(i, w));
+    for (int w = 0; w < per_slice * s.nsplit; ++w) {
+      natural[kind_of[i]].push_back(make_int2(i, w));
+      // the task's panel steps; a whole diagonal 128-tile takes three quarters of the time
+      const int split = w / per_slice, tile = w - split * per_slice;
+      const long long k0 = (long long)split * per, k1 = std::min<long long>(k0 + per, nk[i]);
+      double wt = (double)(k1 - k0);
+      if (!macro && s.bm == 128) {
+        int I = (int)((std::sqrt(8.0 * tile + 1.0) - 1.0) * 0.5);
+        while (I * (I + 1) / 2 > tile) --I;
+        while ((I + 1) * (I + 2) / 2 <= tile) ++I;
+        const int J = tile - I * (I + 1) / 2;
+        if (I == J && (I + 1) * 128 <= items[i].c) wt *= 0.75;
+      }
+      weight[kind_of[i]].push_back(wt);
+    }
     if (!s.direct) {
       const int sub = kfac::ceil_div(items[i].c, 64);
       for (int b = 0; b < sub * (sub + 1) / 2; ++b) fin.push_back(make_int2(i, b));
@@ -1366,8 +1418,8 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
   std::vector<int2> tasks;
   for (int k = 0; k < kGroupKinds; ++k) {
     g->task0[k] = (int)tasks.size();
-    g->ntask[k] = (int)natural[k].size();
-    deal_to_xcds(tasks, natural[k]);
+    deal_to_xcds(tasks, natural[k], weight[k]);
+    g->ntask[k] = (int)tasks.size() - g->task0[k];
   }
   g->ftask0 = (int)tasks.size();
   g->nftask = (int)fin.size();

@@ -434,7 +434,9 @@ __device__ __forceinline__ float fetch(const float *lds, int row, int k) {
 // the matrix cores (its block of the tile is not needed: above the diagonal of a
 // symmetric product, or past the end of the matrix); its accumulators stay as
 // they are.
-template <int WM, int WN, bool SAME, bool RS, class LA, class LB>
+// MASK: bit im * WN + in set = this wave computes block (im, in) of its 2 x 2
+// (compile time, so that a wave that owns fewer blocks carries no test per MFMA).
+template <int WM, int WN, bool SAME, bool RS, class LA, class LB, unsigned MASK = 0xffffffffu>
 __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int rowA0, int rowB0,
                                               long long kbeg, long long kend, float *ldsA,
                                               float *ldsB, floatx16 (&acc)[WM][WN], float *rs,
@@ -479,7 +481,8 @@ __device__ __forceinline__ void mainloop_impl(const LA &la, const LB &lb, int ro
       for (int im = 0; im < WM; ++im)
 #pragma unroll
         for (int in = 0; in < WN; ++in)
-          acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
+          if (MASK & (1u << (im * WN + in)))
+            acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[im], b[in], acc[im][in], 0, 0, 0);
     }
     }
     __syncthreads();
@@ -514,6 +517,29 @@ __device__ __forceinline__ bool syrk_wave_active(int row0A, int row0B, int dt,
                                                  int wave = threadIdx.x >> 6) {
   const int ra = row0A + (wave >> 1) * WM * 32, rb = row0B + (wave & 1) * WM * 32;
   return ra + WM * 32 > rb && ra < dt && rb < dt;
+}
+
+// The diagonal 128-tile of a symmetric product needs 10 of its 16 blocks of 32 x
+// 32 (the lower triangle).  Dealt by 64 x 64 quadrant, three waves compute four
+// blocks each (two of them above the diagonal) and the fourth wave nothing; here
+// the wave of the unused quadrant takes over the lower block row of quadrant
+// (1, 0) and the diagonal quadrants skip their upper block: 3, 2, 2 and 3 blocks,
+// three quarters of the time.
+//   role     the wave index (2 x 2 layout) whose accumulator coordinates this wave uses
+//   compute  bit im * 2 + in: block (im, in) is multiplied out
+//   store    bit im * 2 + in: block (im, in) is this wave's to write (a block that
+//            is not computed but stored holds zeros)
+struct DiagRole {
+  int role;
+  unsigned compute, store;
+};
+__device__ __forceinline__ DiagRole diag_tile_role(int wave) {
+  switch (wave) {
+    case 0: return DiagRole{0, 0xdu, 0xfu};    // quadrant (0,0): blocks (0,0) (1,0) (1,1)
+    case 3: return DiagRole{3, 0xdu, 0xfu};    // quadrant (1,1)
+    case 2: return DiagRole{2, 0x3u, 0x3u};    // quadrant (1,0), upper block row
+    default: return DiagRole{2, 0xcu, 0xcu};   // the wave of quadrant (0,1): quadrant (1,0), lower block row
+  }
 }
 
 // Set every accumulator element of this lane to f(row, col), row / col relative
@@ -553,6 +579,25 @@ __device__ __forceinline__ void for_each_acc(floatx16 (&acc)[WM][WN], F f,
       }
 }
 
+// for_each_acc over the blocks whose bit (im * WN + in) is set in `mask`
+template <int WM, int WN, class F>
+__device__ __forceinline__ void for_each_acc_masked(floatx16 (&acc)[WM][WN], unsigned mask, F f, int wave) {
+  const int lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int im = 0; im < WM; ++im)
+#pragma unroll
+    for (int in = 0; in < WN; ++in) {
+      if (!(mask & (1u << (im * WN + in)))) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = (wm * WM + im) * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int col = (wn * WN + in) * 32 + (lane & 31);
+        f(row, col, acc[im][in][v]);
+      }
+    }
+}
+
 template <int WM, int WN>
 __device__ __forceinline__ void zero_acc(floatx16 (&acc)[WM][WN]) {
 #pragma unroll
@@ -570,10 +615,12 @@ __device__ __forceinline__ void zero_acc(floatx16 (&acc)[WM][WN]) {
 // diagonal of a diagonal tile is skipped (it is the mirror of the one below),
 // and a quadrant on the diagonal writes its upper triangle from its lower one.
 // Rows and columns below dt (the tiled part); d is the leading dimension of C.
+// `store`: the blocks of this wave's 2 x 2 that are its to write (see DiagRole).
 template <int WM>
 __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, int I, int J,
                                            int dt, int d, float alpha, float beta,
-                                           float *__restrict__ C, int wave = threadIdx.x >> 6) {
+                                           float *__restrict__ C, int wave = threadIdx.x >> 6,
+                                           unsigned store = 0xffffffffu) {
   constexpr int BM = 64 * WM;
   float(*t)[65] = reinterpret_cast<float(*)[65]>(lds);
   const int lc = threadIdx.x & 63, lr0 = threadIdx.x >> 6;
@@ -582,7 +629,7 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
     if (I == J && qm < qn) continue;
     const bool diag = I == J && qm == qn;
     __syncthreads();
-    for_each_acc<WM, WM>(acc, [&](int r, int c, float v) {
+    for_each_acc_masked<WM, WM>(acc, store, [&](int r, int c, float v) {
       if (r / 64 == qm && c / 64 == qn) t[r % 64][c % 64] = v;
     }, wave);
     __syncthreads();

@@ -607,7 +607,14 @@ extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int
   for (int p = 0; p < 2; ++p) {
     double per_wg[kPreKinds];
     for (int k = 0; k < kPreKinds; ++k) {
-      per_wg[k] = work[p][k] / 2304.0;
+      // ~4096 workgroups per launch: five rounds of 3 x 256.  Measured on ResNet-50 (kernel
+      // time of the six launches / whole phase with its finish launches): 2304 tasks 1.89 /
+      // 2.04 ms, 3072 1.69 / 1.95, 4608 1.61 / 1.97, 6144 1.60 / 2.02, 9216 1.61 / 2.11: shorter
+      // tasks shorten the tail of a launch, more k-slices lengthen the finish.
+      // KFAC_PRECOND_TASKS is a tuning override.
+      double ntasks = 4096.0;
+      if (const char *env = getenv("KFAC_PRECOND_TASKS")) ntasks = std::max(1.0, atof(env));
+      per_wg[k] = work[p][k] / ntasks;
       if (per_wg[k] < 32.0) per_wg[k] = 32.0;
       if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override
         const double val = atof(env);
