@@ -790,8 +790,9 @@ __global__ __launch_bounds__(THREADS, 2) void lauum_kernel(InvTables tb, int tas
       if (I == 0 && threadIdx.x == 0) out[(long long)(d - 1) * d + d - 1] = sigma;
     }
   }
-  // through an LDS transpose, so that the mirror is written in row segments too
-  write_tile<2>(acc, lds, I, J, dc, d, 1.f, 0.f, out);
+  // through LDS, so that the mirror is written in row segments too
+  static_assert(kWholeTileLdsFloats <= kTileLdsFloats, "the tile must fit the panels' LDS");
+  write_whole_tile(acc, lds, I, J, dc, d, out);
 }
 
 // Dynamic LDS.  The trailing update ("rest") asks for 81 KB although it uses 74:

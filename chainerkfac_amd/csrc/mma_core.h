@@ -662,5 +662,71 @@ __device__ __forceinline__ void write_tile(floatx16 (&acc)[WM][WM], float *lds, 
   }
 }
 
+// The finished 128 x 128 tile (I, J), I >= J, and its mirror image written to C
+// (leading dimension d, rows and columns below dt) in one go: the whole tile is
+// laid out in LDS (128 x 129 floats) once, then every thread stores 16 bytes at
+// a time (at float granularity: rows of an odd-sized matrix do not start on
+// 16-byte boundaries), rows of the tile and rows of the mirrored tile alike.
+// For C = acc (no scaling, no accumulation); ends without a barrier.
+constexpr int kWholeTileLdsFloats = 128 * 129;
+__device__ __forceinline__ void write_whole_tile(floatx16 (&acc)[2][2], float *lds, int I, int J, int dt,
+                                                 int d, float *__restrict__ C) {
+  typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+  constexpr int LD = 129;
+  __syncthreads();   // the main loop's last LDS reads
+  for_each_acc<2, 2>(acc, [&](int r, int c, float v) { lds[r * LD + c] = v; });
+  __syncthreads();
+  const int q = (threadIdx.x & 31) * 4;    // four columns
+  const int r0 = threadIdx.x >> 5;         // 8 rows per pass
+  const int row0 = I * 128, col0 = J * 128;
+  const bool diag = I == J;
+#pragma unroll 4
+  for (int p = 0; p < 16; ++p) {
+    const int lr = r0 + 8 * p;
+    const int r = row0 + lr, c = col0 + q;
+    if (r >= dt) continue;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (!diag || q + e <= lr) ? lds[lr * LD + q + e] : lds[(q + e) * LD + lr];
+    float *dst = C + (long long)r * d + c;
+    if (c + 3 < dt) {
+      floatx4u o;
+      o.x = v[0];
+      o.y = v[1];
+      o.z = v[2];
+      o.w = v[3];
+      *reinterpret_cast<floatx4u *>(dst) = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c + e < dt) dst[e] = v[e];
+    }
+  }
+  if (diag) return;
+  // mirrored tile (J, I): its row lr is column lr of the tile
+#pragma unroll 4
+  for (int p = 0; p < 16; ++p) {
+    const int lr = r0 + 8 * p;
+    const int r = col0 + lr, c = row0 + q;
+    if (r >= dt) continue;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = lds[(q + e) * LD + lr];
+    float *dst = C + (long long)r * d + c;
+    if (c + 3 < dt) {
+      floatx4u o;
+      o.x = v[0];
+      o.y = v[1];
+      o.z = v[2];
+      o.w = v[3];
+      *reinterpret_cast<floatx4u *>(dst) = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c + e < dt) dst[e] = v[e];
+    }
+  }
+}
+
 }  // namespace mma
 }  // namespace kfac
