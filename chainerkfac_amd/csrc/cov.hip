@@ -1179,7 +1179,22 @@ __global__ __launch_bounds__(256) void finish_group_kernel(const GroupItemStatic
   float sum[16];
 #pragma unroll
   for (int p = 0; p < 16; ++p) sum[p] = 0.f;
-  for (int k = 0; k < s.nsplit; ++k) {
+  // four slices' loads in flight at a time (the sums stay in slice order)
+  int k = 0;
+  for (; k + 4 <= s.nsplit; k += 4) {
+    float x[4][16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float *pk = p0 + (k + q) * slot;
+#pragma unroll
+      for (int p = 0; p < 16; ++p) x[q][p] = pk[(lr0 + 4 * p) * bm + lc];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int p = 0; p < 16; ++p) sum[p] += x[q][p];
+  }
+  for (; k < s.nsplit; ++k) {
     const float *pk = p0 + k * slot;
 #pragma unroll
     for (int p = 0; p < 16; ++p) sum[p] += pk[(lr0 + 4 * p) * bm + lc];

@@ -518,8 +518,17 @@ __global__ __launch_bounds__(256) void gemm_group_finish_kernel(const PreStatic 
   const int tile = (i / bm) * s.tn + j / bm;
   const float *p = ws + s.part_off + (long long)tile * bm * bm + (i % bm) * bm + (j % bm);
   const long long stride = (long long)ntiles * bm * bm;
+  // eight slices' loads in flight at a time (the sum stays in slice order)
   float sum = 0.f;
-  for (int k = 0; k < s.nsplit[PHASE]; ++k) sum += p[k * stride];
+  int k = 0;
+  for (; k + 8 <= s.nsplit[PHASE]; k += 8) {
+    float x[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) x[q] = p[(k + q) * stride];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sum += x[q];
+  }
+  for (; k < s.nsplit[PHASE]; ++k) sum += p[k * stride];
   if (PHASE == 0)
     (ws + s.t_off)[(long long)i * s.ldT + j] = sum;
   else if (j < s.dW)
