@@ -369,18 +369,29 @@ __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
   float *__restrict__ dst = tile_ptr(tb, s, I, J);
   const int c4 = (threadIdx.x & 31) * 4;
   const int r0 = threadIdx.x >> 5;
-#pragma unroll 4
+  // 16-byte loads at float granularity (the rows of an odd-sized matrix do not start on
+  // 16-byte boundaries); the quads cut by the edge of the matrix go element by element
+  typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+#pragma unroll 8
   for (int p = 0; p < NB / 8; ++p) {
     const int rl = r0 + 8 * p;
     const int r = I * NB + rl;
     const int c = J * NB + c4;
     float v[4];
+    if (r < dc && c + 3 < dc) {
+      const floatx4u x = *reinterpret_cast<const floatx4u *>(src + (long long)r * d + c);
+      v[0] = x.x;
+      v[1] = x.y;
+      v[2] = x.z;
+      v[3] = x.w;
+    } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int ce = c + e;
-      float x = (r == ce) ? 1.f : 0.f;
-      if (r < dc && ce < dc) x = src[(long long)r * d + ce];
-      v[e] = x;
+      for (int e = 0; e < 4; ++e) {
+        const int ce = c + e;
+        float x = (r == ce) ? 1.f : 0.f;
+        if (r < dc && ce < dc) x = src[(long long)r * d + ce];
+        v[e] = x;
+      }
     }
     *reinterpret_cast<float4 *>(dst + rl * NB + c4) = make_float4(v[0], v[1], v[2], v[3]);
   }
