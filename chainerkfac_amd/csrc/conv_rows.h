@@ -73,21 +73,17 @@ struct RowsCfg {
 // operand values it feeds to the matrix cores into rs[im]: rs ends as the sum
 // over this lane's sample of row (wave_m * WM + im) * 32 + lane % 32; the other
 // sample's half is in lane ^ 32.
-// `wave` is the wave's index in the workgroup (its share of the staging), `role`
-// the wave index whose blocks of the tile it multiplies out, MASK (bit im * WM + in)
-// which of them: the waves of a whole diagonal 128-tile share its ten blocks
-// (DiagRole); everywhere else role = wave and MASK = all.
-template <class Cfg, bool SAME, unsigned MASK = 0xffffffffu>
+template <class Cfg, bool SAME>
 __device__ __forceinline__ void rows_mainloop(const RowsGeom &g, int row0A, int row0B,
                                               long long sbeg, long long send, float *smem,
                                               floatx16 (&acc)[Cfg::WM][Cfg::WM],
-                                              float (&rs)[Cfg::WM], int wave, int role) {
+                                              float (&rs)[Cfg::WM], int wave) {
   constexpr int WM = Cfg::WM, KK = Cfg::KK, K = Cfg::K, S = Cfg::S, P = Cfg::P;
   constexpr int RIN = Cfg::RIN, WR = Cfg::WR, RSZ = Cfg::RSZ, REGION = Cfg::REGION;
   constexpr int PARTS = Cfg::PARTS, NK = Cfg::NK, CH = Cfg::CH, NCOL = Cfg::NCOL;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wm = role >> 1, wn = role & 1;
+  const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane & 31, lk = lane >> 5;
   const int HW = g.H * g.W;
   constexpr int regA = 0, regB = SAME ? 0 : 2 * REGION;
@@ -178,7 +174,7 @@ __device__ __forceinline__ void rows_mainloop(const RowsGeom &g, int row0A, int 
 
   // a wave whose 64 x 64 block lies above the diagonal or past the end of the
   // factor stages like the others but leaves the matrix cores to them
-  const bool active = MASK != 0xffffffffu || syrk_wave_active<WM>(row0A, row0B, g.d_patch, role);
+  const bool active = syrk_wave_active<WM>(row0A, row0B, g.d_patch, wave);
   if (sbeg < send) issue();
   for (long long s = sbeg; s < send; ++s) {
     stash();
@@ -230,9 +226,8 @@ __device__ __forceinline__ void rows_mainloop(const RowsGeom &g, int row0A, int 
           for (int im = 0; im < WM; ++im)
 #pragma unroll
             for (int in = 0; in < WM; ++in)
-              if (MASK & (1u << (im * WM + in)))
-                acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][e][im], b[cur][e][in],
-                                                                   acc[im][in], 0, 0, 0);
+              acc[im][in] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][e][im], b[cur][e][in],
+                                                                 acc[im][in], 0, 0, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);

@@ -400,12 +400,6 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_rows_kernel(RowsGeom g, long 
   const int tiles = (dt + BM - 1) / BM;
   int split, tile, I, J;
   work_decode(blockIdx.x, ntile * nsplit, ntile, tiles, split, tile, I, J);
-  const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
-  float *mine = partial + split * slot;
-  // the four waves of a whole diagonal 128-tile share its ten blocks (DiagRole).  Giving
-  // such tiles longer k-slices in return (their workgroups finish earlier) was measured
-  // slower: a step's staging does not shrink with its MFMA count.
-  const bool whole_diag = WM == 2 && I == J && (I + 1) * BM <= dt;
   // padding columns, the planes of zeros and everything else not staged later
   for (int e = threadIdx.x; e < Cfg::lds_floats(false); e += THREADS) smem[e] = 0.f;
   __syncthreads();
@@ -418,33 +412,21 @@ __global__ __launch_bounds__(THREADS, 2) void syrk_rows_kernel(RowsGeom g, long 
 #pragma unroll
   for (int im = 0; im < WM; ++im) rs[im] = 0.f;
   const int wave = threadIdx.x >> 6;
-  int role = wave;
-  unsigned store = 0xfu, rowmask = 0x3u;
-  if (whole_diag) {
-    const DiagRole r = diag_tile_role(wave);
-    role = r.role;
-    store = r.store;
-    rowmask = r.compute == 0xdu ? 0x3u : (r.compute == 0x3u ? 0x1u : 0x2u);
-    if (r.compute == 0xdu)
-      rows_mainloop<Cfg, true, 0xdu>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave, role);
-    else if (r.compute == 0x3u)
-      rows_mainloop<Cfg, true, 0x3u>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave, role);
-    else
-      rows_mainloop<Cfg, true, 0xcu>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave, role);
-  } else if (I == J) {
-    rows_mainloop<Cfg, true>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave, wave);
-  } else {
-    rows_mainloop<Cfg, false>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave, wave);
-  }
+  if (I == J)
+    rows_mainloop<Cfg, true>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave);
+  else
+    rows_mainloop<Cfg, false>(g, I * BM, J * BM, sbeg, send, smem, acc, rs, wave);
+  const long long slot = (long long)ntile * (BM * BM) + (long long)tiles * BM;
+  float *mine = partial + split * slot;
   if (ones && I == J)
     write_rowsums<WM>(rs, I, dt, d, direct, count, alpha, beta, mine + (long long)ntile * (BM * BM), C,
-                      role, rowmask);
+                      wave);
   if (direct) {
-    write_tile<WM>(acc, smem, I, J, dt, d, alpha, beta, C, role, store);
+    write_tile<WM>(acc, smem, I, J, dt, d, alpha, beta, C, wave);
     return;
   }
   float *out = mine + (long long)tile * (BM * BM);
-  for_each_acc_masked<WM, WM>(acc, store, [&](int r, int c, float v) { out[r * BM + c] = v; }, role);
+  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; }, wave);
 }
 
 // One workgroup per 64x64 sub-block (si >= sj) of C.  The number of slices is a
