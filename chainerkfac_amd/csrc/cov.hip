@@ -702,7 +702,7 @@ int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int
   g.x_bytes = (unsigned)((long long)n * c * h * w * (long long)sizeof(float));
   const long long total_steps = (long long)(n / 2) * g.rgroups;
   const float count = (float)((long long)n * ho * Cfg::WS);
-  if (d - ones <= 320) return 1;   // small factors: 64-tiles of the general kernel
+  if (d - ones <= 256) return 1;   // small factors: 64-tiles of the general kernel
   constexpr size_t lds = (size_t)Cfg::lds_floats(false) * sizeof(float);
   constexpr int occ = (160 * 1024) / lds >= 3 ? 3 : (int)((160 * 1024) / lds);
   const SyrkPlan p = plan_rows(d - ones, 64 * Cfg::WM, total_steps, Cfg::NK * Cfg::WM * Cfg::WM * 64 / 2400.0, occ);
@@ -752,10 +752,22 @@ int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, in
     return run_conv_rows<RowsCfg<2, K, S, P, WS, RT, PAD>>(x, n, c, h, w, ho, d, ones, alpha,     \
                                                            beta, C, ws, ws_bytes, stream);        \
   }
+  // (kernel, stride, padding, output width, output rows per step, plane padding: the
+  // smallest that leaves the 32 operand rows of a block on 32 different banks of 64)
   KFAC_ROWS_CASE(3, 1, 1, 56, 1, 0)
   KFAC_ROWS_CASE(3, 1, 1, 28, 2, 1)
   KFAC_ROWS_CASE(3, 1, 1, 14, 7, 3)
   KFAC_ROWS_CASE(3, 1, 1, 7, 7, 9)
+  // the strided 3x3 convolutions of ResNet-D (56 -> 28, 28 -> 14) and its 112-wide stem.  (14 -> 7
+  // with the whole 7x7 output per step needs 65 KB of LDS, two workgroups per CU, and was
+  // measured slower than the halo-region kernel: 443 against 364 us for 512 channels.)
+  KFAC_ROWS_CASE(3, 2, 1, 28, 1, 1)
+  KFAC_ROWS_CASE(3, 2, 1, 14, 2, 6)
+  KFAC_ROWS_CASE(3, 1, 1, 112, 1, 1)
+  // CIFAR-sized images
+  KFAC_ROWS_CASE(3, 1, 1, 32, 2, 0)
+  KFAC_ROWS_CASE(3, 1, 1, 16, 4, 8)
+  KFAC_ROWS_CASE(3, 1, 1, 8, 8, 11)
 #undef KFAC_ROWS_CASE
   return 1;
 }

@@ -77,6 +77,13 @@ CONV_CASES = [
     (2, 150, 7, 7, 3, 1, 1, True),      # 1351: eleven tile rows, panels that start mid-channel
     (6, 64, 14, 14, 3, 1, 1, True),     # three sample pairs
     (2, 48, 28, 28, 3, 1, 1, True),     # 433
+    # the same kernel's other geometries: 112-wide rows, stride 2 (28/14/7-wide outputs), CIFAR widths
+    (2, 32, 112, 112, 3, 1, 1, False),  # 288: the stem of ResNet-D, 64-tiles with a ragged fifth
+    (2, 30, 112, 112, 3, 1, 1, True),   # 271
+    (2, 64, 56, 56, 3, 2, 1, False),    # stride 2, 28-wide outputs, one row per step
+    (2, 40, 28, 28, 3, 2, 1, True),     # stride 2, 14-wide outputs, two rows per step
+    (4, 64, 14, 14, 3, 2, 1, False),    # stride 2, 7-wide outputs (halo-region kernel)
+    (2, 64, 32, 32, 3, 1, 1, True),     # 32-wide rows, two per step
 ]
 
 
