@@ -702,7 +702,9 @@ int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int
   g.x_bytes = (unsigned)((long long)n * c * h * w * (long long)sizeof(float));
   const long long total_steps = (long long)(n / 2) * g.rgroups;
   const float count = (float)((long long)n * ho * Cfg::WS);
-  if (d - ones <= 256) return 1;   // small factors: 64-tiles of the general kernel
+  // small factors: 64-tiles of the general kernel (a 7x7 kernel has 49 taps per channel: 3
+  // channels are a factor of 147 rows, and the element gather it would otherwise take is slow)
+  if (d - ones <= (Cfg::K == 7 ? 128 : 256)) return 1;
   constexpr size_t lds = (size_t)Cfg::lds_floats(false) * sizeof(float);
   constexpr int occ = (160 * 1024) / lds >= 3 ? 3 : (int)((160 * 1024) / lds);
   const SyrkPlan p = plan_rows(d - ones, 64 * Cfg::WM, total_steps, Cfg::NK * Cfg::WM * Cfg::WM * 64 / 2400.0, occ);
@@ -764,6 +766,8 @@ int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, in
   KFAC_ROWS_CASE(3, 2, 1, 28, 1, 1)
   KFAC_ROWS_CASE(3, 2, 1, 14, 2, 6)
   KFAC_ROWS_CASE(3, 1, 1, 112, 1, 1)
+  // the 7x7 stride-2 stem of ResNet at 224 x 224
+  KFAC_ROWS_CASE(7, 2, 3, 112, 1, 0)
   // CIFAR-sized images
   KFAC_ROWS_CASE(3, 1, 1, 32, 2, 0)
   KFAC_ROWS_CASE(3, 1, 1, 16, 4, 8)

@@ -84,6 +84,7 @@ CONV_CASES = [
     (2, 40, 28, 28, 3, 2, 1, True),     # stride 2, 14-wide outputs, two rows per step
     (4, 64, 14, 14, 3, 2, 1, False),    # stride 2, 7-wide outputs (halo-region kernel)
     (2, 64, 32, 32, 3, 1, 1, True),     # 32-wide rows, two per step
+    (2, 3, 224, 224, 7, 2, 3, True),    # 148: the ImageNet stem, 112-wide outputs
 ]
 
 
