@@ -489,7 +489,7 @@ def run_inverse_config(args, name, cfg):
     }, dims
 
 
-def write_per_layer(path, layers):
+def write_per_layer(path, layers, config='c3'):
     """Per-layer roofline table of the covariance kernels (markdown): every distinct
     convolution / linear shape of the workload, its A and G factor timed alone on one
     stream (HIP events inside the library around the SYRK launch, empty bracket
@@ -553,7 +553,7 @@ def write_per_layer(path, layers):
         del x, gy
     with open(path, 'w') as f:
         f.write('# Covariance kernels layer by layer (every distinct convolution / linear shape of the workload)\n\n'
-                'Command (one MI355X, repository root):\n\n```\npython3 bench.py --config c3 --no-cpu --no-dense-field '
+                'Command (one MI355X, repository root):\n\n```\npython3 bench.py --config {} --no-cpu --no-dense-field '
                 '--steps 5 --per-layer {}\n```\n\n'
                 'Each factor is computed alone, by the single-factor entry point, on one stream; "SYRK kernel us" is '
                 'the duration of its SYRK launch (HIP events inside the library around the launch, 10 repetitions, the '
@@ -562,7 +562,7 @@ def write_per_layer(path, layers):
                 'batch-norm layers) do not run alone but in a handful of grouped launches, so their rows here show the '
                 'latency floor of a single launch, not their cost in the step. GFLOP = M d (d+1); flop/B = that over '
                 'the bytes of the input tensor read once plus the factor written once; roofline cap = min(157.3 '
-                'TFLOP/s FP32 MFMA, flop/B x 8 TB/s).\n\n'.format(path, empty * 1e3))
+                'TFLOP/s FP32 MFMA, flop/B x 8 TB/s).\n\n'.format(config, path, empty * 1e3))
         f.write('| layer (x count) | factor | d | rows M | GFLOP | SYRK kernel us | TFLOP/s | flop/B | roofline cap TFLOP/s '
                 '| fraction of cap |\n|---|---|---:|---:|---:|---:|---:|---:|---:|---:|\n')
         for desc, count, fac, d, M, gf, us, tf, ai, cap, frac in rows:
@@ -935,7 +935,7 @@ def main():
     else:
         result = run_step_config(args, args.config, cfg)
         if args.per_layer:
-            write_per_layer(args.per_layer, cfg['layers'])
+            write_per_layer(args.per_layer, cfg['layers'], args.config)
     if not args.no_cpu:
         result['cpu_baseline'] = run_cpu_baseline(args.config, cfg)
     print(json.dumps(result))
