@@ -31,6 +31,7 @@
 #include "common.h"
 #include "conv_halo.h"
 #include "conv_rows.h"
+#include "conv_shift.h"
 #include "mma_core.h"
 
 namespace {
@@ -776,6 +777,111 @@ int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, in
   return 1;
 }
 
+// The shifted-correlation route (conv_shift.h) for a 3x3, stride-1, padding-1
+// convolution: 1 when the shape is left to the patch-product kernels (few
+// channels, tiny images, workspace too small).
+template <int WM>
+int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float beta, float *C, void *ws,
+                   size_t ws_bytes, hipStream_t stream) {
+  using namespace kfac::shift;
+  constexpr int BM = 64 * WM;
+  const int c = pl.C, h = pl.H, w = pl.W, n = pl.n;
+  pl.tiles = kfac::ceil_div(c, BM);
+  const int ntile = pl.tiles * pl.tiles;
+  int np = 0;
+  auto add = [&](unsigned base_off, int L, int line_len, int da, int db, int amax, int bmax, int out,
+                 int out_t) {
+    Product &p = pl.prod[np++];
+    p.base_off = base_off;
+    p.L = (unsigned)L;
+    p.line_len = (unsigned)line_len;
+    p.da = (short)da; p.db = (short)db; p.amax = (short)amax; p.bmax = (short)bmax;
+    p.K = n * L;
+    p.out = (short)out; p.out_t = (short)out_t;
+  };
+  for (int di = 0; di <= 2; ++di)
+    for (int dj = (di == 0 ? 0 : -2); dj <= 2; ++dj)
+      add(0, h * w, w, di, dj, h, w, (di + 2) * 5 + dj + 2, (2 - di) * 5 + 2 - dj);
+  for (int last = 0; last < 2; ++last)
+    for (int dj = 0; dj <= 2; ++dj)
+      add(last ? (unsigned)(h - 1) * w : 0u, w, w, 0, dj, 1, w, 25 + 5 * last + dj + 2, 25 + 5 * last + 2 - dj);
+  for (int last = 0; last < 2; ++last)
+    for (int di = 0; di <= 2; ++di)
+      add(last ? (unsigned)(w - 1) : 0u, h, 1, di, 0, h, 1, 35 + 5 * last + di + 2, 35 + 5 * last + 2 - di);
+  for (int lr = 0; lr < 2; ++lr)
+    for (int lc = 0; lc < 2; ++lc)
+      add((lr ? (unsigned)(h - 1) * w : 0u) + (lc ? (unsigned)(w - 1) : 0u), 1, 1, 0, 0, 1, 1,
+          45 + 2 * lr + lc, 45 + 2 * lr + lc);
+  if (np != kProducts) return kfac::fail(KFAC_EINVAL, "internal: %d products", np);
+  // slices of about equal length over all products, ~target workgroups in all
+  long long units = 0;
+  for (int i = 0; i < np; ++i) units += (long long)ntile * kfac::ceil_div(pl.prod[i].K, KT);
+  long long target = WM == 1 ? 1024 : 1536;
+  if (const char *env = getenv("KFAC_SHIFT_TARGET")) target = std::max(1ll, atoll(env));   // tuning override
+  long long per = std::max<long long>(6, kfac::ceil_div(units, target));
+  int total = 0;
+  for (int i = 0; i < np; ++i) {
+    Product &p = pl.prod[i];
+    const long long nk = kfac::ceil_div(p.K, KT);
+    const long long ns = kfac::ceil_div(nk, per);
+    const long long len = kfac::ceil_div(nk, ns);
+    p.nsplit = (int)kfac::ceil_div(nk, len);
+    p.klen = (int)len * KT;
+    p.task0 = total;
+    total += ntile * p.nsplit;
+  }
+  pl.total = total;
+  const int nchunk = std::min(n, 8);
+  const size_t partial_floats = (size_t)total * BM * BM;
+  const size_t array_floats = (size_t)kArrays * c * c;
+  const size_t sums_floats = (size_t)nchunk * c * kChannelSums;
+  if (ws == nullptr || ws_bytes < (partial_floats + array_floats + sums_floats) * sizeof(float)) return 1;
+  float *partial = static_cast<float *>(ws);
+  float *arrays = partial + partial_floats;
+  float *sums = arrays + array_floats;
+  if (ones) {
+    hipLaunchKernelGGL(channel_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums);
+    KFAC_HIP_CHECK(hipGetLastError());
+  }
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
+    hipLaunchKernelGGL((corr_kernel<WM>), dim3(total), dim3(THREADS), 0, stream, pl, partial);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  const int nb = kfac::ceil_div(c, 32);
+  hipLaunchKernelGGL((corr_finish_kernel<WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
+                     arrays);
+  KFAC_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL(assemble_kernel, dim3(c, kfac::ceil_div(c, 64)), dim3(256), 0, stream, pl, arrays, sums,
+                     nchunk, d, ones, (float)((long long)n * h * w), alpha, beta, C);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+int try_conv_shift(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
+                   int pw, int d, int ones, float alpha, float beta, float *C, void *ws, size_t ws_bytes,
+                   hipStream_t stream) {
+  if (kh != 3 || kw != 3 || sy != 1 || sx != 1 || ph != 1 || pw != 1) return 1;
+  int min_c = 64;
+  if (const char *env = getenv("KFAC_CONV_SHIFT")) {   // tuning override: 0 = off, else the least channel count
+    min_c = atoi(env);
+    if (min_c <= 0) return 1;
+  }
+  if (c < min_c || h < 4 || w < 4 || h > 32767 || w > 32767) return 1;
+  kfac::shift::Plan pl;
+  memset(&pl, 0, sizeof(pl));
+  pl.x = x;
+  pl.sample_stride = (unsigned)((long long)c * h * w);
+  pl.row_stride = (unsigned)(h * w);
+  pl.line_stride = (unsigned)w;
+  pl.C = c; pl.H = h; pl.W = w; pl.n = n;
+  // 128-tiles unless 64-tiles waste much less on a channel count that is not a multiple of 128
+  const long long t64 = kfac::ceil_div(c, 64), t128 = kfac::ceil_div(c, 128);
+  if (1.15 * (double)(t64 * t64) < 4.0 * (double)(t128 * t128))
+    return run_conv_shift<1>(pl, d, ones, alpha, beta, C, ws, ws_bytes, stream);
+  return run_conv_shift<2>(pl, d, ones, alpha, beta, C, ws, ws_bytes, stream);
+}
+
 bool kc_vec_ok(const float *base, long long sample_stride, long long row_stride, int L) {
   return (sample_stride % 4 == 0) && (row_stride % 4 == 0) && (L % 4 == 0) &&
          (reinterpret_cast<uintptr_t>(base) % 16 == 0);
@@ -922,6 +1028,11 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
     l64.line_stride = l128.line_stride = (unsigned)(sy * w);
     l64.px_stride = l128.px_stride = (unsigned)sx;
     return run_syrk(l64, l128, d, ones, K, alpha, beta, C, ws, ws_bytes, s);
+  }
+  {
+    const int rc = try_conv_shift(x, n, c, h, w, kh, kw, sy, sx, ph, pw, d, ones, alpha, beta, C, ws,
+                                  ws_bytes, s);
+    if (rc <= 0) return rc;   // 1 = shape left to the patch-product kernels
   }
   {
     const int rc = try_conv_rows(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, d, ones, alpha, beta, C,

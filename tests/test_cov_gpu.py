@@ -88,12 +88,74 @@ CONV_CASES = [
 ]
 
 
+def takes_shift_route(c, h, w, k, s, p):
+    """3x3 / stride 1 / padding 1 with at least 64 channels: computed from shifted correlations of
+    the input unless KFAC_CONV_SHIFT=0 leaves it to the patch-product kernels."""
+    return k == 3 and s == 1 and p == 1 and c >= 64 and h >= 4 and w >= 4
+
+
+@pytest.fixture
+def patch_product_route(monkeypatch):
+    def switch(on):
+        if on:
+            monkeypatch.setenv('KFAC_CONV_SHIFT', '0')
+        else:
+            monkeypatch.delenv('KFAC_CONV_SHIFT', raising=False)
+    return switch
+
+
 @pytest.mark.parametrize('n,c,h,w,k,s,p,bias', CONV_CASES)
-def test_conv_A(n, c, h, w, k, s, p, bias):
+def test_conv_A(n, c, h, w, k, s, p, bias, patch_product_route):
     from chainerkfac_amd import ops
     x = np.random.default_rng(c * h + k).standard_normal((n, c, h, w)).astype(np.float32)
+    ref = O.conv_A(x, k, s, p, bias)
     A = ops.cov_conv_a(torch.from_numpy(x).cuda(), k, s, p, bias, 1.0 / n)
-    check(A, O.conv_A(x, k, s, p, bias))
+    check(A, ref)
+    if takes_shift_route(c, h, w, k, s, p):
+        # the same shape through the patch-product kernels
+        patch_product_route(True)
+        B = ops.cov_conv_a(torch.from_numpy(x).cuda(), k, s, p, bias, 1.0 / n)
+        patch_product_route(False)
+        check(B, ref)
+        assert rel_err(A.cpu().numpy(), B.cpu().numpy()) < 1e-5
+
+
+SHIFT_CASES = [
+    # n, c, h, w, bias: 3x3 / 1 / 1 shapes of the shifted-correlation route
+    (1, 64, 4, 4, True),        # the smallest image it takes: border strips are half the image
+    (3, 64, 5, 9, True),        # odd batch, H != W
+    (2, 96, 12, 10, False),     # one 128-tile, a quarter of it padding
+    (2, 200, 6, 7, True),       # two 128-tiles per side, the second ragged
+    (1, 64, 20, 112, True),     # long image rows
+    (2, 64, 56, 56, False),     # 3136 pixels: k-slices that start inside an image
+    (2, 256, 14, 14, True),     # four tiles per product
+    (5, 130, 7, 7, True),       # channel count just past a tile
+    (2, 64, 1000, 4, True),     # tall and narrow: column strips of 1000 pixels
+]
+
+
+@pytest.mark.parametrize('n,c,h,w,bias', SHIFT_CASES)
+def test_conv_A_shift_route(n, c, h, w, bias):
+    from chainerkfac_amd import ops
+    assert takes_shift_route(c, h, w, 3, 1, 1)
+    x = np.random.default_rng(c + h * w).standard_normal((n, c, h, w)).astype(np.float32)
+    x += 0.5    # non-zero mean: the ones column is not just noise
+    A = ops.cov_conv_a(torch.from_numpy(x).cuda(), 3, 1, 1, bias, 1.0 / n)
+    check(A, O.conv_A(x, 3, 1, 1, bias))
+
+
+def test_conv_A_shift_route_border_terms():
+    """An input that is zero except on the image border and corners: every entry of the factor is
+    then made of the border corrections (row / column strips and corner pixels) alone."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(3)
+    x = np.zeros((2, 64, 6, 8), np.float32)
+    x[:, :, 0, :] = r.standard_normal((2, 64, 8))
+    x[:, :, -1, :] = r.standard_normal((2, 64, 8))
+    x[:, :, :, 0] = r.standard_normal((2, 64, 6))
+    x[:, :, :, -1] = r.standard_normal((2, 64, 6))
+    A = ops.cov_conv_a(torch.from_numpy(x).cuda(), 3, 1, 1, True, 0.5)
+    check(A, O.conv_A(x, 3, 1, 1, True))
 
 
 @pytest.mark.parametrize('n,c,ho,wo', [(2, 5, 3, 3), (4, 64, 16, 16), (3, 130, 7, 7), (2, 256, 4, 4),
