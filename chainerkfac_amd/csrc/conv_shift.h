@@ -104,169 +104,272 @@ using namespace kfac::mma;
 //   [45, 49)  corner pixels: 45 + 2 * (last row) + (last column)
 constexpr int kArrays = 49;
 constexpr int kProducts = 29;
+constexpr int kGroups = 11;
 constexpr int kChannelSums = 9;   // whole image, first / last row, first / last column, 4 corners
 
-struct Product {
-  unsigned base_off;   // first element of the domain within an image plane
-  unsigned L;          // k-values per sample: pixels of the domain
-  unsigned line_len;   // p -> (a, b) = (p / line_len, p % line_len)
-  short da, db;        // the second operand's shift
-  short amax, bmax;    // bounds of a + da, b + db
+// Products that share their first operand and differ in the second operand's
+// shift along the domain are computed together, ns (3 or 5) at a time.  A domain
+// is a set of pixels per sample, numbered p < L: the whole image (three groups,
+// one per row shift di: column shifts 0..2 for di = 0, whose negative ones are
+// transposes, and -2..2 for di = 1, 2), the first or last image row (column shifts
+// 0..2), the first or last image column (row shifts 0..2, which move along the
+// column) or one corner pixel.
+//   memory:  pixel p of sample s, channel c at
+//            base[s * sample_stride + c * row_stride + (p / mem_line) * line_stride + p % mem_line]
+//   shift e (= dj0 + 0 .. ns - 1) of row shift di:  p -> p + di * vline + e, inside the
+//   domain if  p / vline + di < amax  and  0 <= p % vline + e < vline
+// The whole image and its first / last row are read from the input tensor; the
+// first / last column and the corners from a compact copy of the two border columns
+// ([2][n][C][H], written by edge_sums_kernel), where a column is contiguous.
+struct ShiftGroup {
+  const float *base;
+  unsigned sample_stride, row_stride, line_stride;
+  unsigned L, mem_line, vline;
+  short di, dj0, ns, amax;
   int K;               // reduction length: samples * L
-  int klen;            // k-values per slice (a multiple of KT)
+  int klen, nsplit;    // k-values per slice (a multiple of KT), slices
+  int task0;           // first work item of the group
+  unsigned part_off;   // its partial tiles: [item][shift][rows of the A tile][64]
+};
+
+// Where the slices of one product's partial sums lie in the workspace, element
+// (row, col) of slice s at  part_off + s * split_stride
+//   + ((row / tile_rows) * tiles_j + col / 64) * tile_stride + (row % tile_rows) * 64 + col % 64,
+// and the arrays it becomes.
+struct Product {
+  unsigned part_off, split_stride, tile_stride;
   int nsplit;
-  int task0;           // first work item; the item's index is also its partial tile's
   short out, out_t;    // array written as it is / transposed (equal: symmetric product)
 };
 
 struct Plan {
   const float *x;
-  unsigned sample_stride, row_stride, line_stride;   // C H W, H W, W
+  unsigned sample_stride, row_stride;   // C H W, H W
   int C, H, W, n;
-  int tiles;    // per side
-  int total;    // work items
+  int tiles_a, tiles_b;     // tile grid: 64 * WM first-operand channels x 64 second-operand channels
+  int nsmall, total;        // work items of the groups 3.. (strips and corners), and of all groups
+  ShiftGroup grp[kGroups];
   Product prod[kProducts];
 };
 
-// Work item -> (product, tile, slice).  Consecutive workgroup ids go round-robin
-// to the 8 XCDs; each XCD takes a contiguous run of the item list, in which the
-// tiles of one slice of one product follow each other (they share operand panels).
+// Consecutive workgroup ids go round-robin to the 8 XCDs; each XCD takes a
+// contiguous run of the item list, in which the tiles of one slice of one group
+// follow each other (they share operand panels).
 __device__ __forceinline__ int item_of_block(int bid, int total) {
   const int xcd = bid % 8, idx = bid / 8;
   const int base = total / 8, rem = total % 8;
   return xcd * base + (xcd < rem ? xcd : rem) + idx;
 }
 
-template <int WM>
-__global__ __launch_bounds__(THREADS, 3) void corr_kernel(Plan pl, float *__restrict__ partial) {
-  constexpr int BM = 64 * WM;
-  __shared__ float lds[2 * Panel<BM>::kFloats];
-  float *ldsA = lds, *ldsB = lds + Panel<BM>::kFloats;
-  const int w = item_of_block(blockIdx.x, pl.total);
-  int p = 0;
-  while (p + 1 < kProducts && pl.prod[p + 1].task0 <= w) ++p;
-  const Product &pr = pl.prod[p];
-  const int ntile = pl.tiles * pl.tiles;
-  const int q = w - pr.task0;
+// k runs over (sample, pixel of the domain).  The workgroup stages 32 k-values of
+// its 64 * WM first-operand channels and the 36 values from di * vline - 2 places on
+// of its 64 second-operand channels; the NS shifts read the latter at NS
+// consecutive offsets.  Where a shifted pixel falls outside the domain is the same
+// for all channels: one 32-bit mask per shift and panel, applied to the operand
+// values as they are read (as 64-bit lane masks in scalar registers: one select
+// per value).  Per panel a wave issues 16 * WM * NS matrix instructions for
+// (8 * WM + 9) global loads of its lanes; one product at a time (WM * WM
+// instructions for 16 * WM loads per step) is bound by the loads.
+constexpr int kShiftCols = 36;
+constexpr int kShiftStride = 37;   // odd: the 32 rows of an operand read on 32 banks
+
+template <int WM, int NS>
+__device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGroup &g, int q, float *lds,
+                                                 float *__restrict__ partial) {
+  constexpr int BMA = 64 * WM;
+  float *ldsA = lds, *ldsB = lds + Panel<BMA>::kFloats;
+  const int ntile = pl.tiles_a * pl.tiles_b;
   const int split = q / ntile, tile = q - split * ntile;
-  const int I = tile / pl.tiles, J = tile - I * pl.tiles;
-  LoaderShift<BM> la, lb;
-  la.base = lb.base = pl.x + pr.base_off;
-  la.sample_stride = lb.sample_stride = pl.sample_stride;
-  la.row_stride = lb.row_stride = pl.row_stride;
-  la.L = lb.L = pr.L;
-  la.line_len = lb.line_len = pr.line_len;
-  la.line_stride = lb.line_stride = pl.line_stride;
-  la.amax = lb.amax = pr.amax;
-  la.bmax = lb.bmax = pr.bmax;
-  la.rows_valid = lb.rows_valid = pl.C;
+  const int I = tile / pl.tiles_b, J = tile - I * pl.tiles_b;
+  const unsigned L = g.L, mem_line = g.mem_line, vline = g.vline;
+  const int K = g.K;
+  LoaderShift<BMA> la;
+  la.base = g.base;
+  la.sample_stride = g.sample_stride;
+  la.row_stride = g.row_stride;
+  la.L = L;
+  la.line_len = mem_line;
+  la.line_stride = g.line_stride;
+  la.amax = 0x7fffffff;
+  la.bmax = 0x7fffffff;
+  la.rows_valid = pl.C;
   la.da = la.db = 0;
-  lb.da = pr.da;
-  lb.db = pr.db;
-  la.init(nullptr, I * BM);
-  lb.init(nullptr, J * BM);
-  const long long kbeg = (long long)split * pr.klen;
-  long long kend = kbeg + pr.klen;
-  if (kend > pr.K) kend = pr.K;
-  floatx16 acc[WM][WM];
-  zero_acc<WM, WM>(acc);
-  mainloop<WM, WM, false>(la, lb, I * BM, J * BM, kbeg, kend, ldsA, ldsB, acc);
-  float *out = partial + (long long)w * (BM * BM);
-  for_each_acc<WM, WM>(acc, [&](int r, int c, float v) { out[r * BM + c] = v; });
+  la.init(nullptr, I * BMA);
+  const int tid = team_tid();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane & 31, lk = lane >> 5;
+  // second operand: 32 columns x 8 row passes, then 4 columns x 64 rows
+  const int jm = tid & 31, rm = tid >> 5;
+  const int je = 32 + (tid & 3), re = tid >> 2;
+  const int shift = g.di * (int)vline - 2;
+  unsigned rowoff[8];
+  unsigned rowok = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = J * 64 + rm + 8 * i;
+    rowoff[i] = (unsigned)(row < pl.C ? row : pl.C - 1) * g.row_stride;
+    if (row < pl.C) rowok |= 1u << i;
+  }
+  const int rowe = J * 64 + re;
+  const unsigned rowoff_e = (unsigned)(rowe < pl.C ? rowe : pl.C - 1) * g.row_stride;
+  const long long kbeg = (long long)split * g.klen;
+  long long kend = kbeg + g.klen;
+  if (kend > K) kend = K;
+  floatx16 acc[NS][WM];
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+#pragma unroll
+    for (int im = 0; im < WM; ++im)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[s][im][v] = 0.f;
+  typename LoaderShift<BMA>::Regs ra;
+  float rb[9];
+  auto load_b = [&](long long k0) {
+    auto offset_of = [&](int j) {
+      long long kk = k0 + shift + j;
+      kk = kk < 0 ? 0 : (kk >= K ? K - 1 : kk);   // any element of the tensor will do: masked when read
+      const unsigned ku = (unsigned)kk, s = ku / L, p = ku - s * L;
+      const unsigned line = p / mem_line;
+      return s * g.sample_stride + line * g.line_stride + (p - line * mem_line);
+    };
+    const unsigned om = offset_of(jm), oe = offset_of(je);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) rb[i] = gload1(g.base, (om + rowoff[i]) * 4u);
+    rb[8] = gload1(g.base, (oe + rowoff_e) * 4u);
+  };
+  if (kbeg < kend) {
+    la.load(ra, 0, kbeg, kend);
+    load_b(kbeg);
+  }
+  for (long long k0 = kbeg; k0 < kend; k0 += KT) {
+    la.store(ra, ldsA);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ldsB[(rm + 8 * i) * kShiftStride + jm] = ((rowok >> i) & 1u) ? rb[i] : 0.f;
+    ldsB[re * kShiftStride + je] = rowe < pl.C ? rb[8] : 0.f;
+    __syncthreads();
+    if (k0 + KT < kend) {
+      la.load(ra, 0, k0 + KT, kend);
+      load_b(k0 + KT);
+    }
+    // validity of the NS shifted pixels of this panel's 32 k-values: bit k of m[s]
+    unsigned m[NS];
+    {
+      const long long kg = k0 + (lane & 31);
+      const unsigned kc = kg < kend ? (unsigned)kg : 0u;
+      const unsigned pix = kc % L;
+      const unsigned a = pix / vline, b = pix - a * vline;
+      const bool row_in = kg < kend && (int)a + g.di < g.amax;
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        m[s] = __builtin_amdgcn_readfirstlane(
+            (unsigned)__ballot(row_in && (unsigned)((int)b + g.dj0 + s) < vline));
+    }
+    const float *pa = ldsA + (wm * WM * 32 + lrow) * Panel<BMA>::kRowKStride + lk;
+    const float *pb = ldsB + (wn * 32 + lrow) * kShiftStride + lk + 2 + g.dj0;
+    // operands of step kk + 1 are read from LDS before the matrix instructions of
+    // step kk issue (the scheduling barriers keep the compiler from sinking the
+    // reads to their first use, which would expose the LDS latency in every step)
+    float a[2][WM], b[2][NS];
+#pragma unroll
+    for (int im = 0; im < WM; ++im) a[0][im] = pa[im * 32 * Panel<BMA>::kRowKStride];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) b[0][s] = pb[s];
+#pragma unroll
+    for (int kk = 0; kk < KT / 2; ++kk) {
+      const int cur = kk & 1, nxt = cur ^ 1;
+      if (kk + 1 < KT / 2) {
+#pragma unroll
+        for (int im = 0; im < WM; ++im) a[nxt][im] = pa[im * 32 * Panel<BMA>::kRowKStride + 2 * kk + 2];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) b[nxt][s] = pb[2 * kk + 2 + s];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        // lanes 0..31 hold k = 2 kk, lanes 32..63 k = 2 kk + 1: the lane mask of the
+        // valid ones, built from two bits of the panel's mask in scalar registers
+        const unsigned lo = 0u - ((m[s] >> (2 * kk)) & 1u), hi = 0u - ((m[s] >> (2 * kk + 1)) & 1u);
+        const unsigned long long lanes = ((unsigned long long)hi << 32) | lo;
+        const float v = __builtin_amdgcn_inverse_ballot_w64(lanes) ? b[cur][s] : 0.f;
+#pragma unroll
+        for (int im = 0; im < WM; ++im)
+          acc[s][im] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][im], v, acc[s][im], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+  }
+  float *out = partial + g.part_off + (long long)q * (NS * BMA * 64);
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+#pragma unroll
+    for (int im = 0; im < WM; ++im)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = (wm * WM + im) * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        out[(s * BMA + row) * 64 + wn * 32 + (lane & 31)] = acc[s][im][v];
+      }
 }
 
-// Sums the slices of one 32 x 32 block of one product and writes it to the
-// product's array and, transposed, to the array of the opposite offset.  A
-// symmetric product (offset zero) is written from its lower triangle.
+// The strips and corners first (few items, bound by latency: they start early and
+// run beside the rest), then the whole-image groups.
 template <int WM>
-__global__ __launch_bounds__(256) void corr_finish_kernel(Plan pl, const float *__restrict__ partial,
-                                                          float *__restrict__ arrays) {
-  constexpr int BM = 64 * WM;
-  __shared__ float t[32][33];
-  const int nb = (pl.C + 31) / 32;
-  const int p = blockIdx.x / (nb * nb);
-  const int b = blockIdx.x - p * (nb * nb);
-  const int bi = b / nb, bj = b - bi * nb;
-  const Product &pr = pl.prod[p];
-  const bool sym = pr.out == pr.out_t;
-  if (sym && bi < bj) return;
-  const int ntile = pl.tiles * pl.tiles;
-  const int r = threadIdx.x >> 3, c4 = (threadIdx.x & 7) * 4;
-  const int row = bi * 32 + r, col = bj * 32 + c4;
-  const int tile = (row / BM) * pl.tiles + col / BM;
-  const float4 *src = reinterpret_cast<const float4 *>(
-      partial + ((long long)pr.task0 + tile) * (BM * BM) + (row % BM) * BM + col % BM);
-  const long long step4 = (long long)ntile * (BM * BM) / 4;
-  float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-  int s = 0;
-  for (; s + 8 <= pr.nsplit; s += 8) {
-    float4 v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = src[(s + e) * step4];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      a.x += v[e].x;
-      a.y += v[e].y;
-      a.z += v[e].z;
-      a.w += v[e].w;
-    }
+__global__ __launch_bounds__(THREADS, 2) void corr_kernel(Plan pl, float *__restrict__ partial) {
+  __shared__ float lds[Panel<64 * WM>::kFloats + 64 * kShiftStride];
+  int w = blockIdx.x;
+  if (w >= pl.nsmall) w = pl.nsmall + item_of_block(w - pl.nsmall, pl.total - pl.nsmall);
+  int gi = 0;
+  if (w >= pl.nsmall) {
+    gi = w >= pl.grp[2].task0 ? 2 : (w >= pl.grp[1].task0 ? 1 : 0);
+  } else {
+    gi = 3;
+    while (gi + 1 < kGroups && pl.grp[gi + 1].task0 <= w) ++gi;
   }
-  for (; s < pr.nsplit; ++s) {
-    const float4 v = src[s * step4];
-    a.x += v.x;
-    a.y += v.y;
-    a.z += v.z;
-    a.w += v.w;
-  }
-  t[r][c4] = a.x;
-  t[r][c4 + 1] = a.y;
-  t[r][c4 + 2] = a.z;
-  t[r][c4 + 3] = a.w;
-  __syncthreads();
-  const int C = pl.C;
-  float *o = arrays + (long long)pr.out * C * C;
-  float *ot = arrays + (long long)pr.out_t * C * C;
-  const int lc = threadIdx.x & 31, lr0 = threadIdx.x >> 5;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int lr = lr0 + 8 * e;
-    const int gr = bi * 32 + lr, gc = bj * 32 + lc;
-    if (sym && bi == bj) {
-      if (gr < C && gc < C) o[(long long)gr * C + gc] = lc <= lr ? t[lr][lc] : t[lc][lr];
-      continue;
-    }
-    if (gr < C && gc < C) o[(long long)gr * C + gc] = t[lr][lc];
-    const int tr = bj * 32 + lr, tc = bi * 32 + lc;   // block (bj, bi) of the transposed array
-    if (tr < C && tc < C) ot[(long long)tr * C + tc] = t[lc][lr];
-  }
+  const ShiftGroup &g = pl.grp[gi];
+  if (g.ns == 3)
+    corr_shifts_body<WM, 3>(pl, g, w - g.task0, lds, partial);
+  else
+    corr_shifts_body<WM, 5>(pl, g, w - g.task0, lds, partial);
 }
 
-// Per-channel sums over the samples of chunk blockIdx.y (every gridDim.y-th
-// sample): sums[chunk][c][0..8] = whole image, first row, last row, first column,
-// last column, corners (first,first) (first,last) (last,first) (last,last).
-__global__ __launch_bounds__(256) void channel_sums_kernel(Plan pl, float *__restrict__ sums) {
+// One pass over the input before the products: the per-channel sums that make the
+// ones column, over the samples of chunk blockIdx.y (a contiguous range),
+//   sums[chunk][c][0..8] = whole image, first row, last row, first column, last
+//   column, corners (first,first) (first,last) (last,first) (last,last),
+// and the compact copy of the first and last image column, edges[last][s][c][u].
+__global__ __launch_bounds__(256) void edge_sums_kernel(Plan pl, float *__restrict__ sums,
+                                                        float *__restrict__ edges) {
   __shared__ float red[4][kChannelSums];
-  const int c = blockIdx.x;
+  const int c = blockIdx.x, chunk = blockIdx.y, nchunk = gridDim.y;
   const int H = pl.H, W = pl.W, HW = H * W;
+  const int per = (pl.n + nchunk - 1) / nchunk;
+  const int s0 = chunk * per, s1 = s0 + per < pl.n ? s0 + per : pl.n;
   float acc[kChannelSums];
 #pragma unroll
   for (int e = 0; e < kChannelSums; ++e) acc[e] = 0.f;
-  for (int s = blockIdx.y; s < pl.n; s += gridDim.y) {
-    const float *plane = pl.x + (long long)s * pl.sample_stride + (long long)c * pl.row_stride;
-    for (int p = threadIdx.x; p < HW; p += 256) {
-      const float v = plane[p];
-      const int u = p / W, q = p - u * W;
-      const bool r0 = u == 0, r1 = u == H - 1, c0 = q == 0, c1 = q == W - 1;
-      acc[0] += v;
-      if (r0) acc[1] += v;
-      if (r1) acc[2] += v;
-      if (c0) acc[3] += v;
-      if (c1) acc[4] += v;
-      if (r0 && c0) acc[5] += v;
-      if (r0 && c1) acc[6] += v;
-      if (r1 && c0) acc[7] += v;
-      if (r1 && c1) acc[8] += v;
+  const float *base = pl.x + (long long)c * pl.row_stride;
+  float *e0 = edges + (long long)c * H, *e1 = e0 + (long long)pl.n * pl.C * H;
+  for (int e = s0 * HW + (int)threadIdx.x; e < s1 * HW; e += 256) {
+    const int s = e / HW, p = e - s * HW;
+    const float v = base[(long long)s * pl.sample_stride + p];
+    const int u = p / W, q = p - u * W;
+    const bool r0 = u == 0, r1 = u == H - 1, c0 = q == 0, c1 = q == W - 1;
+    acc[0] += v;
+    if (r0) acc[1] += v;
+    if (r1) acc[2] += v;
+    if (c0) {
+      acc[3] += v;
+      e0[(long long)s * pl.C * H + u] = v;
     }
+    if (c1) {
+      acc[4] += v;
+      e1[(long long)s * pl.C * H + u] = v;
+    }
+    if (r0 && c0) acc[5] += v;
+    if (r0 && c1) acc[6] += v;
+    if (r1 && c0) acc[7] += v;
+    if (r1 && c1) acc[8] += v;
   }
 #pragma unroll
   for (int e = 0; e < kChannelSums; ++e) {
@@ -276,8 +379,86 @@ __global__ __launch_bounds__(256) void channel_sums_kernel(Plan pl, float *__res
   }
   __syncthreads();
   if (threadIdx.x < kChannelSums)
-    sums[((long long)blockIdx.y * pl.C + c) * kChannelSums + threadIdx.x] =
+    sums[((long long)chunk * pl.C + c) * kChannelSums + threadIdx.x] =
         red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+}
+
+// Sums the slices of one block of one product and writes it to the product's
+// array and, transposed, to the array of the opposite offset.  A symmetric
+// product (offset zero) is written from its lower triangle.  G = 1: blocks of 32 x
+// 32, every thread sums all slices of its four elements; G = 4 (many slices, few
+// blocks): blocks of 16 x 16, four threads share an element's slices (s = g, g +
+// 4, ...) and their sums are added in a fixed order.
+template <int G, int WM>
+__global__ __launch_bounds__(256) void corr_finish_kernel(Plan pl, const float *__restrict__ partial,
+                                                          float *__restrict__ arrays) {
+  constexpr int B = G == 1 ? 32 : 16;
+  constexpr int tile_rows = 64 * WM;
+  __shared__ float t[G][B][B + 1];
+  const int blk = blockIdx.x;
+  const int nb = (pl.C + B - 1) / B;
+  const int p = blk / (nb * nb);
+  const int b = blk - p * (nb * nb);
+  const int bi = b / nb, bj = b - bi * nb;
+  const Product &pr = pl.prod[p];
+  const bool sym = pr.out == pr.out_t;
+  if (sym && bi < bj) return;
+  const int tid = threadIdx.x % (256 / G), grp = threadIdx.x / (256 / G);
+  const int r = tid / (B / 4), c4 = (tid % (B / 4)) * 4;
+  const int row = bi * B + r, col = bj * B + c4;
+  const int ti = row / tile_rows, tj = col / 64;
+  const float4 *src = reinterpret_cast<const float4 *>(
+      partial + pr.part_off + (long long)(ti * pl.tiles_b + tj) * pr.tile_stride +
+      (row - ti * tile_rows) * 64 + (col - tj * 64));
+  const long long step4 = pr.split_stride / 4;
+  float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+  int s = grp;
+  for (; s + 7 * G < pr.nsplit; s += 8 * G) {
+    float4 v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = src[(s + e * G) * step4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      a.x += v[e].x;
+      a.y += v[e].y;
+      a.z += v[e].z;
+      a.w += v[e].w;
+    }
+  }
+  for (; s < pr.nsplit; s += G) {
+    const float4 v = src[s * step4];
+    a.x += v.x;
+    a.y += v.y;
+    a.z += v.z;
+    a.w += v.w;
+  }
+  t[grp][r][c4] = a.x;
+  t[grp][r][c4 + 1] = a.y;
+  t[grp][r][c4 + 2] = a.z;
+  t[grp][r][c4 + 3] = a.w;
+  __syncthreads();
+  const int C = pl.C;
+  float *o = arrays + (long long)pr.out * C * C;
+  float *ot = arrays + (long long)pr.out_t * C * C;
+  const int lc = threadIdx.x % B, lr0 = threadIdx.x / B;
+  auto total = [&](int i, int j) {
+    float v = t[0][i][j];
+#pragma unroll
+    for (int g = 1; g < G; ++g) v += t[g][i][j];
+    return v;
+  };
+#pragma unroll
+  for (int e = 0; e < B * B / 256; ++e) {
+    const int lr = lr0 + (256 / B) * e;
+    const int gr = bi * B + lr, gc = bj * B + lc;
+    if (sym && bi == bj) {
+      if (gr < C && gc < C) o[(long long)gr * C + gc] = lc <= lr ? total(lr, lc) : total(lc, lr);
+      continue;
+    }
+    if (gr < C && gc < C) o[(long long)gr * C + gc] = total(lr, lc);
+    const int tr = bj * B + lr, tc = bi * B + lc;   // block (bj, bi) of the transposed array
+    if (tr < C && tc < C) ot[(long long)tr * C + tc] = total(lc, lr);
+  }
 }
 
 // Entry ((c,i,j), (c',i',j')) of the factor from the arrays' values at [c][c'],

@@ -786,71 +786,144 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   using namespace kfac::shift;
   constexpr int BM = 64 * WM;
   const int c = pl.C, h = pl.H, w = pl.W, n = pl.n;
-  pl.tiles = kfac::ceil_div(c, BM);
-  const int ntile = pl.tiles * pl.tiles;
-  int np = 0;
-  auto add = [&](unsigned base_off, int L, int line_len, int da, int db, int amax, int bmax, int out,
-                 int out_t) {
-    Product &p = pl.prod[np++];
-    p.base_off = base_off;
-    p.L = (unsigned)L;
-    p.line_len = (unsigned)line_len;
-    p.da = (short)da; p.db = (short)db; p.amax = (short)amax; p.bmax = (short)bmax;
-    p.K = n * L;
-    p.out = (short)out; p.out_t = (short)out_t;
-  };
-  for (int di = 0; di <= 2; ++di)
-    for (int dj = (di == 0 ? 0 : -2); dj <= 2; ++dj)
-      add(0, h * w, w, di, dj, h, w, (di + 2) * 5 + dj + 2, (2 - di) * 5 + 2 - dj);
-  for (int last = 0; last < 2; ++last)
-    for (int dj = 0; dj <= 2; ++dj)
-      add(last ? (unsigned)(h - 1) * w : 0u, w, w, 0, dj, 1, w, 25 + 5 * last + dj + 2, 25 + 5 * last + 2 - dj);
-  for (int last = 0; last < 2; ++last)
-    for (int di = 0; di <= 2; ++di)
-      add(last ? (unsigned)(w - 1) : 0u, h, 1, di, 0, h, 1, 35 + 5 * last + di + 2, 35 + 5 * last + 2 - di);
-  for (int lr = 0; lr < 2; ++lr)
-    for (int lc = 0; lc < 2; ++lc)
-      add((lr ? (unsigned)(h - 1) * w : 0u) + (lc ? (unsigned)(w - 1) : 0u), 1, 1, 0, 0, 1, 1,
-          45 + 2 * lr + lc, 45 + 2 * lr + lc);
-  if (np != kProducts) return kfac::fail(KFAC_EINVAL, "internal: %d products", np);
-  // slices of about equal length over all products, ~target workgroups in all
-  long long units = 0;
-  for (int i = 0; i < np; ++i) units += (long long)ntile * kfac::ceil_div(pl.prod[i].K, KT);
-  long long target = WM == 1 ? 1024 : 1536;
-  if (const char *env = getenv("KFAC_SHIFT_TARGET")) target = std::max(1ll, atoll(env));   // tuning override
-  long long per = std::max<long long>(6, kfac::ceil_div(units, target));
-  int total = 0;
-  for (int i = 0; i < np; ++i) {
-    Product &p = pl.prod[i];
-    const long long nk = kfac::ceil_div(p.K, KT);
-    const long long ns = kfac::ceil_div(nk, per);
-    const long long len = kfac::ceil_div(nk, ns);
-    p.nsplit = (int)kfac::ceil_div(nk, len);
-    p.klen = (int)len * KT;
-    p.task0 = total;
-    total += ntile * p.nsplit;
-  }
-  pl.total = total;
-  const int nchunk = std::min(n, 8);
-  const size_t partial_floats = (size_t)total * BM * BM;
+  pl.tiles_a = kfac::ceil_div(c, BM);
+  pl.tiles_b = kfac::ceil_div(c, 64);
+  const int ntab = pl.tiles_a * pl.tiles_b;
+  // workspace: [partial tiles | arrays | channel sums | border columns]; the last two
+  // have sizes known up front and are placed from the end
+  const int nchunk = std::max(1, std::min(n, 1024 / c));
   const size_t array_floats = (size_t)kArrays * c * c;
   const size_t sums_floats = (size_t)nchunk * c * kChannelSums;
-  if (ws == nullptr || ws_bytes < (partial_floats + array_floats + sums_floats) * sizeof(float)) return 1;
+  const size_t edge_floats = (size_t)2 * n * c * h;
+  const size_t tail_floats = array_floats + sums_floats + edge_floats + 64;
+  if (ws == nullptr || ws_bytes < tail_floats * sizeof(float)) return 1;
   float *partial = static_cast<float *>(ws);
-  float *arrays = partial + partial_floats;
+  float *arrays = partial + (ws_bytes / sizeof(float) - tail_floats) / 4 * 4;
   float *sums = arrays + array_floats;
-  if (ones) {
-    hipLaunchKernelGGL(channel_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums);
-    KFAC_HIP_CHECK(hipGetLastError());
+  float *edges = sums + sums_floats;
+  // groups: whole image (di = 0, 1, 2), first / last row, first / last column, corners
+  auto group = [&](int gi, const float *base, long long sample_stride, int row_stride, int line_stride, int L,
+                   int mem_line, int vline, int di, int dj0, int ns, int amax) {
+    ShiftGroup &g = pl.grp[gi];
+    g.base = base;
+    g.sample_stride = (unsigned)sample_stride; g.row_stride = (unsigned)row_stride;
+    g.line_stride = (unsigned)line_stride;
+    g.L = (unsigned)L; g.mem_line = (unsigned)mem_line; g.vline = (unsigned)vline;
+    g.di = (short)di; g.dj0 = (short)dj0; g.ns = (short)ns; g.amax = (short)amax;
+    g.K = n * L;
+  };
+  const long long xs = (long long)c * h * w, es = (long long)c * h;
+  group(0, pl.x, xs, h * w, w, h * w, h * w, w, 0, 0, 3, h);
+  group(1, pl.x, xs, h * w, w, h * w, h * w, w, 1, -2, 5, h);
+  group(2, pl.x, xs, h * w, w, h * w, h * w, w, 2, -2, 5, h);
+  for (int last = 0; last < 2; ++last) {
+    group(3 + last, pl.x + (last ? (h - 1) * w : 0), xs, h * w, w, w, w, w, 0, 0, 3, 1);
+    const float *col = edges + (size_t)last * n * c * h;
+    group(5 + last, col, es, h, h, h, h, h, 0, 0, 3, 1);
   }
+  for (int lr = 0; lr < 2; ++lr)
+    for (int lc = 0; lc < 2; ++lc)
+      group(7 + 2 * lr + lc, edges + (size_t)lc * n * c * h + (lr ? h - 1 : 0), es, h, h, 1, 1, 1, 0, 0, 3, 1);
+  // Slices of the whole-image groups: the workgroups of a launch run two to a CU,
+  // 512 at a time (three with 64 first-operand channels), and a group of ns shifts does ns tile products per panel.  Among
+  // the slice counts (s5 for the two groups of five shifts, s3 for the group of
+  // three) the pair with the least rounds x longest item, plus what an item costs
+  // besides its panels (prologue, partial tiles written and summed).
+  const long long nk = kfac::ceil_div(n * h * w, KT);
+  long long best_s5 = 1, best_s3 = 1;
+  double best_cost = 0.0, best_longest = 1.0;
+  const long long max_items = 4096;
+  for (long long s5 = 1; s5 <= nk && ntab * (2 * s5 + 1) <= max_items; ++s5) {
+    const long long len5 = kfac::ceil_div(nk, s5);
+    if (kfac::ceil_div(nk, len5) != s5) continue;
+    // the slice count of the three-shift group whose items are no longer than these
+    long long len3 = std::min(nk, std::max<long long>(1, 5 * len5 / 3));
+    const long long s3 = kfac::ceil_div(nk, len3);
+    len3 = kfac::ceil_div(nk, s3);
+    const long long items = ntab * (2 * s5 + s3);
+    if (items > max_items) continue;
+    const double longest = (double)std::max(5 * len5, 3 * len3);
+    const double rounds = (double)kfac::ceil_div<long long>(items, WM == 1 ? 768 : 512);
+    // an item's fixed cost in units of one shift-panel
+    const double cost = rounds * (longest + 6.0) + 0.004 * (double)items;
+    if (best_cost == 0.0 || cost < best_cost) {
+      best_cost = cost;
+      best_s5 = s5;
+      best_s3 = s3;
+      best_longest = longest;
+    }
+  }
+  if (const char *env = getenv("KFAC_SHIFT_SLICES")) {   // tuning override: "s5,s3"
+    long long a = 0, b = 0;
+    if (sscanf(env, "%lld,%lld", &a, &b) == 2 && a >= 1 && b >= 1) {
+      best_s5 = std::min(a, nk);
+      best_s3 = std::min(b, nk);
+      best_longest = (double)std::max(5 * kfac::ceil_div(nk, best_s5), 3 * kfac::ceil_div(nk, best_s3));
+    }
+  }
+  // items: strips and corners first (block order), then the whole-image groups
+  size_t partial_floats = 0;
+  int total = 0;
+  auto slice = [&](int gi, long long ns) {
+    ShiftGroup &g = pl.grp[gi];
+    const long long gk = kfac::ceil_div(g.K, KT);
+    const long long len = kfac::ceil_div(gk, std::max(1ll, std::min(ns, gk)));
+    g.nsplit = (int)kfac::ceil_div(gk, len);
+    g.klen = (int)len * KT;
+    g.task0 = total;
+    g.part_off = (unsigned)partial_floats;
+    total += ntab * g.nsplit;
+    partial_floats += (size_t)ntab * g.nsplit * g.ns * BM * 64;
+  };
+  for (int gi = 3; gi < kGroups; ++gi) {
+    const long long gk = kfac::ceil_div(pl.grp[gi].K, KT);
+    slice(gi, kfac::ceil_div<long long>(3 * gk, std::max<long long>(3, (long long)best_longest)));
+  }
+  pl.nsmall = total;
+  slice(0, best_s3);
+  slice(1, best_s5);
+  slice(2, best_s5);
+  pl.total = total;
+  // products -> (group, shift)
+  int np = 0;
+  auto product = [&](int gi, int e, int out, int out_t) {
+    const ShiftGroup &g = pl.grp[gi];
+    Product &p = pl.prod[np++];
+    p.nsplit = g.nsplit;
+    p.tile_stride = (unsigned)(g.ns * BM * 64);
+    p.split_stride = (unsigned)ntab * p.tile_stride;
+    p.part_off = g.part_off + (unsigned)((e - g.dj0) * BM * 64);
+    p.out = (short)out;
+    p.out_t = (short)out_t;
+  };
+  for (int di = 0; di <= 2; ++di)
+    for (int dj = (di == 0 ? 0 : -2); dj <= 2; ++dj) product(di, dj, (di + 2) * 5 + dj + 2, (2 - di) * 5 + 2 - dj);
+  for (int last = 0; last < 2; ++last)
+    for (int dj = 0; dj <= 2; ++dj) product(3 + last, dj, 25 + 5 * last + dj + 2, 25 + 5 * last + 2 - dj);
+  for (int last = 0; last < 2; ++last)
+    for (int di = 0; di <= 2; ++di) product(5 + last, di, 35 + 5 * last + di + 2, 35 + 5 * last + 2 - di);
+  for (int lr = 0; lr < 2; ++lr)
+    for (int lc = 0; lc < 2; ++lc) product(7 + 2 * lr + lc, 0, 45 + 2 * lr + lc, 45 + 2 * lr + lc);
+  if (np != kProducts) return kfac::fail(KFAC_EINVAL, "internal: %d products", np);
+  if (partial_floats >= (1ull << 32) || partial + partial_floats > arrays) return 1;
+  hipLaunchKernelGGL(edge_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums, edges);
+  KFAC_HIP_CHECK(hipGetLastError());
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
-    hipLaunchKernelGGL((corr_kernel<WM>), dim3(total), dim3(THREADS), 0, stream, pl, partial);
+    hipLaunchKernelGGL((corr_kernel<WM>), dim3(pl.total), dim3(THREADS), 0, stream, pl, partial);
   }
   KFAC_HIP_CHECK(hipGetLastError());
-  const int nb = kfac::ceil_div(c, 32);
-  hipLaunchKernelGGL((corr_finish_kernel<WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
-                     arrays);
+  int max_split = 1;
+  for (int i = 0; i < np; ++i) max_split = std::max(max_split, pl.prod[i].nsplit);
+  if (max_split >= 32 && c <= 128) {
+    const int nb = kfac::ceil_div(c, 16);
+    hipLaunchKernelGGL((corr_finish_kernel<4, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
+                       arrays);
+  } else {
+    const int nb = kfac::ceil_div(c, 32);
+    hipLaunchKernelGGL((corr_finish_kernel<1, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
+                       arrays);
+  }
   KFAC_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL(assemble_kernel, dim3(c, kfac::ceil_div(c, 64)), dim3(256), 0, stream, pl, arrays, sums,
                      nchunk, d, ones, (float)((long long)n * h * w), alpha, beta, C);
@@ -873,7 +946,6 @@ int try_conv_shift(const float *x, int n, int c, int h, int w, int kh, int kw, i
   pl.x = x;
   pl.sample_stride = (unsigned)((long long)c * h * w);
   pl.row_stride = (unsigned)(h * w);
-  pl.line_stride = (unsigned)w;
   pl.C = c; pl.H = h; pl.W = w; pl.n = n;
   // 128-tiles unless 64-tiles waste much less on a channel count that is not a multiple of 128
   const long long t64 = kfac::ceil_div(c, 64), t128 = kfac::ceil_div(c, 128);
