@@ -345,6 +345,10 @@ def run_step_config(args, name, cfg):
     syrk_n, syrk_raw_ms = fam['syrk']
     syrk_ms = max(syrk_raw_ms - syrk_n * empty, 1e-9)
     achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
+    # what the matrix cores are actually given: 3x3 stride-1 convolutions compute their A factor from
+    # shifted correlations, about a third of the multiply-adds of the patch product
+    cov_executed = float(W.cov_flops_executed(layers, batch)) * acc_iters
+    achieved_executed = cov_executed / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
     total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
     executed_flops = flops['cov'] + dense_inverse_flops + flops['precondition']
     traffic = read_traffic() if name == 'c3' else None
@@ -385,12 +389,18 @@ def run_step_config(args, name, cfg):
         'inverse_info_nonzero': info_bad,
         'wire_format': wire_stats,
         'roofline': {
-            'kernel': 'covariance SYRK family (syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
+            'kernel': 'covariance SYRK family (shift::corr_kernel, syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
             'bound': 'mfma',
             'achieved': round(achieved, 2),
             'peak': FP32_MFMA_PEAK_TFLOPS,
             'unit': 'TFLOP/s',
             'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+            # `achieved` divides the algorithmic work M d (d+1) of every factor by the kernels' time; the
+            # multiply-adds issued are fewer where a factor is built from shifted correlations
+            'executed': {'gflop_per_step': round(cov_executed / 1e9, 1),
+                         'algorithmic_gflop_per_step': round(flops['cov'] / 1e9, 1),
+                         'achieved': round(achieved_executed, 2),
+                         'frac': round(achieved_executed / FP32_MFMA_PEAK_TFLOPS, 4)},
             'launches': syrk_n,
             'avg_launch_ms': round(syrk_ms / max(syrk_n, 1), 4),
             'avg_launch_ms_with_event_bracket': round(syrk_raw_ms / max(syrk_n, 1), 4),
@@ -547,9 +557,13 @@ def write_per_layer(path, layers, config='c3'):
         in_a, in_g = x.numel() * 4.0, gy.numel() * 4.0
         for fac, d, t, in_bytes in (('A', dA, ta, in_a), ('G', dG, tg, in_g)):
             flop = float(M) * d * (d + 1)
+            issued = flop
+            if fac == 'A' and W.takes_shift_route(layer):   # shifted correlations: fewer multiply-adds than M d (d+1)
+                issued = float(W.cov_flops_executed([layer], BATCH)) - float(M) * dG * (dG + 1)
             ai = flop / (in_bytes + 4.0 * d * d)
             cap = min(FP32_MFMA_PEAK_TFLOPS, ai * HBM_PEAK_GBPS / 1e3)
-            rows.append((desc, count, fac, d, M, flop / 1e9, t * 1e3, flop / t / 1e9, ai, cap, flop / t / 1e9 / cap))
+            rows.append((desc, count, fac, d, M, flop / 1e9, issued / 1e9, t * 1e3, flop / t / 1e9, issued / t / 1e9,
+                         ai, cap, issued / t / 1e9 / cap))
         del x, gy
     with open(path, 'w') as f:
         f.write('# Covariance kernels layer by layer (every distinct convolution / linear shape of the workload)\n\n'
@@ -560,14 +574,18 @@ def write_per_layer(path, layers, config='c3'):
                 '{:.1f} us an empty event bracket measures subtracted); the kernels that sum split-K partial tiles are '
                 'not in it. In a K-FAC step the small factors (at most 8 GFLOP: most 1x1 convolutions, linear and '
                 'batch-norm layers) do not run alone but in a handful of grouped launches, so their rows here show the '
-                'latency floor of a single launch, not their cost in the step. GFLOP = M d (d+1); flop/B = that over '
-                'the bytes of the input tensor read once plus the factor written once; roofline cap = min(157.3 '
-                'TFLOP/s FP32 MFMA, flop/B x 8 TB/s).\n\n'.format(config, path, empty * 1e3))
-        f.write('| layer (x count) | factor | d | rows M | GFLOP | SYRK kernel us | TFLOP/s | flop/B | roofline cap TFLOP/s '
-                '| fraction of cap |\n|---|---|---:|---:|---:|---:|---:|---:|---:|---:|\n')
-        for desc, count, fac, d, M, gf, us, tf, ai, cap, frac in rows:
-            f.write('| {} (x{}) | {} | {} | {} | {:.2f} | {:.1f} | {:.1f} | {:.0f} | {:.1f} | {:.2f} |\n'.format(
-                desc, count, fac, d, M, gf, us, tf, ai, cap, frac))
+                'latency floor of a single launch, not their cost in the step. GFLOP = M d (d+1), the work of the '
+                'patch / activation product; "issued" is what the kernel gives the matrix cores, which is less for the A '
+                'factor of a 3x3 stride-1 convolution (29 shifted correlations of C x C instead of a 9C x 9C product); '
+                'flop/B = M d (d+1) over the bytes of the input tensor read once plus the factor written once; roofline '
+                'cap = min(157.3 TFLOP/s FP32 MFMA, flop/B x 8 TB/s); the last column is the issued rate over the cap.'
+                '\n\n'.format(config, path, empty * 1e3))
+        f.write('| layer (x count) | factor | d | rows M | GFLOP | GFLOP issued | SYRK kernel us | TFLOP/s (M d (d+1)) | '
+                'TFLOP/s issued | flop/B | roofline cap TFLOP/s | issued / cap |\n'
+                '|---|---|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|\n')
+        for desc, count, fac, d, M, gf, gi, us, tf, ti, ai, cap, frac in rows:
+            f.write('| {} (x{}) | {} | {} | {} | {:.2f} | {:.2f} | {:.1f} | {:.1f} | {:.1f} | {:.0f} | {:.1f} | {:.2f} |\n'.format(
+                desc, count, fac, d, M, gf, gi, us, tf, ti, ai, cap, frac))
 
 
 def _cpu_threads():
@@ -698,8 +716,8 @@ def _csv_rows(directory, suffix):
 
 
 KERNEL_FAMILIES = (
-    ('covariance SYRK family', ('syrk_',)),
-    ('split-K finish of the covariances', ('finish_', 'reduce_kernel')),
+    ('covariance SYRK family', ('syrk_', 'shift::corr_kernel')),
+    ('split-K finish of the covariances', ('finish_', 'reduce_kernel', 'shift::assemble', 'shift::edge_sums')),
     ('inverse tile kernels', ('diag_kernel', 'update_kernel', 'lauum_kernel', 'panel_kernel', 'copy_in', 'copy_out',
                               'trtri', 'potrf', 'small_inverse')),
     ('preconditioning GEMMs', ('gemm_',)),
@@ -832,7 +850,7 @@ def summarize_traffic(fetch_dir, write_dir, out_path, command):
     per_kernel = {}
     for d, counter, key in ((fetch_dir, 'FETCH_SIZE', 'fetch'), (write_dir, 'WRITE_SIZE', 'write')):
         rows = load(d, counter)
-        syrk = [v for k, v in rows if 'syrk_' in k]
+        syrk = [v for k, v in rows if 'syrk_' in k or 'shift::corr_kernel' in k]
         cal = [v for k, v in rows if 'stream_copy_kernel' in k]
         if not syrk or not cal:
             raise SystemExit('no {} rows for the SYRK family or the calibration copy under {}'.format(counter, d))
@@ -861,7 +879,7 @@ def summarize_traffic(fetch_dir, write_dir, out_path, command):
              'counters are scaled by {:.3f} and {:.3f} to get KiB.'.format(
                  out['fetch_counter_for_256MiB_copy'], out['write_counter_for_256MiB_copy'],
                  out['fetch_scale'], out['write_scale']), '',
-             'Covariance SYRK family (`syrk_*`, {} launches in the run): **fetch {:.1f} MiB + write {:.1f} MiB = '
+             'Covariance SYRK family (`syrk_*` and `shift::corr_kernel`, {} launches in the run): **fetch {:.1f} MiB + write {:.1f} MiB = '
              '{:.1f} MiB per launch** ({:.4g} bytes, the `roofline.traffic` of bench.py).'.format(
                  out['launches'], out['fetch_bytes_per_launch'] / 2 ** 20, out['write_bytes_per_launch'] / 2 ** 20,
                  total / 2 ** 20, total), '',

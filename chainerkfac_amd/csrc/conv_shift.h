@@ -350,26 +350,53 @@ __global__ __launch_bounds__(256) void edge_sums_kernel(Plan pl, float *__restri
   for (int e = 0; e < kChannelSums; ++e) acc[e] = 0.f;
   const float *base = pl.x + (long long)c * pl.row_stride;
   float *e0 = edges + (long long)c * H, *e1 = e0 + (long long)pl.n * pl.C * H;
-  for (int e = s0 * HW + (int)threadIdx.x; e < s1 * HW; e += 256) {
-    const int s = e / HW, p = e - s * HW;
-    const float v = base[(long long)s * pl.sample_stride + p];
-    const int u = p / W, q = p - u * W;
-    const bool r0 = u == 0, r1 = u == H - 1, c0 = q == 0, c1 = q == W - 1;
-    acc[0] += v;
-    if (r0) acc[1] += v;
-    if (r1) acc[2] += v;
-    if (c0) {
-      acc[3] += v;
-      e0[(long long)s * pl.C * H + u] = v;
+  if (W % 4 == 0 && (reinterpret_cast<uintptr_t>(pl.x) & 15) == 0) {
+    // four pixels of one image row at a time
+    const int Q = HW / 4;
+    for (int e = s0 * Q + (int)threadIdx.x; e < s1 * Q; e += 256) {
+      const int s = e / Q, p = (e - s * Q) * 4;
+      const float4 v = *reinterpret_cast<const float4 *>(base + (long long)s * pl.sample_stride + p);
+      const int u = p / W, q = p - u * W;
+      const bool r0 = u == 0, r1 = u == H - 1, c0 = q == 0, c1 = q + 4 == W;
+      const float t = (v.x + v.y) + (v.z + v.w);
+      acc[0] += t;
+      if (r0) acc[1] += t;
+      if (r1) acc[2] += t;
+      if (c0) {
+        acc[3] += v.x;
+        e0[(long long)s * pl.C * H + u] = v.x;
+        if (r0) acc[5] += v.x;
+        if (r1) acc[7] += v.x;
+      }
+      if (c1) {
+        acc[4] += v.w;
+        e1[(long long)s * pl.C * H + u] = v.w;
+        if (r0) acc[6] += v.w;
+        if (r1) acc[8] += v.w;
+      }
     }
-    if (c1) {
-      acc[4] += v;
-      e1[(long long)s * pl.C * H + u] = v;
+  } else {
+    for (int e = s0 * HW + (int)threadIdx.x; e < s1 * HW; e += 256) {
+      const int s = e / HW, p = e - s * HW;
+      const float v = base[(long long)s * pl.sample_stride + p];
+      const int u = p / W, q = p - u * W;
+      const bool r0 = u == 0, r1 = u == H - 1, c0 = q == 0, c1 = q == W - 1;
+      acc[0] += v;
+      if (r0) acc[1] += v;
+      if (r1) acc[2] += v;
+      if (c0) {
+        acc[3] += v;
+        e0[(long long)s * pl.C * H + u] = v;
+      }
+      if (c1) {
+        acc[4] += v;
+        e1[(long long)s * pl.C * H + u] = v;
+      }
+      if (r0 && c0) acc[5] += v;
+      if (r0 && c1) acc[6] += v;
+      if (r1 && c0) acc[7] += v;
+      if (r1 && c1) acc[8] += v;
     }
-    if (r0 && c0) acc[5] += v;
-    if (r0 && c1) acc[6] += v;
-    if (r1 && c0) acc[7] += v;
-    if (r1 && c1) acc[8] += v;
   }
 #pragma unroll
   for (int e = 0; e < kChannelSums; ++e) {
@@ -473,8 +500,9 @@ __device__ __forceinline__ float assemble(const float (*arr)[CHUNK], int cl, int
   return v;
 }
 
-// Writes the 9 rows of channel blockIdx.x, columns of the 64 channels of chunk
-// blockIdx.y: out = alpha * value + beta * out.  The workgroups of chunk 0 also
+// Writes the 9 rows of channel blockIdx.x (a third of them per blockIdx.z when the
+// grid has three layers), columns of the 64 channels of chunk blockIdx.y: out =
+// alpha * value + beta * out.  The workgroups of chunk 0 also
 // write the ones column and row of their 9 rows (and the first of them the corner).
 __global__ __launch_bounds__(256) void assemble_kernel(Plan pl, const float *__restrict__ arrays,
                                                         const float *__restrict__ sums, int nchunk_sums,
@@ -497,7 +525,8 @@ __global__ __launch_bounds__(256) void assemble_kernel(Plan pl, const float *__r
   }
   __syncthreads();
   const int ncol = width * 9;
-  for (int ij = 0; ij < 9; ++ij) {
+  const int rows_per = 9 / gridDim.z;   // gridDim.z = 1 or 3: a small factor is spread over more workgroups
+  for (int ij = blockIdx.z * rows_per; ij < (int)(blockIdx.z + 1) * rows_per; ++ij) {
     const int i = ij / 3, j = ij - 3 * i;
     float *dst = out + (long long)(c * 9 + ij) * d + c0 * 9;
     for (int t = threadIdx.x; t < ncol; t += 256) {
@@ -508,7 +537,7 @@ __global__ __launch_bounds__(256) void assemble_kernel(Plan pl, const float *__r
       dst[t] = v;
     }
   }
-  if (ones && blockIdx.y == 0 && threadIdx.x < 9) {
+  if (ones && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < 9) {
     const int ij = threadIdx.x, i = ij / 3, j = ij - 3 * i;
     float v = cs[0];
     if (i != 1) v -= cs[i == 0 ? 2 : 1];

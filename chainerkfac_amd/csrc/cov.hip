@@ -925,7 +925,7 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
                        arrays);
   }
   KFAC_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL(assemble_kernel, dim3(c, kfac::ceil_div(c, 64)), dim3(256), 0, stream, pl, arrays, sums,
+  hipLaunchKernelGGL(assemble_kernel, dim3(c, kfac::ceil_div(c, 64), c <= 128 ? 3 : 1), dim3(256), 0, stream, pl, arrays, sums,
                      nchunk, d, ones, (float)((long long)n * h * w), alpha, beta, C);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;

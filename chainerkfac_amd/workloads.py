@@ -153,6 +153,33 @@ def flops(layers, batch):
     return dict(cov=cov, inverse=inv, precondition=pre)
 
 
+def takes_shift_route(layer):
+    """Whether the library computes the layer's A factor from shifted correlations of
+    the input (3x3, stride 1, padding 1, at least 64 channels, images of at least 4 x 4:
+    the conditions of try_conv_shift in csrc/cov.hip) rather than as a product of
+    patch matrices."""
+    return (layer['kind'] == 'conv' and layer['k'] == 3 and layer['s'] == 1 and layer['p'] == 1 and
+            layer['c_in'] >= 64 and layer['h'] >= 4 and layer['w'] >= 4)
+
+
+def cov_flops_executed(layers, batch):
+    """Multiply-add work (2 flop each) that the covariance kernels issue for one step,
+    where it differs from the algorithmic M d (d+1) of flops(): a factor on the
+    shifted-correlation route takes 13 whole-image products of C x C, 6 over one image
+    row, 6 over one image column and 4 over one pixel, each computed in full."""
+    total = 0
+    for layer in layers:
+        m = cov_rows(layer, batch)
+        dims = factor_dims(layer)
+        for i, d in enumerate(dims):
+            if i == 0 and takes_shift_route(layer):
+                c, h, w = layer['c_in'], layer['h'], layer['w']
+                total += 2 * c * c * batch * (13 * h * w + 6 * w + 6 * h + 4)
+            else:
+                total += m * d * (d + 1)
+    return total
+
+
 def build_resnet50_v1(device='cuda', generator=None, n_class=1000, bias=True):
     """The network behind the ``resnet50_v1`` layer table as a callable chain of
     ``chainerkfac_amd.links``: bottleneck topology of the reference's
