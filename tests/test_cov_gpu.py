@@ -131,6 +131,7 @@ SHIFT_CASES = [
     (2, 256, 14, 14, True),     # four tiles per product
     (5, 130, 7, 7, True),       # channel count just past a tile
     (2, 64, 1000, 4, True),     # tall and narrow: column strips of 1000 pixels
+    (2, 1024, 5, 4, False),     # 8 x 16 tiles per product, a reduction shorter than one panel
 ]
 
 
@@ -142,6 +143,25 @@ def test_conv_A_shift_route(n, c, h, w, bias):
     x += 0.5    # non-zero mean: the ones column is not just noise
     A = ops.cov_conv_a(torch.from_numpy(x).cuda(), 3, 1, 1, bias, 1.0 / n)
     check(A, O.conv_A(x, 3, 1, 1, bias))
+
+
+def test_conv_A_shift_route_unaligned_input_and_accumulation():
+    """An input that starts one float past a 16-byte boundary (a view into a larger buffer), and
+    beta = 1 accumulation onto an existing factor with its ones row and column."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(11)
+    n, c, h, w = 2, 64, 8, 12
+    buf = torch.zeros(n * c * h * w + 1, device='cuda')
+    xs = [r.standard_normal((n, c, h, w)).astype(np.float32) + 0.25 for _ in range(2)]
+    out = None
+    acc = None
+    for i, x in enumerate(xs):
+        buf[1:].copy_(torch.from_numpy(x).reshape(-1))
+        xv = buf[1:].view(n, c, h, w)
+        assert xv.data_ptr() % 16 == 4
+        out = ops.cov_conv_a(xv, 3, 1, 1, True, (1.0 / n) / 2, beta=0.0 if i == 0 else 1.0, out=out)
+        acc = O.accumulate_covs(acc, [O.conv_A(x, 3, 1, 1, True)], 2)
+    check(out, acc[0])
 
 
 def test_conv_A_shift_route_border_terms():
