@@ -777,6 +777,91 @@ int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, in
   return 1;
 }
 
+// Slices of the whole-image groups of the shifted-correlation route: the workgroups
+// of a launch run two to a CU, 512 at a time (three with 64 first-operand channels),
+// and a group of ns shifts does ns tile products per panel.  Among the slice counts
+// (s5 for the two groups of five shifts, s3 for the group of three) the pair with
+// the least rounds x longest item, plus what an item costs besides its panels
+// (prologue, partial tiles written and summed).  ntab: tile pairs per product, nk:
+// panels of the whole reduction.
+struct ShiftSlices {
+  long long s5, s3;
+  double longest;   // shift-panels of the longest item
+};
+constexpr long long kShiftMaxItems = 1024;
+
+ShiftSlices plan_shift_slices(int wm, int ntab, long long nk) {
+  long long best_s5 = 1, best_s3 = 1;
+  double best_cost = 0.0, best_longest = (double)(5 * nk);
+  for (long long s5 = 1; s5 <= nk && ntab * (2 * s5 + 1) <= kShiftMaxItems; ++s5) {
+    const long long len5 = kfac::ceil_div(nk, s5);
+    if (kfac::ceil_div(nk, len5) != s5) continue;
+    // the slice count of the three-shift group whose items are no longer than these
+    long long len3 = std::min(nk, std::max<long long>(1, 5 * len5 / 3));
+    const long long s3 = kfac::ceil_div(nk, len3);
+    len3 = kfac::ceil_div(nk, s3);
+    const long long items = ntab * (2 * s5 + s3);
+    if (items > kShiftMaxItems) continue;
+    const double longest = (double)std::max(5 * len5, 3 * len3);
+    const double rounds = (double)kfac::ceil_div<long long>(items, wm == 1 ? 768 : 512);
+    // an item's fixed cost in units of one shift-panel
+    const double cost = rounds * (longest + 6.0) + 0.004 * (double)items;
+    if (best_cost == 0.0 || cost < best_cost) {
+      best_cost = cost;
+      best_s5 = s5;
+      best_s3 = s3;
+      best_longest = longest;
+    }
+  }
+  if (const char *env = getenv("KFAC_SHIFT_SLICES")) {   // tuning override: "s5,s3"
+    long long a = 0, b = 0;
+    if (sscanf(env, "%lld,%lld", &a, &b) == 2 && a >= 1 && b >= 1) {
+      best_s5 = std::min(a, nk);
+      best_s3 = std::min(b, nk);
+      best_longest = (double)std::max(5 * kfac::ceil_div(nk, best_s5), 3 * kfac::ceil_div(nk, best_s3));
+    }
+  }
+  return ShiftSlices{best_s5, best_s3, best_longest};
+}
+
+// Slices of a strip or corner group of gk panels: items about as long as the others'.
+long long shift_strip_slices(long long gk, double longest) {
+  return kfac::ceil_div<long long>(3 * gk, std::max<long long>(3, (long long)longest));
+}
+
+// 64-row first-operand tiles unless 128 rows waste no more on the channel count
+int shift_wm(int c) {
+  const long long t64 = kfac::ceil_div(c, 64), t128 = kfac::ceil_div(c, 128);
+  return 1.15 * (double)(t64 * t64) < 4.0 * (double)(t128 * t128) ? 1 : 2;
+}
+
+bool shift_route_takes(int c, int h, int w) {
+  int min_c = 64;
+  if (const char *env = getenv("KFAC_CONV_SHIFT")) {   // tuning override: 0 = off, else the least channel count
+    min_c = atoi(env);
+    if (min_c <= 0) return false;
+  }
+  return c >= min_c && h >= 4 && w >= 4 && h <= 32767 && w <= 32767;
+}
+
+// Upper bound of the workspace floats the route takes for c channels and `rows` =
+// samples x pixels (the image's sides are not known here: at least 4 each).
+size_t shift_ws_floats_bound(int c, long long rows) {
+  const int wm = shift_wm(c), bm = 64 * wm;
+  const int ntab = kfac::ceil_div(c, bm) * kfac::ceil_div(c, 64);
+  const long long nk = kfac::ceil_div<long long>(rows, KT);
+  const ShiftSlices sl = plan_shift_slices(wm, ntab, nk);
+  size_t floats = (size_t)ntab * (size_t)(2 * sl.s5 * 5 + sl.s3 * 3) * bm * 64;
+  // 8 strip / corner groups of three shifts; a strip has at most rows / 4 k-values
+  const long long strip =
+      shift_strip_slices(kfac::ceil_div<long long>(kfac::ceil_div<long long>(rows, 4), KT), sl.longest);
+  floats += (size_t)8 * ntab * (size_t)std::max(1ll, strip) * 3 * bm * 64;
+  floats += (size_t)kfac::shift::kArrays * c * c;
+  floats += (size_t)1024 * kfac::shift::kChannelSums + (size_t)c * 16;   // sums: at most 1024 (chunk, channel) pairs
+  floats += (size_t)c * (size_t)kfac::ceil_div<long long>(rows, 2);      // border columns: 2 n c h, h <= rows / (4 n)
+  return floats + 256;
+}
+
 // The shifted-correlation route (conv_shift.h) for a 3x3, stride-1, padding-1
 // convolution: 1 when the shape is left to the patch-product kernels (few
 // channels, tiny images, workspace too small).
@@ -796,7 +881,15 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   const size_t sums_floats = (size_t)nchunk * c * kChannelSums;
   const size_t edge_floats = (size_t)2 * n * c * h;
   const size_t tail_floats = array_floats + sums_floats + edge_floats + 64;
-  if (ws == nullptr || ws_bytes < tail_floats * sizeof(float)) return 1;
+  // a workspace smaller than the route needs sends the factor to the patch-product
+  // kernels (KFAC_CONV_SHIFT_STRICT: an error instead, for the test of the workspace query)
+  auto too_small = [&](size_t need_floats) {
+    if (getenv("KFAC_CONV_SHIFT_STRICT"))
+      return kfac::fail(KFAC_ENOMEM, "shifted-correlation workspace too small: %zu < %zu bytes", ws_bytes,
+                        need_floats * sizeof(float));
+    return 1;
+  };
+  if (ws == nullptr || ws_bytes < tail_floats * sizeof(float)) return too_small(tail_floats);
   float *partial = static_cast<float *>(ws);
   float *arrays = partial + (ws_bytes / sizeof(float) - tail_floats) / 4 * 4;
   float *sums = arrays + array_floats;
@@ -824,43 +917,10 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   for (int lr = 0; lr < 2; ++lr)
     for (int lc = 0; lc < 2; ++lc)
       group(7 + 2 * lr + lc, edges + (size_t)lc * n * c * h + (lr ? h - 1 : 0), es, h, h, 1, 1, 1, 0, 0, 3, 1);
-  // Slices of the whole-image groups: the workgroups of a launch run two to a CU,
-  // 512 at a time (three with 64 first-operand channels), and a group of ns shifts does ns tile products per panel.  Among
-  // the slice counts (s5 for the two groups of five shifts, s3 for the group of
-  // three) the pair with the least rounds x longest item, plus what an item costs
-  // besides its panels (prologue, partial tiles written and summed).
   const long long nk = kfac::ceil_div(n * h * w, KT);
-  long long best_s5 = 1, best_s3 = 1;
-  double best_cost = 0.0, best_longest = 1.0;
-  const long long max_items = 4096;
-  for (long long s5 = 1; s5 <= nk && ntab * (2 * s5 + 1) <= max_items; ++s5) {
-    const long long len5 = kfac::ceil_div(nk, s5);
-    if (kfac::ceil_div(nk, len5) != s5) continue;
-    // the slice count of the three-shift group whose items are no longer than these
-    long long len3 = std::min(nk, std::max<long long>(1, 5 * len5 / 3));
-    const long long s3 = kfac::ceil_div(nk, len3);
-    len3 = kfac::ceil_div(nk, s3);
-    const long long items = ntab * (2 * s5 + s3);
-    if (items > max_items) continue;
-    const double longest = (double)std::max(5 * len5, 3 * len3);
-    const double rounds = (double)kfac::ceil_div<long long>(items, WM == 1 ? 768 : 512);
-    // an item's fixed cost in units of one shift-panel
-    const double cost = rounds * (longest + 6.0) + 0.004 * (double)items;
-    if (best_cost == 0.0 || cost < best_cost) {
-      best_cost = cost;
-      best_s5 = s5;
-      best_s3 = s3;
-      best_longest = longest;
-    }
-  }
-  if (const char *env = getenv("KFAC_SHIFT_SLICES")) {   // tuning override: "s5,s3"
-    long long a = 0, b = 0;
-    if (sscanf(env, "%lld,%lld", &a, &b) == 2 && a >= 1 && b >= 1) {
-      best_s5 = std::min(a, nk);
-      best_s3 = std::min(b, nk);
-      best_longest = (double)std::max(5 * kfac::ceil_div(nk, best_s5), 3 * kfac::ceil_div(nk, best_s3));
-    }
-  }
+  const ShiftSlices sl = plan_shift_slices(WM, ntab, nk);
+  const long long best_s5 = sl.s5, best_s3 = sl.s3;
+  const double best_longest = sl.longest;
   // items: strips and corners first (block order), then the whole-image groups
   size_t partial_floats = 0;
   int total = 0;
@@ -877,7 +937,7 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   };
   for (int gi = 3; gi < kGroups; ++gi) {
     const long long gk = kfac::ceil_div(pl.grp[gi].K, KT);
-    slice(gi, kfac::ceil_div<long long>(3 * gk, std::max<long long>(3, (long long)best_longest)));
+    slice(gi, shift_strip_slices(gk, best_longest));
   }
   pl.nsmall = total;
   slice(0, best_s3);
@@ -905,7 +965,8 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   for (int lr = 0; lr < 2; ++lr)
     for (int lc = 0; lc < 2; ++lc) product(7 + 2 * lr + lc, 0, 45 + 2 * lr + lc, 45 + 2 * lr + lc);
   if (np != kProducts) return kfac::fail(KFAC_EINVAL, "internal: %d products", np);
-  if (partial_floats >= (1ull << 32) || partial + partial_floats > arrays) return 1;
+  if (partial_floats >= (1ull << 32)) return 1;
+  if (partial + partial_floats > arrays) return too_small(partial_floats + tail_floats + 4);
   hipLaunchKernelGGL(edge_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums, edges);
   KFAC_HIP_CHECK(hipGetLastError());
   {
@@ -935,22 +996,14 @@ int try_conv_shift(const float *x, int n, int c, int h, int w, int kh, int kw, i
                    int pw, int d, int ones, float alpha, float beta, float *C, void *ws, size_t ws_bytes,
                    hipStream_t stream) {
   if (kh != 3 || kw != 3 || sy != 1 || sx != 1 || ph != 1 || pw != 1) return 1;
-  int min_c = 64;
-  if (const char *env = getenv("KFAC_CONV_SHIFT")) {   // tuning override: 0 = off, else the least channel count
-    min_c = atoi(env);
-    if (min_c <= 0) return 1;
-  }
-  if (c < min_c || h < 4 || w < 4 || h > 32767 || w > 32767) return 1;
+  if (!shift_route_takes(c, h, w)) return 1;
   kfac::shift::Plan pl;
   memset(&pl, 0, sizeof(pl));
   pl.x = x;
   pl.sample_stride = (unsigned)((long long)c * h * w);
   pl.row_stride = (unsigned)(h * w);
   pl.C = c; pl.H = h; pl.W = w; pl.n = n;
-  // 128-tiles unless 64-tiles waste much less on a channel count that is not a multiple of 128
-  const long long t64 = kfac::ceil_div(c, 64), t128 = kfac::ceil_div(c, 128);
-  if (1.15 * (double)(t64 * t64) < 4.0 * (double)(t128 * t128))
-    return run_conv_shift<1>(pl, d, ones, alpha, beta, C, ws, ws_bytes, stream);
+  if (shift_wm(c) == 1) return run_conv_shift<1>(pl, d, ones, alpha, beta, C, ws, ws_bytes, stream);
   return run_conv_shift<2>(pl, d, ones, alpha, beta, C, ws, ws_bytes, stream);
 }
 
@@ -1015,7 +1068,6 @@ extern "C" size_t kfac_cov_workspace_bytes(int d, int64_t rows) {
   // upper bound over every kernel and reduction length: no plan uses more than
   // max_splits(tiles) k-slices (plus the slots of the pre-reduction), with 64- or
   // 128-tiles, with or without a ones column (the tile grid then covers d - 1 rows)
-  (void)rows;
   size_t need = 0;
   for (int dt = d > 1 ? d - 1 : d; dt <= d; ++dt)
     for (int bm = 64; bm <= 128; bm *= 2) {
@@ -1027,6 +1079,10 @@ extern "C" size_t kfac_cov_workspace_bytes(int d, int64_t rows) {
       p.nreduced = p.nsplit > kFinishSplits ? kFinishSplits : 0;
       need = std::max(need, syrk_ws_floats(p));
     }
+  // the shifted-correlation route of a 3x3 convolution's A factor (d = 9 c or 9 c + 1)
+  for (int ones = 0; ones <= 1 && rows > 0; ++ones)
+    if ((d - ones) % 9 == 0 && shift_route_takes((d - ones) / 9, 4, 4))
+      need = std::max(need, shift_ws_floats_bound((d - ones) / 9, rows));
   return need * sizeof(float);
 }
 

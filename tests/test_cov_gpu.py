@@ -164,6 +164,29 @@ def test_conv_A_shift_route_unaligned_input_and_accumulation():
     check(out, acc[0])
 
 
+@pytest.mark.parametrize('n,c,h,w', [(32, 64, 56, 56), (32, 128, 28, 28), (8, 256, 14, 14), (4, 512, 7, 7),
+                                     (2, 64, 4, 200), (3, 96, 9, 5)])
+def test_workspace_query_covers_the_shift_route(n, c, h, w, monkeypatch):
+    """A workspace of exactly kfac_cov_workspace_bytes(d, rows) is enough for the shifted-correlation
+    route (with KFAC_CONV_SHIFT_STRICT a workspace that is too small for it is an error instead of a
+    silent change of route)."""
+    from chainerkfac_amd import _lib, device as _dev
+    lib = _lib.load()
+    monkeypatch.setenv('KFAC_CONV_SHIFT_STRICT', '1')
+    d = 9 * c + 1
+    nbytes = lib.kfac_cov_workspace_bytes(d, n * h * w)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device='cuda')
+    x = torch.randn(n, c, h, w, device='cuda')
+    out = torch.empty(d, d, device='cuda')
+    _lib.check(lib.kfac_cov_conv_a_f32(x.data_ptr(), n, c, h, w, 3, 3, 1, 1, 1, 1, 1, 1.0 / n, 0.0, out.data_ptr(),
+                                       ws.data_ptr(), nbytes, _dev.stream_handle(None)))
+    torch.cuda.synchronize()
+    # and one byte less than the route's tail is refused in strict mode
+    with pytest.raises(Exception):
+        _lib.check(lib.kfac_cov_conv_a_f32(x.data_ptr(), n, c, h, w, 3, 3, 1, 1, 1, 1, 1, 1.0 / n, 0.0,
+                                           out.data_ptr(), ws.data_ptr(), 1024, _dev.stream_handle(None)))
+
+
 def test_conv_A_shift_route_border_terms():
     """An input that is zero except on the image border and corners: every entry of the factor is
     then made of the border corrections (row / column strips and corner pixels) alone."""
