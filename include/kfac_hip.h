@@ -92,7 +92,12 @@ int kfac_unpack_f16(kfac_pack_plan_t plan, const void *buf, int64_t buf_nelems,
  * (1) Kronecker-factor construction:  C = beta*C + alpha * P^T P
  *     beta = 1, alpha = scale/acc_iters gives the running accumulation of
  *     optimizers/kfac.py:294-304; beta = 0 the plain covariance.
- *     All of them need kfac_cov_workspace_bytes(d, rows) bytes of workspace.
+ *     All of them need kfac_cov_workspace_bytes(d, rows) bytes of workspace,
+ *     d the side of C and rows the length of the reduction (samples, times
+ *     output pixels for a convolution).  With less, a factor that has several
+ *     routes takes one that fits (rows <= 0 asks for the bound of the routes
+ *     whose need does not depend on it); with too little for any, the call
+ *     fails with KFAC_ENOMEM.
  * --------------------------------------------------------------------- */
 size_t kfac_cov_workspace_bytes(int d, int64_t rows);
 
