@@ -29,15 +29,15 @@
 namespace kfac {
 namespace mma {
 
-// Operand of one product: rows = channels, k = (sample, p), p < L running over the
-// product's domain (a whole image, one image row, one image column or one pixel);
-//   p -> (a, b) = (p / line_len, p % line_len),
-//   element = base[sample * sample_stride + row * row_stride + (a + da) * line_stride + (b + db)]
-// if 0 <= a + da < amax and 0 <= b + db < bmax, else 0.  Dword loads, the 32 lanes
-// of a half-wave on 32 consecutive k of one row (the layout of LoaderKC's scalar
-// variant).
+// First operand of a group of products: rows = channels, k = (sample, p), p < L
+// running over the group's domain (a whole image, one image row, one border column
+// or one pixel):
+//   element = base[sample * sample_stride + row * row_stride + (p / line_len) * line_stride + p % line_len],
+// 0 for rows >= rows_valid and k past the end of the slice.  Dword loads, the 32
+// lanes of a half-wave on 32 consecutive k of one row (the layout of LoaderKC's
+// scalar variant).
 template <int ROWS>
-struct LoaderShift {
+struct LoaderDomain {
   static constexpr bool kKRow = false;
   static constexpr int NR = ROWS / 8;   // rows per thread
   struct Regs {
@@ -47,26 +47,23 @@ struct LoaderShift {
   const float *base;
   unsigned sample_stride, row_stride;
   unsigned L, line_len, line_stride;
-  int da, db, amax, bmax;
   int rows_valid;
   int first_row;
   unsigned last_off;
 
-  __device__ __forceinline__ void init(float *, int row0) {
+  __device__ __forceinline__ void init(int row0) {
     first_row = row0 + (team_tid() >> 5);
     last_off = (unsigned)(rows_valid > 0 ? rows_valid - 1 : 0) * row_stride;
   }
 
-  __device__ __forceinline__ void load(Regs &r, int, long long k0, long long k_end) const {
+  __device__ __forceinline__ void load(Regs &r, long long k0, long long k_end) const {
     const long long kg = k0 + (team_tid() & 31);
-    const bool kin = kg < k_end;
-    const unsigned kc = kin ? (unsigned)kg : 0u;
+    r.kvalid = kg < k_end;
+    const unsigned kc = r.kvalid ? (unsigned)kg : 0u;
     const unsigned s = kc / L;
     const unsigned p = kc - s * L;
-    const unsigned a0 = p / line_len;
-    const int a = (int)a0 + da, b = (int)(p - a0 * line_len) + db;
-    r.kvalid = kin && (unsigned)a < (unsigned)amax && (unsigned)b < (unsigned)bmax;
-    const unsigned koff = r.kvalid ? s * sample_stride + (unsigned)a * line_stride + (unsigned)b : 0u;
+    const unsigned a = p / line_len;
+    const unsigned koff = s * sample_stride + a * line_stride + (p - a * line_len);
     int fr = first_row;
     asm volatile("" : "+v"(fr));   // keep the NR row offsets out of registers (see LoaderKC)
     const unsigned off0 = (unsigned)fr * row_stride;
@@ -183,18 +180,15 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
   const int I = tile / pl.tiles_b, J = tile - I * pl.tiles_b;
   const unsigned L = g.L, mem_line = g.mem_line, vline = g.vline;
   const int K = g.K;
-  LoaderShift<BMA> la;
+  LoaderDomain<BMA> la;
   la.base = g.base;
   la.sample_stride = g.sample_stride;
   la.row_stride = g.row_stride;
   la.L = L;
   la.line_len = mem_line;
   la.line_stride = g.line_stride;
-  la.amax = 0x7fffffff;
-  la.bmax = 0x7fffffff;
   la.rows_valid = pl.C;
-  la.da = la.db = 0;
-  la.init(nullptr, I * BMA);
+  la.init(I * BMA);
   const int tid = team_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -223,7 +217,7 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
     for (int im = 0; im < WM; ++im)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[s][im][v] = 0.f;
-  typename LoaderShift<BMA>::Regs ra;
+  typename LoaderDomain<BMA>::Regs ra;
   float rb[9];
   auto load_b = [&](long long k0) {
     auto offset_of = [&](int j) {
@@ -239,7 +233,7 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
     rb[8] = gload1(g.base, (oe + rowoff_e) * 4u);
   };
   if (kbeg < kend) {
-    la.load(ra, 0, kbeg, kend);
+    la.load(ra, kbeg, kend);
     load_b(kbeg);
   }
   for (long long k0 = kbeg; k0 < kend; k0 += KT) {
@@ -249,7 +243,7 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
     ldsB[re * kShiftStride + je] = rowe < pl.C ? rb[8] : 0.f;
     __syncthreads();
     if (k0 + KT < kend) {
-      la.load(ra, 0, k0 + KT, kend);
+      la.load(ra, k0 + KT, kend);
       load_b(k0 + KT);
     }
     // validity of the NS shifted pixels of this panel's 32 k-values: bit k of m[s]
