@@ -349,8 +349,8 @@ def run_step_config(args, name, cfg):
     # shifted correlations, about a third of the multiply-adds of the patch product
     cov_executed = float(W.cov_flops_executed(layers, batch)) * acc_iters
     achieved_executed = cov_executed / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
+    executed_flops = cov_executed + dense_inverse_flops + flops['precondition']
     total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
-    executed_flops = flops['cov'] + dense_inverse_flops + flops['precondition']
     traffic = read_traffic() if name == 'c3' else None
     result = {
         'metric': METRIC,
@@ -371,11 +371,13 @@ def run_step_config(args, name, cfg):
                    'hip_graph': not args.no_graph, 'lanes': args.lanes, 'macro_tiles': bool(args.macro_tiles),
                    'bn_inverse': 'woodbury rank-{} ({} blocks)'.format(batch, len(lowrank)) if lowrank else 'dense'},
         # rates use the flops actually executed; the *_reference_work entries divide the work of the
-        # reference's algorithm (every factor inverted densely) by the same times
+        # reference's algorithm (every factor a patch / activation product, every factor inverted densely)
+        # by the same times
         'tflops': {
             'step': round(executed_flops / ms_per_step / 1e9, 2),
-            'cov_inv': round((flops['cov'] + dense_inverse_flops) / ((phase_ms['cov'] + phase_ms['inverse'])) / 1e9, 2),
-            'cov': round(flops['cov'] / phase_ms['cov'] / 1e9, 2),
+            'cov_inv': round((cov_executed + dense_inverse_flops) / ((phase_ms['cov'] + phase_ms['inverse'])) / 1e9, 2),
+            'cov': round(cov_executed / phase_ms['cov'] / 1e9, 2),
+            'cov_reference_work': round(flops['cov'] / phase_ms['cov'] / 1e9, 2),
             'inverse': round(dense_inverse_flops / phase_ms['inverse'] / 1e9, 2),
             'precondition': round(flops['precondition'] / phase_ms['precondition'] / 1e9, 2),
             'frac_of_fp32_mfma_peak': round(executed_flops / ms_per_step / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4),
@@ -384,7 +386,7 @@ def run_step_config(args, name, cfg):
         },
         'phase_ms': {k: round(v, 3) for k, v in phase_ms.items()},
         'gflop': dict({k: round(v / 1e9, 1) for k, v in flops.items()},
-                      inverse_executed=round(dense_inverse_flops / 1e9, 1)),
+                      inverse_executed=round(dense_inverse_flops / 1e9, 1), cov_executed=round(cov_executed / 1e9, 1)),
         'kernel_ms': {k: {'launches': n, 'total_ms': round(ms - n * empty, 3)} for k, (n, ms) in fam.items() if n},
         'inverse_info_nonzero': info_bad,
         'wire_format': wire_stats,
