@@ -118,11 +118,21 @@ constexpr int kChannelSums = 9;   // whole image, first / last row, first / last
 // The whole image and its first / last row are read from the input tensor; the
 // first / last column and the corners from a compact copy of the two border columns
 // ([2][n][C][H], written by edge_sums_kernel), where a column is contiguous.
+// Layers of at most 32 channels would fill a quarter of a 64 x 64 tile.  Their
+// whole-image groups are `stacked`: the 64 first-operand rows are the channels at
+// row shift 0 and, 32 rows on, the same channels one image row up (X(c, u - 1, v):
+// against a second operand at row shift di that is the product of row shift di + 1),
+// the 64 second-operand rows the channels and, 32 rows on, the same channels three
+// columns on -- so the four 32 x 32 blocks of a tile and its three column offsets
+// are the products of row shifts di, di + 1 and column shifts dj0 .. dj0 + 5.
+// stacked = 2: both first-operand halves; 1: only the first (the waves of the
+// second issue no matrix instructions); 0: plain rows = channels.
 struct ShiftGroup {
   const float *base;
   unsigned sample_stride, row_stride, line_stride;
   unsigned L, mem_line, vline;
   short di, dj0, ns, amax;
+  int stacked;
   int K;               // reduction length: samples * L
   int klen, nsplit;    // k-values per slice (a multiple of KT), slices
   int task0;           // first work item of the group
@@ -170,9 +180,10 @@ __device__ __forceinline__ int item_of_block(int bid, int total) {
 constexpr int kShiftCols = 36;
 constexpr int kShiftStride = 37;   // odd: the 32 rows of an operand read on 32 banks
 
-template <int WM, int NS>
+template <int WM, int NS, bool STACKED = false>
 __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGroup &g, int q, float *lds,
                                                  float *__restrict__ partial) {
+  static_assert(!STACKED || WM == 1, "stacked groups use 64-row tiles");
   constexpr int BMA = 64 * WM;
   float *ldsA = lds, *ldsB = lds + Panel<BMA>::kFloats;
   const int ntile = pl.tiles_a * pl.tiles_b;
@@ -189,6 +200,10 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
   la.line_stride = g.line_stride;
   la.rows_valid = pl.C;
   la.init(I * BMA);
+  if (STACKED) {   // all of a thread's rows are rows of one half: channel = row % 32
+    la.first_row = team_tid() >> 5;
+    la.rows_valid = pl.C;
+  }
   const int tid = team_tid();
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -201,11 +216,11 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
   unsigned rowok = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int row = J * 64 + rm + 8 * i;
+    const int row = STACKED ? (rm + 8 * i) & 31 : J * 64 + rm + 8 * i;
     rowoff[i] = (unsigned)(row < pl.C ? row : pl.C - 1) * g.row_stride;
     if (row < pl.C) rowok |= 1u << i;
   }
-  const int rowe = J * 64 + re;
+  const int rowe = STACKED ? re & 31 : J * 64 + re;
   const unsigned rowoff_e = (unsigned)(rowe < pl.C ? rowe : pl.C - 1) * g.row_stride;
   const long long kbeg = (long long)split * g.klen;
   long long kend = kbeg + g.klen;
@@ -227,23 +242,53 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
       const unsigned line = p / mem_line;
       return s * g.sample_stride + line * g.line_stride + (p - line * mem_line);
     };
-    const unsigned om = offset_of(jm), oe = offset_of(je);
+    const unsigned om = offset_of(jm), oe = offset_of(je + (STACKED && re >= 32 ? 3 : 0));
+    const unsigned om1 = STACKED ? offset_of(jm + 3) : om;   // rows 32..: three columns on
 #pragma unroll
-    for (int i = 0; i < 8; ++i) rb[i] = gload1(g.base, (om + rowoff[i]) * 4u);
+    for (int i = 0; i < 8; ++i) rb[i] = gload1(g.base, ((STACKED && i >= 4 ? om1 : om) + rowoff[i]) * 4u);
     rb[8] = gload1(g.base, (oe + rowoff_e) * 4u);
   };
+  // first operand of a stacked group: rows 32.. are the channels one image row up
+  auto load_a = [&](long long k0) {
+    if (!STACKED) {
+      la.load(ra, k0, kend);
+      return;
+    }
+    const long long kg = k0 + jm;
+    ra.kvalid = kg < kend;
+    const long long kc = ra.kvalid ? kg : 0;
+    auto offset_at = [&](long long kk) {
+      const unsigned ku = (unsigned)(kk < 0 ? 0 : kk), s = ku / L, p = ku - s * L;
+      return s * g.sample_stride + p;   // whole images: pixels are contiguous
+    };
+    const unsigned o0 = offset_at(kc), o1 = offset_at(kc - (long long)vline);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = (rm + 8 * i) & 31;
+      ra.v[i] = gload1(g.base, ((i >= 4 ? o1 : o0) + (unsigned)(row < pl.C ? row : pl.C - 1) * g.row_stride) * 4u);
+    }
+  };
+  auto store_a = [&]() {
+    if (!STACKED) {
+      la.store(ra, ldsA);
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      ldsA[(rm + 8 * i) * Panel<BMA>::kRowKStride + jm] = (ra.kvalid && ((rm + 8 * i) & 31) < pl.C) ? ra.v[i] : 0.f;
+  };
   if (kbeg < kend) {
-    la.load(ra, kbeg, kend);
+    load_a(kbeg);
     load_b(kbeg);
   }
   for (long long k0 = kbeg; k0 < kend; k0 += KT) {
-    la.store(ra, ldsA);
+    store_a();
 #pragma unroll
     for (int i = 0; i < 8; ++i) ldsB[(rm + 8 * i) * kShiftStride + jm] = ((rowok >> i) & 1u) ? rb[i] : 0.f;
     ldsB[re * kShiftStride + je] = rowe < pl.C ? rb[8] : 0.f;
     __syncthreads();
     if (k0 + KT < kend) {
-      la.load(ra, k0 + KT, kend);
+      load_a(k0 + KT);
       load_b(k0 + KT);
     }
     // validity of the NS shifted pixels of this panel's 32 k-values: bit k of m[s]
@@ -253,12 +298,16 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
       const unsigned kc = kg < kend ? (unsigned)kg : 0u;
       const unsigned pix = kc % L;
       const unsigned a = pix / vline, b = pix - a * vline;
-      const bool row_in = kg < kend && (int)a + g.di < g.amax;
+      // stacked: this wave's blocks are row shift di + wm (first operand one row up:
+      // not for the first image row) and column shifts dj0 + 3 wn + s
+      const bool row_in = kg < kend && (int)a + g.di < g.amax && (!STACKED || (int)a >= wm);
+      const int dj_first = g.dj0 + (STACKED ? 3 * wn : 0);
 #pragma unroll
       for (int s = 0; s < NS; ++s)
         m[s] = __builtin_amdgcn_readfirstlane(
-            (unsigned)__ballot(row_in && (unsigned)((int)b + g.dj0 + s) < vline));
+            (unsigned)__ballot(row_in && (unsigned)((int)b + dj_first + s) < vline));
     }
+    const bool active = !STACKED || wm < g.stacked;
     const float *pa = ldsA + (wm * WM * 32 + lrow) * Panel<BMA>::kRowKStride + lk;
     const float *pb = ldsB + (wn * 32 + lrow) * kShiftStride + lk + 2 + g.dj0;
     // operands of step kk + 1 are read from LDS before the matrix instructions of
@@ -269,6 +318,7 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
     for (int im = 0; im < WM; ++im) a[0][im] = pa[im * 32 * Panel<BMA>::kRowKStride];
 #pragma unroll
     for (int s = 0; s < NS; ++s) b[0][s] = pb[s];
+    if (active) {
 #pragma unroll
     for (int kk = 0; kk < KT / 2; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
@@ -291,6 +341,7 @@ __device__ __forceinline__ void corr_shifts_body(const Plan &pl, const ShiftGrou
           acc[s][im] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][im], v, acc[s][im], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
     }
     __syncthreads();
   }
@@ -321,6 +372,12 @@ __global__ __launch_bounds__(THREADS, 2) void corr_kernel(Plan pl, float *__rest
     while (gi + 1 < kGroups && pl.grp[gi + 1].task0 <= w) ++gi;
   }
   const ShiftGroup &g = pl.grp[gi];
+  if constexpr (WM == 1) {
+    if (g.stacked) {
+      corr_shifts_body<1, 3, true>(pl, g, w - g.task0, lds, partial);
+      return;
+    }
+  }
   if (g.ns == 3)
     corr_shifts_body<WM, 3>(pl, g, w - g.task0, lds, partial);
   else

@@ -824,6 +824,15 @@ ShiftSlices plan_shift_slices(int wm, int ntab, long long nk) {
   return ShiftSlices{best_s5, best_s3, best_longest};
 }
 
+// Stacked groups (one tile pair, two groups of three column offsets): equal slices,
+// about 720 items in all for the 768 slots of three workgroups per CU.
+ShiftSlices plan_stacked_slices(long long nk) {
+  const long long want = std::max<long long>(1, std::min<long long>(360, nk / 8));
+  const long long len = kfac::ceil_div(nk, want);
+  const long long ns = kfac::ceil_div(nk, len);
+  return ShiftSlices{ns, ns, (double)(3 * len)};
+}
+
 // Slices of a strip or corner group of gk panels: items about as long as the others'.
 long long shift_strip_slices(long long gk, double longest) {
   return kfac::ceil_div<long long>(3 * gk, std::max<long long>(3, (long long)longest));
@@ -835,13 +844,18 @@ int shift_wm(int c) {
   return 1.15 * (double)(t64 * t64) < 4.0 * (double)(t128 * t128) ? 1 : 2;
 }
 
+// Layers of 28..32 channels take the route with stacked operand tiles (conv_shift.h).
+bool shift_stacked(int c) { return c >= 28 && c <= 32; }
+
 bool shift_route_takes(int c, int h, int w) {
   int min_c = 64;
+  bool stacked_on = true;
   if (const char *env = getenv("KFAC_CONV_SHIFT")) {   // tuning override: 0 = off, else the least channel count
     min_c = atoi(env);
     if (min_c <= 0) return false;
+    stacked_on = min_c <= 32;
   }
-  return c >= min_c && h >= 4 && w >= 4 && h <= 32767 && w <= 32767;
+  return (c >= min_c || (stacked_on && shift_stacked(c))) && h >= 4 && w >= 4 && h <= 32767 && w <= 32767;
 }
 
 // Upper bound of the workspace floats the route takes for c channels and `rows` =
@@ -850,8 +864,10 @@ size_t shift_ws_floats_bound(int c, long long rows) {
   const int wm = shift_wm(c), bm = 64 * wm;
   const int ntab = kfac::ceil_div(c, bm) * kfac::ceil_div(c, 64);
   const long long nk = kfac::ceil_div<long long>(rows, KT);
-  const ShiftSlices sl = plan_shift_slices(wm, ntab, nk);
-  size_t floats = (size_t)ntab * (size_t)(2 * sl.s5 * 5 + sl.s3 * 3) * bm * 64;
+  const bool stacked = shift_stacked(c);
+  const ShiftSlices sl = stacked ? plan_stacked_slices(nk) : plan_shift_slices(wm, ntab, nk);
+  size_t floats = stacked ? (size_t)(sl.s5 + sl.s3) * 3 * bm * 64
+                          : (size_t)ntab * (size_t)(2 * sl.s5 * 5 + sl.s3 * 3) * bm * 64;
   // 8 strip / corner groups of three shifts; a strip has at most rows / 4 k-values
   const long long strip =
       shift_strip_slices(kfac::ceil_div<long long>(kfac::ceil_div<long long>(rows, 4), KT), sl.longest);
@@ -903,12 +919,23 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
     g.line_stride = (unsigned)line_stride;
     g.L = (unsigned)L; g.mem_line = (unsigned)mem_line; g.vline = (unsigned)vline;
     g.di = (short)di; g.dj0 = (short)dj0; g.ns = (short)ns; g.amax = (short)amax;
+    g.stacked = 0;
     g.K = n * L;
   };
   const long long xs = (long long)c * h * w, es = (long long)c * h;
-  group(0, pl.x, xs, h * w, w, h * w, h * w, w, 0, 0, 3, h);
-  group(1, pl.x, xs, h * w, w, h * w, h * w, w, 1, -2, 5, h);
-  group(2, pl.x, xs, h * w, w, h * w, h * w, w, 2, -2, 5, h);
+  const bool stacked = shift_stacked(c);
+  if (stacked) {
+    // row shifts 0 and 1 from one group (both halves of the first operand), row shift 2 from another
+    group(0, pl.x, xs, h * w, w, h * w, h * w, w, 0, -2, 3, h);
+    group(1, pl.x, xs, h * w, w, h * w, h * w, w, 2, -2, 3, h);
+    group(2, pl.x, xs, h * w, w, h * w, h * w, w, 2, -2, 3, h);   // no items
+    pl.grp[0].stacked = 2;
+    pl.grp[1].stacked = 1;
+  } else {
+    group(0, pl.x, xs, h * w, w, h * w, h * w, w, 0, 0, 3, h);
+    group(1, pl.x, xs, h * w, w, h * w, h * w, w, 1, -2, 5, h);
+    group(2, pl.x, xs, h * w, w, h * w, h * w, w, 2, -2, 5, h);
+  }
   for (int last = 0; last < 2; ++last) {
     group(3 + last, pl.x + (last ? (h - 1) * w : 0), xs, h * w, w, w, w, w, 0, 0, 3, 1);
     const float *col = edges + (size_t)last * n * c * h;
@@ -918,7 +945,7 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
     for (int lc = 0; lc < 2; ++lc)
       group(7 + 2 * lr + lc, edges + (size_t)lc * n * c * h + (lr ? h - 1 : 0), es, h, h, 1, 1, 1, 0, 0, 3, 1);
   const long long nk = kfac::ceil_div(n * h * w, KT);
-  const ShiftSlices sl = plan_shift_slices(WM, ntab, nk);
+  const ShiftSlices sl = stacked ? plan_stacked_slices(nk) : plan_shift_slices(WM, ntab, nk);
   const long long best_s5 = sl.s5, best_s3 = sl.s3;
   const double best_longest = sl.longest;
   // items: strips and corners first (block order), then the whole-image groups
@@ -942,7 +969,15 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   pl.nsmall = total;
   slice(0, best_s3);
   slice(1, best_s5);
-  slice(2, best_s5);
+  if (stacked) {
+    ShiftGroup &g = pl.grp[2];   // empty
+    g.nsplit = 0;
+    g.klen = KT;
+    g.task0 = total;
+    g.part_off = (unsigned)partial_floats;
+  } else {
+    slice(2, best_s5);
+  }
   pl.total = total;
   // products -> (group, shift)
   int np = 0;
@@ -957,7 +992,16 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
     p.out_t = (short)out_t;
   };
   for (int di = 0; di <= 2; ++di)
-    for (int dj = (di == 0 ? 0 : -2); dj <= 2; ++dj) product(di, dj, (di + 2) * 5 + dj + 2, (2 - di) * 5 + 2 - dj);
+    for (int dj = (di == 0 ? 0 : -2); dj <= 2; ++dj) {
+      if (!stacked) {
+        product(di, dj, (di + 2) * 5 + dj + 2, (2 - di) * 5 + 2 - dj);
+        continue;
+      }
+      // block (a, b) of the stacked tile at column offset e: row shift di0 + a, column shift -2 + 3 b + e
+      const int gi = di == 2 ? 1 : 0, a = di == 2 ? 0 : di, b = (dj + 2) / 3, e = (dj + 2) % 3;
+      product(gi, -2 + e, (di + 2) * 5 + dj + 2, (2 - di) * 5 + 2 - dj);
+      pl.prod[np - 1].part_off += (unsigned)(a * 32 * 64 + b * 32);
+    }
   for (int last = 0; last < 2; ++last)
     for (int dj = 0; dj <= 2; ++dj) product(3 + last, dj, 25 + 5 * last + dj + 2, 25 + 5 * last + 2 - dj);
   for (int last = 0; last < 2; ++last)

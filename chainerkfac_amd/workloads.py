@@ -155,11 +155,11 @@ def flops(layers, batch):
 
 def takes_shift_route(layer):
     """Whether the library computes the layer's A factor from shifted correlations of
-    the input (3x3, stride 1, padding 1, at least 64 channels, images of at least 4 x 4:
-    the conditions of try_conv_shift in csrc/cov.hip) rather than as a product of
-    patch matrices."""
+    the input (3x3, stride 1, padding 1, at least 64 channels or 28..32, images of at
+    least 4 x 4: the conditions of try_conv_shift in csrc/cov.hip) rather than as a
+    product of patch matrices."""
     return (layer['kind'] == 'conv' and layer['k'] == 3 and layer['s'] == 1 and layer['p'] == 1 and
-            layer['c_in'] >= 64 and layer['h'] >= 4 and layer['w'] >= 4)
+            (layer['c_in'] >= 64 or 28 <= layer['c_in'] <= 32) and layer['h'] >= 4 and layer['w'] >= 4)
 
 
 def cov_flops_executed(layers, batch):
@@ -174,7 +174,12 @@ def cov_flops_executed(layers, batch):
         for i, d in enumerate(dims):
             if i == 0 and takes_shift_route(layer):
                 c, h, w = layer['c_in'], layer['h'], layer['w']
-                total += 2 * c * c * batch * (13 * h * w + 6 * w + 6 * h + 4)
+                if c <= 32:
+                    # stacked tiles: 18 blocks of 32 x 32 over the whole image (13 of them needed),
+                    # strips and corners as three-shift groups on a 64 x 64 tile
+                    total += 2 * batch * (18 * 32 * 32 * h * w + 3 * 64 * 64 * (2 * w + 2 * h + 4))
+                else:
+                    total += 2 * c * c * batch * (13 * h * w + 6 * w + 6 * h + 4)
             else:
                 total += m * d * (d + 1)
     return total

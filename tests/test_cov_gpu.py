@@ -89,9 +89,10 @@ CONV_CASES = [
 
 
 def takes_shift_route(c, h, w, k, s, p):
-    """3x3 / stride 1 / padding 1 with at least 64 channels: computed from shifted correlations of
-    the input unless KFAC_CONV_SHIFT=0 leaves it to the patch-product kernels."""
-    return k == 3 and s == 1 and p == 1 and c >= 64 and h >= 4 and w >= 4
+    """3x3 / stride 1 / padding 1 with at least 64 channels (or 28..32, with stacked operand tiles):
+    computed from shifted correlations of the input unless KFAC_CONV_SHIFT=0 leaves it to the
+    patch-product kernels."""
+    return k == 3 and s == 1 and p == 1 and (c >= 64 or 28 <= c <= 32) and h >= 4 and w >= 4
 
 
 @pytest.fixture
@@ -132,6 +133,11 @@ SHIFT_CASES = [
     (5, 130, 7, 7, True),       # channel count just past a tile
     (2, 64, 1000, 4, True),     # tall and narrow: column strips of 1000 pixels
     (2, 1024, 5, 4, False),     # 8 x 16 tiles per product, a reduction shorter than one panel
+    # 28..32 channels: stacked tiles (two row shifts x two column offsets of the same 32 channels)
+    (2, 32, 112, 112, False),   # ResNet-50-D's stem
+    (3, 32, 9, 7, True),        # odd sizes, odd batch
+    (2, 30, 16, 16, True),      # fewer than 32 channels
+    (1, 28, 4, 4, True),
 ]
 
 
