@@ -565,9 +565,20 @@ __global__ __launch_bounds__(256) void assemble_kernel(Plan pl, const float *__r
   const int C = pl.C;
   const int c = blockIdx.x, c0 = blockIdx.y * CHUNK;
   const int width = (C - c0 < CHUNK) ? C - c0 : CHUNK;
-  for (int e = threadIdx.x; e < kArrays * CHUNK; e += 256) {
+  // all of a thread's loads in flight before the first is stored
+  constexpr int kPer = (kArrays * CHUNK + 255) / 256;
+  float stage[kPer];
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    const int e = threadIdx.x + 256 * k;
     const int a = e / CHUNK, cl = e - a * CHUNK;
-    arr[a][cl] = cl < width ? arrays[((long long)a * C + c) * C + c0 + cl] : 0.f;
+    stage[k] = (a < kArrays && cl < width) ? arrays[((long long)a * C + c) * C + c0 + cl] : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    const int e = threadIdx.x + 256 * k;
+    const int a = e / CHUNK, cl = e - a * CHUNK;
+    if (a < kArrays) arr[a][cl] = stage[k];
   }
   if (ones && blockIdx.y == 0 && threadIdx.x < kChannelSums) {
     float v = 0.f;
@@ -580,7 +591,9 @@ __global__ __launch_bounds__(256) void assemble_kernel(Plan pl, const float *__r
   for (int ij = blockIdx.z * rows_per; ij < (int)(blockIdx.z + 1) * rows_per; ++ij) {
     const int i = ij / 3, j = ij - 3 * i;
     float *dst = out + (long long)(c * 9 + ij) * d + c0 * 9;
-    for (int t = threadIdx.x; t < ncol; t += 256) {
+#pragma unroll
+    for (int t = threadIdx.x; t < CHUNK * 9; t += 256) {
+      if (t >= ncol) break;
       const int cl = t / 9, ij2 = t - 9 * cl;
       const int i2 = ij2 / 3, j2 = ij2 - 3 * i2;
       float v = alpha * assemble<CHUNK>(arr, cl, i, j, i2, j2);
