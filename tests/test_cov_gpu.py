@@ -193,6 +193,25 @@ def test_workspace_query_covers_the_shift_route(n, c, h, w, monkeypatch):
                                            out.data_ptr(), ws.data_ptr(), 1024, _dev.stream_handle(None)))
 
 
+def test_conv_A_shift_route_random_shapes():
+    """Seeded random geometries of the shifted-correlation route (both tile modes, ragged channel
+    counts, images from 4 x 4 up, reductions shorter and longer than a panel, with and without the
+    ones column) against the oracle."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(2024)
+    for _ in range(40):
+        c = int(r.integers(28, 33)) if r.random() < 0.3 else int(r.integers(64, 200))
+        n, h, w = int(r.integers(1, 6)), int(r.integers(4, 24)), int(r.integers(4, 24))
+        bias = bool(r.integers(0, 2))
+        assert takes_shift_route(c, h, w, 3, 1, 1)
+        x = (r.standard_normal((n, c, h, w)) + r.standard_normal()).astype(np.float32)
+        A = ops.cov_conv_a(torch.from_numpy(x).cuda(), 3, 1, 1, bias, 1.0 / n)
+        try:
+            check(A, O.conv_A(x, 3, 1, 1, bias))
+        except AssertionError as e:
+            raise AssertionError('shape n={} c={} h={} w={} bias={}: {}'.format(n, c, h, w, bias, e))
+
+
 def test_conv_A_shift_route_border_terms():
     """An input that is zero except on the image border and corners: every entry of the factor is
     then made of the border corrections (row / column strips and corner pixels) alone."""
