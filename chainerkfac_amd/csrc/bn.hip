@@ -6,6 +6,8 @@
 // written.  One wave owns one (sample, channel) slab.
 // Replaces chainerkfac/optimizers/fisher_blocks/normalizations/
 // batch_normalization.py:86-119.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace {
@@ -70,6 +72,56 @@ __global__ __launch_bounds__(kThreads) void bn_stats_kernel(
       a += dv * dv;
       b += gv;
       g += gv * dv;
+    }
+  }
+  a = group_sum<LPS>(a);
+  b = group_sum<LPS>(b);
+  g = group_sum<LPS>(g);
+  if (lane == 0) {
+    smean[slab] = mean;
+    sm2[slab] = a;
+    sg[slab] = b;
+    sgx[slab] = g;
+  }
+}
+
+// The same for slabs of at most 4 * LPS * Q pixels whose rows are 16-byte aligned:
+// the lane's Q quads of x stay in registers between the two sweeps (x is loaded
+// once, all loads of a sweep are in flight together), and so do those of gy.
+template <int LPS, int Q>
+__global__ __launch_bounds__(kThreads) void bn_stats_reg_kernel(
+    const float *__restrict__ x, const float *__restrict__ gy, int nslab, int hw,
+    float *__restrict__ smean, float *__restrict__ sm2, float *__restrict__ sg,
+    float *__restrict__ sgx) {
+  int slab = (blockIdx.x * kThreads + threadIdx.x) / LPS;
+  if (slab >= nslab) slab = nslab - 1;
+  const int lane = threadIdx.x % LPS;
+  const float4 *x4 = reinterpret_cast<const float4 *>(x + (long long)slab * hw);
+  const float4 *g4 = reinterpret_cast<const float4 *>(gy + (long long)slab * hw);
+  const int nq = hw / 4;
+  float4 xv[Q], gv[Q];
+#pragma unroll
+  for (int k = 0; k < Q; ++k) {
+    const int i = lane + k * LPS;
+    xv[k] = i < nq ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int k = 0; k < Q; ++k) {
+    const int i = lane + k * LPS;
+    gv[k] = i < nq ? g4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int k = 0; k < Q; ++k) acc += (xv[k].x + xv[k].y) + (xv[k].z + xv[k].w);
+  const float mean = group_sum<LPS>(acc) / (float)hw;
+  float a = 0.f, b = 0.f, g = 0.f;
+#pragma unroll
+  for (int k = 0; k < Q; ++k) {
+    if (lane + k * LPS < nq) {
+      const float d0 = xv[k].x - mean, d1 = xv[k].y - mean, d2 = xv[k].z - mean, d3 = xv[k].w - mean;
+      a += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      b += (gv[k].x + gv[k].y) + (gv[k].z + gv[k].w);
+      g += (gv[k].x * d0 + gv[k].y * d1) + (gv[k].z * d2 + gv[k].w * d3);
     }
   }
   a = group_sum<LPS>(a);
@@ -155,7 +207,15 @@ extern "C" int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, i
   const int nslab = n * c;
   float *smean = static_cast<float *>(ws);
   float *sm2 = smean + nslab, *sg = sm2 + nslab, *sgx = sg + nslab;
-  if (hw <= 256)
+  const bool vec =
+      (hw & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gy)) & 15) == 0;
+  if (vec && hw <= 4 * 16 * 4 && !getenv("KFAC_BN_STATS_LOOP"))
+    hipLaunchKernelGGL((bn_stats_reg_kernel<16, 4>), dim3(kfac::ceil_div(nslab, kThreads / 16)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  else if (vec && hw > 256 && hw <= 4 * 64 * 13 && !getenv("KFAC_BN_STATS_LOOP"))
+    hipLaunchKernelGGL((bn_stats_reg_kernel<64, 13>), dim3(kfac::ceil_div(nslab, kThreads / 64)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  else if (hw <= 256)
     hipLaunchKernelGGL(bn_stats_kernel<16>, dim3(kfac::ceil_div(nslab, kThreads / 16)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
   else
