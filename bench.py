@@ -326,6 +326,20 @@ def run_step_config(args, name, cfg):
         arrays = [[(cov, True) for fb in opt.fblocks for cov in fb.covs]]
     wire_stats, _ = wire_format(arrays, dev, lib)
 
+    # the momentum rule over all parameters (the reference's next call after the preconditioning,
+    # optimizers/kfac.py:250-252): not part of `value`, timed the same way as the phases
+    def update_phase():
+        opt.update_params()
+
+    update_ms = {}
+    for label, batched in (('batched', True), ('per_parameter', False)):
+        opt.batch_param_updates = batched
+        update_phase()
+        update_ms[label] = timed(update_phase if args.no_graph else capture(update_phase))
+    opt.batch_param_updates = True
+    n_param_arrays = len(list(model.params()))
+    n_params = sum(p.data.numel() for p in model.params())
+
     # dominant kernel family, timed launch by launch inside the library (one stream: with lanes,
     # launches overlap and the time between a launch's events is shared with others)
     opt._lanes.n = 0
@@ -390,6 +404,13 @@ def run_step_config(args, name, cfg):
         'kernel_ms': {k: {'launches': n, 'total_ms': round(ms - n * empty, 3)} for k, (n, ms) in fam.items() if n},
         'inverse_info_nonzero': info_bad,
         'wire_format': wire_stats,
+        # v = momentum v - lr kfgrad; param += v over every parameter: 20 bytes per element
+        'param_update': {'parameters': n_params, 'arrays': n_param_arrays,
+                         'one_launch_ms': round(update_ms['batched'], 4),
+                         'launch_per_parameter_ms': round(update_ms['per_parameter'], 4),
+                         'one_launch_tb_s': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12, 3),
+                         'frac_of_hbm_peak': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
+                         'in_value': False},
         'roofline': {
             'kernel': 'covariance SYRK family (shift::corr_kernel, syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
             'bound': 'mfma',

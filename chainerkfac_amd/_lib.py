@@ -72,6 +72,10 @@ PROTOTYPES = {
     'kfac_precond_bn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_precond_bn_static_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp]),
     'kfac_momentum_update_f32': (c_int, [c_vp, c_vp, c_vp, c_i64, c_f, c_f, c_vp]),
+    'kfac_momentum_batch_create': (c_int, [c_vp]),
+    'kfac_momentum_batch_destroy': (c_int, [c_vp]),
+    'kfac_momentum_update_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_f, c_f, c_f,
+                                                 c_vp]),
     'kfac_stream_copy_f32': (c_int, [c_vp, c_vp, c_i64, c_vp]),
     'kfac_timing_enable': (c_int, [c_int]),
     'kfac_timing_read': (c_int, [c_int, c_i64p, c_dp]),

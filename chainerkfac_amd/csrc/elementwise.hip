@@ -122,15 +122,101 @@ __global__ __launch_bounds__(kThreads) void add_diag_batched_kernel(const DiagIt
   }
 }
 
+// v = momentum * v - lr * g; p += v: the one expression of the single and of the
+// batched kernel (so that both round alike).
+__device__ __forceinline__ void momentum_step(float &p, float &v, float g, float lr, float momentum) {
+  const float nv = momentum * v - lr * g;
+  v = nv;
+  p += nv;
+}
+
 __global__ __launch_bounds__(kThreads) void momentum_kernel(
     float *__restrict__ p, float *__restrict__ v, const float *__restrict__ g,
     long long n, float lr, float momentum) {
   long long i = (long long)blockIdx.x * kThreads + threadIdx.x;
   const long long stride = (long long)gridDim.x * kThreads;
-  for (; i < n; i += stride) {
-    const float nv = momentum * v[i] - lr * g[i];
-    v[i] = nv;
-    p[i] += nv;
+  for (; i < n; i += stride) momentum_step(p[i], v[i], g[i], lr, momentum);
+}
+
+// The momentum rule of many parameters in one launch.  A unit is kMomentumUnit
+// consecutive elements of one parameter; `owner` gives a workgroup its entry
+// with one load.
+constexpr int kMomentumQuads = 2;                                // 16-byte accesses per thread
+constexpr int kMomentumUnit = kThreads * 4 * kMomentumQuads;     // elements per workgroup
+constexpr int kEntryGradF16 = 1, kEntryWriteBack = 2, kEntryAligned = 4;
+
+struct MomentumEntry {
+  float *param;               // float32 values that are updated (the master copy of a float16 parameter)
+  float *v;
+  void *grad;                 // float32, or float16 with kEntryGradF16
+  unsigned short *param_f16;  // float16 parameter that receives the rounded result, or null
+  long long n;
+  int unit0;                  // first unit of this entry
+  int flags;
+};
+
+typedef float floatx4a __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx4a __attribute__((ext_vector_type(4)));
+
+template <bool SCALE>
+__device__ __forceinline__ float scaled_grad(float g, float loss_scale) {
+  return SCALE ? g / loss_scale : g;   // an IEEE division, as the reference's in-place `/=`
+}
+
+template <bool SCALE>
+__global__ __launch_bounds__(kThreads) void momentum_batched_kernel(
+    const MomentumEntry *__restrict__ entries, const int *__restrict__ owner, float lr,
+    float momentum, float loss_scale) {
+  const MomentumEntry t = entries[owner[blockIdx.x]];
+  const long long base = (long long)((int)blockIdx.x - t.unit0) * kMomentumUnit;
+  const bool g16 = t.flags & kEntryGradF16;
+  const bool wb = SCALE && (t.flags & kEntryWriteBack) && !g16;
+#pragma unroll
+  for (int q = 0; q < kMomentumQuads; ++q) {
+    const long long i = base + ((long long)q * kThreads + threadIdx.x) * 4;
+    if (i >= t.n) continue;
+    if ((t.flags & kEntryAligned) && i + 4 <= t.n) {
+      floatx4a p = *reinterpret_cast<floatx4a *>(t.param + i);
+      floatx4a v = *reinterpret_cast<floatx4a *>(t.v + i);
+      floatx4a g;
+      if (g16) {
+        const halfx4a h = *reinterpret_cast<const halfx4a *>(static_cast<const _Float16 *>(t.grad) + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) g[e] = (float)h[e];
+      } else {
+        g = *reinterpret_cast<const floatx4a *>(static_cast<const float *>(t.grad) + i);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float ge = scaled_grad<SCALE>(g[e], loss_scale);
+        float pe = p[e], ve = v[e];
+        momentum_step(pe, ve, ge, lr, momentum);
+        g[e] = ge;
+        p[e] = pe;
+        v[e] = ve;
+      }
+      if (wb) *reinterpret_cast<floatx4a *>(static_cast<float *>(t.grad) + i) = g;
+      *reinterpret_cast<floatx4a *>(t.v + i) = v;
+      *reinterpret_cast<floatx4a *>(t.param + i) = p;
+      if (t.param_f16) {
+        halfx4a h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = (_Float16)p[e];
+        *reinterpret_cast<halfx4a *>(reinterpret_cast<_Float16 *>(t.param_f16) + i) = h;
+      }
+    } else {
+      const long long end = i + 4 < t.n ? i + 4 : t.n;
+      for (long long j = i; j < end; ++j) {
+        float g = g16 ? (float)static_cast<const _Float16 *>(t.grad)[j] : static_cast<const float *>(t.grad)[j];
+        g = scaled_grad<SCALE>(g, loss_scale);
+        float p = t.param[j], v = t.v[j];
+        momentum_step(p, v, g, lr, momentum);
+        if (wb) static_cast<float *>(t.grad)[j] = g;
+        t.v[j] = v;
+        t.param[j] = p;
+        if (t.param_f16) reinterpret_cast<_Float16 *>(t.param_f16)[j] = (_Float16)p;
+      }
+    }
   }
 }
 
@@ -215,6 +301,86 @@ extern "C" int kfac_momentum_update_f32(float *param, float *v, const float *gra
   hipLaunchKernelGGL(momentum_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0,
                      kfac::as_stream(stream), param, v, grad, (long long)nelems, lr,
                      momentum);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+struct kfac_momentum_batch {
+  std::vector<MomentumEntry> entries;
+  std::vector<int> owner;
+  kfac::DevTableRing entry_table, owner_table;
+};
+
+extern "C" int kfac_momentum_batch_create(kfac_momentum_batch_t *out) {
+  KFAC_REQUIRE(out != nullptr, "batch_out is null");
+  *out = new (std::nothrow) kfac_momentum_batch;
+  if (!*out) return kfac::fail(KFAC_ENOMEM, "out of host memory");
+  return KFAC_OK;
+}
+
+extern "C" int kfac_momentum_batch_destroy(kfac_momentum_batch_t batch) {
+  delete batch;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_momentum_update_batched_f32(kfac_momentum_batch_t batch, int count,
+                                                float *const *params, float *const *vs,
+                                                void *const *grads, const int64_t *nelems,
+                                                const int32_t *flags, void *const *params_f16,
+                                                float lr, float momentum, float loss_scale,
+                                                void *stream) {
+  KFAC_REQUIRE(batch != nullptr, "batch is null");
+  KFAC_REQUIRE(count >= 0, "count < 0");
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(params && vs && grads && nelems, "null table");
+  KFAC_REQUIRE(loss_scale == loss_scale && loss_scale != 0.f, "loss_scale must be a non-zero number (1 = none)");
+  batch->entries.clear();
+  batch->owner.clear();
+  long long units = 0;
+  for (int i = 0; i < count; ++i) {
+    KFAC_REQUIRE(nelems[i] >= 0, "parameter %d: nelems < 0", i);
+    if (nelems[i] == 0) continue;
+    KFAC_REQUIRE(params[i] && vs[i] && grads[i], "parameter %d: null pointer", i);
+    const int f = flags ? flags[i] : 0;
+    KFAC_REQUIRE((f & ~(KFAC_MOMENTUM_GRAD_F16 | KFAC_MOMENTUM_WRITE_BACK_GRAD)) == 0,
+                 "parameter %d: unknown flag bits %d", i, f);
+    MomentumEntry e;
+    memset(&e, 0, sizeof(e));   // the table is compared bytewise with the uploaded one
+    e.param = params[i];
+    e.v = vs[i];
+    e.grad = grads[i];
+    e.param_f16 = params_f16 ? static_cast<unsigned short *>(params_f16[i]) : nullptr;
+    e.n = nelems[i];
+    e.unit0 = (int)units;
+    e.flags = ((f & KFAC_MOMENTUM_GRAD_F16) ? kEntryGradF16 : 0) |
+              ((f & KFAC_MOMENTUM_WRITE_BACK_GRAD) ? kEntryWriteBack : 0);
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(e.param) | reinterpret_cast<uintptr_t>(e.v) |
+                           ((f & KFAC_MOMENTUM_GRAD_F16) ? 2 * reinterpret_cast<uintptr_t>(e.grad)
+                                                         : reinterpret_cast<uintptr_t>(e.grad)) |
+                           2 * reinterpret_cast<uintptr_t>(e.param_f16);
+    if (bits % 16 == 0) e.flags |= kEntryAligned;
+    const long long u = kfac::ceil_div<long long>(e.n, kMomentumUnit);
+    units += u;
+    KFAC_REQUIRE(units < 0x7fffffffLL, "too many elements");
+    batch->owner.insert(batch->owner.end(), (size_t)u, (int)batch->entries.size());
+    batch->entries.push_back(e);
+  }
+  if (units == 0) return KFAC_OK;
+  hipStream_t s = kfac::as_stream(stream);
+  const void *d_entries = nullptr, *d_owner = nullptr;
+  if (int rc = batch->entry_table.set(batch->entries.data(), sizeof(MomentumEntry) * batch->entries.size(), s,
+                                      &d_entries))
+    return rc;
+  if (int rc = batch->owner_table.set(batch->owner.data(), sizeof(int) * batch->owner.size(), s, &d_owner))
+    return rc;
+  if (loss_scale != 1.f)
+    hipLaunchKernelGGL(momentum_batched_kernel<true>, dim3((unsigned)units), dim3(kThreads), 0, s,
+                       static_cast<const MomentumEntry *>(d_entries), static_cast<const int *>(d_owner), lr,
+                       momentum, loss_scale);
+  else
+    hipLaunchKernelGGL(momentum_batched_kernel<false>, dim3((unsigned)units), dim3(kThreads), 0, s,
+                       static_cast<const MomentumEntry *>(d_entries), static_cast<const int *>(d_owner), lr,
+                       momentum, loss_scale);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }

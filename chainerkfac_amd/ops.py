@@ -602,3 +602,66 @@ def momentum_update(param, v, grad, lr, momentum, stream=None):
     _lib.check(_lib.load().kfac_momentum_update_f32(
         param.data_ptr(), v.data_ptr(), grad.data_ptr(), param.numel(), lr, momentum,
         _dev.stream_handle(stream)))
+
+
+class _MomentumBatch(object):
+    def __init__(self):
+        h = ctypes.c_void_p()
+        _lib.check(_lib.load().kfac_momentum_batch_create(ctypes.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        try:
+            h, self._h = self._h, None
+            if h is not None:
+                _lib._lib.kfac_momentum_batch_destroy(h)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+
+_momentum_batches = None
+
+
+def momentum_update_batched(params, vs, grads, lr, momentum, loss_scale=None, write_back=None,
+                            params_f16=None, stream=None):
+    """The momentum rule of a list of parameters in one launch (in place).
+
+    ``params`` and ``vs`` are float32; ``grads`` float32 or float16.  With a
+    ``loss_scale`` every gradient is divided by it first, and where
+    ``write_back[i]`` is true (float32 gradients only) the quotient replaces the
+    gradient.  ``params_f16[i]`` (or None) is a float16 array that receives the
+    rounded new values of ``params[i]``."""
+    global _momentum_batches
+    n = len(params)
+    if not (len(vs) == len(grads) == n):
+        raise ValueError('one velocity and one gradient per parameter')
+    if n == 0:
+        return
+    write_back = [False] * n if write_back is None else list(write_back)
+    params_f16 = [None] * n if params_f16 is None else list(params_f16)
+    if not (len(write_back) == len(params_f16) == n):
+        raise ValueError('one flag and one float16 array (or None) per parameter')
+    flags = []
+    for p, v, g, wb, h in zip(params, vs, grads, write_back, params_f16):
+        for t, nm in ((p, 'param'), (v, 'v')):
+            _dev.require_gpu_tensor(t, nm)
+        if g.dtype not in (torch.float32, torch.float16) or not g.is_cuda or not g.is_contiguous():
+            raise ValueError('grad must be a contiguous float32 or float16 GPU tensor')
+        if v.numel() != p.numel() or g.numel() != p.numel():
+            raise ValueError('param, v and grad differ in size')
+        if h is not None and (h.dtype != torch.float16 or not h.is_cuda or not h.is_contiguous()
+                              or h.numel() != p.numel()):
+            raise ValueError('params_f16 entries must be contiguous float16 GPU tensors of the parameter\'s size')
+        if wb and g.dtype != torch.float32:
+            raise ValueError('only a float32 gradient can receive the divided values')
+        flags.append((1 if g.dtype == torch.float16 else 0) | (2 if wb else 0))
+    if _momentum_batches is None:
+        _momentum_batches = _PlanCache(16)
+    key = (tuple(p.data_ptr() for p in params), tuple(g.data_ptr() for g in grads))
+    batch = _momentum_batches.get(key, _MomentumBatch)
+    _lib.check(_lib.load().kfac_momentum_update_batched_f32(
+        batch._h, n, _lib.ptr_array([p.data_ptr() for p in params]),
+        _lib.ptr_array([v.data_ptr() for v in vs]), _lib.ptr_array([g.data_ptr() for g in grads]),
+        _lib.i64_array([p.numel() for p in params]), _lib.i32_array(flags),
+        _lib.ptr_array([_dev.ptr(h) for h in params_f16]), lr, momentum,
+        1.0 if loss_scale is None else float(loss_scale), _dev.stream_handle(stream)))

@@ -165,6 +165,43 @@ class KFACUpdateRule(object):
                 param.grad /= param._loss_scale
         self.update_core(param)
 
+    def batched_job(self, param):
+        """What ``update`` would hand to the momentum kernel, for
+        ``ops.momentum_update_batched``: the rule's bookkeeping is done here
+        (step count, state, float32 master copy), the arithmetic -- division by
+        the loss scale, the rule, the float16 copy -- is left to the one launch
+        that takes all parameters.  Returns None when there is nothing to update,
+        or ``NotImplemented`` when the parameter has to go through ``update``
+        (arrays the batched kernel does not take)."""
+        import torch
+        if not self.enabled:
+            return None
+        grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
+        data = param.data
+        if grad is not None and not (
+                grad.is_cuda and grad.is_contiguous() and grad.dtype in (torch.float32, torch.float16)
+                and data.is_cuda and data.is_contiguous() and data.dtype in (torch.float32, torch.float16)
+                and (data.dtype == torch.float16 or grad.dtype == torch.float32)):
+            return NotImplemented
+        self.t += 1
+        if self.state is None:
+            self.init_state(param)
+        half = data.dtype == torch.float16
+        if half and self._fp32_param is None:
+            self._fp32_param = data.float()
+        if grad is None:
+            return None
+        lr = self.hyperparam.lr
+        lr_pre = self.hyperparam.lr_pre
+        momentum = self.hyperparam.momentum
+        if self.adjust_momentum and lr < lr_pre:
+            momentum *= lr / lr_pre
+        return {'param': self._fp32_param if half else data, 'v': self.state['v'], 'grad': grad,
+                'param_f16': data if half else None,
+                # the reference divides the float32 gradient in place (kfac.py:76-78) and a
+                # float16 parameter's through a float32 copy (kfac.py:69-75)
+                'write_back': not half, 'key': (float(lr), float(momentum), param._loss_scale)}
+
     def update_core(self, param, data=None, grad=None):
         if grad is None:
             grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
@@ -199,6 +236,10 @@ class KFAC(object):
     #: kernels are too small to fill the GPU alone); 0 keeps everything on the
     #: caller's stream.  Read at ``setup``.
     lanes = 3
+
+    #: apply the momentum rule of all parameters with one launch per set of
+    #: hyperparameters (normally one) instead of one launch per parameter
+    batch_param_updates = True
 
     def __init__(self, lr=_default_hyperparam.lr, momentum=_default_hyperparam.momentum,
                  cov_ema_decay=_default_hyperparam.cov_ema_decay,
@@ -368,13 +409,31 @@ class KFAC(object):
         self.update_kfgrads(self.fblocks)
 
         if not self.only_pic_update_weight:
-            for param in self.target.params():
-                param.update()
+            self.update_params()
 
         self.reallocate_cleared_grads()
         self.call_hooks('post')
         self.acc_aware_iterations += 1
         self.observation['acc_aware_iterations'] = self.acc_aware_iterations
+
+    def update_params(self):
+        """``param.update()`` for every parameter (reference kfac.py:250-252).  With
+        ``batch_param_updates`` the K-FAC rules that share their hyperparameters
+        run as one launch over all their parameters instead of one each."""
+        jobs = {}
+        for param in self.target.params():
+            rule = param.update_rule
+            job = NotImplemented
+            if self.batch_param_updates and type(rule) is KFACUpdateRule:
+                job = rule.batched_job(param)
+            if job is NotImplemented:
+                param.update()
+            elif job is not None:
+                jobs.setdefault(job['key'], []).append(job)
+        for (lr, momentum, loss_scale), group in jobs.items():
+            ops.momentum_update_batched(
+                [j['param'] for j in group], [j['v'] for j in group], [j['grad'] for j in group], lr, momentum,
+                loss_scale, [j['write_back'] for j in group], [j['param_f16'] for j in group])
 
     # ---- accumulation over acc_iters micro-batches -----------------------
     def accumulate(self):

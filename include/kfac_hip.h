@@ -352,6 +352,35 @@ int kfac_momentum_update_f32(float *param, float *v, const float *grad,
                              int64_t nelems, float lr, float momentum,
                              void *stream);
 
+/* The same rule for many parameters in one launch, with the loss-scale and
+ * float16 handling of KFACUpdateRule.update (optimizers/kfac.py:63-85) folded
+ * in.  For every element of parameter i:
+ *   g = grads[i][e] (float32, or float16 with KFAC_MOMENTUM_GRAD_F16);
+ *   if loss_scale != 1:  g = g / loss_scale (an IEEE division), and with
+ *     KFAC_MOMENTUM_WRITE_BACK_GRAD and a float32 gradient the quotient is
+ *     stored back (the reference divides `kfgrad` in place, kfac.py:76-78);
+ *   v = momentum*v - lr*g;  params[i][e] += v  (float32: the master copy of a
+ *     float16 parameter, kfac.py:64-68);
+ *   if params_f16 and params_f16[i]:  params_f16[i][e] = float16(params[i][e])
+ *     (what Chainer's use_fp32_update copies back into the parameter).
+ * lr and momentum are common to the call: parameters whose rules carry other
+ * hyperparameters go into a call of their own.  `flags` and `params_f16` may
+ * be null.  Arrays need no alignment (16-byte aligned ones are moved 16 bytes
+ * per lane).  The batch object keeps the device-side tables between calls and
+ * rewrites them only when the arguments change (a rewrite synchronises the
+ * stream, and is refused while the stream is being captured). */
+typedef struct kfac_momentum_batch *kfac_momentum_batch_t;
+#define KFAC_MOMENTUM_GRAD_F16 1
+#define KFAC_MOMENTUM_WRITE_BACK_GRAD 2
+int kfac_momentum_batch_create(kfac_momentum_batch_t *batch_out);
+int kfac_momentum_batch_destroy(kfac_momentum_batch_t batch);
+int kfac_momentum_update_batched_f32(kfac_momentum_batch_t batch, int count,
+                                     float *const *params, float *const *vs,
+                                     void *const *grads, const int64_t *nelems,
+                                     const int32_t *flags, void *const *params_f16,
+                                     float lr, float momentum, float loss_scale,
+                                     void *stream);
+
 /* ------------------------------------------------------------------------
  * Per-kernel timing for benchmarks (no counterpart in the reference, which
  * has no instrumentation).  While enabled, every launch of the kernel

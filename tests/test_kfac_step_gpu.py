@@ -394,6 +394,49 @@ def test_plain_gradient_path_divides_by_loss_scale():
     assert rel(b.fc.W.data.cpu().numpy(), a.fc.W.data.cpu().numpy()) < 1e-4
 
 
+@pytest.mark.parametrize('loss_scale', [None, 64.0])
+def test_batched_parameter_updates_match_the_per_parameter_rule(loss_scale):
+    """KFAC.batch_param_updates: one momentum launch over all parameters leaves the same
+    parameters, velocities, (divided) gradients and step counts as one rule call per
+    parameter (momentum and lr_pre exercised over three steps, adjust_momentum on)."""
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import KFAC
+
+    def lossfun(m, x, t):
+        return TF.cross_entropy(m(x), t)
+
+    nets = []
+    for batched in (True, False):
+        gen = torch.Generator(device='cpu').manual_seed(7)
+        src = build_cnn(L, 'cpu', gen)
+        model = build_cnn(L, 'cuda', None)
+        copy_params(src, model)
+        opt = KFAC(lr=1e-2, momentum=0.9, cov_ema_decay=0.9, damping=1e-2, loss_scale=loss_scale,
+                   adjust_momentum=True).setup(model)
+        opt.batch_param_updates = batched
+        for step, (x, t) in enumerate(cnn_batches(3)):
+            if step == 2:
+                opt.hyperparam.lr_pre, opt.hyperparam.lr = opt.hyperparam.lr, 0.5 * opt.hyperparam.lr
+            opt.update(lossfun, model, torch.from_numpy(x).cuda(), torch.from_numpy(t).cuda())
+        torch.cuda.synchronize()
+        nets.append(model)
+    a, b = nets
+    pb = dict(b.namedparams())
+    # (two runs of the same configuration already differ in the last bits: the backward pass
+    # of the network is not run-to-run deterministic; that the two kernels round alike is
+    # tested on fixed arrays in test_precond_gpu.py)
+    for name, p in a.namedparams():
+        q = pb[name]
+        assert rel(p.data.cpu().numpy(), q.data.cpu().numpy()) < 1e-3, name
+        assert rel(p.update_rule.state['v'].cpu().numpy(), q.update_rule.state['v'].cpu().numpy()) < 1e-3, name
+        assert p.update_rule.t == q.update_rule.t == 3
+        for attr in ('grad', 'kfgrad'):
+            ga, gb = getattr(p, attr, None), getattr(q, attr, None)
+            assert (ga is None) == (gb is None)
+            if ga is not None and name != '/conv1/b':   # (a zero gradient up to rounding noise)
+                assert rel(ga.cpu().numpy(), gb.cpu().numpy()) < 1e-3, (name, attr)
+
+
 def test_side_streams_do_not_change_results(monkeypatch):
     """The per-layer kernels dealt onto side streams are the same launches on the
     same data: factors, inverses and preconditioned gradients are bit-identical to
@@ -578,8 +621,11 @@ def test_float16_activations_and_gradients_are_cast_up():
     assert (got - full).norm() <= 2e-3 * full.norm()
 
 
-def test_float16_parameter_is_updated_through_a_float32_master_copy():
-    """reference kfac.py:64-85: the update runs on a float32 copy; the float16 parameter follows."""
+@pytest.mark.parametrize('batched', [False, True])
+def test_float16_parameter_is_updated_through_a_float32_master_copy(batched):
+    """reference kfac.py:64-85: the update runs on a float32 copy; the float16 parameter follows.
+    ``batched``: through the rule's job for the one launch that takes all parameters."""
+    from chainerkfac_amd import ops
     from chainerkfac_amd.optimizers.kfac import KFACUpdateRule, Hyperparameter
 
     class P(object):
@@ -598,7 +644,15 @@ def test_float16_parameter_is_updated_through_a_float32_master_copy():
     for _ in range(3):
         p.kfgrad = (torch.randn(257, device='cuda', generator=g) * 8.0).half()
         kf = p.kfgrad.double() / 8.0
-        rule.update(p)
+        kf16 = p.kfgrad.clone()
+        if batched:
+            job = rule.batched_job(p)
+            lr, momentum, loss_scale = job['key']
+            ops.momentum_update_batched([job['param']], [job['v']], [job['grad']], lr, momentum, loss_scale,
+                                        [job['write_back']], [job['param_f16']])
+        else:
+            rule.update(p)
+        assert torch.equal(p.kfgrad, kf16)   # divided in a float32 copy, not in place
         v = 0.9 * v - 0.01 * kf
         master = master + v
         assert p.data.dtype == torch.float16

@@ -120,6 +120,62 @@ def test_axpby_and_momentum_update():
     np.testing.assert_allclose(pd.cpu().numpy(), p, rtol=1e-6, atol=1e-7)
 
 
+@pytest.mark.parametrize('loss_scale', [None, 128.0, 3.0])
+def test_momentum_update_batched(loss_scale):
+    """One launch for the rule of many parameters (optimizers/kfac.py:63-116): ragged sizes
+    around the unit size, empty arrays, arrays that start off a 16-byte boundary, float16
+    gradients and float16 parameters behind a float32 master copy, with and without a loss
+    scale.  Against the oracle's rule on the divided gradients, bit-exact against the
+    single-parameter kernel, and the divided gradient is stored where it is asked for."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(11)
+    sizes = [0, 1, 5, 2047, 2048, 2049, 100003, 3 * 4096, 777, 6144]
+    lr, momentum = 0.05, 0.9
+    params, vs, grads, wbs, halves, expect = [], [], [], [], [], []
+    for k, n in enumerate(sizes):
+        off = k % 3   # views that start 0, 4 or 8 bytes past an aligned address
+        p = torch.from_numpy(r.standard_normal(n + 3).astype(np.float32)).cuda()[off:off + n]
+        v = torch.from_numpy(r.standard_normal(n + 3).astype(np.float32)).cuda()[off:off + n]
+        g16 = k % 4 == 1
+        g = torch.from_numpy(r.standard_normal(n + 3).astype(np.float16 if g16 else np.float32)).cuda()[off:off + n]
+        h = torch.zeros(n + 3, dtype=torch.float16, device='cuda')[off:off + n] if k % 4 in (1, 2) else None
+        wb = (not g16) and k % 2 == 0
+        pe, ve, ge = p.cpu().numpy().copy(), v.cpu().numpy().copy(), g.cpu().numpy().astype(np.float32)
+        if loss_scale is not None:
+            ge = ge / np.float32(loss_scale)
+        single = None
+        if n:
+            # the single-parameter kernel on copies (divided by a device scalar: a true division)
+            ps, vs1 = p.clone(), v.clone()
+            gs = g.float() if loss_scale is None else g.float() / torch.tensor(loss_scale, device='cuda')
+            ops.momentum_update(ps, vs1, gs.contiguous(), lr, momentum)
+            single = (ps, vs1)
+        O.momentum_update(pe, ve, ge, lr, momentum)
+        params.append(p); vs.append(v); grads.append(g); wbs.append(wb); halves.append(h)
+        expect.append((pe, ve, ge, single, g.clone()))
+    ops.momentum_update_batched(params, vs, grads, lr, momentum, loss_scale, wbs, halves)
+    torch.cuda.synchronize()
+    for p, v, g, wb, h, (pe, ve, ge, single, g0) in zip(params, vs, grads, wbs, halves, expect):
+        np.testing.assert_allclose(v.cpu().numpy(), ve, rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(p.cpu().numpy(), pe, rtol=1e-6, atol=1e-6)
+        if single is not None:
+            assert torch.equal(p, single[0]) and torch.equal(v, single[1])
+        if wb and loss_scale is not None:
+            assert np.array_equal(g.cpu().numpy(), ge)
+        else:
+            assert torch.equal(g, g0)
+        if h is not None:
+            assert torch.equal(h, p.half())
+    # the same call again goes through the cached tables; a changed list rewrites them
+    ops.momentum_update_batched(params, vs, grads, lr, momentum, loss_scale, wbs, halves)
+    ops.momentum_update_batched(params[3:6], vs[3:6], grads[3:6], lr, momentum)
+    torch.cuda.synchronize()
+    with pytest.raises(ValueError):
+        ops.momentum_update_batched(params[:2], vs[:1], grads[:2], lr, momentum)
+    with pytest.raises(ValueError):
+        ops.momentum_update_batched([params[1]], [vs[1]], [grads[1]], lr, momentum, 2.0, [True])
+
+
 def test_grouped_preconditioning_matches_the_single_calls():
     """All layers' products in one grouped call: 64- and 128-tiles, with and without bias,
     aligned and odd dimensions, several k-slices; against float64 and the single calls."""
