@@ -340,6 +340,27 @@ def run_step_config(args, name, cfg):
     n_param_arrays = len(list(model.params()))
     n_params = sum(p.data.numel() for p in model.params())
 
+    # the moving average of all factors in a step that has history (cov_ema_decay = 0.99, the
+    # reference's default; the first step, which `value` times for c3 - c5, only aliases)
+    for fb in opt.fblocks:
+        fb.cov_ema_decay, fb.cov_emas = 0.99, None
+
+    def ema_phase():
+        opt.update_cov_emas(opt.fblocks)
+
+    ema_phase()   # the first call copies
+    ema_ms = {}
+    for label, batched in (('batched', True), ('per_array', False)):
+        opt.batch_elementwise = batched
+        ema_phase()
+        ema_ms[label] = timed(ema_phase if args.no_graph else capture(ema_phase))
+    opt.batch_elementwise = True
+    n_factor_arrays = sum(len(fb.covs) for fb in opt.fblocks)
+    n_factor_elems = sum(c.numel() for fb in opt.fblocks for c in fb.covs)
+    for fb in opt.fblocks:
+        fb.cov_ema_decay, fb.cov_emas = cfg['decay'], None
+    inv_phase()   # back to this configuration's own averages and inverses
+
     # dominant kernel family, timed launch by launch inside the library (one stream: with lanes,
     # launches overlap and the time between a launch's events is shared with others)
     opt._lanes.n = 0
@@ -411,6 +432,13 @@ def run_step_config(args, name, cfg):
                          'one_launch_tb_s': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12, 3),
                          'frac_of_hbm_peak': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
                          'in_value': False},
+        # ema = 0.99 cov + 0.01 ema over every factor: 12 bytes per element
+        'moving_average': {'elements': n_factor_elems, 'arrays': n_factor_arrays,
+                           'one_launch_ms': round(ema_ms['batched'], 4),
+                           'launch_per_array_ms': round(ema_ms['per_array'], 4),
+                           'one_launch_tb_s': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12, 3),
+                           'frac_of_hbm_peak': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
+                           'in_value': False},
         'roofline': {
             'kernel': 'covariance SYRK family (shift::corr_kernel, syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
             'bound': 'mfma',

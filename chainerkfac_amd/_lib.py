@@ -46,6 +46,9 @@ PROTOTYPES = {
     'kfac_bn_grad_matrix_f32': (c_int, [c_vp, c_vp, c_int, c_int, c_int, c_f, c_f, c_int, c_int,
                                         c_vp, c_vp, c_sz, c_vp]),
     'kfac_axpby_f32': (c_int, [c_vp, c_vp, c_i64, c_f, c_f, c_vp]),
+    'kfac_axpby_batch_create': (c_int, [c_vp]),
+    'kfac_axpby_batch_destroy': (c_int, [c_vp]),
+    'kfac_axpby_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_vp, c_f, c_f, c_vp]),
     'kfac_inverse_plan_create': (c_int, [c_int, c_i32p, c_vpp]),
     'kfac_inverse_plan_workspace_bytes': (c_sz, [c_vp]),
     'kfac_inverse_plan_destroy': (c_int, [c_vp]),

@@ -85,6 +85,10 @@ namespace {
 
 constexpr int kThreads = 256;
 
+// a x + b y: the one expression of the single and of the batched kernel (so that
+// both round alike)
+__device__ __forceinline__ float axpby_value(float x, float y, float a, float b) { return a * x + b * y; }
+
 __global__ __launch_bounds__(kThreads) void axpby_kernel(
     const float *__restrict__ x, float *__restrict__ y, long long n, float a, float b) {
   long long i = (long long)blockIdx.x * kThreads + threadIdx.x;
@@ -93,7 +97,48 @@ __global__ __launch_bounds__(kThreads) void axpby_kernel(
   if (b == 0.f) {
     for (; i < n; i += stride) y[i] = a * x[i];
   } else {
-    for (; i < n; i += stride) y[i] = a * x[i] + b * y[i];
+    for (; i < n; i += stride) y[i] = axpby_value(x[i], y[i], a, b);
+  }
+}
+
+// Work of the batched elementwise kernels: a unit is kBatchUnit consecutive
+// elements of one array pair; `owner` gives a workgroup its entry with one load.
+constexpr int kBatchQuads = 2;                             // 16-byte accesses per thread
+constexpr int kBatchUnit = kThreads * 4 * kBatchQuads;     // elements per workgroup
+typedef float floatx4a __attribute__((ext_vector_type(4)));
+
+struct AxpbyEntry {
+  const float *x;
+  float *y;
+  long long n;
+  int unit0;     // first unit of this entry
+  int aligned;   // both arrays start on 16-byte boundaries
+};
+
+template <bool OVERWRITE>
+__global__ __launch_bounds__(kThreads) void axpby_batched_kernel(
+    const AxpbyEntry *__restrict__ entries, const int *__restrict__ owner, float a, float b) {
+  const AxpbyEntry t = entries[owner[blockIdx.x]];
+  const long long base = (long long)((int)blockIdx.x - t.unit0) * kBatchUnit;
+#pragma unroll
+  for (int q = 0; q < kBatchQuads; ++q) {
+    const long long i = base + ((long long)q * kThreads + threadIdx.x) * 4;
+    if (i >= t.n) continue;
+    if (t.aligned && i + 4 <= t.n) {
+      const floatx4a x = *reinterpret_cast<const floatx4a *>(t.x + i);
+      floatx4a y;
+      if (OVERWRITE) {
+        y = a * x;
+      } else {
+        y = *reinterpret_cast<const floatx4a *>(t.y + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = axpby_value(x[e], y[e], a, b);
+      }
+      *reinterpret_cast<floatx4a *>(t.y + i) = y;
+    } else {
+      const long long end = i + 4 < t.n ? i + 4 : t.n;
+      for (long long j = i; j < end; ++j) t.y[j] = OVERWRITE ? a * t.x[j] : axpby_value(t.x[j], t.y[j], a, b);
+    }
   }
 }
 
@@ -141,8 +186,8 @@ __global__ __launch_bounds__(kThreads) void momentum_kernel(
 // The momentum rule of many parameters in one launch.  A unit is kMomentumUnit
 // consecutive elements of one parameter; `owner` gives a workgroup its entry
 // with one load.
-constexpr int kMomentumQuads = 2;                                // 16-byte accesses per thread
-constexpr int kMomentumUnit = kThreads * 4 * kMomentumQuads;     // elements per workgroup
+constexpr int kMomentumQuads = kBatchQuads;
+constexpr int kMomentumUnit = kBatchUnit;
 constexpr int kEntryGradF16 = 1, kEntryWriteBack = 2, kEntryAligned = 4;
 
 struct MomentumEntry {
@@ -155,7 +200,6 @@ struct MomentumEntry {
   int flags;
 };
 
-typedef float floatx4a __attribute__((ext_vector_type(4)));
 typedef _Float16 halfx4a __attribute__((ext_vector_type(4)));
 
 template <bool SCALE>
@@ -381,6 +425,69 @@ extern "C" int kfac_momentum_update_batched_f32(kfac_momentum_batch_t batch, int
     hipLaunchKernelGGL(momentum_batched_kernel<false>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const MomentumEntry *>(d_entries), static_cast<const int *>(d_owner), lr,
                        momentum, loss_scale);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+struct kfac_axpby_batch {
+  std::vector<AxpbyEntry> entries;
+  std::vector<int> owner;
+  kfac::DevTableRing entry_table, owner_table;
+};
+
+extern "C" int kfac_axpby_batch_create(kfac_axpby_batch_t *out) {
+  KFAC_REQUIRE(out != nullptr, "batch_out is null");
+  *out = new (std::nothrow) kfac_axpby_batch;
+  if (!*out) return kfac::fail(KFAC_ENOMEM, "out of host memory");
+  return KFAC_OK;
+}
+
+extern "C" int kfac_axpby_batch_destroy(kfac_axpby_batch_t batch) {
+  delete batch;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_axpby_batched_f32(kfac_axpby_batch_t batch, int count, const float *const *xs,
+                                      float *const *ys, const int64_t *nelems, float a, float b,
+                                      void *stream) {
+  KFAC_REQUIRE(batch != nullptr, "batch is null");
+  KFAC_REQUIRE(count >= 0, "count < 0");
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(xs && ys && nelems, "null table");
+  batch->entries.clear();
+  batch->owner.clear();
+  long long units = 0;
+  for (int i = 0; i < count; ++i) {
+    KFAC_REQUIRE(nelems[i] >= 0, "pair %d: nelems < 0", i);
+    if (nelems[i] == 0) continue;
+    KFAC_REQUIRE(xs[i] && ys[i], "pair %d: null pointer", i);
+    AxpbyEntry e;
+    memset(&e, 0, sizeof(e));   // the table is compared bytewise with the uploaded one
+    e.x = xs[i];
+    e.y = ys[i];
+    e.n = nelems[i];
+    e.unit0 = (int)units;
+    e.aligned = (reinterpret_cast<uintptr_t>(e.x) | reinterpret_cast<uintptr_t>(e.y)) % 16 == 0;
+    const long long u = kfac::ceil_div<long long>(e.n, kBatchUnit);
+    units += u;
+    KFAC_REQUIRE(units < 0x7fffffffLL, "too many elements");
+    batch->owner.insert(batch->owner.end(), (size_t)u, (int)batch->entries.size());
+    batch->entries.push_back(e);
+  }
+  if (units == 0) return KFAC_OK;
+  hipStream_t s = kfac::as_stream(stream);
+  const void *d_entries = nullptr, *d_owner = nullptr;
+  if (int rc = batch->entry_table.set(batch->entries.data(), sizeof(AxpbyEntry) * batch->entries.size(), s,
+                                      &d_entries))
+    return rc;
+  if (int rc = batch->owner_table.set(batch->owner.data(), sizeof(int) * batch->owner.size(), s, &d_owner))
+    return rc;
+  if (b == 0.f)
+    hipLaunchKernelGGL(axpby_batched_kernel<true>, dim3((unsigned)units), dim3(kThreads), 0, s,
+                       static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
+  else
+    hipLaunchKernelGGL(axpby_batched_kernel<false>, dim3((unsigned)units), dim3(kThreads), 0, s,
+                       static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }

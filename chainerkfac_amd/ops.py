@@ -220,6 +220,46 @@ def axpby(x, y, a, b, stream=None):
     return y
 
 
+class _AxpbyBatch(object):
+    def __init__(self):
+        h = ctypes.c_void_p()
+        _lib.check(_lib.load().kfac_axpby_batch_create(ctypes.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        try:
+            h, self._h = self._h, None
+            if h is not None:
+                _lib._lib.kfac_axpby_batch_destroy(h)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+
+_axpby_batches = None
+
+
+def axpby_batched(xs, ys, a, b, stream=None):
+    """ys[i] = a*xs[i] + b*ys[i] for a list of array pairs in one launch (in place)."""
+    global _axpby_batches
+    if len(xs) != len(ys):
+        raise ValueError('one y per x')
+    if not xs:
+        return ys
+    for x, y in zip(xs, ys):
+        _dev.require_gpu_tensor(x, 'x')
+        _dev.require_gpu_tensor(y, 'y')
+        if x.numel() != y.numel():
+            raise ValueError('size mismatch')
+    if _axpby_batches is None:
+        _axpby_batches = _PlanCache(16)
+    key = (tuple(x.data_ptr() for x in xs), tuple(y.data_ptr() for y in ys))
+    batch = _axpby_batches.get(key, _AxpbyBatch)
+    _lib.check(_lib.load().kfac_axpby_batched_f32(
+        batch._h, len(xs), _lib.ptr_array(key[0]), _lib.ptr_array(key[1]),
+        _lib.i64_array([x.numel() for x in xs]), a, b, _dev.stream_handle(stream)))
+    return ys
+
+
 def add_diag(M, v0, v1=None, split=None, stream=None):
     """diag(M)[i] += v0 for i < split else v1 (float64 sum, float32 store)."""
     _dev.require_gpu_tensor(M, 'M')

@@ -181,8 +181,17 @@ class FisherBlock(object):
                 ema.copy_(cov)
                 self.cov_emas.append(ema)
         else:
-            for cov, cov_ema in zip(self.covs, self.cov_emas):
+            for cov, cov_ema in self.cov_ema_pairs():
                 ops.axpby(cov, cov_ema, r, 1 - r)
+
+    def cov_ema_pairs(self):
+        """The (covariance, moving average) pairs of a step that does average
+        (not the first one, decay != 1), else None: what ``KFAC.update_cov_emas``
+        hands to one launch for all blocks."""
+        if self.cov_ema_decay == 1.0 or self.cov_emas is None:
+            return None
+        self.check_attr('covs')
+        return list(zip(self.covs, self.cov_emas))
 
     # ---- damping + inverse ------------------------------------------------
     def _inv_buffers(self):

@@ -109,6 +109,12 @@ class FisherBlockBatchNormalization(FisherBlock):
         super(FisherBlockBatchNormalization, self).update_cov_emas()
         self._ema_is_single_factor = first or self.cov_ema_decay == 1.0
 
+    def cov_ema_pairs(self):
+        pairs = super(FisherBlockBatchNormalization, self).cov_ema_pairs()
+        if pairs is not None:
+            self._ema_is_single_factor = False   # the average now has history
+        return pairs
+
     def lowrank_inverse_args(self):
         """``(U, split, d_gamma, d_beta)`` when the damped moving average is exactly
         ``U^T U / n + diag(d_gamma | d_beta)`` with U this step's per-sample

@@ -241,6 +241,10 @@ class KFAC(object):
     #: hyperparameters (normally one) instead of one launch per parameter
     batch_param_updates = True
 
+    #: moving averages of all factors and the gradient accumulation of all
+    #: parameters as one launch each instead of one per array
+    batch_elementwise = True
+
     def __init__(self, lr=_default_hyperparam.lr, momentum=_default_hyperparam.momentum,
                  cov_ema_decay=_default_hyperparam.cov_ema_decay,
                  damping=_default_hyperparam.damping, stab_coeff=16.0,
@@ -458,7 +462,9 @@ class KFAC(object):
             self.acc_count, self.acc_iters))
 
     def accumulate_grads(self):
-        """acc_grad += grad / acc_iters for every parameter."""
+        """acc_grad += grad / acc_iters for every parameter (one launch for those
+        that start their sum, one for those that continue it)."""
+        first, later = [], []
         for param in self.target.params():
             if param.grad is None:
                 continue
@@ -467,9 +473,15 @@ class KFAC(object):
                 if buf is None or buf.shape != param.grad.shape:
                     buf = param._acc_grad_buf = param.grad.new_empty(param.grad.shape)
                 param.acc_grad = buf
-                ops.axpby(param.grad.contiguous(), buf, 1 / self.acc_iters, 0.0)
+                first.append((param.grad.contiguous(), buf))
             else:
-                ops.axpby(param.grad.contiguous(), param.acc_grad, 1 / self.acc_iters, 1.0)
+                later.append((param.grad.contiguous(), param.acc_grad))
+        for pairs, b in ((first, 0.0), (later, 1.0)):
+            if self.batch_elementwise:
+                ops.axpby_batched([x for x, _ in pairs], [y for _, y in pairs], 1 / self.acc_iters, b)
+            else:
+                for x, y in pairs:
+                    ops.axpby(x, y, 1 / self.acc_iters, b)
 
     def accumulate_covs(self):
         """The covariance kernels already added this micro-batch's factors, scaled
@@ -485,9 +497,18 @@ class KFAC(object):
         self.precondition(fblocks)
 
     def update_cov_emas(self, fblocks):
+        """``fblock.update_cov_emas()`` for every block (reference kfac.py:306-308); the
+        moving averages of the blocks that share a decay run as one launch."""
         self.finish_covs()   # factors computed by the hooks
+        averaging = {}
         for fblock in fblocks:
-            fblock.update_cov_emas()
+            pairs = fblock.cov_ema_pairs() if self.batch_elementwise else None
+            if pairs is None:
+                fblock.update_cov_emas()
+            else:
+                averaging.setdefault(fblock.cov_ema_decay, []).extend(pairs)
+        for r, pairs in averaging.items():
+            ops.axpby_batched([c for c, _ in pairs], [e for _, e in pairs], r, 1 - r)
 
     #: run the preconditioning products of all connection blocks as one grouped call
     #: (a few launches for the whole network); False calls every block's

@@ -183,6 +183,21 @@ int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, int c,
 int kfac_axpby_f32(const float *x, float *y, int64_t nelems, float a, float b,
                    void *stream);
 
+/* The same for `count` pairs of arrays in one launch (one a and b for all):
+ * the moving average of every factor of the network
+ * (`for fblock in fblocks: fblock.update_cov_emas()`, kfac.py:306-308 over
+ * fisher_block.py:155-163) or `accumulate_grads` over all parameters
+ * (kfac.py:286-294).  Arrays need no alignment.  The batch object keeps the
+ * device-side tables between calls and rewrites them only when the arguments
+ * change (a rewrite synchronises the stream, and is refused while the stream
+ * is being captured). */
+typedef struct kfac_axpby_batch *kfac_axpby_batch_t;
+int kfac_axpby_batch_create(kfac_axpby_batch_t *batch_out);
+int kfac_axpby_batch_destroy(kfac_axpby_batch_t batch);
+int kfac_axpby_batched_f32(kfac_axpby_batch_t batch, int count,
+                           const float *const *xs, float *const *ys,
+                           const int64_t *nelems, float a, float b, void *stream);
+
 /* ------------------------------------------------------------------------
  * (2) Damping and the damped inverse
  * --------------------------------------------------------------------- */

@@ -396,7 +396,8 @@ def test_plain_gradient_path_divides_by_loss_scale():
 
 @pytest.mark.parametrize('loss_scale', [None, 64.0])
 def test_batched_parameter_updates_match_the_per_parameter_rule(loss_scale):
-    """KFAC.batch_param_updates: one momentum launch over all parameters leaves the same
+    """KFAC.batch_param_updates and batch_elementwise: one momentum launch over all parameters
+    (and one moving-average launch over all factors) leaves the same
     parameters, velocities, (divided) gradients and step counts as one rule call per
     parameter (momentum and lr_pre exercised over three steps, adjust_momentum on)."""
     from chainerkfac_amd import links as L
@@ -413,7 +414,7 @@ def test_batched_parameter_updates_match_the_per_parameter_rule(loss_scale):
         copy_params(src, model)
         opt = KFAC(lr=1e-2, momentum=0.9, cov_ema_decay=0.9, damping=1e-2, loss_scale=loss_scale,
                    adjust_momentum=True).setup(model)
-        opt.batch_param_updates = batched
+        opt.batch_param_updates = opt.batch_elementwise = batched
         for step, (x, t) in enumerate(cnn_batches(3)):
             if step == 2:
                 opt.hyperparam.lr_pre, opt.hyperparam.lr = opt.hyperparam.lr, 0.5 * opt.hyperparam.lr

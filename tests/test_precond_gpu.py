@@ -120,6 +120,38 @@ def test_axpby_and_momentum_update():
     np.testing.assert_allclose(pd.cpu().numpy(), p, rtol=1e-6, atol=1e-7)
 
 
+def test_axpby_batched():
+    """y = a x + b y for many array pairs in one launch: ragged sizes around the unit size,
+    empty arrays, arrays that start off a 16-byte boundary; bit-exact against the single-pair
+    kernel, and b == 0 overwrites without reading y."""
+    from chainerkfac_amd import ops
+    r = np.random.default_rng(5)
+    sizes = [0, 1, 7, 2047, 2048, 2049, 100003, 3 * 4096, 65 * 65, 4609]
+    xs, ys, singles = [], [], []
+    for k, n in enumerate(sizes):
+        off = k % 3
+        x = torch.from_numpy(r.standard_normal(n + 3).astype(np.float32)).cuda()[off:off + n]
+        yoff = (off + (k // 3) % 2) % 3   # both aligned, one aligned, none aligned
+        y = torch.from_numpy(r.standard_normal(n + 3).astype(np.float32)).cuda()[yoff:yoff + n]
+        xs.append(x); ys.append(y)
+        singles.append(ops.axpby(x.contiguous(), y.clone(), 0.99, 0.01) if n else y.clone())
+    expect = [np.float32(0.99) * x.cpu().numpy() + np.float32(0.01) * y.cpu().numpy() for x, y in zip(xs, ys)]
+    ops.axpby_batched(xs, ys, 0.99, 0.01)
+    torch.cuda.synchronize()
+    for y, single, e in zip(ys, singles, expect):
+        assert torch.equal(y, single)
+        np.testing.assert_allclose(y.cpu().numpy(), e, rtol=1e-6, atol=1e-7)
+    nans = [torch.full_like(y, float('nan')) for y in ys]
+    ops.axpby_batched(xs, nans, 0.5, 0.0)
+    torch.cuda.synchronize()
+    for x, y in zip(xs, nans):
+        assert np.array_equal(y.cpu().numpy(), np.float32(0.5) * x.cpu().numpy())
+    with pytest.raises(ValueError):
+        ops.axpby_batched(xs[:2], ys[:1], 1.0, 1.0)
+    with pytest.raises(ValueError):
+        ops.axpby_batched([xs[2]], [ys[3]], 1.0, 1.0)
+
+
 @pytest.mark.parametrize('loss_scale', [None, 128.0, 3.0])
 def test_momentum_update_batched(loss_scale):
     """One launch for the rule of many parameters (optimizers/kfac.py:63-116): ragged sizes
