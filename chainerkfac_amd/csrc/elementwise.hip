@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kThreads) void axpby_kernel(
 
 // Work of the batched elementwise kernels: a unit is kBatchUnit consecutive
 // elements of one array pair; `owner` gives a workgroup its entry with one load.
-constexpr int kBatchQuads = 2;                             // 16-byte accesses per thread
+constexpr int kBatchQuads = 1;                             // 16-byte accesses per thread
 constexpr int kBatchUnit = kThreads * 4 * kBatchQuads;     // elements per workgroup
 typedef float floatx4a __attribute__((ext_vector_type(4)));
 
