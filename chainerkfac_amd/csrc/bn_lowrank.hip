@@ -38,6 +38,7 @@ constexpr int NMAX = kfac::kChol32;   // largest batch size
 constexpr int CHUNK = 128;            // columns per gram / apply workgroup
 constexpr int SLS = NMAX + 1;         // LDS row stride of the n x n matrix
 constexpr int TILE = 64;              // output tile of the outer product
+typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 struct LrTables {
   const float *const *U;    // [count] (n x w), row-major
@@ -48,6 +49,7 @@ struct LrTables {
   const float *db;          // [count]
   const int *chunk_cs;      // [count+1] cumulative chunk counts
   const int *tile_cs;       // [count+1] cumulative tile counts (tiles per side squared)
+  const int *tile_owner;    // [tiles] block of every output tile (one load instead of a search)
   const long long *v_off;   // [count] float offset of V in the workspace
   double *part;             // [chunks][NMAX*NMAX]
   double *winv;             // [count][NMAX*NMAX]  U32 = (L^-1)^T
@@ -98,28 +100,41 @@ __global__ __launch_bounds__(256) void lr_gram_kernel(LrTables tb, int count, in
   }
 }
 
-// One wave per block: S, its Cholesky factor and winv = (L^-1)^T.
-__global__ __launch_bounds__(64) void lr_factor_kernel(LrTables tb) {
+// One workgroup per block: S (all waves sum the chunks' partial Gram matrices,
+// several loads in flight per thread), its Cholesky factor (wave 0) and
+// winv = (L^-1)^T.
+constexpr int kFactorThreads = 256;
+__global__ __launch_bounds__(kFactorThreads) void lr_factor_kernel(LrTables tb) {
   __shared__ double S[NMAX * SLS];
   const int l = blockIdx.x;
-  const int lane = threadIdx.x;
   const int c_lo = tb.chunk_cs[l], c_hi = tb.chunk_cs[l + 1];
 #pragma unroll
-  for (int q = 0; q < NMAX * NMAX / 64; ++q) {
-    const int e = lane + 64 * q;
+  for (int q = 0; q < NMAX * NMAX / kFactorThreads; ++q) {
+    const int e = threadIdx.x + kFactorThreads * q;
     const int a = e / NMAX, b = e % NMAX;
+    const double *__restrict__ src = tb.part + (long long)c_lo * (NMAX * NMAX) + e;
+    // in chunk order, whatever the unrolling: the sum does not depend on it
     double acc = a == b ? 1.0 : 0.0;
-    for (int c = c_lo; c < c_hi; ++c) acc += tb.part[(long long)c * (NMAX * NMAX) + e];
+    int c = c_lo;
+    for (; c + 8 <= c_hi; c += 8, src += 8 * NMAX * NMAX) {
+      double v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(long long)u * (NMAX * NMAX)];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; c < c_hi; ++c, src += NMAX * NMAX) acc += *src;
     S[a * SLS + b] = acc;
   }
   __syncthreads();
-  const int bad = kfac::chol_inv_32<SLS>(S, 0);
+  int bad = 0;
+  if (threadIdx.x < 64) bad = kfac::chol_inv_32<SLS>(S, 0);
   __syncthreads();
-  if (lane == 0) tb.info[l] = bad;
+  if (threadIdx.x == 0) tb.info[l] = bad;
   double *__restrict__ dst = tb.winv + (long long)l * (NMAX * NMAX);
 #pragma unroll
-  for (int q = 0; q < NMAX * NMAX / 64; ++q) {
-    const int e = lane + 64 * q;
+  for (int q = 0; q < NMAX * NMAX / kFactorThreads; ++q) {
+    const int e = threadIdx.x + kFactorThreads * q;
     const int m = e / NMAX, r = e % NMAX;
     dst[e] = r >= m ? S[m * SLS + r] : 0.0;   // winv[m][r] = (L^-1)[r][m]
   }
@@ -153,7 +168,7 @@ __global__ __launch_bounds__(CHUNK) void lr_apply_kernel(LrTables tb, int count,
 __global__ __launch_bounds__(256) void lr_outer_kernel(LrTables tb, int count) {
   __shared__ float Vi[NMAX][TILE + 4];
   __shared__ float Vj[NMAX][TILE + 4];
-  const int l = find_slot(tb.tile_cs, count, blockIdx.x);
+  const int l = tb.tile_owner[blockIdx.x];
   const int w = tb.w[l];
   const int tiles = (w + TILE - 1) / TILE;
   const int t = blockIdx.x - tb.tile_cs[l];
@@ -165,34 +180,25 @@ __global__ __launch_bounds__(256) void lr_outer_kernel(LrTables tb, int count) {
     Vj[k][c] = j0 + c < w ? V[(long long)k * w + j0 + c] : 0.f;
   }
   __syncthreads();
-  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
-  float acc[4][4];
+  // four waves, one 32 x 32 quadrant each: 16 matrix instructions over the NMAX rows of V.
+  // v_mfma_f32_32x32x2_f32 takes A[i][k] and B[k][j] with i, j = lane % 32, k = lane / 32
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, lk = lane >> 5;
+  floatx16 acc;
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-    for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
-#pragma unroll 8
-  for (int k = 0; k < NMAX; ++k) {
-    float av[4], bv[4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a) av[a] = Vi[k][ty * 4 + a];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) bv[b] = Vj[k][tx * 4 + b];
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b) acc[a][b] += av[a] * bv[b];
-  }
+  for (int kk = 0; kk < NMAX / 2; ++kk)
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Vi[2 * kk + lk][wm * 32 + li], Vj[2 * kk + lk][wn * 32 + li], acc,
+                                               0, 0, 0);
+  // accumulator element v of a lane: row 8 (v / 4) + 4 (lane / 32) + v % 4, column lane % 32
   float *__restrict__ out = tb.out[l];
+  const int c = j0 + wn * 32 + li;
 #pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int r = i0 + ty * 4 + a;
-    if (r >= w) continue;
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int c = j0 + tx * 4 + b;
-      if (c < w) out[(long long)r * w + c] = (r == c ? 1.0f / damp_of(tb, l, r) : 0.f) - acc[a][b];
-    }
+  for (int v = 0; v < 16; ++v) {
+    const int r = i0 + wm * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+    if (r < w && c < w) out[(long long)r * w + c] = (r == c ? 1.0f / damp_of(tb, l, r) : 0.f) - acc[v];
   }
 }
 
@@ -206,7 +212,7 @@ struct kfac_bn_lowrank_plan {
   size_t v_floats = 0;
   std::vector<const void *> u_host, out_host;
   std::vector<float> dg_host, db_host;
-  kfac::DevTable d_u, d_out, d_w, d_split, d_dg, d_db, d_chunk, d_tile, d_voff;
+  kfac::DevTable d_u, d_out, d_w, d_split, d_dg, d_db, d_chunk, d_tile, d_tile_owner, d_voff;
 };
 
 extern "C" int kfac_bn_lowrank_plan_create(int count, int n, const int32_t *widths,
@@ -251,6 +257,11 @@ extern "C" int kfac_bn_lowrank_plan_create(int count, int n, const int32_t *widt
   up(p->d_split, p->split.data(), sizeof(int) * count);
   up(p->d_chunk, chunk_cs.data(), sizeof(int) * (count + 1));
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
+  {
+    std::vector<int> owner((size_t)p->tiles);
+    for (int i = 0; i < count; ++i) std::fill(owner.begin() + tile_cs[i], owner.begin() + tile_cs[i + 1], i);
+    up(p->d_tile_owner, owner.data(), sizeof(int) * owner.size());
+  }
   up(p->d_voff, voff.data(), sizeof(long long) * count);
   if (rc != KFAC_OK) {
     delete p;
@@ -314,6 +325,7 @@ extern "C" int kfac_bn_lowrank_inverse_batched_f32(kfac_bn_lowrank_plan_t plan,
   tb.db = plan->d_db.as<const float>();
   tb.chunk_cs = plan->d_chunk.as<const int>();
   tb.tile_cs = plan->d_tile.as<const int>();
+  tb.tile_owner = plan->d_tile_owner.as<const int>();
   tb.v_off = plan->d_voff.as<const long long>();
   uintptr_t base = (reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255;
   tb.part = reinterpret_cast<double *>(base);
@@ -321,7 +333,7 @@ extern "C" int kfac_bn_lowrank_inverse_batched_f32(kfac_bn_lowrank_plan_t plan,
   tb.V = reinterpret_cast<float *>(tb.winv + (size_t)count * NMAX * NMAX);
   tb.info = info_dev;
   hipLaunchKernelGGL(lr_gram_kernel, dim3(plan->chunks), dim3(256), 0, s, tb, count, plan->n);
-  hipLaunchKernelGGL(lr_factor_kernel, dim3(count), dim3(64), 0, s, tb);
+  hipLaunchKernelGGL(lr_factor_kernel, dim3(count), dim3(kFactorThreads), 0, s, tb);
   hipLaunchKernelGGL(lr_apply_kernel, dim3(plan->chunks), dim3(CHUNK), 0, s, tb, count, plan->n);
   hipLaunchKernelGGL(lr_outer_kernel, dim3(plan->tiles), dim3(256), 0, s, tb, count);
   KFAC_HIP_CHECK(hipGetLastError());
