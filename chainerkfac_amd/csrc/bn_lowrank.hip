@@ -195,10 +195,13 @@ __global__ __launch_bounds__(256) void lr_outer_kernel(LrTables tb, int count) {
   // accumulator element v of a lane: row 8 (v / 4) + 4 (lane / 32) + v % 4, column lane % 32
   float *__restrict__ out = tb.out[l];
   const int c = j0 + wn * 32 + li;
+  // D^-1 only meets the quadrants on the diagonal (a wave-uniform test): the others are
+  // stored as they are, without a division per element
+  const float dinv = (i0 + wm * 32 == j0 + wn * 32 && c < w) ? 1.0f / damp_of(tb, l, c) : 0.f;
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     const int r = i0 + wm * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-    if (r < w && c < w) out[(long long)r * w + c] = (r == c ? 1.0f / damp_of(tb, l, r) : 0.f) - acc[v];
+    if (r < w && c < w) out[(long long)r * w + c] = (r == c ? dinv : 0.f) - acc[v];
   }
 }
 
