@@ -326,40 +326,57 @@ def run_step_config(args, name, cfg):
         arrays = [[(cov, True) for fb in opt.fblocks for cov in fb.covs]]
     wire_stats, _ = wire_format(arrays, dev, lib)
 
-    # the momentum rule over all parameters (the reference's next call after the preconditioning,
-    # optimizers/kfac.py:250-252): not part of `value`, timed the same way as the phases
-    def update_phase():
-        opt.update_params()
+    extras = {}
+    if not args.no_extras:
+        # the momentum rule over all parameters (the reference's next call after the preconditioning,
+        # optimizers/kfac.py:250-252): not part of `value`, timed the same way as the phases
+        def update_phase():
+            opt.update_params()
 
-    update_ms = {}
-    for label, batched in (('batched', True), ('per_parameter', False)):
-        opt.batch_param_updates = batched
-        update_phase()
-        update_ms[label] = timed(update_phase if args.no_graph else capture(update_phase))
-    opt.batch_param_updates = True
-    n_param_arrays = len(list(model.params()))
-    n_params = sum(p.data.numel() for p in model.params())
+        update_ms = {}
+        for label, batched in (('batched', True), ('per_parameter', False)):
+            opt.batch_param_updates = batched
+            update_phase()
+            update_ms[label] = timed(update_phase if args.no_graph else capture(update_phase))
+        opt.batch_param_updates = True
+        n_param_arrays = len(list(model.params()))
+        n_params = sum(p.data.numel() for p in model.params())
 
-    # the moving average of all factors in a step that has history (cov_ema_decay = 0.99, the
-    # reference's default; the first step, which `value` times for c3 - c5, only aliases)
-    for fb in opt.fblocks:
-        fb.cov_ema_decay, fb.cov_emas = 0.99, None
+        # the moving average of all factors in a step that has history (cov_ema_decay = 0.99, the
+        # reference's default; the first step, which `value` times for c3 - c5, only aliases)
+        for fb in opt.fblocks:
+            fb.cov_ema_decay, fb.cov_emas = 0.99, None
 
-    def ema_phase():
-        opt.update_cov_emas(opt.fblocks)
+        def ema_phase():
+            opt.update_cov_emas(opt.fblocks)
 
-    ema_phase()   # the first call copies
-    ema_ms = {}
-    for label, batched in (('batched', True), ('per_array', False)):
-        opt.batch_elementwise = batched
-        ema_phase()
-        ema_ms[label] = timed(ema_phase if args.no_graph else capture(ema_phase))
-    opt.batch_elementwise = True
-    n_factor_arrays = sum(len(fb.covs) for fb in opt.fblocks)
-    n_factor_elems = sum(c.numel() for fb in opt.fblocks for c in fb.covs)
-    for fb in opt.fblocks:
-        fb.cov_ema_decay, fb.cov_emas = cfg['decay'], None
-    inv_phase()   # back to this configuration's own averages and inverses
+        ema_phase()   # the first call copies
+        ema_ms = {}
+        for label, batched in (('batched', True), ('per_array', False)):
+            opt.batch_elementwise = batched
+            ema_phase()
+            ema_ms[label] = timed(ema_phase if args.no_graph else capture(ema_phase))
+        opt.batch_elementwise = True
+        n_factor_arrays = sum(len(fb.covs) for fb in opt.fblocks)
+        n_factor_elems = sum(c.numel() for fb in opt.fblocks for c in fb.covs)
+        for fb in opt.fblocks:
+            fb.cov_ema_decay, fb.cov_emas = cfg['decay'], None
+        inv_phase()   # back to this configuration's own averages and inverses
+        extras = {
+            # v = momentum v - lr kfgrad; param += v over every parameter: 20 bytes per element
+            'param_update': {'parameters': n_params, 'arrays': n_param_arrays,
+                             'one_launch_ms': round(update_ms['batched'], 4),
+                             'launch_per_parameter_ms': round(update_ms['per_parameter'], 4),
+                             'one_launch_tb_s': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12, 3),
+                             'frac_of_hbm_peak': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
+                             'in_value': False},
+            # ema = 0.99 cov + 0.01 ema over every factor: 12 bytes per element
+            'moving_average': {'elements': n_factor_elems, 'arrays': n_factor_arrays,
+                               'one_launch_ms': round(ema_ms['batched'], 4),
+                               'launch_per_array_ms': round(ema_ms['per_array'], 4),
+                               'one_launch_tb_s': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12, 3),
+                               'frac_of_hbm_peak': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
+                               'in_value': False}}
 
     # dominant kernel family, timed launch by launch inside the library (one stream: with lanes,
     # launches overlap and the time between a launch's events is shared with others)
@@ -425,20 +442,6 @@ def run_step_config(args, name, cfg):
         'kernel_ms': {k: {'launches': n, 'total_ms': round(ms - n * empty, 3)} for k, (n, ms) in fam.items() if n},
         'inverse_info_nonzero': info_bad,
         'wire_format': wire_stats,
-        # v = momentum v - lr kfgrad; param += v over every parameter: 20 bytes per element
-        'param_update': {'parameters': n_params, 'arrays': n_param_arrays,
-                         'one_launch_ms': round(update_ms['batched'], 4),
-                         'launch_per_parameter_ms': round(update_ms['per_parameter'], 4),
-                         'one_launch_tb_s': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12, 3),
-                         'frac_of_hbm_peak': round(20.0 * n_params / (update_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
-                         'in_value': False},
-        # ema = 0.99 cov + 0.01 ema over every factor: 12 bytes per element
-        'moving_average': {'elements': n_factor_elems, 'arrays': n_factor_arrays,
-                           'one_launch_ms': round(ema_ms['batched'], 4),
-                           'launch_per_array_ms': round(ema_ms['per_array'], 4),
-                           'one_launch_tb_s': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12, 3),
-                           'frac_of_hbm_peak': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
-                           'in_value': False},
         'roofline': {
             'kernel': 'covariance SYRK family (shift::corr_kernel, syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
             'bound': 'mfma',
@@ -462,6 +465,7 @@ def run_step_config(args, name, cfg):
             'traffic_unit': 'bytes/launch',
         },
     }
+    result.update(extras)
     if name == 'c3' and lowrank and not args.no_dense_field:
         # the reference's algorithm inverts the batch-norm blocks densely as well: the same step with
         # the Woodbury shortcut switched off, as a second figure
@@ -619,7 +623,7 @@ def write_per_layer(path, layers, config='c3'):
     with open(path, 'w') as f:
         f.write('# Covariance kernels layer by layer (every distinct convolution / linear shape of the workload)\n\n'
                 'Command (one MI355X, repository root):\n\n```\npython3 bench.py --config {} --no-cpu --no-dense-field '
-                '--steps 5 --per-layer {}\n```\n\n'
+                '--no-extras --steps 5 --per-layer {}\n```\n\n'
                 'Each factor is computed alone, by the single-factor entry point, on one stream; "SYRK kernel us" is '
                 'the duration of its SYRK launch (HIP events inside the library around the launch, 10 repetitions, the '
                 '{:.1f} us an empty event bracket measures subtracted); the kernels that sum split-K partial tiles are '
@@ -962,6 +966,9 @@ def main():
                          'rank-32 Woodbury form, which yields the same dense inverse)')
     ap.add_argument('--no-dense-field', action='store_true',
                     help='skip the second measurement of c3 with all batch-norm blocks inverted densely')
+    ap.add_argument('--no-extras', action='store_true',
+                    help='skip the measurements beside the step (momentum rule of all parameters, moving average '
+                         'of all factors): profiling runs')
     ap.add_argument('--lanes', type=int, default=3,
                     help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
     ap.add_argument('--macro-tiles', action='store_true',
