@@ -252,10 +252,12 @@ def axpby_batched(xs, ys, a, b, stream=None):
             raise ValueError('size mismatch')
     if _axpby_batches is None:
         _axpby_batches = _PlanCache(16)
-    key = (tuple(x.data_ptr() for x in xs), tuple(y.data_ptr() for y in ys))
-    batch = _axpby_batches.get(key, _AxpbyBatch)
+    # one batch object per list of destinations (they persist; the sources of a gradient
+    # accumulation need not, and the object keeps its last few tables)
+    xp, yp = tuple(x.data_ptr() for x in xs), tuple(y.data_ptr() for y in ys)
+    batch = _axpby_batches.get(yp, _AxpbyBatch)
     _lib.check(_lib.load().kfac_axpby_batched_f32(
-        batch._h, len(xs), _lib.ptr_array(key[0]), _lib.ptr_array(key[1]),
+        batch._h, len(xs), _lib.ptr_array(xp), _lib.ptr_array(yp),
         _lib.i64_array([x.numel() for x in xs]), a, b, _dev.stream_handle(stream)))
     return ys
 
@@ -697,8 +699,9 @@ def momentum_update_batched(params, vs, grads, lr, momentum, loss_scale=None, wr
         flags.append((1 if g.dtype == torch.float16 else 0) | (2 if wb else 0))
     if _momentum_batches is None:
         _momentum_batches = _PlanCache(16)
-    key = (tuple(p.data_ptr() for p in params), tuple(g.data_ptr() for g in grads))
-    batch = _momentum_batches.get(key, _MomentumBatch)
+    # one batch object per list of parameters (gradient arrays may be new ones every step;
+    # the object keeps its last few tables)
+    batch = _momentum_batches.get(tuple(p.data_ptr() for p in params), _MomentumBatch)
     _lib.check(_lib.load().kfac_momentum_update_batched_f32(
         batch._h, n, _lib.ptr_array([p.data_ptr() for p in params]),
         _lib.ptr_array([v.data_ptr() for v in vs]), _lib.ptr_array([g.data_ptr() for g in grads]),
