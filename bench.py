@@ -161,7 +161,7 @@ def timed_steps(run, steps):
     return mean, each[len(each) // 2]
 
 
-def timed(fn, reps=5):
+def timed(fn, reps=11):
     import torch
     pairs = _events(reps)
     torch.cuda.synchronize()
@@ -173,16 +173,39 @@ def timed(fn, reps=5):
     return sorted(e0.elapsed_time(e1) for e0, e1 in pairs)[reps // 2]
 
 
+FAMILY_IDS = (('syrk', 0), ('inv_update', 1), ('inv_lauum', 2), ('gemm', 3), ('pack', 4), ('unpack', 5), ('copy', 6),
+              ('cov_aux', 7), ('bn_stats', 8), ('inv_call', 9), ('gemm_aux', 10))
+
+
 def family_times(lib):
+    """(launches, summed ms between the HIP events) of every timed kernel family since timing was enabled."""
     from chainerkfac_amd import _lib
     fam = {}
-    for name, fid in (('syrk', 0), ('inv_update', 1), ('inv_lauum', 2), ('gemm', 3), ('pack', 4), ('unpack', 5),
-                      ('copy', 6)):
+    for name, fid in FAMILY_IDS:
         n = ctypes.c_int64()
         ms = ctypes.c_double()
         _lib.check(lib.kfac_timing_read(fid, ctypes.byref(n), ctypes.byref(ms)))
         fam[name] = (n.value, ms.value)
     return fam
+
+
+def family_roofline(label, kernels, flop, members, fam, empty, note, reference_flop=None):
+    """Roofline entry of one kernel family: `flop` is the work its kernels are given (issued
+    multiply-adds x 2), the time is the sum of the event brackets of `members` (each bracket less
+    what an empty bracket measures)."""
+    n = sum(fam[m][0] for m in members)
+    ms = sum(max(fam[m][1] - fam[m][0] * empty, 0.0) for m in members)
+    rate = flop / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+    out = {'kernel': kernels, 'bound': 'mfma', 'achieved': round(rate, 2), 'peak': FP32_MFMA_PEAK_TFLOPS,
+           'unit': 'TFLOP/s', 'frac': round(rate / FP32_MFMA_PEAK_TFLOPS, 4),
+           'gflop_per_step': round(flop / 1e9, 1), 'kernel_ms_per_step': round(ms, 4), 'brackets': n,
+           'avg_bracket_ms': round(ms / max(n, 1), 4), 'timed': note}
+    if reference_flop is not None and ms > 0:
+        # the work of the reference's algorithm for the same result over the same time: a labelled
+        # extra, not a utilisation (it exceeds the peak where this build issues fewer flops)
+        out['reference_work_gflop_per_step'] = round(reference_flop / 1e9, 1)
+        out['reference_work_rate'] = round(reference_flop / (ms * 1e-3) / 1e12, 2)
+    return out
 
 
 def read_traffic():
@@ -378,7 +401,14 @@ def run_step_config(args, name, cfg):
                                'frac_of_hbm_peak': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
                                'in_value': False}}
 
-    # dominant kernel family, timed launch by launch inside the library (one stream: with lanes,
+    # the same step launched kernel by kernel from the host (what a caller of the drop-in classes
+    # gets without capturing a graph of its own)
+    eager_ms = None
+    if not args.no_graph and not args.no_extras:
+        step()
+        eager_ms, _ = timed_steps(step, max(args.steps // 2, 5))
+
+    # every kernel family, timed bracket by bracket inside the library (one stream: with lanes,
     # launches overlap and the time between a launch's events is shared with others)
     opt._lanes.n = 0
     _lib.check(lib.kfac_timing_enable(1))
@@ -394,16 +424,41 @@ def run_step_config(args, name, cfg):
     dense_inverse_flops = flops['inverse'] - sum(float(fb.cov_emas[0].shape[0]) ** 3 for fb in lowrank)
 
     empty = bracket_ms()
-    syrk_n, syrk_raw_ms = fam['syrk']
-    syrk_ms = max(syrk_raw_ms - syrk_n * empty, 1e-9)
-    achieved = flops['cov'] / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
     # what the matrix cores are actually given: 3x3 stride-1 convolutions compute their A factor from
     # shifted correlations, about a third of the multiply-adds of the patch product
     cov_executed = float(W.cov_flops_executed(layers, batch)) * acc_iters
-    achieved_executed = cov_executed / (syrk_ms * 1e-3) / 1e12 if syrk_n > 0 else 0.0
     executed_flops = cov_executed + dense_inverse_flops + flops['precondition']
     total_flops = flops['cov'] + flops['inverse'] + flops['precondition']
+    one_stream = 'launches on one stream (--lanes 0 for this pass), HIP events around each launch, empty bracket subtracted'
+    families = {
+        'cov_syrk': family_roofline(
+            'cov_syrk', 'covariance SYRK family: shift::corr_kernel, syrk_rows_kernel, syrk_group_kernel, syrk_kernel, '
+            'syrk_conv_kernel and the kernels around them (edge_sums, corr_finish, assemble, finish_group, finish, reduce)',
+            cov_executed, ('syrk', 'cov_aux'), fam, empty, one_stream, reference_flop=flops['cov']),
+        'inverse_tiles': family_roofline(
+            'inverse_tiles', 'batched dense inverse: copy_in, diag, update, panel, border, lauum kernels',
+            dense_inverse_flops, ('inv_call',), fam, empty,
+            'd^3 flop of the densely inverted factors over the time between the first and the last launch of the '
+            'batched call (its kernels overlap on three streams, so their durations do not add up)',
+            reference_flop=flops['inverse']),
+        'precond_gemm': family_roofline(
+            'precond_gemm', 'preconditioning GEMMs: gemm_group_kernel (both phases), gemm_group_finish_kernel, '
+            'gemv_kernel + bn_select_kernel of the batch-norm blocks',
+            flops['precondition'], ('gemm', 'gemm_aux'), fam, empty, one_stream),
+    }
+    main_syrk = family_roofline('', '', cov_executed, ('syrk',), fam, empty, '')
+    families['cov_syrk']['main_kernels_only'] = {
+        'launches': main_syrk['brackets'], 'kernel_ms_per_step': main_syrk['kernel_ms_per_step'],
+        'achieved': main_syrk['achieved'], 'frac': main_syrk['frac']}
     traffic = read_traffic() if name == 'c3' else None
+    families['cov_syrk']['traffic_main_kernels'] = traffic
+    families['cov_syrk']['traffic_unit'] = 'bytes/launch of the main kernels'
+    dominant = max(families, key=lambda k: families[k]['kernel_ms_per_step'])
+    roofline = dict(families[dominant])
+    roofline['family'] = dominant
+    roofline['traffic'] = traffic if dominant == 'cov_syrk' else None
+    roofline['event_bracket_ms'] = round(empty, 4)
+    roofline['families'] = families
     result = {
         'metric': METRIC,
         'value': round(ms_per_step, 4),
@@ -420,6 +475,7 @@ def run_step_config(args, name, cfg):
         'data': 'synthetic',
         'config': {'workload': cfg['workload'], 'name': name, 'batch': batch,
                    'factors': len(W.all_factor_dims(layers)), 'damping': cfg['damping'], 'acc_iters': acc_iters,
+                   'cov_ema_decay': cfg['decay'],
                    'hip_graph': not args.no_graph, 'lanes': args.lanes, 'macro_tiles': bool(args.macro_tiles),
                    'bn_inverse': 'woodbury rank-{} ({} blocks)'.format(batch, len(lowrank)) if lowrank else 'dense'},
         # rates use the flops actually executed; the *_reference_work entries divide the work of the
@@ -437,34 +493,16 @@ def run_step_config(args, name, cfg):
             'inverse_reference_work': round(flops['inverse'] / phase_ms['inverse'] / 1e9, 2),
         },
         'phase_ms': {k: round(v, 3) for k, v in phase_ms.items()},
+        'phase_ms_timed': 'each phase as its own HIP graph, median of 11 replays',
         'gflop': dict({k: round(v / 1e9, 1) for k, v in flops.items()},
                       inverse_executed=round(dense_inverse_flops / 1e9, 1), cov_executed=round(cov_executed / 1e9, 1)),
         'kernel_ms': {k: {'launches': n, 'total_ms': round(ms - n * empty, 3)} for k, (n, ms) in fam.items() if n},
         'inverse_info_nonzero': info_bad,
         'wire_format': wire_stats,
-        'roofline': {
-            'kernel': 'covariance SYRK family (shift::corr_kernel, syrk_rows_kernel, syrk_group_kernel, syrk_kernel)',
-            'bound': 'mfma',
-            'achieved': round(achieved, 2),
-            'peak': FP32_MFMA_PEAK_TFLOPS,
-            'unit': 'TFLOP/s',
-            'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
-            # `achieved` divides the algorithmic work M d (d+1) of every factor by the kernels' time; the
-            # multiply-adds issued are fewer where a factor is built from shifted correlations
-            'executed': {'gflop_per_step': round(cov_executed / 1e9, 1),
-                         'algorithmic_gflop_per_step': round(flops['cov'] / 1e9, 1),
-                         'achieved': round(achieved_executed, 2),
-                         'frac': round(achieved_executed / FP32_MFMA_PEAK_TFLOPS, 4)},
-            'launches': syrk_n,
-            'avg_launch_ms': round(syrk_ms / max(syrk_n, 1), 4),
-            'avg_launch_ms_with_event_bracket': round(syrk_raw_ms / max(syrk_n, 1), 4),
-            'event_bracket_ms': round(empty, 4),
-            'timed': 'launches on one stream (--lanes 0 for this pass), HIP events around each launch, '
-                     'empty bracket subtracted',
-            'traffic': traffic,
-            'traffic_unit': 'bytes/launch',
-        },
+        'roofline': roofline,
     }
+    if eager_ms is not None:
+        result['eager_ms_per_step'] = round(eager_ms, 4)
     result.update(extras)
     if name == 'c3' and lowrank and not args.no_dense_field:
         # the reference's algorithm inverts the batch-norm blocks densely as well: the same step with
@@ -481,6 +519,23 @@ def run_step_config(args, name, cfg):
             'inverse_ms': round(inv_dense, 3),
             'inverse_tflops': round(flops['inverse'] / inv_dense / 1e9, 2),
             'step_tflops': round(total_flops / dense_ms / 1e9, 2)}
+        # a step with history: cov_ema_decay = 0.99 (the reference's default), so every factor is averaged
+        # into its moving average (one launch over all factors) and every batch-norm block is inverted
+        # densely (its moving average is no longer this step's rank-n matrix)
+        opt.bn_lowrank_inverse = True
+        for fb in opt.fblocks:
+            fb.cov_ema_decay, fb.cov_emas = 0.99, None
+        for _ in range(2):
+            step()      # the first call copies, the second averages
+        torch.cuda.synchronize()
+        run_steady = step if args.no_graph else capture(step)
+        steady_ms, steady_median = timed_steps(run_steady, max(args.steps // 2, 5))
+        result['steady_state'] = {
+            'cov_ema_decay': 0.99, 'bn_inverse': 'dense', 'ms_per_step': round(steady_ms, 4),
+            'ms_per_step_median': round(steady_median, 4),
+            'step_tflops_reference_work': round(total_flops / steady_ms / 1e9, 2)}
+        for fb in opt.fblocks:
+            fb.cov_ema_decay, fb.cov_emas = cfg['decay'], None
     return result
 
 
@@ -545,13 +600,76 @@ def run_inverse_config(args, name, cfg):
         'inverse_info_nonzero': int((info != 0).sum().item()),
         'max_residual': worst,      # max over sizes of ||M M^-1 - I||_F / sqrt(d); the bound is 1e-3
         'roofline': {
-            'kernel': 'batched inverse (copy_in, step, panel, update, lauum kernels)', 'bound': 'mfma',
+            'family': 'inverse_tiles',
+            'kernel': 'batched dense inverse: copy_in, diag, update, panel, border, lauum kernels', 'bound': 'mfma',
             'achieved': round(achieved, 2), 'peak': FP32_MFMA_PEAK_TFLOPS, 'unit': 'TFLOP/s',
             'frac': round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
             'timed': 'd^3 flop per matrix over the wall time of the whole batched call (its kernels overlap on two '
                      'streams, so their durations do not add up)',
             'traffic': None},
     }, dims
+
+
+def run_real_network(steps=5, warmup=2):
+    """``KFAC.update(lossfun)`` on the ResNet-50 built from the link classes (batch 32 @ 224): a
+    real forward and backward pass under the function hooks, then moving average, damped inverse,
+    preconditioning and the momentum rule, launched from the host with no HIP graph.  Gradient and
+    activation buffers are whatever torch's autograd hands out each step."""
+    import torch
+    import torch.nn.functional as TF
+    from chainerkfac_amd import workloads as W
+    from chainerkfac_amd.optimizers import KFAC
+    dev = torch.device('cuda:0')
+    gen = torch.Generator(device=dev).manual_seed(3)
+    model = W.build_resnet50_v1(device=dev, generator=gen)
+    x = torch.randn(BATCH, 3, 224, 224, device=dev, generator=gen)
+    t = torch.randint(0, 1000, (BATCH,), device=dev, generator=gen)
+
+    def lossfun():
+        return TF.cross_entropy(model(x), t)
+
+    def wall(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n
+
+    def plain():
+        model.cleargrads()
+        lossfun().backward()
+
+    for _ in range(warmup):
+        plain()
+    plain_ms = wall(plain, steps)
+    opt = KFAC(lr=1e-3, damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0).setup(model)
+    for _ in range(warmup):
+        opt.update(lossfun)
+    update_ms = wall(lambda: opt.update(lossfun), steps)
+    return {'workload': 'KFAC.update(lossfun) on the link-built ResNet-50 v1 (bias), batch 32 @224, 161 factors, '
+                        'eager (no HIP graph), torch autograd for the forward / backward pass',
+            'steps': steps, 'ms_per_update': round(update_ms, 3),
+            'forward_backward_only_ms': round(plain_ms, 3),
+            'kfac_part_ms': round(update_ms - plain_ms, 3), 'in_value': False}
+
+
+def compact(result):
+    """The few figures of another configuration's line that go into the default line."""
+    roof = result['roofline']
+    out = {'workload': result['config']['workload'], 'ms_per_step': result['value'], 'steps': result['steps'],
+           'roofline': {k: roof.get(k) for k in ('family', 'kernel', 'achieved', 'unit', 'frac') if k in roof}}
+    if 'phase_ms' in result:
+        out['phase_ms'] = result['phase_ms']
+    if 'families' in roof:
+        out['family_frac'] = {k: v['frac'] for k, v in roof['families'].items()}
+    if result['config'].get('name') == 'c5':
+        w = result['wire_format']
+        out['wire_format'] = {'arrays': w['arrays'], 'triangular': w['triangular'],
+                              'pack': w['pack'], 'unpack': w['unpack'], 'stream_copy': w['stream_copy']}
+    if 'max_residual' in result:
+        out['max_residual'] = result['max_residual']
+    return out
 
 
 def write_per_layer(path, layers, config='c3'):
@@ -969,11 +1087,14 @@ def main():
     ap.add_argument('--no-extras', action='store_true',
                     help='skip the measurements beside the step (momentum rule of all parameters, moving average '
                          'of all factors): profiling runs')
+    ap.add_argument('--no-other-configs', action='store_true',
+                    help='c3 only: skip the short runs of c1, c2, c4 and c5 and the real-network step that the '
+                         'default line carries beside its own figures')
     ap.add_argument('--lanes', type=int, default=3,
                     help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
     ap.add_argument('--macro-tiles', action='store_true',
                     help='grouped covariance launches use the macro-tile kernel for slabs of several 128-tiles '
-                         '(KFAC_GROUP_MACRO=1: less HBM traffic, about 1 %% slower)')
+                         '(library option group_macro = 1: less HBM traffic, about 1 %% slower)')
     ap.add_argument('--per-layer', metavar='PATH', default=None,
                     help='also time the covariance kernels of every distinct layer shape alone and write a '
                          'markdown roofline table to PATH')
@@ -1004,7 +1125,8 @@ def main():
         summarize_mfma(args.summarize_mfma[0], args.summarize_mfma[1], args.profiled_command)
         return
     if args.macro_tiles:
-        os.environ['KFAC_GROUP_MACRO'] = '1'
+        from chainerkfac_amd import _lib
+        _lib.set_option('group_macro', 1)
     cfg = configs()[args.config]
     if args.config == 'c4':
         result, _ = run_inverse_config(args, args.config, cfg)
@@ -1012,6 +1134,30 @@ def main():
         result = run_step_config(args, args.config, cfg)
         if args.per_layer:
             write_per_layer(args.per_layer, cfg['layers'], args.config)
+    if args.config == 'c3' and not args.no_other_configs:
+        # the other configurations of the benchmark definition, shorter runs of the same code paths
+        # (their full lines: --config c1 | c2 | c4 | c5), and the drop-in step on a real network
+        import copy
+        import gc
+        import torch
+        others = {}
+        for name, steps in (('c1', 50), ('c2', 50), ('c4', 20), ('c5', 5)):
+            gc.collect()
+            torch.cuda.empty_cache()
+            sub = copy.copy(args)
+            sub.config, sub.steps, sub.warmup = name, steps, 1
+            sub.no_extras = sub.no_dense_field = True
+            sub.per_layer = None
+            sub_cfg = configs()[name]
+            if name == 'c4':
+                line, _ = run_inverse_config(sub, name, sub_cfg)
+            else:
+                line = run_step_config(sub, name, sub_cfg)
+            others[name] = compact(line)
+        result['other_configs'] = others
+        gc.collect()
+        torch.cuda.empty_cache()
+        result['real_network'] = run_real_network()
     if not args.no_cpu:
         result['cpu_baseline'] = run_cpu_baseline(args.config, cfg)
     print(json.dumps(result))

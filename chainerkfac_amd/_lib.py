@@ -25,6 +25,11 @@ c_sz = ctypes.c_size_t
 PROTOTYPES = {
     'kfac_abi_version': (c_int, []),
     'kfac_last_error_string': (ctypes.c_char_p, []),
+    'kfac_option_set': (c_int, [ctypes.c_char_p, c_d]),
+    'kfac_option_unset': (c_int, [ctypes.c_char_p]),
+    'kfac_option_get': (c_int, [ctypes.c_char_p, c_dp, ctypes.POINTER(c_int)]),
+    'kfac_option_count': (c_int, []),
+    'kfac_option_name': (ctypes.c_char_p, [c_int]),
     'kfac_packed_nelems': (c_i64, [c_int, c_i64p, c_i32p]),
     'kfac_pack_plan_create': (c_int, [c_int, c_vpp, c_i64p, c_i32p, c_i32p, c_vpp]),
     'kfac_pack_plan_set_ptrs': (c_int, [c_vp, c_vpp, c_vp]),
@@ -73,6 +78,11 @@ PROTOTYPES = {
     'kfac_precond_group_run_f32': (c_int, [c_vp, c_vpp, c_vpp, c_vpp, c_vpp, c_vpp, c_vpp, c_vp, c_sz, c_vp]),
     'kfac_precond_bn_workspace_bytes': (c_sz, [c_int]),
     'kfac_precond_bn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    'kfac_precond_bn_batch_create': (c_int, [c_vp]),
+    'kfac_precond_bn_batch_destroy': (c_int, [c_vp]),
+    'kfac_precond_bn_batched_workspace_bytes': (c_sz, [c_int, c_i32p]),
+    'kfac_precond_bn_batched_f32': (c_int, [c_vp, c_int, c_vpp, c_i32p, c_vpp, c_i32p, c_vpp, c_vpp, c_vpp, c_vpp,
+                                            c_vp, c_sz, c_vp]),
     'kfac_precond_bn_static_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp]),
     'kfac_momentum_update_f32': (c_int, [c_vp, c_vp, c_vp, c_i64, c_f, c_f, c_vp]),
     'kfac_momentum_batch_create': (c_int, [c_vp]),
@@ -117,6 +127,41 @@ def check(status):
     if status != 0:
         msg = load().kfac_last_error_string().decode('utf-8', 'replace')
         raise KfacHipError('libkfac_hip error {}: {}'.format(status, msg))
+
+
+def set_option(name, value):
+    """Sets a tuning option of the library (None restores the built-in default)."""
+    lib = load()
+    if value is None:
+        check(lib.kfac_option_unset(name.encode()))
+    else:
+        check(lib.kfac_option_set(name.encode(), float(value)))
+
+
+def get_option(name):
+    """The value an option was set to, or None while the built-in default is in force."""
+    value, is_set = ctypes.c_double(), ctypes.c_int()
+    check(load().kfac_option_get(name.encode(), ctypes.byref(value), ctypes.byref(is_set)))
+    return value.value if is_set.value else None
+
+
+class options(object):
+    """``with options(inverse_group=3): ...`` -- options set for the block, restored after."""
+
+    def __init__(self, **values):
+        self._values = values
+        self._saved = {}
+
+    def __enter__(self):
+        for k, v in self._values.items():
+            self._saved[k] = get_option(k)
+            set_option(k, v)
+        return self
+
+    def __exit__(self, *exc):
+        for k, v in self._saved.items():
+            set_option(k, v)
+        return False
 
 
 def i32_array(values):

@@ -100,14 +100,41 @@ class ArrayPacker(object):
         self._cache = {}
         self._max_cached = max_cached
 
-    def _info(self, arrays):
+    def _info(self, arrays, stream=None):
         key = _key_of(arrays)
-        info = self._cache.get(key)
+        info = self._cache.pop(key, None)
+        if info is None:
+            info = self._rebind(key, arrays, stream)
         if info is None:
             if len(self._cache) >= self._max_cached:
                 self._cache.pop(next(iter(self._cache)))
-            info = self._cache[key] = _ArraysInfo(arrays)
+            info = _ArraysInfo(arrays)
+        self._cache[key] = info      # most recently used last
         return info
+
+    def _rebind(self, key, arrays, stream):
+        """A cached descriptor of the same layout pointed at other arrays (gradient arrays
+        move from step to step): only the pointer table is uploaded again.  The two most
+        recent descriptors of a layout are left alone (lists that alternate keep theirs),
+        and so is one that a captured HIP graph replays against (the library refuses to
+        change it)."""
+        layout = tuple(k[1:] for k in key)
+        same = [k for k in self._cache if tuple(e[1:] for e in k) == layout]
+        if len(same) < 2:
+            return None
+        flat = [_dev.require_gpu_tensor(a, 'array') for local in arrays for a, _ in local]
+        for old_key in same[:-1]:
+            info = self._cache[old_key]
+            try:
+                _lib.check(_lib.load().kfac_pack_plan_set_ptrs(
+                    info.plan, _lib.ptr_array([a.data_ptr() for a in flat]), _dev.stream_handle(stream)))
+            except _lib.KfacHipError:
+                continue
+            del self._cache[old_key]
+            info.arrays = flat
+            info.key = key
+            return info
+        return None
 
     def get_nelems(self, arrays):
         return _utility.get_nelems(arrays)
@@ -131,7 +158,7 @@ class ArrayPacker(object):
 
     def _pack_arrays_to_buffer(self, arrays, gpu_buf, buf_dtype=np.float32, target=-1,
                                stream=None, debug=False):
-        info = self._info(arrays)
+        info = self._info(arrays, stream)
         if debug and self.rank == 0:
             info.show()
         kind = self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)
@@ -142,7 +169,7 @@ class ArrayPacker(object):
 
     def _unpack_arrays_from_buffer(self, arrays, gpu_buf, buf_dtype=np.float32, target=-1,
                                    divisor=1, stream=None, debug=False):
-        info = self._info(arrays)
+        info = self._info(arrays, stream)
         if debug and self.rank == 0:
             info.show()
         kind = self._check_buf(gpu_buf, buf_dtype, info.buf_size_total)

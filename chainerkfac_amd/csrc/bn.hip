@@ -209,10 +209,12 @@ extern "C" int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, i
   float *sm2 = smean + nslab, *sg = sm2 + nslab, *sgx = sg + nslab;
   const bool vec =
       (hw & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gy)) & 15) == 0;
-  if (vec && hw <= 4 * 16 * 4 && !getenv("KFAC_BN_STATS_LOOP"))
+  kfac::TimedLaunch timed(KFAC_TIMED_BN, s);
+  const bool stats_loop = kfac::option_int(kfac::kOptBnStatsLoop, 0) != 0;   // tuning override
+  if (vec && hw <= 4 * 16 * 4 && !stats_loop)
     hipLaunchKernelGGL((bn_stats_reg_kernel<16, 4>), dim3(kfac::ceil_div(nslab, kThreads / 16)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
-  else if (vec && hw > 256 && hw <= 4 * 64 * 13 && !getenv("KFAC_BN_STATS_LOOP"))
+  else if (vec && hw > 256 && hw <= 4 * 64 * 13 && !stats_loop)
     hipLaunchKernelGGL((bn_stats_reg_kernel<64, 13>), dim3(kfac::ceil_div(nslab, kThreads / 64)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
   else if (hw <= 256)

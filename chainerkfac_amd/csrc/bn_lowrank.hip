@@ -254,7 +254,7 @@ extern "C" int kfac_bn_lowrank_plan_create(int count, int n, const int32_t *widt
   p->tiles = tile_cs[count];
   int rc = KFAC_OK;
   auto up = [&](kfac::DevTable &t, const void *h, size_t b) {
-    if (rc == KFAC_OK) rc = t.set(h, b, nullptr);
+    if (rc == KFAC_OK) rc = t.set_sync(h, b);
   };
   up(p->d_w, p->w.data(), sizeof(int) * count);
   up(p->d_split, p->split.data(), sizeof(int) * count);

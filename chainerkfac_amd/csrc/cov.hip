@@ -61,7 +61,7 @@ long long max_splits(int ntile) {
 SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
   SyrkPlan p;
   int bm64_max = 520;   // measured: 64-tiles win up to d = 512 (more workgroups, 4x smaller partial tiles)
-  if (const char *env = getenv("KFAC_SYRK_BM64_MAX")) bm64_max = atoi(env);   // tuning override
+  bm64_max = kfac::option_int(kfac::kOptSyrkBm64Max, bm64_max);   // tuning override
   p.bm = d <= bm64_max ? 64 : 128;
   // A short reduction (batch-norm blocks: K = batch size) is all output traffic:
   // 64-tiles spread the stores over four times as many workgroups.
@@ -99,9 +99,9 @@ SyrkPlan plan_syrk_panels(int d, long long nk, int panel_len) {
     }
     ns = best_ns;
   }
-  // tuning override: KFAC_SYRK_SPLITS=<n> forces the split count
-  if (const char *env = getenv("KFAC_SYRK_SPLITS")) {
-    const long long forced = atoll(env);
+  // tuning override: option syrk_splits forces the split count
+  if (kfac::option_is_set(kfac::kOptSyrkSplits)) {
+    const long long forced = (long long)kfac::option_value(kfac::kOptSyrkSplits, 0);
     if (forced >= 1) ns = forced < nk ? forced : nk;
   }
   if (ns > max_splits(p.ntile)) ns = max_splits(p.ntile);
@@ -147,8 +147,8 @@ SyrkPlan plan_rows(int d, int bm, long long steps, double step_us, int occ) {
       best_c = c;
     }
   }
-  if (const char *env = getenv("KFAC_SYRK_SPLITS")) {   // tuning override
-    const long long forced = atoll(env);
+  if (kfac::option_is_set(kfac::kOptSyrkSplits)) {   // tuning override
+    const long long forced = (long long)kfac::option_value(kfac::kOptSyrkSplits, 0);
     if (forced >= 1) best_c = std::min(forced, cmax);
   }
   const long long per = kfac::ceil_div(steps, best_c);
@@ -506,6 +506,7 @@ int finish_partials(const SyrkPlan &p, int d, int ones, float count, float alpha
   const float *fin = partial;
   int nfin = p.nsplit;
   const long long slot = (long long)syrk_slot_floats(p);
+  kfac::TimedLaunch timed(KFAC_TIMED_COV_AUX, stream);
   if (p.nreduced) {
     const long long slot4 = slot / 4;
     float *red = partial + (size_t)p.nsplit * slot;
@@ -735,7 +736,7 @@ int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int
 int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, int sy, int sx, int ph,
                   int pw, int ho, int wo, int d, int ones, float alpha, float beta, float *C,
                   void *ws, size_t ws_bytes, hipStream_t stream) {
-  if (getenv("KFAC_CONV_ROWS_OFF")) return 1;   // tuning override: the general kernels only
+  if (kfac::option_int(kfac::kOptConvRows, 1) == 0) return 1;   // tuning override: the general kernels only
   if (n % 2 != 0 || kh != kw || sy != sx || ph != pw) return 1;
   if ((long long)n * c * h * w * (long long)sizeof(float) >= (1ll << 31)) return 1;
   // 128-tiles feed the matrix cores with half the LDS traffic of 64-tiles, but a
@@ -746,7 +747,7 @@ int try_conv_rows(const float *x, int n, int c, int h, int w, int kh, int kw, in
   const int dt = d - ones;
   const long long t64 = kfac::ceil_div(dt, 64), t128 = kfac::ceil_div(dt, 128);
   bool small_tiles = 1.15 * (double)(t64 * (t64 + 1) / 2) < 4.0 * (double)(t128 * (t128 + 1) / 2);
-  if (const char *env = getenv("KFAC_ROWS_WM")) small_tiles = atoi(env) == 1;   // tuning override
+  if (kfac::option_is_set(kfac::kOptRowsWm)) small_tiles = kfac::option_int(kfac::kOptRowsWm, 2) == 1;   // tuning override
 #define KFAC_ROWS_CASE(K, S, P, WS, RT, PAD)                                                      \
   if (kh == K && sy == S && ph == P && wo == WS && ho % RT == 0) {                                \
     if (small_tiles)                                                                              \
@@ -813,9 +814,10 @@ ShiftSlices plan_shift_slices(int wm, int ntab, long long nk) {
       best_longest = longest;
     }
   }
-  if (const char *env = getenv("KFAC_SHIFT_SLICES")) {   // tuning override: "s5,s3"
-    long long a = 0, b = 0;
-    if (sscanf(env, "%lld,%lld", &a, &b) == 2 && a >= 1 && b >= 1) {
+  if (kfac::option_is_set(kfac::kOptShiftSlices5) && kfac::option_is_set(kfac::kOptShiftSlices3)) {   // tuning override
+    const long long a = (long long)kfac::option_value(kfac::kOptShiftSlices5, 0);
+    const long long b = (long long)kfac::option_value(kfac::kOptShiftSlices3, 0);
+    if (a >= 1 && b >= 1) {
       best_s5 = std::min(a, nk);
       best_s3 = std::min(b, nk);
       best_longest = (double)std::max(5 * kfac::ceil_div(nk, best_s5), 3 * kfac::ceil_div(nk, best_s3));
@@ -850,8 +852,8 @@ bool shift_stacked(int c) { return c >= 28 && c <= 32; }
 bool shift_route_takes(int c, int h, int w) {
   int min_c = 64;
   bool stacked_on = true;
-  if (const char *env = getenv("KFAC_CONV_SHIFT")) {   // tuning override: 0 = off, else the least channel count
-    min_c = atoi(env);
+  if (kfac::option_is_set(kfac::kOptConvShift)) {   // tuning override: 0 = off, else the least channel count
+    min_c = kfac::option_int(kfac::kOptConvShift, min_c);
     if (min_c <= 0) return false;
     stacked_on = min_c <= 32;
   }
@@ -898,9 +900,9 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   const size_t edge_floats = (size_t)2 * n * c * h;
   const size_t tail_floats = array_floats + sums_floats + edge_floats + 64;
   // a workspace smaller than the route needs sends the factor to the patch-product
-  // kernels (KFAC_CONV_SHIFT_STRICT: an error instead, for the test of the workspace query)
+  // kernels (option conv_shift_strict: an error instead, for the test of the workspace query)
   auto too_small = [&](size_t need_floats) {
-    if (getenv("KFAC_CONV_SHIFT_STRICT"))
+    if (kfac::option_int(kfac::kOptConvShiftStrict, 0) != 0)
       return kfac::fail(KFAC_ENOMEM, "shifted-correlation workspace too small: %zu < %zu bytes", ws_bytes,
                         need_floats * sizeof(float));
     return 1;
@@ -1011,7 +1013,10 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   if (np != kProducts) return kfac::fail(KFAC_EINVAL, "internal: %d products", np);
   if (partial_floats >= (1ull << 32)) return 1;
   if (partial + partial_floats > arrays) return too_small(partial_floats + tail_floats + 4);
-  hipLaunchKernelGGL(edge_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums, edges);
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_COV_AUX, stream);
+    hipLaunchKernelGGL(edge_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums, edges);
+  }
   KFAC_HIP_CHECK(hipGetLastError());
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
@@ -1020,6 +1025,7 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   KFAC_HIP_CHECK(hipGetLastError());
   int max_split = 1;
   for (int i = 0; i < np; ++i) max_split = std::max(max_split, pl.prod[i].nsplit);
+  kfac::TimedLaunch timed_post(KFAC_TIMED_COV_AUX, stream);   // the two launches that follow
   if (max_split >= 32 && c <= 128) {
     const int nb = kfac::ceil_div(c, 16);
     hipLaunchKernelGGL((corr_finish_kernel<4, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
@@ -1657,21 +1663,19 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     // 64-tiles and, in a grouped launch, need not be many to fill the GPU; 64-tiles for
     // narrow factors (padding) and for short reductions over many tiles (all output
     // traffic: smaller tiles spread the stores over more workgroups).
-    // KFAC_GROUP_BM64_MAX is a tuning override.
-    int bm64_max = 160;
-    if (const char *env = getenv("KFAC_GROUP_BM64_MAX")) bm64_max = atoi(env);
+    // Option group_bm64_max is a tuning override.
+    const int bm64_max = kfac::option_int(kfac::kOptGroupBm64Max, 160);
     s.bm = (it.c <= bm64_max || nk[i] <= 4) ? 64 : 128;
     s.tiles = kfac::ceil_div(it.c, s.bm);
     s.ntile = s.tiles * (s.tiles + 1) / 2;
     kind_of[i] = (s.bm == 64 ? 0 : 4) + (s.kind == KFAC_COV_SLAB ? 0 : 2) + (s.vec ? 0 : 1);
     // Slabs of several 128-tiles with a reduction long enough to cut into slices can take
-    // the macro-tile kernel, KFAC_GROUP_MACRO=1.  Off by default: on ResNet-50 it cuts the
+    // the macro-tile kernel, option group_macro = 1.  Off by default: on ResNet-50 it cuts the
     // HBM fetch of the grouped launches by 30 % (the launches' total traffic from 1.77 to
     // 1.58 times the algorithmic bytes) at the same kernel time, but its workgroups own a
     // CU each, so they need more and shorter k-slices to balance, and the extra partial
     // tiles make the finish launch 70 us longer: 1 % of a step.
-    const char *macro_env = getenv("KFAC_GROUP_MACRO");
-    const bool macro_on = macro_env && atoi(macro_env) != 0;
+    const bool macro_on = kfac::option_int(kfac::kOptGroupMacro, 0) != 0;
     if (macro_on && s.bm == 128 && s.kind == KFAC_COV_SLAB && s.tiles >= 2 && nk[i] >= 16) {
       kind_of[i] = kMacroKind0 + (s.vec ? 0 : 1);
       const int mt = (s.tiles + 1) / 2;
@@ -1688,17 +1692,16 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
   for (int k = 0; k < kGroupKinds; ++k) {
     per_wg[k] = work[k] / 2304.0;
     if (per_wg[k] < 32.0) per_wg[k] = 32.0;
-    if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override: panel units per workgroup
-      const double v = atof(env);
+    {   // tuning override: panel units per workgroup
+      const double v = kfac::option_value(kfac::kOptGroupPanels, 0.0);
       if (v >= 1.0) per_wg[k] = v;
     }
   }
   // a macro-tile workgroup has a CU to itself: ~6 rounds of 256 (measured: fewer, longer
   // workgroups balance worse, more gain nothing), at least 8 panels each
-  // (work counted in panels per macro-tile; KFAC_GROUP_MACRO_TASKS is a tuning override)
+  // (work counted in panels per macro-tile; option group_macro_tasks is a tuning override)
   for (int k = kMacroKind0; k < kGroupKinds; ++k) {
-    double ntasks = 1536.0;
-    if (const char *env = getenv("KFAC_GROUP_MACRO_TASKS")) ntasks = std::max(1.0, atof(env));
+    const double ntasks = std::max(1.0, kfac::option_value(kfac::kOptGroupMacroTasks, 1536.0));
     per_wg[k] = std::max(8.0, work[k] / ntasks);
   }
   // A launch of several rounds of workgroups ends with the GPU draining: the last
@@ -1706,12 +1709,13 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
   // (measured on ResNet-50's launch of 128-tiles: 2.4 of 3 workgroup slots occupied on
   // average, the last 300-500 us of 1.9 ms on a half-empty GPU).  So the last third of
   // every factor's reduction is cut into slices of half the length, and those tasks go
-  // to the end of every XCD's run.  KFAC_GROUP_GRADED=0 switches this off.
+  // to the end of every XCD's run.  Option group_graded = 0 switches this off.
   bool graded_on = true;
   int graded_part = 3;   // the last 1 / graded_part of a reduction is halved
-  if (const char *env = getenv("KFAC_GROUP_GRADED")) {   // tuning override: 0 = off, n >= 2: the last n-th
-    graded_on = atoi(env) != 0;
-    if (atoi(env) >= 2) graded_part = atoi(env);
+  if (kfac::option_is_set(kfac::kOptGroupGraded)) {   // tuning override: 0 = off, n >= 2: the last n-th
+    const int v = kfac::option_int(kfac::kOptGroupGraded, 1);
+    graded_on = v != 0;
+    if (v >= 2) graded_part = v;
   }
   double ntasks_kind[kGroupKinds] = {};
   for (int i = 0; i < count; ++i) {
@@ -1785,8 +1789,8 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
   g->nftask = (int)fin.size();
   tasks.insert(tasks.end(), fin.begin(), fin.end());
   if (tasks.empty()) tasks.push_back(make_int2(0, 0));
-  int rc = g->d_items.set(g->items.data(), sizeof(GroupItemStatic) * (size_t)count, nullptr);
-  if (rc == KFAC_OK) rc = g->d_tasks.set(tasks.data(), sizeof(int2) * tasks.size(), nullptr);
+  int rc = g->d_items.set_sync(g->items.data(), sizeof(GroupItemStatic) * (size_t)count);
+  if (rc == KFAC_OK) rc = g->d_tasks.set_sync(tasks.data(), sizeof(int2) * tasks.size());
   if (rc != KFAC_OK) {
     delete g;
     return rc;
@@ -1861,6 +1865,7 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (group->nftask > 0) {
+    kfac::TimedLaunch timed(KFAC_TIMED_COV_AUX, s);
     hipLaunchKernelGGL(finish_group_kernel, dim3(group->nftask), dim3(256), 0, s, st, dy,
                        tasks + group->ftask0, base);
     KFAC_HIP_CHECK(hipGetLastError());

@@ -78,8 +78,8 @@ extern "C" int kfac_damp_plan_create(int count, const int32_t *dimsA, const int3
   auto *p = new (std::nothrow) kfac_damp_plan;
   if (!p) return kfac::fail(KFAC_ENOMEM, "out of host memory");
   p->count = count;
-  int rc = p->d_dA.set(dimsA, sizeof(int) * count, nullptr);
-  if (rc == KFAC_OK) rc = p->d_dG.set(dimsG, sizeof(int) * count, nullptr);
+  int rc = p->d_dA.set_sync(dimsA, sizeof(int) * count);
+  if (rc == KFAC_OK) rc = p->d_dG.set_sync(dimsG, sizeof(int) * count);
   if (rc != KFAC_OK) {
     delete p;
     return rc;

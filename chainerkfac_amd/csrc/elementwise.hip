@@ -1,6 +1,10 @@
 // Small bandwidth-bound helpers of the K-FAC step: axpby (moving average and
 // unfused accumulation), diagonal damping and the momentum update rule.
+#include <cctype>
+#include <cstdlib>
+#include <mutex>
 #include <new>
+#include <string>
 #include <vector>
 
 #include "common.h"
@@ -26,20 +30,21 @@ double g_total_ms[KFAC_TIMED_FAMILIES];
 
 bool timing_on() { return g_timing; }
 
-void timing_begin(int family, hipStream_t stream) {
+int timing_begin(int family, hipStream_t stream) {
   TimedRec r;
   r.family = family;
-  if (hipEventCreate(&r.start) != hipSuccess) return;
+  if (hipEventCreate(&r.start) != hipSuccess) return -1;
   if (hipEventCreate(&r.stop) != hipSuccess) {
     (void)hipEventDestroy(r.start);
-    return;
+    return -1;
   }
   (void)hipEventRecord(r.start, stream);
   g_open.push_back(r);
+  return (int)g_open.size() - 1;
 }
 
-void timing_end(hipStream_t stream) {
-  if (!g_open.empty()) (void)hipEventRecord(g_open.back().stop, stream);
+void timing_end(int index, hipStream_t stream) {
+  if (index >= 0 && index < (int)g_open.size()) (void)hipEventRecord(g_open[index].stop, stream);
 }
 
 static void timing_collect() {
@@ -76,6 +81,82 @@ extern "C" int kfac_timing_read(int family, int64_t *launches, double *total_ms)
   *launches = kfac::g_launches[family];
   *total_ms = kfac::g_total_ms[family];
   return KFAC_OK;
+}
+
+namespace kfac {
+namespace {
+const char *const kOptionNames[kOptCount] = {
+    "syrk_bm64_max",   "syrk_splits",      "conv_rows",       "rows_wm",          "shift_slices5",
+    "shift_slices3",   "conv_shift",       "conv_shift_strict", "group_bm64_max", "group_macro",
+    "group_panels",    "group_macro_tasks", "group_graded",   "inverse_group",    "inverse_border",
+    "inverse_lookahead", "inverse_rest_lds", "inverse_align", "precond_tasks",    "bn_stats_loop"};
+struct OptionState {
+  bool set[kOptCount] = {};
+  double value[kOptCount] = {};
+};
+OptionState &option_state() {
+  static OptionState st;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    for (int i = 0; i < kOptCount; ++i) {
+      std::string env = "KFAC_";
+      for (const char *c = kOptionNames[i]; *c; ++c) env += (char)toupper((unsigned char)*c);
+      if (const char *v = getenv(env.c_str())) {
+        char *end = nullptr;
+        const double x = strtod(v, &end);
+        if (end != v) {
+          st.set[i] = true;
+          st.value[i] = x;
+        }
+      }
+    }
+  });
+  return st;
+}
+int option_index(const char *name) {
+  if (name)
+    for (int i = 0; i < kOptCount; ++i)
+      if (strcmp(name, kOptionNames[i]) == 0) return i;
+  return -1;
+}
+}  // namespace
+bool option_is_set(Option o) { return option_state().set[o]; }
+double option_value(Option o, double unset_value) {
+  const OptionState &st = option_state();
+  return st.set[o] ? st.value[o] : unset_value;
+}
+}  // namespace kfac
+
+extern "C" int kfac_option_set(const char *name, double value) {
+  const int i = kfac::option_index(name);
+  KFAC_REQUIRE(i >= 0, "unknown option '%s'", name ? name : "(null)");
+  kfac::OptionState &st = kfac::option_state();
+  st.set[i] = true;
+  st.value[i] = value;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_option_unset(const char *name) {
+  const int i = kfac::option_index(name);
+  KFAC_REQUIRE(i >= 0, "unknown option '%s'", name ? name : "(null)");
+  kfac::option_state().set[i] = false;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_option_get(const char *name, double *value, int *is_set) {
+  const int i = kfac::option_index(name);
+  KFAC_REQUIRE(i >= 0, "unknown option '%s'", name ? name : "(null)");
+  KFAC_REQUIRE(value && is_set, "null pointer");
+  const kfac::OptionState &st = kfac::option_state();
+  *is_set = st.set[i] ? 1 : 0;
+  *value = st.set[i] ? st.value[i] : 0.0;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_option_count(void) { return kfac::kOptCount; }
+
+extern "C" const char *kfac_option_name(int index) {
+  return index >= 0 && index < kfac::kOptCount ? kfac::kOptionNames[index] : nullptr;
 }
 
 extern "C" int kfac_abi_version(void) { return KFAC_ABI_VERSION; }

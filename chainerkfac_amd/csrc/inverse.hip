@@ -912,8 +912,8 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     KFAC_REQUIRE(dims[i] > 0 && dims[i] <= 46340, "matrix %d: bad dimension %d", i, dims[i]);
   auto *p = new (std::nothrow) kfac_inverse_plan;
   if (!p) return kfac::fail(KFAC_ENOMEM, "out of host memory");
-  if (const char *e = getenv("KFAC_INVERSE_GROUP")) {   // tuning override
-    const int g = atoi(e);
+  {   // tuning override
+    const int g = kfac::option_int(kfac::kOptInverseGroup, p->group);
     if (g >= 1 && g <= 64) p->group = g;
   }
   p->count = count;
@@ -926,9 +926,8 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   p->nt.resize(count);
   size_t total = 0;
   // matrices of 128 m + 1 rows are inverted from their leading 128 m x 128 m block
-  // (KFAC_INVERSE_BORDER=0 tiles them whole, for comparisons)
-  bool border_on = true;
-  if (const char *e = getenv("KFAC_INVERSE_BORDER")) border_on = atoi(e) != 0;
+  // (option inverse_border = 0 tiles them whole, for comparisons)
+  const bool border_on = kfac::option_int(kfac::kOptInverseBorder, 1) != 0;
   std::vector<int> core(count);
   std::vector<long long> vec_off(count, -1);
   std::vector<int> border_slots;
@@ -957,14 +956,14 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   std::vector<int2> natural;
   p->with_diag.resize(p->max_t);
   p->rest.resize(p->max_t);
-  if (const char *e = getenv("KFAC_INVERSE_LOOKAHEAD")) p->lookahead = atoi(e) != 0;
+  p->lookahead = kfac::option_int(kfac::kOptInverseLookahead, 1) != 0;
   // The rest asks for more LDS than it uses, 81 KB: then one of its workgroups
   // fits a CU, not two, and a step or panel workgroup always finds room beside
   // it instead of queueing behind the rest for a slot (measured: the rest alone
-  // loses 14 %, the sweep as a whole gains).  KFAC_INVERSE_REST_LDS overrides.
+  // loses 14 %, the sweep as a whole gains).  Option inverse_rest_lds overrides.
   p->rest_lds = kRestLdsBytes;
-  if (const char *e = getenv("KFAC_INVERSE_REST_LDS")) {
-    const long v = atol(e);
+  {
+    const long v = (long)kfac::option_value(kfac::kOptInverseRestLds, 0.0);
     if (v >= (long)kTileLdsBytes && v <= 160 * 1024) p->rest_lds = (size_t)v;
   }
   auto pack = [](int s, int a, int b) { return make_int2(s, a | (b << 16)); };
@@ -973,10 +972,10 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   // beside the late steps of the largest ones, which on their own leave most of
   // the GPU idle (few tiles, one dependent launch after another); aligning the
   // starts piles all matrices onto the early steps, which are the ones that are
-  // already throughput-bound.  KFAC_INVERSE_ALIGN=<percent> (0 = starts, 100 =
+  // already throughput-bound.  Option inverse_align = <percent> (0 = starts, 100 =
   // ends) is a tuning override.
   int align = 100;
-  if (const char *e = getenv("KFAC_INVERSE_ALIGN")) align = std::min(100, std::max(0, atoi(e)));
+  align = std::min(100, std::max(0, kfac::option_int(kfac::kOptInverseAlign, align)));
   std::vector<int> shift(count);
   for (int s = 0; s < count; ++s) shift[s] = (p->max_t - p->nt[s]) * align / 100;
   std::vector<BorderTask> btasks;
@@ -1183,7 +1182,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   if (tasks.empty()) tasks.push_back(TileTask{0, 0, 0, 0, 0});
   int rc = KFAC_OK;
   auto up = [&](kfac::DevTable &t, const void *h, size_t b) {
-    if (rc == KFAC_OK) rc = t.set(h, b, nullptr);
+    if (rc == KFAC_OK) rc = t.set_sync(h, b);
   };
   up(p->d_dim, dim.data(), sizeof(int) * count);
   up(p->d_core, core.data(), sizeof(int) * count);
@@ -1298,6 +1297,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.ws = reinterpret_cast<float *>(base);
   tb.info = info_dev;
 
+  kfac::TimedLaunch timed_call(KFAC_TIMED_INV_CALL, s);   // copy-in to the final product (the side streams rejoin `s`)
   hipLaunchKernelGGL(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
   KFAC_HIP_CHECK(hipGetLastError());
   // Side stream: after the last column of a group, the rest of its trailing

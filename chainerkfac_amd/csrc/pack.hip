@@ -414,9 +414,8 @@ extern "C" int kfac_pack_plan_create(int n_arrays, const void *const *ptrs,
   p->unpack_units = (int)uunits;
   p->ptrs.assign(ptrs, ptrs + n_arrays);
   int rc = KFAC_OK;
-  hipStream_t s = nullptr;
   auto up = [&](kfac::DevTable &t, const void *h, size_t b) {
-    if (rc == KFAC_OK) rc = t.set(h, b, s);
+    if (rc == KFAC_OK) rc = t.set_sync(h, b);
   };
   up(p->d_ptrs, p->ptrs.data(), sizeof(void *) * n_arrays);
   up(p->d_tri, tri.data(), sizeof(int) * n_arrays);

@@ -159,13 +159,10 @@ LoaderKS<ROWS, VEC> colop_ks(const float *base, long long ld, int rows_valid, co
   return l;
 }
 
-// y = F g with g = [g0 ; g1]; one wave per row.
-__global__ __launch_bounds__(256) void gemv_kernel(const float *__restrict__ F, int d,
-                                                   const float *__restrict__ g0, int n0,
-                                                   const float *__restrict__ g1,
-                                                   float *__restrict__ y) {
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= d) return;
+// Row `row` of y = F g with g = [g0 ; g1], by one wave (the result is valid in lane 0).
+__device__ __forceinline__ float gemv_row(const float *__restrict__ F, int d, int row,
+                                          const float *__restrict__ g0, int n0,
+                                          const float *__restrict__ g1) {
   const int lane = threadIdx.x & 63;
   const float *fr = F + (long long)row * d;
   float acc = 0.f;
@@ -193,16 +190,25 @@ __global__ __launch_bounds__(256) void gemv_kernel(const float *__restrict__ F, 
     for (int j = lane; j < d; j += 64) acc += fr[j] * (j < n0 ? g0[j] : g1[j - n0]);
   }
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o, 64);
-  if (lane == 0) y[row] = acc;
+  return acc;
+}
+
+// y = F g with g = [g0 ; g1]; one wave per row.
+__global__ __launch_bounds__(256) void gemv_kernel(const float *__restrict__ F, int d,
+                                                   const float *__restrict__ g0, int n0,
+                                                   const float *__restrict__ g1,
+                                                   float *__restrict__ y) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= d) return;
+  const float acc = gemv_row(F, d, row, g0, n0, g1);
+  if ((threadIdx.x & 63) == 0) y[row] = acc;
 }
 
 // One workgroup: if any y is NaN the outputs are the raw gradients.
-__global__ __launch_bounds__(1024) void bn_select_kernel(const float *__restrict__ y, int d,
-                                                         const float *__restrict__ g0, int n0,
-                                                         const float *__restrict__ g1,
-                                                         float *__restrict__ k0,
-                                                         float *__restrict__ k1,
-                                                         int *__restrict__ flag) {
+__device__ __forceinline__ void bn_select(const float *__restrict__ y, int d,
+                                          const float *__restrict__ g0, int n0,
+                                          const float *__restrict__ g1, float *__restrict__ k0,
+                                          float *__restrict__ k1, int *__restrict__ flag) {
   __shared__ int any;
   if (threadIdx.x == 0) any = 0;
   __syncthreads();
@@ -218,6 +224,43 @@ __global__ __launch_bounds__(1024) void bn_select_kernel(const float *__restrict
       k1[i - n0] = bad ? g1[i - n0] : y[i];
   }
   if (flag && threadIdx.x == 0) *flag = bad;
+}
+
+__global__ __launch_bounds__(1024) void bn_select_kernel(const float *__restrict__ y, int d,
+                                                         const float *__restrict__ g0, int n0,
+                                                         const float *__restrict__ g1,
+                                                         float *__restrict__ k0,
+                                                         float *__restrict__ k1,
+                                                         int *__restrict__ flag) {
+  bn_select(y, d, g0, n0, g1, k0, k1, flag);
+}
+
+// The same two kernels over a list of batch-norm blocks: a unit is four rows of
+// one block's product (one wave per row, the single-block kernel's arithmetic),
+// the selection takes one workgroup per block.
+struct BnPreItem {
+  const float *F, *g0, *g1;
+  float *k0, *k1;
+  int *flag;
+  long long y_off;   // floats from the workspace base
+  int d, n0;
+};
+
+__global__ __launch_bounds__(256) void gemv_batched_kernel(const BnPreItem *__restrict__ items,
+                                                           const int2 *__restrict__ units,
+                                                           float *__restrict__ ws) {
+  const int2 u = units[blockIdx.x];   // (item, first row)
+  const BnPreItem it = items[u.x];
+  const int row = u.y + (threadIdx.x >> 6);
+  if (row >= it.d) return;
+  const float acc = gemv_row(it.F, it.d, row, it.g0, it.n0, it.g1);
+  if ((threadIdx.x & 63) == 0) ws[it.y_off + row] = acc;
+}
+
+__global__ __launch_bounds__(1024) void bn_select_batched_kernel(const BnPreItem *__restrict__ items,
+                                                                 const float *__restrict__ ws) {
+  const BnPreItem it = items[blockIdx.x];
+  bn_select(ws + it.y_off, it.d, it.g0, it.n0, it.g1, it.k0, it.k1, it.flag);
 }
 
 template <class LA64, class LB64, class LA128, class LB128>
@@ -240,6 +283,7 @@ int launch_gemm(const LA64 &a64, const LB64 &b64, const LA128 &a128, const LB128
   KFAC_HIP_CHECK(hipGetLastError());
   if (part) {
     const long long total = (long long)M * N;
+    kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, stream);
     hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)kfac::ceil_div<long long>(total, 256)),
                        dim3(256), 0, stream, part, p.nsplit, ntiles, p.tn, 64 * p.w, M, N, C0, ld0,
                        n_main, C1);
@@ -364,6 +408,7 @@ extern "C" int kfac_precond_bn_static_f32(const float *Finv, int d, const float 
   hipStream_t s = kfac::as_stream(stream);
   // y[0, d) is written in full by the product before the selection reads it, so
   // nothing of an earlier call's contents is ever seen and nothing needs clearing
+  kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
   hipLaunchKernelGGL(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
                      n_gamma, g_beta, y);
   hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
@@ -389,10 +434,78 @@ extern "C" int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamm
     return kfac::fail(KFAC_ENOMEM, "batch-norm preconditioning workspace too small");
   hipStream_t s = kfac::as_stream(stream);
   float *y = static_cast<float *>(ws);
+  kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
   hipLaunchKernelGGL(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
                      n_gamma, g_beta, y);
   hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
                      kf_gamma, kf_beta, nan_flag_dev);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+struct kfac_precond_bn_batch {
+  std::vector<BnPreItem> items;
+  std::vector<int2> units;
+  kfac::DevTableRing item_table;
+  kfac::DevTable unit_table;
+};
+
+extern "C" int kfac_precond_bn_batch_create(kfac_precond_bn_batch_t *batch_out) {
+  KFAC_REQUIRE(batch_out != nullptr, "batch_out is null");
+  *batch_out = new (std::nothrow) kfac_precond_bn_batch;
+  return *batch_out ? KFAC_OK : kfac::fail(KFAC_ENOMEM, "out of host memory");
+}
+
+extern "C" int kfac_precond_bn_batch_destroy(kfac_precond_bn_batch_t batch) {
+  delete batch;
+  return KFAC_OK;
+}
+
+extern "C" size_t kfac_precond_bn_batched_workspace_bytes(int count, const int32_t *dims) {
+  size_t floats = 0;
+  for (int i = 0; i < count; ++i)
+    if (dims && dims[i] > 0) floats += ((size_t)dims[i] + 3) / 4 * 4;
+  return floats * sizeof(float);
+}
+
+extern "C" int kfac_precond_bn_batched_f32(kfac_precond_bn_batch_t batch, int count,
+                                           const float *const *Finv, const int32_t *dims,
+                                           const float *const *g_gamma, const int32_t *n_gamma,
+                                           const float *const *g_beta, float *const *kf_gamma,
+                                           float *const *kf_beta, int32_t *const *nan_flags,
+                                           void *ws, size_t ws_bytes, void *stream) {
+  KFAC_REQUIRE(batch != nullptr, "batch is null");
+  KFAC_REQUIRE(count >= 0, "count < 0");
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(Finv && dims && g_gamma && n_gamma && g_beta && kf_gamma && kf_beta, "null table");
+  if (ws == nullptr || ws_bytes < kfac_precond_bn_batched_workspace_bytes(count, dims))
+    return kfac::fail(KFAC_ENOMEM, "batch-norm preconditioning workspace too small");
+  batch->items.resize(count);
+  batch->units.clear();
+  long long off = 0;
+  for (int i = 0; i < count; ++i) {
+    const int d = dims[i], n0 = n_gamma[i];
+    KFAC_REQUIRE(d > 0 && n0 >= 0 && n0 <= d, "block %d: sizes %d of %d", i, n0, d);
+    KFAC_REQUIRE(Finv[i] != nullptr, "block %d: Finv is null", i);
+    KFAC_REQUIRE(n0 == 0 || (g_gamma[i] && kf_gamma[i]), "block %d: gamma pointers are null", i);
+    KFAC_REQUIRE(n0 == d || (g_beta[i] && kf_beta[i]), "block %d: beta pointers are null", i);
+    batch->items[i] = BnPreItem{Finv[i],     g_gamma[i], g_beta[i], kf_gamma[i],
+                                kf_beta[i],  nan_flags ? nan_flags[i] : nullptr,
+                                off,         d,          n0};
+    off += ((long long)d + 3) / 4 * 4;
+    for (int r = 0; r < d; r += 4) batch->units.push_back(make_int2(i, r));
+  }
+  hipStream_t s = kfac::as_stream(stream);
+  const void *d_items = nullptr;
+  if (int rc = batch->item_table.set(batch->items.data(), sizeof(BnPreItem) * (size_t)count, s, &d_items))
+    return rc;
+  if (int rc = batch->unit_table.set(batch->units.data(), sizeof(int2) * batch->units.size(), s)) return rc;
+  kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
+  hipLaunchKernelGGL(gemv_batched_kernel, dim3((unsigned)batch->units.size()), dim3(256), 0, s,
+                     static_cast<const BnPreItem *>(d_items), batch->unit_table.as<const int2>(),
+                     static_cast<float *>(ws));
+  hipLaunchKernelGGL(bn_select_batched_kernel, dim3(count), dim3(1024), 0, s,
+                     static_cast<const BnPreItem *>(d_items), static_cast<const float *>(ws));
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
@@ -620,13 +733,12 @@ extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int
       // time of the six launches / whole phase with its finish launches): 2304 tasks 1.89 /
       // 2.04 ms, 3072 1.69 / 1.95, 4608 1.61 / 1.97, 6144 1.60 / 2.02, 9216 1.61 / 2.11: shorter
       // tasks shorten the tail of a launch, more k-slices lengthen the finish.
-      // KFAC_PRECOND_TASKS is a tuning override.
-      double ntasks = 4096.0;
-      if (const char *env = getenv("KFAC_PRECOND_TASKS")) ntasks = std::max(1.0, atof(env));
+      // Option precond_tasks is a tuning override.
+      const double ntasks = std::max(1.0, kfac::option_value(kfac::kOptPrecondTasks, 4096.0));
       per_wg[k] = work[p][k] / ntasks;
       if (per_wg[k] < 32.0) per_wg[k] = 32.0;
-      if (const char *env = getenv("KFAC_GROUP_PANELS")) {   // tuning override
-        const double val = atof(env);
+      {   // tuning override
+        const double val = kfac::option_value(kfac::kOptGroupPanels, 0.0);
         if (val >= 1.0) per_wg[k] = val;
       }
     }
@@ -669,8 +781,8 @@ extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int
     tasks.insert(tasks.end(), fin[p].begin(), fin[p].end());
   }
   if (tasks.empty()) tasks.push_back(make_int2(0, 0));
-  int rc = g->d_items.set(g->items.data(), sizeof(PreStatic) * (size_t)count, nullptr);
-  if (rc == KFAC_OK) rc = g->d_tasks.set(tasks.data(), sizeof(int2) * tasks.size(), nullptr);
+  int rc = g->d_items.set_sync(g->items.data(), sizeof(PreStatic) * (size_t)count);
+  if (rc == KFAC_OK) rc = g->d_tasks.set_sync(tasks.data(), sizeof(int2) * tasks.size());
   if (rc != KFAC_OK) {
     delete g;
     return rc;
@@ -734,6 +846,7 @@ extern "C" int kfac_precond_group_run_f32(kfac_precond_group_t group, const floa
     }
     KFAC_HIP_CHECK(hipGetLastError());
     if (group->nftask[p] > 0) {
+      kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
       if (p == 0)
         hipLaunchKernelGGL(gemm_group_finish_kernel<0>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
                            tasks + group->ftask0[p], base);

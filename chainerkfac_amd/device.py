@@ -1,5 +1,7 @@
 """Device-memory plumbing: torch-ROCm tensors carry the buffers, raw pointers go
 to the C ABI.  Nothing here computes."""
+import threading
+
 import torch
 
 from . import _lib
@@ -26,7 +28,9 @@ def ptr(t):
 def stream_handle(stream=None):
     """hipStream_t (as int) of ``stream`` or of torch's current stream."""
     if stream is None:
-        stream = torch.cuda.current_stream()
+        # the raw handle without building a torch.cuda.Stream object (this is on the path of
+        # every kernel launch)
+        return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
     if isinstance(stream, int):
         return stream
     return stream.cuda_stream
@@ -48,22 +52,28 @@ class Workspace(object):
         return self._buf
 
 
+# Scratch buffers of work queued on the caller's own stream (no lane), by kind.
 _default_workspaces = {}
-_current_lane = None   # index of the lane whose work is being queued (None: the caller's stream)
+# The lane whose work is being queued by this thread: (Lanes object, lane index) or None.
+_queueing = threading.local()
 
 
 def current_lane():
     """Index of the lane whose work is being queued, None on the caller's stream."""
-    return _current_lane
+    cur = getattr(_queueing, 'lane', None)
+    return None if cur is None else cur[1]
 
 
 def workspace(kind, nbytes, device):
     """Scratch buffer of ``kind`` for the lane being queued on (work on
-    different lanes runs concurrently and must not share scratch memory)."""
-    key = (kind, _current_lane)
-    ws = _default_workspaces.get(key)
+    different lanes runs concurrently and must not share scratch memory; the
+    lanes of different ``Lanes`` objects are different streams and have their
+    own buffers)."""
+    cur = getattr(_queueing, 'lane', None)
+    table, key = (_default_workspaces, kind) if cur is None else (cur[0].workspaces, (kind, cur[1]))
+    ws = table.get(key)
     if ws is None:
-        ws = _default_workspaces[key] = Workspace()
+        ws = table[key] = Workspace()
     return ws.get(nbytes, device)
 
 
@@ -75,19 +85,22 @@ class Lanes(object):
     when they share a stream.  ``run`` deals such work onto ``n`` streams in
     turn; every piece first waits for what the caller's stream has queued so far
     (its inputs), and ``join`` makes the caller's stream wait for all of it.
-    With ``n`` = 0 everything runs on the caller's stream.
+    With ``n`` = 0 everything runs on the caller's stream.  The scratch buffers
+    of the work queued on a lane belong to this object.
     """
 
     def __init__(self, n=0):
         self.n = int(n)
+        self.workspaces = {}
         self._streams = {}
         self._turn = 0
         self._busy = []
 
     def _pool(self, device):
         pool = self._streams.get(device)
-        if pool is None:
-            pool = self._streams[device] = [torch.cuda.Stream(device=device) for _ in range(self.n)]
+        if pool is None or len(pool) < self.n:
+            pool = self._streams[device] = (pool or []) + [
+                torch.cuda.Stream(device=device) for _ in range(self.n - len(pool or []))]
         return pool
 
     def run(self, fn, tensors=()):
@@ -98,18 +111,18 @@ class Lanes(object):
             return fn()
         main = torch.cuda.current_stream()
         pool = self._pool(main.device)
-        global _current_lane
         index = self._turn % self.n
         lane = pool[index]
         self._turn += 1
         lane.wait_stream(main)
-        outer = _current_lane
-        _current_lane = index
+        outer = getattr(_queueing, 'lane', None)
+        _queueing.lane = (self, index)
+        torch.cuda.set_stream(lane)
         try:
-            with torch.cuda.stream(lane):
-                out = fn()
+            out = fn()
         finally:
-            _current_lane = outer
+            torch.cuda.set_stream(main)
+            _queueing.lane = outer
         for t in tensors:
             if isinstance(t, torch.Tensor) and t.is_cuda:
                 t.record_stream(lane)

@@ -637,6 +637,69 @@ def precond_bn(Finv, g_gamma, g_beta, kf_gamma=None, kf_beta=None, nan_flag=None
     return kf_gamma, kf_beta, nan_flag
 
 
+class _PrecondBnBatch(object):
+    def __init__(self):
+        h = ctypes.c_void_p()
+        _lib.check(_lib.load().kfac_precond_bn_batch_create(ctypes.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        try:
+            h, self._h = self._h, None
+            if h is not None:
+                _lib._lib.kfac_precond_bn_batch_destroy(h)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+
+_precond_bn_batches = None
+
+
+def precond_bn_batched(Finvs, g_gammas, g_betas, kf_gammas, kf_betas, nan_flags, stream=None):
+    """``precond_bn`` for a list of batch-norm blocks in two launches.  Every list has one
+    entry per block; gradient / output entries may be None where a block has no gamma or
+    no beta; ``nan_flags`` entries are one-element int32 tensors."""
+    global _precond_bn_batches
+    n = len(Finvs)
+    if not (len(g_gammas) == len(g_betas) == len(kf_gammas) == len(kf_betas) == len(nan_flags) == n):
+        raise ValueError('one entry per block in every list')
+    if n == 0:
+        return
+    dims, n0s = [], []
+    for F, g, b, kg, kb, flag in zip(Finvs, g_gammas, g_betas, kf_gammas, kf_betas, nan_flags):
+        _dev.require_gpu_tensor(F, 'Finv')
+        d = F.shape[0]
+        ng = 0 if g is None else g.numel()
+        nb = 0 if b is None else b.numel()
+        if F.ndim != 2 or F.shape[1] != d or ng + nb != d:
+            raise ValueError('gradient sizes {}+{} do not match Finv {}'.format(ng, nb, tuple(F.shape)))
+        for t, out, nm in ((g, kg, 'gamma'), (b, kb, 'beta')):
+            if t is not None:
+                _dev.require_gpu_tensor(t, 'g_' + nm)
+                _dev.require_gpu_tensor(out, 'kf_' + nm)
+                if out.numel() != t.numel():
+                    raise ValueError('kf_{} does not match its gradient'.format(nm))
+        if flag is not None:
+            _dev.require_gpu_tensor(flag, 'nan_flag', dtype=torch.int32)
+        dims.append(d)
+        n0s.append(ng)
+    if _precond_bn_batches is None:
+        _precond_bn_batches = _PlanCache(16)
+    # one batch object per list of inverses and outputs (persistent); gradient arrays may move
+    key = tuple(t.data_ptr() for t in Finvs) + tuple(_dev.ptr(t) for t in kf_gammas) + \
+        tuple(_dev.ptr(t) for t in kf_betas)
+    batch = _precond_bn_batches.get(key, _PrecondBnBatch)
+    lib = _lib.load()
+    dims_arr = _lib.i32_array(dims)
+    ws = _dev.workspace('precond_bn', lib.kfac_precond_bn_batched_workspace_bytes(n, dims_arr), Finvs[0].device)
+    _lib.check(lib.kfac_precond_bn_batched_f32(
+        batch._h, n, _lib.ptr_array([t.data_ptr() for t in Finvs]), dims_arr,
+        _lib.ptr_array([_dev.ptr(t) for t in g_gammas]), _lib.i32_array(n0s),
+        _lib.ptr_array([_dev.ptr(t) for t in g_betas]), _lib.ptr_array([_dev.ptr(t) for t in kf_gammas]),
+        _lib.ptr_array([_dev.ptr(t) for t in kf_betas]), _lib.ptr_array([_dev.ptr(t) for t in nan_flags]),
+        ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
+
+
 def momentum_update(param, v, grad, lr, momentum, stream=None):
     """v = momentum*v - lr*grad; param += v (in place)."""
     for t in (param, v, grad):

@@ -88,6 +88,9 @@ class FisherBlock(object):
         #: ops.PendingCovs of the optimizer, or None: where the factors of small
         #: layers wait for one grouped launch instead of being computed on the spot
         self.pending_covs = None
+        #: device.Lanes of the optimizer, or None: side streams for the kernels this
+        #: block launches on its own (they are independent of other layers' work)
+        self.lanes = None
         self._bufs = {}
 
     # ---- identity -------------------------------------------------------
@@ -158,6 +161,12 @@ class FisherBlock(object):
             return (self._buffer('acc_' + key, shape, device), scale / acc_iters,
                     0.0 if acc_index == 0 else 1.0)
         return self._buffer(key, shape, device), scale, 0.0
+
+    def _on_lane(self, fn, tensors=()):
+        """Runs ``fn`` (kernel launches that read ``tensors``) on the next side stream."""
+        if self.lanes is None:
+            return fn()
+        return self.lanes.run(fn, tensors)
 
     def _defer_cov(self, kind, x, ones, rows, out, alpha, beta, stride=1):
         """Hands a factor to the grouped launch if there is one and the factor

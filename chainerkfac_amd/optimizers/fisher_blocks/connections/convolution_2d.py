@@ -28,7 +28,7 @@ class FisherBlockConvolution2D(FisherBlockConnection):
             ho, wo = (x.shape[2] - 1) // stride + 1, (x.shape[3] - 1) // stride + 1
             if self._defer_cov(ops.COV_SLAB, x, has_b, n * ho * wo, out, alpha, beta, stride):
                 return out
-        return ops.cov_conv_a(x, ksize, stride, pad, has_b, alpha, beta, out)
+        return self._on_lane(lambda: ops.cov_conv_a(x, ksize, stride, pad, has_b, alpha, beta, out), (x,))
 
     def compute_G(self, in_data, out_grad_data):
         gy = as_float32(out_grad_data[0])
@@ -39,4 +39,4 @@ class FisherBlockConvolution2D(FisherBlockConnection):
         out, alpha, beta = self._cov_target('G', (c, c), gy.device, scale)
         if self._defer_cov(ops.COV_SLAB, gy, False, n * ho * wo, out, alpha, beta):
             return out
-        return ops.cov_conv_g(gy, alpha, beta, out)
+        return self._on_lane(lambda: ops.cov_conv_g(gy, alpha, beta, out), (gy,))

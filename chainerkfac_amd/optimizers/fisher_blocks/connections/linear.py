@@ -20,7 +20,7 @@ class FisherBlockLinear(FisherBlockConnection):
         out, alpha, beta = self._cov_target('A', (d, d), x.device, 1.0 / n)
         if self._defer_cov(ops.COV_LINEAR, x, has_b, n, out, alpha, beta):
             return out
-        return ops.cov_linear(x, has_b, alpha, beta, out)
+        return self._on_lane(lambda: ops.cov_linear(x, has_b, alpha, beta, out), (x,))
 
     def compute_G(self, in_data, out_grad_data):
         gy = as_float32(out_grad_data[0])
@@ -29,4 +29,4 @@ class FisherBlockLinear(FisherBlockConnection):
         out, alpha, beta = self._cov_target('G', (d_out, d_out), gy.device, scale)
         if self._defer_cov(ops.COV_LINEAR, gy, False, n, out, alpha, beta):
             return out
-        return ops.cov_linear(gy, False, alpha, beta, out)
+        return self._on_lane(lambda: ops.cov_linear(gy, False, alpha, beta, out), (gy,))

@@ -96,13 +96,25 @@ class FisherBlockBatchNormalization(FisherBlock):
         has_gamma = self.link.gamma is not None
         has_beta = self.link.beta is not None
         width = x.shape[1] * (int(has_gamma) + int(has_beta))
-        U = ops.bn_grad_matrix(x, gy, self.link.eps, gy_scale, has_gamma, has_beta,
-                               out=self._buffer('U', (n, width), x.device))
+        U = self._buffer('U', (n, width), x.device)
         self._U = U
         out, alpha, beta = self._cov_target('F', (width, width), x.device, 1.0 / n)
-        if self._defer_cov(ops.COV_LINEAR, U, False, n, out, alpha, beta):
+        eps = self.link.eps
+
+        def stats():
+            ops.bn_grad_matrix(x, gy, eps, gy_scale, has_gamma, has_beta, out=U)
+
+        if self.pending_covs is not None and self.pending_covs.accepts(n, width):
+            self._on_lane(stats, (x, gy))
+            self._defer_cov(ops.COV_LINEAR, U, False, n, out, alpha, beta)
             return out
-        return ops.cov_linear(U, False, alpha, beta, out)
+
+        def stats_and_factor():
+            stats()
+            ops.cov_linear(U, False, alpha, beta, out)
+
+        self._on_lane(stats_and_factor, (x, gy))
+        return out
 
     def update_cov_emas(self):
         first = self.cov_emas is None
@@ -174,19 +186,30 @@ class FisherBlockBatchNormalization(FisherBlock):
         F, v0, v1, split = self.damp_args()
         ops.add_diag(F, v0, v1, split=split)
 
-    def update_kfgrads(self):
+    def kfgrad_operands(self):
+        """``(F_inv, g_gamma, g_beta, kf_gamma, kf_beta, nan_flag)`` of the preconditioning
+        product, with the output buffers this block keeps."""
         self.check_attr('invs')
         gamma, beta = self.link.gamma, self.link.beta
-        g = None if gamma is None else as_float32(gamma.grad)
-        b = None if beta is None else as_float32(beta.grad)
+
+        def grad_of(param):
+            if param is None:
+                return None
+            g = as_float32(param.grad)
+            return g if g.is_contiguous() else g.contiguous()
+
         kg = None if gamma is None else self._buffer('kf_gamma', gamma.shape, gamma.data.device)
         kb = None if beta is None else self._buffer('kf_beta', beta.shape, beta.data.device)
         if self.nan_flag is None:
             import torch
             self.nan_flag = torch.zeros(1, dtype=torch.int32, device=self.invs[0].device)
-        # NaN anywhere in F^-1 grad makes the kernel hand back the raw gradients
-        ops.precond_bn(self.invs[0], g, b, kg, kb, self.nan_flag)
-        # kfgrad in the gradient's own type (reference batch_normalization.py:185-193)
+        return self.invs[0], grad_of(gamma), grad_of(beta), kg, kb, self.nan_flag
+
+    def finish_kfgrads(self):
+        """After the product: ``kfgrad`` in the gradient's own type (reference
+        batch_normalization.py:185-193)."""
+        gamma, beta = self.link.gamma, self.link.beta
+        kg, kb = self._bufs.get('kf_gamma'), self._bufs.get('kf_beta')
         if gamma is not None:
             gamma.kfgrad = kg if gamma.grad.dtype == kg.dtype else kg.to(gamma.grad.dtype)
         if beta is not None:
@@ -197,6 +220,11 @@ class FisherBlockBatchNormalization(FisherBlock):
         # next step.  ``link.debug`` asks for the immediate warning.
         if self.debug():
             self.warn_if_nan()
+
+    def update_kfgrads(self):
+        # NaN anywhere in F^-1 grad makes the kernel hand back the raw gradients
+        ops.precond_bn(*self.kfgrad_operands())
+        self.finish_kfgrads()
 
     def warn_if_nan(self):
         if self.nan_flag is not None and int(self.nan_flag.item()):

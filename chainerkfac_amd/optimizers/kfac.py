@@ -84,6 +84,7 @@ class KFACHook(links.FunctionHook):
         self._owner = {}
         for fb in fblocks:
             fb.pending_covs = pending
+            fb.lanes = lanes
             for p in fb.link.params():
                 self._owner[id(p.data)] = fb
 
@@ -94,21 +95,17 @@ class KFACHook(links.FunctionHook):
                 return fb
         return None
 
-    def _run(self, fn, tensors):
-        if self.lanes is None:
-            return fn()
-        return self.lanes.run(fn, tensors)
-
+    # The blocks deal the kernels they launch themselves onto the lanes; a factor that
+    # only joins the grouped launch costs its hook call no stream switch.
     def forward_postprocess(self, func, in_data):
         fb = self._find(func, in_data)
         if fb is not None:
-            self._run(lambda: fb.forward_postprocess(func, in_data), in_data[:1])
+            fb.forward_postprocess(func, in_data)
 
     def backward_preprocess(self, func, in_data, out_grad_data):
         fb = self._find(func, in_data, out_grad_data)
         if fb is not None:
-            self._run(lambda: fb.backward_preprocess(func, in_data, out_grad_data),
-                      tuple(in_data[:1]) + tuple(out_grad_data))
+            fb.backward_preprocess(func, in_data, out_grad_data)
 
 
 class KFACUpdateRule(object):
@@ -291,7 +288,9 @@ class KFAC(object):
     def setup(self, link):
         self.target = link
         self.t = 0
-        for param in link.params():
+        # the parameters as of now: walking the link tree costs more than a step's launches
+        self._params = list(link.params())
+        for param in self._params:
             param.update_rule = self.create_update_rule()
         self.fblocks = []
         for sub_linkname, sub_link in sorted(link.namedlinks(), key=lambda kv: kv[0]):
@@ -315,7 +314,7 @@ class KFAC(object):
         """Chainer's Optimizer.use_fp32_update: float32 master copies for float16
         parameters (this implementation always keeps them; the flag is recorded)."""
         self._use_fp32_update = flag
-        for param in self.target.params():
+        for param in self._params:
             if param.update_rule is not None:
                 param.update_rule.use_fp32_update(flag)
 
@@ -331,7 +330,7 @@ class KFAC(object):
 
     def reallocate_cleared_grads(self):
         import torch
-        for _, param in self.target.namedparams(False):
+        for param in self._params:
             if hasattr(param, 'kfgrad') and param.kfgrad is None:
                 param.kfgrad = torch.zeros_like(param.data)
             if param.grad is None:
@@ -397,7 +396,7 @@ class KFAC(object):
                     loss.backward()
                 # Chainer's backward(loss_scale=...) stamps the scale on every
                 # parameter that received a gradient; the update rule divides by it
-                for param in self.target.params():
+                for param in self._params:
                     param._loss_scale = self._loss_scale
             del loss
         # the factor kernels of this pass ran on the side streams; the small ones are still to run
@@ -425,7 +424,7 @@ class KFAC(object):
         ``batch_param_updates`` the K-FAC rules that share their hyperparameters
         run as one launch over all their parameters instead of one each."""
         jobs = {}
-        for param in self.target.params():
+        for param in self._params:
             rule = param.update_rule
             job = NotImplemented
             if self.batch_param_updates and type(rule) is KFACUpdateRule:
@@ -442,7 +441,7 @@ class KFAC(object):
     # ---- accumulation over acc_iters micro-batches -----------------------
     def accumulate(self):
         if self.acc_count == 0:
-            for param in self.target.params():
+            for param in self._params:
                 param.acc_grad = None
             for fblock in self.fblocks:
                 fblock.acc_covs = None
@@ -451,7 +450,7 @@ class KFAC(object):
         self.acc_count += 1
         if self.acc_count == self.acc_iters:
             self.acc_count = 0
-            for param in self.target.params():
+            for param in self._params:
                 param.grad = param.acc_grad
             for fblock in self.fblocks:
                 fblock.covs = fblock.acc_covs
@@ -465,7 +464,7 @@ class KFAC(object):
         """acc_grad += grad / acc_iters for every parameter (one launch for those
         that start their sum, one for those that continue it)."""
         first, later = [], []
-        for param in self.target.params():
+        for param in self._params:
             if param.grad is None:
                 continue
             if getattr(param, 'acc_grad', None) is None:
@@ -520,14 +519,24 @@ class KFAC(object):
         grouped call, the other blocks side by side on the lanes."""
         conn = [fb for fb in fblocks if isinstance(fb, FB.FisherBlockConnection)] \
             if self.group_precondition else []
-        grouped = set(id(fb) for fb in conn)
+        norm = [fb for fb in fblocks if isinstance(fb, FB.FisherBlockBatchNormalization)] \
+            if self.group_precondition else []
+        grouped = set(id(fb) for fb in conn + norm)
         for fblock in fblocks:
             if id(fblock) not in grouped:
                 self._lanes.run(fblock.update_kfgrads)
+        if norm:
+            # all batch-norm blocks in two launches, beside the connection blocks' GEMMs
+            operands = [fb.kfgrad_operands() for fb in norm]
+            self._lanes.run(lambda: ops.precond_bn_batched(*[[o[i] for o in operands] for i in range(6)]))
+            for fb in norm:
+                fb.finish_kfgrads()
         if conn:
             operands = [fb.kfgrad_operands() for fb in conn]
             shapes = [(o[0].shape[0], o[1].shape[0], o[3] is not None) for o in operands]
-            bound = tuple(0 if t is None else t.data_ptr() for o in operands for t in o)
+            # a plan per set of persistent buffers (inverses, outputs); the gradient arrays may be
+            # new ones every step and go through the plan's table of per-call pointers
+            bound = tuple(0 if o[i] is None else o[i].data_ptr() for o in operands for i in (0, 1, 4, 5))
             ops.precond_group(shapes, bound).run(*[[o[i] for o in operands] for i in range(6)])
             for fb in conn:
                 fb.finish_kfgrads()

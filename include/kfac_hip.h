@@ -38,6 +38,25 @@ extern "C" {
 int kfac_abi_version(void);
 const char *kfac_last_error_string(void);
 
+/* Tuning options (no counterpart in the reference, which has no tunables on this
+ * path).  Every option has a built-in default that the library chooses itself;
+ * kfac_option_set overrides it for plans created and calls made afterwards,
+ * kfac_option_unset restores the default.  The environment variable
+ * KFAC_<NAME IN CAPITALS> gives an option its starting value; the environment is
+ * read once, when the first option is looked up.  Names (kfac_option_name(i) for
+ * i < kfac_option_count()):
+ *   syrk_bm64_max, syrk_splits, conv_rows, rows_wm, shift_slices5, shift_slices3,
+ *   conv_shift, conv_shift_strict, group_bm64_max, group_macro, group_panels,
+ *   group_macro_tasks, group_graded, inverse_group, inverse_border,
+ *   inverse_lookahead, inverse_rest_lds, inverse_align, precond_tasks,
+ *   bn_stats_loop.
+ * Not thread-safe against concurrent calls into the library. */
+int kfac_option_set(const char *name, double value);
+int kfac_option_unset(const char *name);
+int kfac_option_get(const char *name, double *value, int *is_set);
+int kfac_option_count(void);
+const char *kfac_option_name(int index);
+
 /* ------------------------------------------------------------------------
  * (4) Communicator buffer layout: triangular pack / unpack
  * --------------------------------------------------------------------- */
@@ -51,7 +70,10 @@ int64_t kfac_packed_nelems(int n_arrays, const int64_t *sizes,
 
 /* Descriptor of a list of arrays in buffer order; replaces _ArraysInfo
  * (communicators/pure_nccl_communicator.py:221-279).  The tables are uploaded
- * once; kfac_pack_plan_set_ptrs re-uploads only the pointers. */
+ * once; kfac_pack_plan_set_ptrs re-uploads only the pointers, and only when
+ * they differ from the last ones: the upload is a copy ordered on `stream`, so
+ * the pack / unpack calls that are to see it must be issued on that stream (or
+ * on one that waits for it). */
 typedef struct kfac_pack_plan *kfac_pack_plan_t;
 
 int kfac_pack_plan_create(int n_arrays, const void *const *ptrs,
@@ -341,6 +363,28 @@ int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamma,
                         float *kf_gamma, float *kf_beta, int32_t *nan_flag_dev,
                         void *ws, size_t ws_bytes, void *stream);
 
+/* kfac_precond_bn_f32 for a list of batch-norm blocks in two launches (the products
+ * of all blocks, then the NaN selection of all blocks) instead of two per block;
+ * the arithmetic is the single-block kernels' own, so the results are identical.
+ * Block i: Finv[i] (dims[i] x dims[i]), gradients g_gamma[i] (n_gamma[i] entries)
+ * and g_beta[i] (the rest), outputs kf_gamma[i] / kf_beta[i], flag nan_flags[i]
+ * (device int32; the table or an entry may be NULL).  The batch object keeps the
+ * device-side tables between calls and uploads them again, with copies ordered on
+ * `stream`, only when the arguments change.  Workspace: the sum of the dims
+ * rounded up to multiples of 4, in floats.
+ * Replaces the per-block loop over batch_normalization.py:159-191 of
+ * optimizers/kfac.py:306-310. */
+typedef struct kfac_precond_bn_batch *kfac_precond_bn_batch_t;
+int kfac_precond_bn_batch_create(kfac_precond_bn_batch_t *batch_out);
+int kfac_precond_bn_batch_destroy(kfac_precond_bn_batch_t batch);
+size_t kfac_precond_bn_batched_workspace_bytes(int count, const int32_t *dims);
+int kfac_precond_bn_batched_f32(kfac_precond_bn_batch_t batch, int count,
+                                const float *const *Finv, const int32_t *dims,
+                                const float *const *g_gamma, const int32_t *n_gamma,
+                                const float *const *g_beta, float *const *kf_gamma,
+                                float *const *kf_beta, int32_t *const *nan_flags,
+                                void *ws, size_t ws_bytes, void *stream);
+
 /* kfac_precond_bn_f32 without a workspace argument and without any allocation:
  * the staging vector lives in a device array of KFAC_PRECOND_BN_STATIC_MAX_D
  * floats (32 KiB) that is part of the library image on every GPU the library
@@ -410,7 +454,12 @@ int kfac_momentum_update_batched_f32(kfac_momentum_batch_t batch, int count,
 #define KFAC_TIMED_PACK 4       /* pack kernel                                */
 #define KFAC_TIMED_UNPACK 5     /* unpack kernel                              */
 #define KFAC_TIMED_COPY 6       /* kfac_stream_copy_f32                        */
-#define KFAC_TIMED_FAMILIES 7
+#define KFAC_TIMED_COV_AUX 7    /* covariance: kernels around the main one (border sums, split-K sums,
+                                   assembly of a factor from shifted correlations)                     */
+#define KFAC_TIMED_BN 8         /* batch-norm statistics and per-sample gradient matrix               */
+#define KFAC_TIMED_INV_CALL 9   /* one whole kfac_spd_inverse_batched_f32 call: first launch to last  */
+#define KFAC_TIMED_GEMM_AUX 10  /* preconditioning: split-K sums and the batch-norm GEMV              */
+#define KFAC_TIMED_FAMILIES 11
 
 /* dst[i] = src[i] for nelems floats (16-byte aligned pointers): a plain
  * streaming copy that moves 8 bytes per element, the yardstick that bench.py

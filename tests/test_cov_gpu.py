@@ -90,18 +90,29 @@ CONV_CASES = [
 
 def takes_shift_route(c, h, w, k, s, p):
     """3x3 / stride 1 / padding 1 with at least 64 channels (or 28..32, with stacked operand tiles):
-    computed from shifted correlations of the input unless KFAC_CONV_SHIFT=0 leaves it to the
-    patch-product kernels."""
+    computed from shifted correlations of the input unless the option conv_shift = 0 leaves it to
+    the patch-product kernels."""
     return k == 3 and s == 1 and p == 1 and (c >= 64 or 28 <= c <= 32) and h >= 4 and w >= 4
 
 
 @pytest.fixture
-def patch_product_route(monkeypatch):
+def lib_options():
+    """Sets tuning options of the library for one test and restores the defaults afterwards."""
+    from chainerkfac_amd import _lib
+    touched = []
+
+    def set_option(name, value):
+        touched.append(name)
+        _lib.set_option(name, value)
+    yield set_option
+    for name in touched:
+        _lib.set_option(name, None)
+
+
+@pytest.fixture
+def patch_product_route(lib_options):
     def switch(on):
-        if on:
-            monkeypatch.setenv('KFAC_CONV_SHIFT', '0')
-        else:
-            monkeypatch.delenv('KFAC_CONV_SHIFT', raising=False)
+        lib_options('conv_shift', 0 if on else None)
     return switch
 
 
@@ -172,13 +183,13 @@ def test_conv_A_shift_route_unaligned_input_and_accumulation():
 
 @pytest.mark.parametrize('n,c,h,w', [(32, 64, 56, 56), (32, 128, 28, 28), (8, 256, 14, 14), (4, 512, 7, 7),
                                      (2, 64, 4, 200), (3, 96, 9, 5)])
-def test_workspace_query_covers_the_shift_route(n, c, h, w, monkeypatch):
+def test_workspace_query_covers_the_shift_route(n, c, h, w, lib_options):
     """A workspace of exactly kfac_cov_workspace_bytes(d, rows) is enough for the shifted-correlation
-    route (with KFAC_CONV_SHIFT_STRICT a workspace that is too small for it is an error instead of a
-    silent change of route)."""
+    route (with the option conv_shift_strict a workspace that is too small for it is an error instead
+    of a silent change of route)."""
     from chainerkfac_amd import _lib, device as _dev
     lib = _lib.load()
-    monkeypatch.setenv('KFAC_CONV_SHIFT_STRICT', '1')
+    lib_options('conv_shift_strict', 1)
     d = 9 * c + 1
     nbytes = lib.kfac_cov_workspace_bytes(d, n * h * w)
     ws = torch.empty(nbytes, dtype=torch.uint8, device='cuda')
@@ -342,14 +353,14 @@ def test_grouped_launch_matches_the_single_calls():
     np.testing.assert_allclose(outs[0].cpu().numpy(), O.conv_G(gy) * (0.25 * 14 * 14 / 4), rtol=1e-4, atol=1e-4)
 
 
-def test_grouped_launch_macro_tiles(monkeypatch):
-    """With KFAC_GROUP_MACRO=1 (read when a group is created), slabs of several 128-tiles with
+def test_grouped_launch_macro_tiles(lib_options):
+    """With the option group_macro = 1 (read when a group is created), slabs of several 128-tiles with
     a long reduction take the macro-tile kernel (four teams
     per workgroup, 2 x 2 tiles from four panels staged once): an even and an odd number of
     tiles, a ragged last tile, 16-byte and scalar loads, a ones column, accumulation; against
     float64 and the single-call entry point."""
     from chainerkfac_amd import ops
-    monkeypatch.setenv('KFAC_GROUP_MACRO', '1')
+    lib_options('group_macro', 1)
     r = np.random.default_rng(29)
 
     def t(*shape):

@@ -46,17 +46,20 @@ def test_batched_inverse_mixed_sizes():
         check_inverse(m, o.cpu().numpy())
 
 
-@pytest.mark.parametrize('env,extra', [({'KFAC_INVERSE_ALIGN': '0'}, 3), ({'KFAC_INVERSE_ALIGN': '50'}, 4),
-                                       ({'KFAC_INVERSE_GROUP': '3'}, 5), ({'KFAC_INVERSE_GROUP': '1'}, 6),
-                                       ({'KFAC_INVERSE_LOOKAHEAD': '0'}, 8),
-                                       ({'KFAC_INVERSE_GROUP': '4', 'KFAC_INVERSE_ALIGN': '30'}, 9)])
-def test_schedule_overrides_do_not_change_results(monkeypatch, env, extra):
-    """The tuning overrides (where a matrix joins the sweep, block columns per
+@pytest.mark.parametrize('opts,extra', [({'inverse_align': 0}, 3), ({'inverse_align': 50}, 4),
+                                        ({'inverse_group': 3}, 5), ({'inverse_group': 1}, 6),
+                                        ({'inverse_lookahead': 0}, 8),
+                                        ({'inverse_group': 4, 'inverse_align': 30}, 9)])
+def test_schedule_overrides_do_not_change_results(opts, extra):
+    """The tuning options (where a matrix joins the sweep, block columns per
     group, second stream) only reorder launches.  A plan reads them when it is
     created; `extra` makes the size list, and with it the plan, unique to the case."""
-    from chainerkfac_amd import ops
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    from chainerkfac_amd import _lib, ops
+    with _lib.options(**opts):
+        _run_schedule_case(ops, extra)
+
+
+def _run_schedule_case(ops, extra):
     dims = [900, 641, 640, 385, 300, 129, 128, 40, extra]
     mats = [spd(d, 200 + d) for d in dims]
     outs, info = ops.spd_inverse_batched([torch.from_numpy(m).cuda() for m in mats])
@@ -104,9 +107,9 @@ def test_non_spd_and_nan_are_flagged_per_matrix():
         O.inverse(bad)
 
 
-def test_bordered_matrices(monkeypatch):
+def test_bordered_matrices():
     """Matrices of 128 m + 1 rows (a layer with a bias) are inverted from their leading
-    block plus a border; the result equals the whole-matrix path (KFAC_INVERSE_BORDER=0) to
+    block plus a border; the result equals the whole-matrix path (option inverse_border = 0) to
     rounding, a non-positive last pivot is reported as info = d, and sizes around the rule
     (128 m, 128 m + 2, 129) take their own paths."""
     from chainerkfac_amd import ops
@@ -119,12 +122,12 @@ def test_bordered_matrices(monkeypatch):
     for m, o in zip(mats, outs):
         check_inverse(m, o.cpu().numpy())
     # the same through the whole-matrix path (a plan reads the switch when it is created)
-    monkeypatch.setenv('KFAC_INVERSE_BORDER', '0')
-    whole, info = ops.spd_inverse_batched(dev + [torch.from_numpy(spd(3, 1)).cuda()])
+    from chainerkfac_amd import _lib
+    with _lib.options(inverse_border=0):
+        whole, info = ops.spd_inverse_batched(dev + [torch.from_numpy(spd(3, 1)).cuda()])
     for m, o, w in zip(mats, outs, whole):
         ref64 = np.linalg.inv(m.astype(np.float64))
         assert np.linalg.norm(o.cpu().numpy() - w.cpu().numpy()) <= 2e-4 * np.linalg.norm(ref64)
-    monkeypatch.delenv('KFAC_INVERSE_BORDER')
     # last pivot not positive: SPD leading block, corner too small
     bad = spd(257, 9).astype(np.float64)
     a = bad[:256, 256]
