@@ -42,6 +42,7 @@ PROTOTYPES = {
     'kfac_cov_workspace_bytes': (c_sz, [c_int, c_i64]),
     'kfac_cov_linear_f32': (c_int, [c_vp, c_int, c_int, c_int, c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
     'kfac_cov_conv_a_f32': (c_int, [c_vp] + [c_int] * 11 + [c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
+    'kfac_cov_conv_a_last_route': (c_int, []),
     'kfac_cov_conv_g_f32': (c_int, [c_vp, c_int, c_int, c_int, c_f, c_f, c_vp, c_vp, c_sz, c_vp]),
     'kfac_cov_group_create': (c_int, [c_int, c_vp, c_vpp]),
     'kfac_cov_group_workspace_bytes': (c_sz, [c_vp]),
@@ -54,6 +55,7 @@ PROTOTYPES = {
     'kfac_axpby_batch_create': (c_int, [c_vp]),
     'kfac_axpby_batch_destroy': (c_int, [c_vp]),
     'kfac_axpby_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_vp, c_f, c_f, c_vp]),
+    'kfac_div_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_f, c_vp]),
     'kfac_inverse_plan_create': (c_int, [c_int, c_i32p, c_vpp]),
     'kfac_inverse_plan_workspace_bytes': (c_sz, [c_vp]),
     'kfac_inverse_plan_destroy': (c_int, [c_vp]),
@@ -67,6 +69,8 @@ PROTOTYPES = {
     'kfac_bn_lowrank_plan_destroy': (c_int, [c_vp]),
     'kfac_bn_lowrank_inverse_batched_f32': (c_int, [c_vp, c_vpp, c_vpp, c_dp, c_dp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_add_diag_f32': (c_int, [c_vp, c_int, c_int, c_d, c_d, c_vp]),
+    'kfac_keep_diag_f32': (c_int, [c_vp, c_int, c_vp]),
+    'kfac_recip_add_f32': (c_int, [c_vp, c_i64, c_d, c_d, c_vp, c_i64, c_vp]),
     'kfac_diag_batch_create': (c_int, [c_vp]),
     'kfac_diag_batch_destroy': (c_int, [c_vp]),
     'kfac_add_diag_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),

@@ -1169,6 +1169,12 @@ extern "C" int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, floa
                   beta, C, ws, ws_bytes, kfac::as_stream(stream));
 }
 
+namespace {
+thread_local int last_conv_route = -1;
+}
+
+extern "C" int kfac_cov_conv_a_last_route(void) { return last_conv_route; }
+
 extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, int kh, int kw,
                                    int sy, int sx, int ph, int pw, int append_ones,
                                    float alpha, float beta, float *C, void *ws,
@@ -1187,6 +1193,7 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
   const int ones = append_ones ? 1 : 0;
   const long long K = (long long)n * ho * wo;
   hipStream_t s = kfac::as_stream(stream);
+  last_conv_route = KFAC_CONV_ROUTE_SLAB;
   if (kh == 1 && kw == 1 && sy == 1 && sx == 1 && ph == 0 && pw == 0) {
     // 1x1 convolution: the patch matrix is the NCHW tensor itself
     const int hw = h * w;
@@ -1208,20 +1215,24 @@ extern "C" int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, i
     return run_syrk(l64, l128, d, ones, K, alpha, beta, C, ws, ws_bytes, s);
   }
   {
+    last_conv_route = KFAC_CONV_ROUTE_SHIFT;
     const int rc = try_conv_shift(x, n, c, h, w, kh, kw, sy, sx, ph, pw, d, ones, alpha, beta, C, ws,
                                   ws_bytes, s);
     if (rc <= 0) return rc;   // 1 = shape left to the patch-product kernels
   }
   {
+    last_conv_route = KFAC_CONV_ROUTE_ROWS;
     const int rc = try_conv_rows(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, d, ones, alpha, beta, C,
                                  ws, ws_bytes, s);
     if (rc <= 0) return rc;   // 1 = no instantiation for this shape
   }
   ConvGeom geom;
   if (make_halo_geom(x, n, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo, &geom)) {
+    last_conv_route = KFAC_CONV_ROUTE_HALO;
     const int rc = run_conv_halo(geom, n, d, ones, alpha, beta, C, ws, ws_bytes, s);
     if (rc <= 0) return rc;   // 1 = shape left to the generic kernel
   }
+  last_conv_route = KFAC_CONV_ROUTE_GATHER;
   return run_syrk(make_im<64>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo),
                   make_im<128>(x, c, h, w, kh, kw, sy, sx, ph, pw, ho, wo), d, ones, K, alpha,
                   beta, C, ws, ws_bytes, s);

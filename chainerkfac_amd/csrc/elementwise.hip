@@ -196,7 +196,8 @@ struct AxpbyEntry {
   int aligned;   // both arrays start on 16-byte boundaries
 };
 
-template <bool OVERWRITE>
+// MODE 0: y = a x + b y; 1: y = a x (y is not read); 2: y = x / a (an IEEE division)
+template <int MODE>
 __global__ __launch_bounds__(kThreads) void axpby_batched_kernel(
     const AxpbyEntry *__restrict__ entries, const int *__restrict__ owner, float a, float b) {
   const AxpbyEntry t = entries[owner[blockIdx.x]];
@@ -208,8 +209,11 @@ __global__ __launch_bounds__(kThreads) void axpby_batched_kernel(
     if (t.aligned && i + 4 <= t.n) {
       const floatx4a x = *reinterpret_cast<const floatx4a *>(t.x + i);
       floatx4a y;
-      if (OVERWRITE) {
+      if (MODE == 1) {
         y = a * x;
+      } else if (MODE == 2) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = x[e] / a;
       } else {
         y = *reinterpret_cast<const floatx4a *>(t.y + i);
 #pragma unroll
@@ -218,7 +222,8 @@ __global__ __launch_bounds__(kThreads) void axpby_batched_kernel(
       *reinterpret_cast<floatx4a *>(t.y + i) = y;
     } else {
       const long long end = i + 4 < t.n ? i + 4 : t.n;
-      for (long long j = i; j < end; ++j) t.y[j] = OVERWRITE ? a * t.x[j] : axpby_value(t.x[j], t.y[j], a, b);
+      for (long long j = i; j < end; ++j)
+        t.y[j] = MODE == 1 ? a * t.x[j] : MODE == 2 ? t.x[j] / a : axpby_value(t.x[j], t.y[j], a, b);
     }
   }
 }
@@ -345,6 +350,25 @@ __global__ __launch_bounds__(kThreads) void momentum_batched_kernel(
   }
 }
 
+// M[r][c] = 0 for r != c: 16-byte stores over whole rows where the row allows, the
+// diagonal entry kept.
+__global__ __launch_bounds__(kThreads) void keep_diag_kernel(float *__restrict__ M, int d) {
+  const long long total = (long long)d * d;
+  for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < total;
+       i += (long long)gridDim.x * kThreads) {
+    const long long r = i / d;
+    if (i - r * d != r) M[i] = 0.f;
+  }
+}
+
+// out[i] = 1 / (x[i] + (i < split ? v0 : v1)), the sum and the quotient in float64
+__global__ __launch_bounds__(kThreads) void recip_add_kernel(const float *__restrict__ x, long long split,
+                                                             double v0, double v1, float *__restrict__ out,
+                                                             long long n) {
+  for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < n; i += (long long)gridDim.x * kThreads)
+    out[i] = (float)(1.0 / ((double)x[i] + (i < split ? v0 : v1)));
+}
+
 int grid_for(long long n) {
   long long g = kfac::ceil_div<long long>(n, kThreads);
   const long long cap = 256LL * 32;
@@ -371,6 +395,27 @@ extern "C" int kfac_add_diag_f32(float *M, int d, int split, double v0, double v
   KFAC_REQUIRE(M != nullptr, "M is null");
   hipLaunchKernelGGL(add_diag_kernel, dim3(kfac::ceil_div(d, kThreads)), dim3(kThreads),
                      0, kfac::as_stream(stream), M, d, split, v0, v1);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+extern "C" int kfac_keep_diag_f32(float *M, int d, void *stream) {
+  KFAC_REQUIRE(d >= 0 && d <= 46340, "bad dimension %d", d);
+  if (d == 0) return KFAC_OK;
+  KFAC_REQUIRE(M != nullptr, "M is null");
+  hipLaunchKernelGGL(keep_diag_kernel, dim3(grid_for((long long)d * d)), dim3(kThreads), 0,
+                     kfac::as_stream(stream), M, d);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+extern "C" int kfac_recip_add_f32(const float *x, int64_t split, double v0, double v1, float *out,
+                                  int64_t nelems, void *stream) {
+  KFAC_REQUIRE(nelems >= 0, "nelems < 0");
+  if (nelems == 0) return KFAC_OK;
+  KFAC_REQUIRE(x && out, "null pointer");
+  hipLaunchKernelGGL(recip_add_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0, kfac::as_stream(stream),
+                     x, (long long)split, v0, v1, out, (long long)nelems);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }
@@ -528,9 +573,9 @@ extern "C" int kfac_axpby_batch_destroy(kfac_axpby_batch_t batch) {
   return KFAC_OK;
 }
 
-extern "C" int kfac_axpby_batched_f32(kfac_axpby_batch_t batch, int count, const float *const *xs,
-                                      float *const *ys, const int64_t *nelems, float a, float b,
-                                      void *stream) {
+namespace {
+int run_axpby_batch(kfac_axpby_batch_t batch, int count, const float *const *xs, float *const *ys,
+                    const int64_t *nelems, float a, float b, bool divide, void *stream) {
   KFAC_REQUIRE(batch != nullptr, "batch is null");
   KFAC_REQUIRE(count >= 0, "count < 0");
   if (count == 0) return KFAC_OK;
@@ -563,12 +608,28 @@ extern "C" int kfac_axpby_batched_f32(kfac_axpby_batch_t batch, int count, const
     return rc;
   if (int rc = batch->owner_table.set(batch->owner.data(), sizeof(int) * batch->owner.size(), s, &d_owner))
     return rc;
-  if (b == 0.f)
-    hipLaunchKernelGGL(axpby_batched_kernel<true>, dim3((unsigned)units), dim3(kThreads), 0, s,
+  if (divide)
+    hipLaunchKernelGGL(axpby_batched_kernel<2>, dim3((unsigned)units), dim3(kThreads), 0, s,
+                       static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
+  else if (b == 0.f)
+    hipLaunchKernelGGL(axpby_batched_kernel<1>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
   else
-    hipLaunchKernelGGL(axpby_batched_kernel<false>, dim3((unsigned)units), dim3(kThreads), 0, s,
+    hipLaunchKernelGGL(axpby_batched_kernel<0>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
+}
+}  // namespace
+
+extern "C" int kfac_axpby_batched_f32(kfac_axpby_batch_t batch, int count, const float *const *xs,
+                                      float *const *ys, const int64_t *nelems, float a, float b,
+                                      void *stream) {
+  return run_axpby_batch(batch, count, xs, ys, nelems, a, b, false, stream);
+}
+
+extern "C" int kfac_div_batched_f32(kfac_axpby_batch_t batch, int count, float *const *arrays,
+                                    const int64_t *nelems, float divisor, void *stream) {
+  KFAC_REQUIRE(divisor == divisor && divisor != 0.f, "the divisor must be a non-zero number");
+  return run_axpby_batch(batch, count, arrays, arrays, nelems, divisor, 0.f, true, stream);
 }

@@ -262,6 +262,27 @@ def axpby_batched(xs, ys, a, b, stream=None):
     return ys
 
 
+_div_batches = None
+
+
+def div_batched(arrays, divisor, stream=None):
+    """arrays[i] /= divisor in place for a list of float32 arrays in one launch."""
+    global _div_batches
+    if not arrays:
+        return arrays
+    for a in arrays:
+        _dev.require_gpu_tensor(a, 'array')
+    if _div_batches is None:
+        _div_batches = _PlanCache(4)
+    # one batch object per number of arrays (gradient arrays may be new ones every step; the
+    # object keeps its last few tables)
+    batch = _div_batches.get(len(arrays), _AxpbyBatch)
+    _lib.check(_lib.load().kfac_div_batched_f32(
+        batch._h, len(arrays), _lib.ptr_array([a.data_ptr() for a in arrays]),
+        _lib.i64_array([a.numel() for a in arrays]), float(divisor), _dev.stream_handle(stream)))
+    return arrays
+
+
 def add_diag(M, v0, v1=None, split=None, stream=None):
     """diag(M)[i] += v0 for i < split else v1 (float64 sum, float32 store)."""
     _dev.require_gpu_tensor(M, 'M')
@@ -273,6 +294,26 @@ def add_diag(M, v0, v1=None, split=None, stream=None):
     _lib.check(_lib.load().kfac_add_diag_f32(M.data_ptr(), d, int(split), float(v0), float(v1),
                                              _dev.stream_handle(stream)))
     return M
+
+
+def keep_diag(M, stream=None):
+    """M = diag(diag(M)) in place."""
+    _dev.require_gpu_tensor(M, 'M')
+    if M.ndim != 2 or M.shape[0] != M.shape[1]:
+        raise ValueError('M must be square')
+    _lib.check(_lib.load().kfac_keep_diag_f32(M.data_ptr(), M.shape[0], _dev.stream_handle(stream)))
+    return M
+
+
+def recip_add(x, v0, v1=None, split=None, out=None, stream=None):
+    """1 / (x[i] + (v0 if i < split else v1)) elementwise (float64 arithmetic, float32 result)."""
+    _dev.require_gpu_tensor(x, 'x')
+    out = _out(out, tuple(x.shape), x)
+    if split is None:
+        split, v1 = x.numel(), v0
+    _lib.check(_lib.load().kfac_recip_add_f32(x.data_ptr(), int(split), float(v0), float(v1), out.data_ptr(),
+                                              x.numel(), _dev.stream_handle(stream)))
+    return out
 
 
 class _DiagBatch(object):

@@ -211,13 +211,45 @@ class FisherBlock(object):
         """Add the damping to the diagonals of ``cov_emas`` in place."""
         raise NotImplementedError
 
+    def has_diagonal_factor(self):
+        """True when a factor is kept as its diagonal only (a 1-D array)."""
+        return self.cov_emas is not None and any(c.ndim == 1 for c in self.cov_emas)
+
     def update_invs(self):
         self.check_attr('cov_emas')
-        for c in self.cov_emas:
-            if c.ndim != 2:
-                raise NotImplementedError('diagonal (1-D) factors are not produced on this path')
-        self.damp()
-        self.invs, self.inv_info = ops.spd_inverse_batched(self.cov_emas, outs=self._inv_buffers())
+        if not self.has_diagonal_factor():
+            self.damp()
+            self.invs, self.inv_info = ops.spd_inverse_batched(self.cov_emas, outs=self._inv_buffers())
+            return
+        # A factor kept as a 1-D array is inverted entry by entry, 1 / (cov + diagvals)
+        # (reference fisher_block.py:165-179); the damping values come to the host here
+        # (get_diagvals), which the all-matrix path above avoids.
+        import numpy as np
+        invs, dense, dense_at = [], [], []
+        for i, (c, vals) in enumerate(zip(self.cov_emas, self.get_diagvals())):
+            vals = np.asarray(vals, dtype=np.float64).reshape(-1)
+            changes = np.nonzero(vals != vals[0])[0]
+            split = int(changes[0]) if changes.size else vals.size
+            if not np.all(vals[split:] == vals[-1]):
+                raise ValueError('the damping of a factor must take at most two values')
+            if c.ndim == 1:
+                invs.append(ops.recip_add(c, vals[0], vals[-1], split,
+                                          out=self._buffer('inv{}'.format(i), c.shape, c.device)))
+            elif c.ndim == 2:
+                ops.add_diag(c, vals[0], vals[-1], split=split)
+                dense.append(c)
+                dense_at.append(i)
+                invs.append(None)
+            else:
+                raise ValueError('a factor must be a vector or a square matrix')
+        self.inv_info = None
+        if dense:
+            outs, self.inv_info = ops.spd_inverse_batched(
+                dense, outs=[self._buffer('inv{}'.format(i), self.cov_emas[i].shape, self.cov_emas[i].device)
+                             for i in dense_at])
+            for i, o in zip(dense_at, outs):
+                invs[i] = o
+        self.invs = invs
 
     def get_diagvals(self):
         raise NotImplementedError

@@ -34,9 +34,14 @@ class FisherBlockConvolution2D(FisherBlockConnection):
         gy = as_float32(out_grad_data[0])
         n, c, ho, wo = gy.shape
         scale = self.gy_scale(n) ** 2 / (n * ho * wo)
-        if getattr(self.link, 'diag', False):
-            raise NotImplementedError('link.diag (diagonal G) is not supported on the HIP path')
         out, alpha, beta = self._cov_target('G', (c, c), gy.device, scale)
+        if self.diagonalize or getattr(self.link, 'diag', False):
+            # G = diag(diag(G)), still a c x c matrix (reference convolution_2d.py:57-62, :68-70)
+            def diagonal_factor():
+                ops.cov_conv_g(gy, alpha, beta, out)
+                ops.keep_diag(out)
+            self._on_lane(diagonal_factor, (gy,))
+            return out
         if self._defer_cov(ops.COV_SLAB, gy, False, n * ho * wo, out, alpha, beta):
             return out
         return self._on_lane(lambda: ops.cov_conv_g(gy, alpha, beta, out), (gy,))

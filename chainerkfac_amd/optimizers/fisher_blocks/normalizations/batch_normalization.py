@@ -104,6 +104,14 @@ class FisherBlockBatchNormalization(FisherBlock):
         def stats():
             ops.bn_grad_matrix(x, gy, eps, gy_scale, has_gamma, has_beta, out=U)
 
+        if self.diagonalize:
+            # F = diag(mean(grad^2)): diag(diag(F)), a matrix (reference batch_normalization.py:121-124)
+            def diagonal_factor():
+                stats()
+                ops.cov_linear(U, False, alpha, beta, out)
+                ops.keep_diag(out)
+            self._on_lane(diagonal_factor, (x, gy))
+            return out
         if self.pending_covs is not None and self.pending_covs.accepts(n, width):
             self._on_lane(stats, (x, gy))
             self._defer_cov(ops.COV_LINEAR, U, False, n, out, alpha, beta)
@@ -135,7 +143,7 @@ class FisherBlockBatchNormalization(FisherBlock):
         (accumulation over micro-batches, a moving average with history, factors
         that were averaged over ranks, batches larger than LOWRANK_MAX_BATCH)."""
         U = self._U
-        if U is None or not self._ema_is_single_factor or not self.factor_is_local:
+        if U is None or not self._ema_is_single_factor or not self.factor_is_local or self.diagonalize:
             return None
         if self.acc_state[0] != 1 or U.shape[0] > self.LOWRANK_MAX_BATCH:
             return None

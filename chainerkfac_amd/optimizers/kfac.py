@@ -156,11 +156,16 @@ class KFACUpdateRule(object):
             param.data.copy_(self._fp32_param)
             return
         if param._loss_scale is not None:
+            # the reference's rule divides ``kfgrad`` in place (kfac.py:76-78), Chainer's base
+            # rule, which it then calls, ``grad``: both end up unscaled
             if getattr(param, 'kfgrad', None) is not None:
                 param.kfgrad /= param._loss_scale
-            elif param.grad is not None:
+            if param.grad is not None:
                 param.grad /= param._loss_scale
-        self.update_core(param)
+        grad = param.kfgrad if getattr(param, 'kfgrad', None) is not None else param.grad
+        if grad is not None and grad.dtype != torch.float32:
+            grad = grad.float()      # a float16 gradient of a float32 parameter
+        self.update_core(param, grad=grad)
 
     def batched_job(self, param):
         """What ``update`` would hand to the momentum kernel, for
@@ -195,6 +200,10 @@ class KFACUpdateRule(object):
             momentum *= lr / lr_pre
         return {'param': self._fp32_param if half else data, 'v': self.state['v'], 'grad': grad,
                 'param_f16': data if half else None,
+                # Chainer's base rule divides ``grad`` of a float32 parameter in place as well
+                'raw_grad': param.grad if (not half and grad is not param.grad and param.grad is not None
+                                           and param.grad.dtype == torch.float32
+                                           and param.grad.is_contiguous()) else None,
                 # the reference divides the float32 gradient in place (kfac.py:76-78) and a
                 # float16 parameter's through a float32 copy (kfac.py:69-75)
                 'write_back': not half, 'key': (float(lr), float(momentum), param._loss_scale)}
@@ -437,6 +446,8 @@ class KFAC(object):
             ops.momentum_update_batched(
                 [j['param'] for j in group], [j['v'] for j in group], [j['grad'] for j in group], lr, momentum,
                 loss_scale, [j['write_back'] for j in group], [j['param_f16'] for j in group])
+            if loss_scale is not None:
+                ops.div_batched([j['raw_grad'] for j in group if j['raw_grad'] is not None], loss_scale)
 
     # ---- accumulation over acc_iters micro-batches -----------------------
     def accumulate(self):
@@ -545,10 +556,16 @@ class KFAC(object):
     def update_invs_batched(self, fblocks):
         """``fblock.update_invs()`` for every block, with all damping kernels and
         all inversions issued together."""
-        conn = [fb for fb in fblocks if isinstance(fb, FB.FisherBlockConnection)]
-        other = [fb for fb in fblocks if not isinstance(fb, FB.FisherBlockConnection)]
         for fb in fblocks:
             fb.check_attr('cov_emas')
+        # blocks with a factor kept as its diagonal (a 1-D array) go their own way
+        diagonal = [fb for fb in fblocks if fb.has_diagonal_factor()]
+        for fb in diagonal:
+            fb.update_invs()
+        if diagonal:
+            fblocks = [fb for fb in fblocks if not fb.has_diagonal_factor()]
+        conn = [fb for fb in fblocks if isinstance(fb, FB.FisherBlockConnection)]
+        other = [fb for fb in fblocks if not isinstance(fb, FB.FisherBlockConnection)]
         if conn:
             use_pi = {fb._pi_type == PI_TYPE_TRACENORM for fb in conn}
             if len(use_pi) == 1:

@@ -141,6 +141,17 @@ int kfac_cov_conv_a_f32(const float *x, int n, int c, int h, int w, int kh,
                         float alpha, float beta, float *C, void *ws,
                         size_t ws_bytes, void *stream);
 
+/* Which kernels the calling thread's last kfac_cov_conv_a_f32 call used (the choice
+ * depends on the geometry and, for the shifted correlations, on the size of the
+ * workspace): for tests and benchmarks that must know a shape runs where they
+ * think it does.  -1 before the first call.  No counterpart in the reference. */
+#define KFAC_CONV_ROUTE_SLAB 0    /* 1x1 convolution: the NCHW tensor read in place        */
+#define KFAC_CONV_ROUTE_SHIFT 1   /* 3x3 / 1 / 1: shifted correlations of the input       */
+#define KFAC_CONV_ROUTE_ROWS 2    /* compile-time geometry, whole output rows per step     */
+#define KFAC_CONV_ROUTE_HALO 3    /* halo regions staged in LDS                           */
+#define KFAC_CONV_ROUTE_GATHER 4  /* implicit im2col, element gather                      */
+int kfac_cov_conv_a_last_route(void);
+
 /* P = gy viewed as (n*ho*wo, c) from the NCHW tensor gy, read in place.  With
  * alpha = gy_scale^2/(n*ho*wo) replaces compute_G (convolution_2d.py:43-72). */
 int kfac_cov_conv_g_f32(const float *gy, int n, int c, int howo, float alpha,
@@ -219,6 +230,14 @@ int kfac_axpby_batch_destroy(kfac_axpby_batch_t batch);
 int kfac_axpby_batched_f32(kfac_axpby_batch_t batch, int count,
                            const float *const *xs, float *const *ys,
                            const int64_t *nelems, float a, float b, void *stream);
+
+/* arrays[i][j] /= divisor (an IEEE division, like NumPy's in-place `/=`) for a list
+ * of arrays in one launch: what Chainer's UpdateRule.update does to every
+ * parameter's `grad` of a scaled loss before the rule runs (the reference's rule,
+ * optimizers/kfac.py:63-85, does the same to `kfgrad`).  Takes a batch object of
+ * kfac_axpby_batch_create. */
+int kfac_div_batched_f32(kfac_axpby_batch_t batch, int count, float *const *arrays,
+                         const int64_t *nelems, float divisor, void *stream);
 
 /* ------------------------------------------------------------------------
  * (2) Damping and the damped inverse
@@ -304,6 +323,19 @@ int kfac_bn_lowrank_inverse_batched_f32(kfac_bn_lowrank_plan_t plan,
  * fisher_block.py:175). */
 int kfac_add_diag_f32(float *M, int d, int split, double v0, double v1,
                       void *stream);
+
+/* M = diag(diag(M)): the off-diagonal entries of the d x d matrix are set to zero.
+ * With the factor kernels before it, replaces `G = xp.diag(xp.diag(G))` of a link
+ * with `diag` set (connections/convolution_2d.py:68-70) and the `diagonalize`
+ * branches (convolution_2d.py:57-62, batch_normalization.py:121-124), whose
+ * results are d x d matrices as well. */
+int kfac_keep_diag_f32(float *M, int d, void *stream);
+
+/* out[i] = 1 / (x[i] + (i < split ? v0 : v1)), evaluated in float64 and rounded to
+ * float32: the inverse of a factor that is kept as its diagonal only (a 1-D
+ * array), fisher_block.py:170-171, with the damping of kfac_add_diag_f32. */
+int kfac_recip_add_f32(const float *x, int64_t split, double v0, double v1, float *out,
+                       int64_t nelems, void *stream);
 
 /* The same for `count` matrices in one launch (the damping of all batch-norm
  * blocks of a network: the loop of update_invs, fisher_block.py:165-179, over

@@ -48,19 +48,20 @@ PI_TYPE_TRACENORM = 'tracenorm'
 # Kronecker-factor construction
 # --------------------------------------------------------------------------
 
-def linear_A(x, has_bias=True):
-    """chainerkfac/optimizers/fisher_blocks/connections/linear.py:14-27."""
+def linear_A(x, has_bias=True, diagonalize=False):
+    """chainerkfac/optimizers/fisher_blocks/connections/linear.py:14-27.  With
+    ``diagonalize`` the factor is a vector (:25)."""
     n = x.shape[0]
     if has_bias:
         ones = np.ones(n, dtype=x.dtype)
         x = np.column_stack((x, ones))
     if x.dtype == np.float16:
         x = x.astype(np.float32)
-    return x.T.dot(x) * (1 / n)
+    return (x * x).mean(axis=0) if diagonalize else x.T.dot(x) * (1 / n)
 
 
-def linear_G(gy, loss_scale=None):
-    """linear.py:29-46."""
+def linear_G(gy, loss_scale=None, diagonalize=False):
+    """linear.py:29-46.  With ``diagonalize`` a diagonal matrix (:43-44)."""
     n = gy.shape[0]
     gy_scale = n
     if loss_scale is not None:
@@ -69,7 +70,7 @@ def linear_G(gy, loss_scale=None):
         gy = gy_scale * gy.astype(np.float32)
     else:
         gy = gy_scale * gy
-    return gy.T.dot(gy) * (1 / n)
+    return np.diag((gy * gy).mean(axis=0)) if diagonalize else gy.T.dot(gy) * (1 / n)
 
 
 def conv_out_size(size, k, s, p):
@@ -120,18 +121,28 @@ def conv_A(x, ksize, stride, pad, has_bias=True):
     return col.T.dot(col) * A_scale
 
 
-def conv_G(gy, loss_scale=None):
-    """convolution_2d.py:43-72 (non-diagonal branch)."""
+def conv_G(gy, loss_scale=None, diag=False, diagonalize=False):
+    """convolution_2d.py:43-72.  ``diagonalize`` is the block's own switch (:57-62),
+    ``diag`` the link attribute (:68-70); both return a matrix."""
     gy = gy.transpose(0, 2, 3, 1)
     n, ho, wo, _ = gy.shape
     gy = gy.reshape(n * ho * wo, -1)
     gy_scale = n
     if loss_scale is not None:
         gy_scale *= 1.0 / loss_scale
+    if diagonalize:
+        if gy.dtype == np.float16:
+            gy = gy_scale * gy.astype(np.float32)
+        else:
+            gy = gy_scale * gy
+        return np.diag((gy * gy).mean(axis=0))
     G_scale = 1 / (n * ho * wo) * (gy_scale ** 2)
     if gy.dtype == np.float16:
         gy = gy.astype(np.float32)
-    return gy.T.dot(gy) * G_scale
+    G = gy.T.dot(gy) * G_scale
+    if diag:
+        G = np.diag(np.diag(G))
+    return G
 
 
 def batch_normalize(x, eps):
@@ -176,10 +187,14 @@ def bn_grad_matrix(x, gy, eps, loss_scale=None, has_gamma=True, has_beta=True):
     return grad.astype(x.dtype, copy=False)
 
 
-def bn_F(x, gy, eps, loss_scale=None, has_gamma=True, has_beta=True):
-    """batch_normalization.py:78-131 (non-diagonal branch)."""
+def bn_F(x, gy, eps, loss_scale=None, has_gamma=True, has_beta=True, diagonalize=False):
+    """batch_normalization.py:78-131 (``diagonalize``: :121-124)."""
     grad = bn_grad_matrix(x, gy, eps, loss_scale, has_gamma, has_beta)
     n = x.shape[0]
+    if diagonalize:
+        if grad.dtype == np.float16:
+            grad = grad.astype(np.float32)
+        return np.diag((grad * grad).mean(axis=0))
     F_scale = 1 / n
     if grad.dtype == np.float16:
         grad = grad.astype(np.float32)

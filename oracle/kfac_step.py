@@ -59,7 +59,7 @@ class OracleKFAC(object):
         if rec.kind == 'conv':
             a = rec.attrs
             return [O.conv_A(rec.x, a['ksize'], a['stride'], a['pad'], 'b' in rec.params),
-                    O.conv_G(rec.gy, self.loss_scale)]
+                    O.conv_G(rec.gy, self.loss_scale, diag=a.get('diag', False))]
         return [O.bn_F(rec.x, rec.gy, rec.attrs['eps'], self.loss_scale,
                        'gamma' in rec.params, 'beta' in rec.params)]
 

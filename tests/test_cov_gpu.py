@@ -469,3 +469,98 @@ def test_workspace_too_small_is_reported():
     assert rc == -3 and b'workspace' in lib.kfac_last_error_string()
     rc = lib.kfac_cov_linear_f32(x.data_ptr(), 0, 8, 0, 1.0, 0.0, C.data_ptr(), None, 0, None)
     assert rc == -1
+
+
+def _conv_block(c_in, c_out, k, diag=False, diagonalize=False):
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import fisher_blocks as FB
+    link = L.Convolution2D(c_in, c_out, k, 1, k // 2, device='cuda')
+    if diag:
+        link.diag = True
+    fb = FB.FisherBlockConvolution2D('/conv', link, cov_ema_decay=1.0, damping=1e-3)
+    fb.diagonalize = diagonalize
+    return link, fb
+
+
+@pytest.mark.parametrize('kw', [{'diag': True}, {'diagonalize': True}])
+def test_conv_G_diagonal_branches(kw):
+    """``link.diag`` and the block's ``diagonalize``: G = diag(diag(G)), still a matrix, also when
+    the factor is accumulated over micro-batches (reference convolution_2d.py:56-70)."""
+    from chainerkfac_amd import links as L
+    r = np.random.default_rng(31)
+    link, fb = _conv_block(6, 40, 3, **kw)
+    x = torch.from_numpy(r.standard_normal((4, 6, 9, 9)).astype(np.float32)).cuda()
+    gys = [(r.standard_normal((4, 40, 9, 9)) / 4).astype(np.float32) for _ in range(2)]
+    func = L.Convolution2DFunction()
+    fb.forward_postprocess(func, (x, link.W.data, link.b.data))
+    fb.backward_preprocess(func, (x, link.W.data, link.b.data), (torch.from_numpy(gys[0]).cuda(),))
+    G = fb.covs[1].cpu().numpy()
+    assert G.shape == (40, 40) and np.count_nonzero(G - np.diag(np.diag(G))) == 0
+    np.testing.assert_allclose(G, O.conv_G(gys[0], **kw), rtol=1e-4, atol=1e-7)
+    # two micro-batches: the mean of the two diagonal factors
+    acc = None
+    for i, gy in enumerate(gys):
+        fb.acc_state = (2, i)
+        fb.backward_preprocess(func, (x, link.W.data, link.b.data), (torch.from_numpy(gy).cuda(),))
+        acc = O.accumulate_covs(acc, [O.conv_G(gy, **kw)], 2)
+    G = fb.covs[1].cpu().numpy()
+    assert np.count_nonzero(G - np.diag(np.diag(G))) == 0
+    np.testing.assert_allclose(G, acc[0], rtol=1e-4, atol=1e-7)
+
+
+def test_linear_and_batchnorm_diagonalize():
+    """``diagonalize`` on the other blocks: the linear A factor becomes a vector, G and the
+    batch-norm factor diagonal matrices (reference linear.py:25,43-44, batch_normalization.py:121-124),
+    and the batch-norm block no longer offers its low-rank inverse."""
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import fisher_blocks as FB
+    r = np.random.default_rng(32)
+    lin = L.Linear(33, 20, device='cuda')
+    fb = FB.FisherBlockLinear('/fc', lin, cov_ema_decay=1.0, damping=1e-3)
+    fb.diagonalize = True
+    x = r.standard_normal((16, 33)).astype(np.float32)
+    gy = (r.standard_normal((16, 20)) / 16).astype(np.float32)
+    func = L.LinearFunction()
+    in_data = (torch.from_numpy(x).cuda(), lin.W.data, lin.b.data)
+    fb.forward_postprocess(func, in_data)
+    fb.backward_preprocess(func, in_data, (torch.from_numpy(gy).cuda(),))
+    A, G = (c.cpu().numpy() for c in fb.covs)
+    assert A.shape == (34,) and G.shape == (20, 20)
+    np.testing.assert_allclose(A, O.linear_A(x, True, diagonalize=True), rtol=1e-4)
+    np.testing.assert_allclose(G, O.linear_G(gy, diagonalize=True), rtol=1e-4, atol=1e-7)
+    bn = L.BatchNormalization(12, device='cuda')
+    fbn = FB.FisherBlockBatchNormalization('/bn', bn, cov_ema_decay=1.0, damping=1e-3)
+    fbn.diagonalize = True
+    xb = r.standard_normal((8, 12, 5, 5)).astype(np.float32)
+    gb = (r.standard_normal((8, 12, 5, 5)) / 8).astype(np.float32)
+    fbn.backward_preprocess(L.BatchNormalizationFunction(), (torch.from_numpy(xb).cuda(), bn.gamma.data, bn.beta.data),
+                            (torch.from_numpy(gb).cuda(),))
+    F = fbn.covs[0].cpu().numpy()
+    assert np.count_nonzero(F - np.diag(np.diag(F))) == 0
+    np.testing.assert_allclose(F, O.bn_F(xb, gb, bn.eps, diagonalize=True), rtol=1e-4, atol=1e-7)
+    fbn.update_cov_emas()
+    assert fbn.lowrank_inverse_args() is None
+
+
+@pytest.mark.parametrize('n,c,h,w', [(32, 64, 56, 56), (32, 128, 28, 28), (32, 256, 14, 14), (32, 512, 7, 7),
+                                     (32, 32, 112, 112)])
+def test_resnet_3x3_shapes_take_the_shift_route(n, c, h, w):
+    """The 3x3 convolutions of ResNet-50 (and the 32-channel stem convolution of ResNet-50-D, with
+    stacked tiles) are computed from shifted correlations when called the way the benchmark calls
+    them: through ``ops.cov_conv_a`` with the workspace ``kfac_cov_workspace_bytes`` reports.  A
+    workspace that is too small sends them to the patch-product kernels without an error, so the
+    route is read back from the library."""
+    from chainerkfac_amd import _lib, ops
+    lib = _lib.load()
+    x = torch.randn(n, c, h, w, device='cuda')
+    A = ops.cov_conv_a(x, 3, 1, 1, True, 1.0 / n)
+    assert lib.kfac_cov_conv_a_last_route() == 1      # KFAC_CONV_ROUTE_SHIFT
+    assert torch.equal(A, A.T)
+    # the same call with the route switched off lands on the rows kernels
+    with _lib.options(conv_shift=0):
+        ops.cov_conv_a(x, 3, 1, 1, True, 1.0 / n)
+    assert lib.kfac_cov_conv_a_last_route() == 2      # KFAC_CONV_ROUTE_ROWS
+    # other geometries report their own routes
+    ops.cov_conv_a(torch.randn(2, 16, 9, 9, device='cuda'), 1, 1, 0, True, 0.5)
+    assert lib.kfac_cov_conv_a_last_route() == 0      # KFAC_CONV_ROUTE_SLAB
+    torch.cuda.synchronize()

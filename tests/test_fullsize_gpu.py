@@ -60,10 +60,12 @@ def test_conv_G_full_size(c, hw):
 
 
 def test_inverse_of_all_161_factor_sizes():
-    """The inverse-only configuration: one SPD matrix per factor of ResNet-50 (64 .. 4609)."""
-    from chainerkfac_amd import ops, workloads as W
-    dims = W.all_factor_dims(W.resnet50_v1())
-    assert len(dims) == 161 and max(dims) == 4609
+    """The inverse-only configuration: 161 SPD matrices of ResNet-50's factor sizes, 27^2 .. 4609^2
+    (the list the benchmark's c4 builds)."""
+    import bench
+    from chainerkfac_amd import ops
+    dims = bench.inverse_dims()
+    assert len(dims) == 161 and max(dims) == 4609 and min(dims) == 27
     g = torch.Generator(device='cuda').manual_seed(4)
     mats = []
     for d in dims:

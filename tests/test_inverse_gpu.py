@@ -300,3 +300,44 @@ def test_capture_on_a_forked_stream_keeps_the_inverse_on_that_stream():
         assert info.cpu().tolist() == [0, 0, 0]
         for o, e in zip(outs, eager):
             assert torch.equal(o, e)
+
+
+def test_update_invs_with_a_diagonal_factor():
+    """A factor kept as a vector is inverted entry by entry, 1 / (cov + diagvals), beside the dense
+    inverse of the block's other factor, with pi taken from the vector's sum (reference
+    fisher_block.py:23-42, :165-179); the batched path of the optimizer hands such blocks to it."""
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import KFAC
+    from chainerkfac_amd.optimizers import fisher_blocks as FB
+    r = np.random.default_rng(40)
+    lin = L.Linear(50, 30, device='cuda')
+    fb = FB.FisherBlockLinear('/fc', lin, cov_ema_decay=1.0, damping=1e-2)
+    a = (r.random(51) + 0.1).astype(np.float32)
+    G = spd(30, 77)
+    fb.cov_emas = [torch.from_numpy(a).cuda(), torch.from_numpy(G).cuda()]
+    fb.update_invs()
+    ref_emas = [a.copy(), G.copy()]
+    diagvals, _ = O.connection_diagvals(ref_emas[0], ref_emas[1], 1e-2)
+    ref = O.update_invs(ref_emas, diagvals)
+    assert fb.invs[0].shape == (51,) and fb.invs[1].shape == (30, 30)
+    np.testing.assert_allclose(fb.invs[0].cpu().numpy(), ref[0], rtol=1e-5)
+    assert np.linalg.norm(fb.invs[1].cpu().numpy() - ref[1]) < 1e-3 * np.linalg.norm(ref[1])
+    # the damped matrix is left in cov_emas, the vector untouched (as in the reference)
+    np.testing.assert_allclose(fb.cov_emas[1].cpu().numpy(), ref_emas[1], rtol=1e-6)
+    assert np.array_equal(fb.cov_emas[0].cpu().numpy(), a)
+    # through the optimizer's batched path, next to an ordinary block
+    model = L.Chain()
+    model.a = L.Linear(50, 30, device='cuda')
+    model.b = L.Linear(30, 8, device='cuda')
+    opt = KFAC(damping=1e-2, cov_ema_decay=1.0).setup(model)
+    fa, fbb = opt.fblocks
+    A2, G2 = spd(31, 5), spd(8, 6)
+    fa.cov_emas = [torch.from_numpy(a).cuda(), torch.from_numpy(G).cuda()]
+    fbb.cov_emas = [torch.from_numpy(A2).cuda(), torch.from_numpy(G2).cuda()]
+    opt.update_invs_batched(opt.fblocks)
+    np.testing.assert_allclose(fa.invs[0].cpu().numpy(), ref[0], rtol=1e-5)
+    refb = [A2.copy(), G2.copy()]
+    dv, _ = O.connection_diagvals(refb[0], refb[1], 1e-2)
+    refb = O.update_invs(refb, dv)
+    for got, want in zip(fbb.invs, refb):
+        assert np.linalg.norm(got.cpu().numpy() - want) < 1e-3 * np.linalg.norm(want)

@@ -119,25 +119,32 @@ class Recorder(object):
                 out.append(LayerRecord('linear', name, c['x'], c['gy'], params, grads))
             elif isinstance(link, L.Convolution2D):
                 out.append(LayerRecord('conv', name, c['x'], c['gy'], params, grads, ksize=link.ksize,
-                                       stride=link.stride[0], pad=link.pad[0]))
+                                       stride=link.stride[0], pad=link.pad[0], diag=getattr(link, 'diag', False)))
             else:
                 out.append(LayerRecord('bn', name, c['x'], c['gy'], params, grads, eps=link.eps))
         return out
 
 
-def run_case(build, batches, **hyper):
+def run_case(build, batches, after_first_update=None, prepare=None, **hyper):
+    """``after_first_update(model, ref_model, opt, oracle)`` is called once both sides have made
+    their first parameter update (the only one whose inputs are bit-identical on both sides);
+    ``prepare(model)`` is applied to both models before the optimizers are set up."""
     from chainerkfac_amd import links as L
     from chainerkfac_amd.optimizers import KFAC
     gen = torch.Generator(device='cpu').manual_seed(7)
     ref_model = build(L, 'cpu', gen)
     model = build(L, 'cuda', None)
     copy_params(ref_model, model)
+    if prepare is not None:
+        prepare(model)
+        prepare(ref_model)
     opt = KFAC(**hyper).setup(model)
     oracle = OracleKFAC(**hyper)
 
     def lossfun(m, x, t):
         return TF.cross_entropy(m(x), t)
 
+    updates = 0
     for x, t in batches:
         opt.update(lossfun, model, torch.from_numpy(x).cuda(), torch.from_numpy(t).cuda())
         rec = Recorder(L, ref_model)
@@ -145,12 +152,20 @@ def run_case(build, batches, **hyper):
         with rec.hook():
             loss = lossfun(ref_model, torch.from_numpy(x), torch.from_numpy(t))
             loss.backward()
-        oracle.step(rec.records())   # updates ref_model's parameters in place (shared memory)
+        # updates ref_model's parameters in place (shared memory); False inside an accumulation
+        updates += bool(oracle.step(rec.records()))
+        if updates == 1 and after_first_update is not None:
+            torch.cuda.synchronize()
+            after_first_update(model, ref_model, opt, oracle)
+            after_first_update = None
     torch.cuda.synchronize()
     return model, ref_model, opt, oracle
 
 
-def compare(model, ref_model, opt, oracle, tol_param=1e-3, tol_kf=1e-3):
+def compare(model, ref_model, opt, oracle, tol_param=1e-3, tol_kf=1e-3, loose=None):
+    """Factors 1e-4, inverses 1e-3, preconditioned gradients ``tol_kf``, parameters ``tol_param``;
+    ``loose`` maps a parameter path ('/fc/b') to its own (tol_param, tol_kf)."""
+    loose = loose or {}
     by_name = {fb.linkname: fb for fb in opt.fblocks}
     assert [fb.linkname for fb in opt.fblocks] == sorted(by_name)
     for name, invs in oracle.invs.items():
@@ -162,9 +177,11 @@ def compare(model, ref_model, opt, oracle, tol_param=1e-3, tol_kf=1e-3):
     for (lname, pname), ref in oracle.kfgrads.items():
         got = getattr(by_name[lname].link, pname).kfgrad.cpu().numpy()
         assert got.shape == ref.shape
-        assert rel(got, ref) < tol_kf, (lname, pname)
+        tol = loose.get(lname + '/' + pname, (tol_param, tol_kf))[1]
+        assert rel(got, ref) < tol, (lname, pname, rel(got, ref))
     for (n1, p1), (n2, p2) in zip(sorted(model.namedparams()), sorted(ref_model.namedparams())):
-        assert rel(p1.data.cpu().numpy(), p2.data.numpy()) < tol_param, n1
+        tol = loose.get(n1, (tol_param, tol_kf))[0]
+        assert rel(p1.data.cpu().numpy(), p2.data.numpy()) < tol, (n1, rel(p1.data.cpu().numpy(), p2.data.numpy()))
     assert int((opt.inv_info != 0).sum()) == 0
 
 
@@ -196,16 +213,33 @@ def test_mlp_three_steps_moving_average_and_momentum():
     parameters drift apart by ~1e-6), and the damped inverse of the nearly
     singular softmax-gradient factor amplifies that; the 1e-3 bound of the
     single-step tests is therefore relaxed to 5e-3 for the later steps."""
-    out = run_case(build_mlp, mnist_batches(3, bs=32), lr=1e-2, momentum=0.9, cov_ema_decay=0.9, damping=1e-2)
+    out = run_case(build_mlp, mnist_batches(3, bs=32), after_first_update=compare,
+                   lr=1e-2, momentum=0.9, cov_ema_decay=0.9, damping=1e-2)   # first step: 1e-3
     compare(*out, tol_param=2e-3, tol_kf=5e-3)
     shadow_check(*out)
 
 
 def test_cnn_with_batchnorm_two_steps():
-    out = run_case(build_cnn, cnn_batches(2), lr=1e-2, momentum=0.9, cov_ema_decay=1.0, damping=1e-2,
-                   stab_coeff=16.0)
+    out = run_case(build_cnn, cnn_batches(2), after_first_update=compare,
+                   lr=1e-2, momentum=0.9, cov_ema_decay=1.0, damping=1e-2, stab_coeff=16.0)   # first step: 1e-3
     compare(*out, tol_param=2e-3, tol_kf=5e-3)
     shadow_check(*out)
+
+
+def test_cnn_with_diagonal_G_factor():
+    """``link.diag = True`` on a convolution (a user-settable attribute the reference reads at
+    convolution_2d.py:68-70): G = diag(diag(G)) goes through damping, inverse and preconditioning
+    like any other factor; one step against the oracle."""
+    def prepare(model):
+        model.conv1.diag = True
+        model.conv3.diag = True
+    out = run_case(build_cnn, cnn_batches(1), prepare=prepare, lr=1e-2, momentum=0.9, cov_ema_decay=1.0,
+                   damping=1e-2, stab_coeff=16.0)
+    compare(*out)
+    opt = out[2]
+    for name in ('/conv1', '/conv3'):
+        G = {fb.linkname: fb for fb in opt.fblocks}[name].covs[1].cpu().numpy()
+        assert np.count_nonzero(G - np.diag(np.diag(G))) == 0
 
 
 def kfgrad_errors_vs_float64(A_damped, G_damped, gW, gb, kW, kb):
@@ -265,11 +299,13 @@ def test_cifar_cnn_one_step_config2():
     batches = [(r.standard_normal((128, 3, 32, 32)).astype(np.float32), r.integers(0, 10, 128).astype(np.int64))]
     model, ref_model, opt, oracle = run_case(build_cifar_cnn, batches, lr=1e-3, momentum=0.9,
                                              cov_ema_decay=0.99, damping=1e-3)
-    # (a bias starts at 0, so after one step it is the update itself: same bound as the kfgrads.
-    # The bias row of the last layer rides on the last column of the 4097x4097 inverse, which the
-    # NumPy formula itself gets right to 0.7 % only: 2e-2 between the two float32 results, and the
-    # float64 criterion below for the bias on its own.)
-    compare(model, ref_model, opt, oracle, tol_param=2e-2, tol_kf=2e-2)
+    # The three convolutions meet rel 1e-3 against the oracle.  The last layer's 4097 x 4097 factor
+    # is where two float32 evaluations part: 1e-2 for its weights; its bias row rides on the last
+    # column of that inverse, which the NumPy formula itself gets right to 0.7 % only, so 2e-2
+    # between the two float32 results there (a bias starts at 0, so after one step it is the update
+    # itself) and the float64 criterion below for the bias on its own.
+    compare(model, ref_model, opt, oracle, tol_param=1e-3, tol_kf=1e-3,
+            loose={'/fc/W': (1e-3, 1e-2), '/fc/b': (2e-2, 2e-2)})
     assert [tuple(c.shape) for fb in opt.fblocks for c in fb.covs] == \
         [(28, 28), (64, 64), (577, 577), (128, 128), (1153, 1153), (256, 256), (4097, 4097), (10, 10)]
     ref_links = dict(ref_model.namedlinks())
@@ -295,7 +331,19 @@ def test_cifar_cnn_one_step_config2():
         rkb64 = (rG64 @ rg.astype(np.float64) @ rA64)[:, -1]
         err_hip_b = rel(b.kfgrad.cpu().numpy(), kb64)
         err_ref_b = rel(oracle.kfgrads[(name, 'b')], rkb64)
-        assert err_hip_b < max(2 * err_ref_b, 1e-3), (name, err_hip_b, err_ref_b)
+        assert err_hip_b < max(1.25 * err_ref_b, 2e-4), (name, err_hip_b, err_ref_b)
+    # the bordered-matrix path of the inverse (d = 128 m + 1: 577, 1153, 4097) against the path that
+    # tiles such matrices whole, on this step's damped factors: what separates the two HIP results
+    # is rounding, not the border formula
+    from chainerkfac_amd import _lib, ops
+    mats = [c.clone() for fb in opt.fblocks for c in fb.cov_emas]
+    bordered, _ = ops.spd_inverse_batched(mats)
+    with _lib.options(inverse_border=0):
+        whole, _ = ops.spd_inverse_batched(mats + [torch.eye(3, device='cuda')])
+    for M, a, b in zip(mats, bordered, whole):
+        ref64 = np.linalg.inv(M.cpu().numpy().astype(np.float64))
+        ea, eb = rel(a.cpu().numpy(), ref64), rel(b.cpu().numpy(), ref64)
+        assert ea < max(2 * eb, 1e-5), (M.shape, ea, eb)
 
 
 def test_accumulation_over_micro_batches():
@@ -341,7 +389,8 @@ def test_loss_scale_cancels_end_to_end():
     for name, emas in oracle.cov_emas.items():
         for got, ref in zip(by_name[name].cov_emas, emas):
             assert rel(got.cpu().numpy(), ref) < 1e-4, name
-    # kfgrads were divided by the scale in place; gradients still carry it
+    # kfgrads were divided by the scale in place (reference kfac.py:76-78) and so were the
+    # gradients (Chainer's UpdateRule.update, which the reference's rule calls next)
     for (lname, pname), ref in oracle.kfgrads.items():
         got = getattr(by_name[lname].link, pname).kfgrad.cpu().numpy()
         assert rel(got, ref) < 5e-3, (lname, pname)
@@ -349,7 +398,7 @@ def test_loss_scale_cancels_end_to_end():
     for name, p in model.namedparams():
         # (the bias of conv1 feeds a batch normalisation: its gradient is zero up to rounding noise)
         if name != '/conv1/b':
-            assert rel(p.grad.cpu().numpy(), 128.0 * ref_params[name].grad.numpy()) < 1e-4, name
+            assert rel(p.grad.cpu().numpy(), ref_params[name].grad.numpy()) < 1e-4, name
         assert rel(p.data.cpu().numpy(), ref_params[name].data.numpy()) < 2e-3, name
 
 
@@ -660,3 +709,48 @@ def test_float16_parameter_is_updated_through_a_float32_master_copy(batched):
         # the float16 parameter is the rounded master copy, not an accumulation of rounded steps
         assert torch.equal(p.data, rule._fp32_param.half())
         assert (rule._fp32_param.double() - master).abs().max() <= 1e-5
+
+
+def test_float32_parameter_with_float16_gradients_and_both_divisions():
+    """A float32 parameter whose gradients arrive in float16 (the batched launch does not take the
+    pair and hands it to the per-parameter rule, which casts up), and the two in-place divisions of
+    a scaled loss: ``kfgrad`` by the reference's rule (kfac.py:76-78), ``grad`` by Chainer's
+    UpdateRule.update, also on the batched path."""
+    from chainerkfac_amd import links as L
+    from chainerkfac_amd.optimizers import KFAC
+    from chainerkfac_amd.optimizers.kfac import KFACUpdateRule, Hyperparameter
+
+    class P(object):
+        pass
+
+    g = torch.Generator(device='cuda').manual_seed(8)
+    hp = Hyperparameter()
+    hp.lr, hp.lr_pre, hp.momentum = 0.1, 0.1, 0.0
+    p = P()
+    p.data = torch.randn(100, device='cuda', generator=g)
+    before = p.data.clone()
+    p.grad = torch.randn(100, device='cuda', generator=g).half()
+    p.kfgrad = p.grad.clone()
+    p._loss_scale = None
+    rule = KFACUpdateRule(hp)
+    assert rule.batched_job(p) is NotImplemented
+    rule.t = 0
+    rule.update(p)
+    assert torch.allclose(p.data, before - 0.1 * p.kfgrad.float(), rtol=1e-6, atol=1e-7)
+    # both arrays of a float32 parameter are divided by the loss scale
+    for batched in (False, True):
+        model = L.Chain()
+        model.fc = L.Linear(6, 4, device='cuda')
+        opt = KFAC(lr=0.1, momentum=0.0, loss_scale=4.0).setup(model)
+        opt.batch_param_updates = batched
+        for q in model.params():
+            q.grad = torch.full(q.data.shape, 8.0, device='cuda')
+            q.kfgrad = torch.full(q.data.shape, 2.0, device='cuda')
+            q._loss_scale = 4.0
+        start = [q.data.clone() for q in model.params()]
+        opt.update_params()
+        torch.cuda.synchronize()
+        for q, s0 in zip(model.params(), start):
+            assert torch.equal(q.grad, torch.full_like(q.grad, 2.0))
+            assert torch.equal(q.kfgrad, torch.full_like(q.kfgrad, 0.5))
+            assert torch.allclose(q.data, s0 - 0.1 * 0.5)

@@ -177,3 +177,33 @@ def test_ema_weights_new_cov_by_decay_and_aliases_first():
     assert same[0] is a
     ema = O.update_cov_emas([a], [np.zeros((2, 2), np.float32)], 0.75)
     np.testing.assert_allclose(ema[0], 1.5)   # 0.75 * new + 0.25 * old
+
+
+def test_diagonal_branches_are_the_diagonals_of_the_full_factors():
+    """The ``diagonalize`` / ``link.diag`` branches (linear.py:25,43-44, convolution_2d.py:56-70,
+    batch_normalization.py:121-124) against the diagonal of the float64 Gram matrix written out
+    independently: a vector for the linear A factor, matrices with zero off-diagonals elsewhere."""
+    r = rng(20)
+    x = r.standard_normal((6, 5)).astype(np.float32)
+    xe = np.concatenate([x.astype(np.float64), np.ones((6, 1))], axis=1)
+    A = O.linear_A(x, True, diagonalize=True)
+    assert A.shape == (6,)
+    np.testing.assert_allclose(A, np.einsum('ni,ni->i', xe, xe) / 6, rtol=1e-5)
+    gy = (r.standard_normal((6, 4)) / 6).astype(np.float32)
+    G = O.linear_G(gy, diagonalize=True)
+    g64 = gy.astype(np.float64)
+    assert G.shape == (4, 4) and np.count_nonzero(G - np.diag(np.diag(G))) == 0
+    np.testing.assert_allclose(np.diag(G), 6 * np.einsum('ni,ni->i', g64, g64), rtol=1e-5)
+    gyc = (r.standard_normal((3, 4, 5, 5)) / 3).astype(np.float32)
+    full = O.conv_G(gyc).astype(np.float64)
+    for kw in ({'diag': True}, {'diagonalize': True}):
+        Gc = O.conv_G(gyc, **kw)
+        assert Gc.shape == (4, 4) and np.count_nonzero(Gc - np.diag(np.diag(Gc))) == 0
+        np.testing.assert_allclose(np.diag(Gc), np.diag(full), rtol=1e-5)
+        m = gyc.astype(np.float64).transpose(0, 2, 3, 1).reshape(-1, 4)
+        np.testing.assert_allclose(np.diag(Gc), 3.0 ** 2 / 75 * np.einsum('ni,ni->i', m, m), rtol=1e-5)
+    xb = r.standard_normal((4, 3, 5, 5)).astype(np.float32)
+    gb = (r.standard_normal((4, 3, 5, 5)) / 4).astype(np.float32)
+    F = O.bn_F(xb, gb, 2e-5, diagonalize=True)
+    assert F.shape == (6, 6) and np.count_nonzero(F - np.diag(np.diag(F))) == 0
+    np.testing.assert_allclose(np.diag(F), np.diag(O.bn_F(xb, gb, 2e-5)), rtol=1e-5)
