@@ -212,18 +212,18 @@ extern "C" int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, i
   kfac::TimedLaunch timed(KFAC_TIMED_BN, s);
   const bool stats_loop = kfac::option_int(kfac::kOptBnStatsLoop, 0) != 0;   // tuning override
   if (vec && hw <= 4 * 16 * 4 && !stats_loop)
-    hipLaunchKernelGGL((bn_stats_reg_kernel<16, 4>), dim3(kfac::ceil_div(nslab, kThreads / 16)),
+    KFAC_LAUNCH((bn_stats_reg_kernel<16, 4>), dim3(kfac::ceil_div(nslab, kThreads / 16)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
   else if (vec && hw > 256 && hw <= 4 * 64 * 13 && !stats_loop)
-    hipLaunchKernelGGL((bn_stats_reg_kernel<64, 13>), dim3(kfac::ceil_div(nslab, kThreads / 64)),
+    KFAC_LAUNCH((bn_stats_reg_kernel<64, 13>), dim3(kfac::ceil_div(nslab, kThreads / 64)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
   else if (hw <= 256)
-    hipLaunchKernelGGL(bn_stats_kernel<16>, dim3(kfac::ceil_div(nslab, kThreads / 16)),
+    KFAC_LAUNCH(bn_stats_kernel<16>, dim3(kfac::ceil_div(nslab, kThreads / 16)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
   else
-    hipLaunchKernelGGL(bn_stats_kernel<64>, dim3(kfac::ceil_div(nslab, kThreads / 64)),
+    KFAC_LAUNCH(bn_stats_kernel<64>, dim3(kfac::ceil_div(nslab, kThreads / 64)),
                        dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
-  hipLaunchKernelGGL(bn_finish_kernel, dim3(kfac::ceil_div(c, 64)), dim3(256), 0, s, n, c, hw, eps,
+  KFAC_LAUNCH(bn_finish_kernel, dim3(kfac::ceil_div(c, 64)), dim3(256), 0, s, n, c, hw, eps,
                      gy_scale, has_gamma ? 1 : 0, has_beta ? 1 : 0, smean, sm2, sg, sgx, U);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;

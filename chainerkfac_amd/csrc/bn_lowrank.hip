@@ -335,10 +335,10 @@ extern "C" int kfac_bn_lowrank_inverse_batched_f32(kfac_bn_lowrank_plan_t plan,
   tb.winv = tb.part + (size_t)plan->chunks * NMAX * NMAX;
   tb.V = reinterpret_cast<float *>(tb.winv + (size_t)count * NMAX * NMAX);
   tb.info = info_dev;
-  hipLaunchKernelGGL(lr_gram_kernel, dim3(plan->chunks), dim3(256), 0, s, tb, count, plan->n);
-  hipLaunchKernelGGL(lr_factor_kernel, dim3(count), dim3(kFactorThreads), 0, s, tb);
-  hipLaunchKernelGGL(lr_apply_kernel, dim3(plan->chunks), dim3(CHUNK), 0, s, tb, count, plan->n);
-  hipLaunchKernelGGL(lr_outer_kernel, dim3(plan->tiles), dim3(256), 0, s, tb, count);
+  KFAC_LAUNCH(lr_gram_kernel, dim3(plan->chunks), dim3(256), 0, s, tb, count, plan->n);
+  KFAC_LAUNCH(lr_factor_kernel, dim3(count), dim3(kFactorThreads), 0, s, tb);
+  KFAC_LAUNCH(lr_apply_kernel, dim3(plan->chunks), dim3(CHUNK), 0, s, tb, count, plan->n);
+  KFAC_LAUNCH(lr_outer_kernel, dim3(plan->tiles), dim3(256), 0, s, tb, count);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }

@@ -23,12 +23,26 @@ inline int fail(int code, const char *fmt, ...) {
   return code;
 }
 
+// Host-only mode (option host_only = 1): no call reaches the HIP runtime.  Plans are
+// built, arguments checked, task tables filled and every launch site passed with its
+// grid computed, but nothing is allocated, copied or launched: the planners and their
+// index arithmetic then run on a machine without a GPU, under a host sanitizer.
+bool host_only();
+
 #define KFAC_HIP_CHECK(expr)                                                   \
   do {                                                                         \
-    hipError_t e_ = (expr);                                                    \
-    if (e_ != hipSuccess)                                                      \
-      return ::kfac::fail(KFAC_EHIP, "%s failed: %s (%s:%d)", #expr,           \
-                          hipGetErrorString(e_), __FILE__, __LINE__);          \
+    if (!::kfac::host_only()) {                                                \
+      hipError_t e_ = (expr);                                                  \
+      if (e_ != hipSuccess)                                                    \
+        return ::kfac::fail(KFAC_EHIP, "%s failed: %s (%s:%d)", #expr,         \
+                            hipGetErrorString(e_), __FILE__, __LINE__);        \
+    }                                                                          \
+  } while (0)
+
+// Every kernel launch of the library goes through here.
+#define KFAC_LAUNCH(...)                                                       \
+  do {                                                                         \
+    if (!::kfac::host_only()) hipLaunchKernelGGL(__VA_ARGS__);                 \
   } while (0)
 
 #define KFAC_REQUIRE(cond, ...)                                                \
@@ -50,6 +64,7 @@ class DevTable {
   DevTable(const DevTable &) = delete;
   DevTable &operator=(const DevTable &) = delete;
   ~DevTable() {
+    if (dev_ == &host_only_address_) dev_ = nullptr;
     if (dev_) (void)hipFree(dev_);
     if (staging_) (void)hipHostFree(staging_);
     if (copied_) (void)hipEventDestroy(copied_);
@@ -62,6 +77,7 @@ class DevTable {
   // a graph replays against them, so they must never change again
   bool pinned() const { return pinned_; }
   int set(const void *host, size_t bytes, hipStream_t stream) {
+    if (host_only()) return set_sync(host, bytes);
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cs) != hipSuccess) {
       (void)hipGetLastError();
@@ -114,6 +130,11 @@ class DevTable {
   // Upload that has finished when the call returns (plan creation: the tables are read by
   // launches on whatever streams the plan is used on later).
   int set_sync(const void *host, size_t bytes) {
+    if (host_only()) {   // the contents only: nothing lives on a device
+      shadow_.assign(static_cast<const char *>(host), static_cast<const char *>(host) + bytes);
+      if (!dev_) dev_ = &host_only_address_;
+      return KFAC_OK;
+    }
     if (matches(host, bytes)) return KFAC_OK;
     if (pinned_)
       return ::kfac::fail(KFAC_EINVAL, "a device table that a captured graph replays against would have to change");
@@ -145,6 +166,10 @@ class DevTable {
   std::vector<char> shadow_;
   hipEvent_t copied_ = nullptr;
   bool copy_pending_ = false, pinned_ = false;
+  char host_only_address_ = 0;   // what as<T>() returns in host-only mode (never dereferenced)
+  // the contents last set, for checks of the tables on the host
+ public:
+  const std::vector<char> &shadow() const { return shadow_; }
 };
 
 // A few device copies of a table whose contents alternate between a small number
@@ -226,6 +251,7 @@ enum Option : int {
   kOptInverseAlign,       // inverse: 0 = sweeps start together ... 100 = end together
   kOptPrecondTasks,       // grouped preconditioning: workgroups per launch
   kOptBnStatsLoop,        // 1: batch-norm statistics always by the looping kernel
+  kOptHostOnly,           // 1: host-only mode: plan, check and count, never touch a GPU
   kOptCount
 };
 bool option_is_set(Option o);

@@ -512,7 +512,7 @@ int finish_partials(const SyrkPlan &p, int d, int ones, float count, float alpha
     float *red = partial + (size_t)p.nsplit * slot;
     const int per = kfac::ceil_div(p.nsplit, p.nreduced);
     nfin = kfac::ceil_div(p.nsplit, per);
-    hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)kfac::ceil_div<long long>(slot4, 256), nfin),
+    KFAC_LAUNCH(reduce_kernel, dim3((unsigned)kfac::ceil_div<long long>(slot4, 256), nfin),
                        dim3(256), 0, stream, reinterpret_cast<const float4 *>(partial),
                        reinterpret_cast<float4 *>(red), p.nsplit, per, slot4);
     KFAC_HIP_CHECK(hipGetLastError());
@@ -526,7 +526,7 @@ int finish_partials(const SyrkPlan &p, int d, int ones, float count, float alpha
                                             finish_kernel<4>, finish_kernel<5>, finish_kernel<6>,
                                             finish_kernel<7>, finish_kernel<8>};
   if (nfin < 1 || nfin > kFinishSplits) return kfac::fail(KFAC_EINVAL, "bad slice count %d", nfin);
-  hipLaunchKernelGGL(kerns[nfin - 1], dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, fin, p.ntile,
+  KFAC_LAUNCH(kerns[nfin - 1], dim3(sub * (sub + 1) / 2), dim3(256), 0, stream, fin, p.ntile,
                      p.bm, slot, dt, d, ones, count, alpha, beta, C);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -554,10 +554,10 @@ int run_syrk(const L64 &l64, const L128 &l128, int d, int ones, long long K, flo
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
     if (p.bm == 64)
-      hipLaunchKernelGGL((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
+      KFAC_LAUNCH((syrk_kernel<1, L64>), dim3(grid), dim3(THREADS), 0, stream, l64, K,
                          p.klen, p.ntile, p.nsplit, direct, d, ones, alpha, beta, partial, C);
     else
-      hipLaunchKernelGGL((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
+      KFAC_LAUNCH((syrk_kernel<2, L128>), dim3(grid), dim3(THREADS), 0, stream, l128, K,
                          p.klen, p.ntile, p.nsplit, direct, d, ones, alpha, beta, partial, C);
   }
   KFAC_HIP_CHECK(hipGetLastError());
@@ -668,6 +668,7 @@ int run_conv_halo(const ConvGeom &g, int n, int d, int ones, float alpha, float 
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [] {
+    if (kfac::host_only()) return;
     for (int i = 0; i < 3; ++i)
       for (int j = 0; j < 2; ++j) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kerns[i][j]),
@@ -683,7 +684,7 @@ int run_conv_halo(const ConvGeom &g, int n, int d, int ones, float alpha, float 
   const Kern kern = kerns[g.nk == 50 ? 0 : (g.nk == 56 ? 1 : 2)][mask ? 1 : 0];
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, g, total_steps, p.klen, p.ntile, p.nsplit,
+    KFAC_LAUNCH(kern, grid, block, lds, stream, g, total_steps, p.klen, p.ntile, p.nsplit,
                        direct, d, ones, count, alpha, beta, partial, C);
   }
   KFAC_HIP_CHECK(hipGetLastError());
@@ -714,6 +715,7 @@ int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int
   static std::once_flag once;
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [] {
+    if (kfac::host_only()) return;
     attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(syrk_rows_kernel<Cfg>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   });
@@ -722,7 +724,7 @@ int run_conv_rows(const float *x, int n, int c, int h, int w, int ho, int d, int
   const int direct = p.nsplit == 1 ? 1 : 0;
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
-    hipLaunchKernelGGL((syrk_rows_kernel<Cfg>), dim3(p.ntile * p.nsplit), dim3(THREADS), lds, stream,
+    KFAC_LAUNCH((syrk_rows_kernel<Cfg>), dim3(p.ntile * p.nsplit), dim3(THREADS), lds, stream,
                        g, total_steps, p.klen, p.ntile, p.nsplit, direct, d, ones, count, alpha, beta,
                        partial, C);
   }
@@ -1015,12 +1017,12 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   if (partial + partial_floats > arrays) return too_small(partial_floats + tail_floats + 4);
   {
     kfac::TimedLaunch timed(KFAC_TIMED_COV_AUX, stream);
-    hipLaunchKernelGGL(edge_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums, edges);
+    KFAC_LAUNCH(edge_sums_kernel, dim3(c, nchunk), dim3(256), 0, stream, pl, sums, edges);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream);
-    hipLaunchKernelGGL((corr_kernel<WM>), dim3(pl.total), dim3(THREADS), 0, stream, pl, partial);
+    KFAC_LAUNCH((corr_kernel<WM>), dim3(pl.total), dim3(THREADS), 0, stream, pl, partial);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   int max_split = 1;
@@ -1028,15 +1030,15 @@ int run_conv_shift(kfac::shift::Plan &pl, int d, int ones, float alpha, float be
   kfac::TimedLaunch timed_post(KFAC_TIMED_COV_AUX, stream);   // the two launches that follow
   if (max_split >= 32 && c <= 128) {
     const int nb = kfac::ceil_div(c, 16);
-    hipLaunchKernelGGL((corr_finish_kernel<4, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
+    KFAC_LAUNCH((corr_finish_kernel<4, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
                        arrays);
   } else {
     const int nb = kfac::ceil_div(c, 32);
-    hipLaunchKernelGGL((corr_finish_kernel<1, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
+    KFAC_LAUNCH((corr_finish_kernel<1, WM>), dim3(kProducts * nb * nb), dim3(256), 0, stream, pl, partial,
                        arrays);
   }
   KFAC_HIP_CHECK(hipGetLastError());
-  hipLaunchKernelGGL(assemble_kernel, dim3(c, kfac::ceil_div(c, 64), c <= 128 ? 3 : 1), dim3(256), 0, stream, pl, arrays, sums,
+  KFAC_LAUNCH(assemble_kernel, dim3(c, kfac::ceil_div(c, 64), c <= 128 ? 3 : 1), dim3(256), 0, stream, pl, arrays, sums,
                      nchunk, d, ones, (float)((long long)n * h * w), alpha, beta, C);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -1852,7 +1854,7 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   for (int k = 0; k < kMacroKind0; ++k) {
     if (group->ntask[k] == 0) continue;
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
-    hipLaunchKernelGGL(kerns[k], dim3(group->ntask[k]), dim3(THREADS), 0, s, st, dy,
+    KFAC_LAUNCH(kerns[k], dim3(group->ntask[k]), dim3(THREADS), 0, s, st, dy,
                        tasks + group->task0[k], base);
   }
   static const Kern macro_kerns[2] = {syrk_macro_kernel<LoaderKC<128, true>>,
@@ -1860,6 +1862,7 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   static std::once_flag macro_attr;
   static hipError_t macro_attr_rc = hipSuccess;
   std::call_once(macro_attr, [&] {
+    if (kfac::host_only()) return;
     for (Kern f : macro_kerns) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(f),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1871,13 +1874,13 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   for (int k = kMacroKind0; k < kGroupKinds; ++k) {
     if (group->ntask[k] == 0) continue;
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
-    hipLaunchKernelGGL(macro_kerns[k - kMacroKind0], dim3(group->ntask[k]), dim3(kMacroThreads),
+    KFAC_LAUNCH(macro_kerns[k - kMacroKind0], dim3(group->ntask[k]), dim3(kMacroThreads),
                        kMacroLdsBytes, s, st, dy, tasks + group->task0[k], base);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (group->nftask > 0) {
     kfac::TimedLaunch timed(KFAC_TIMED_COV_AUX, s);
-    hipLaunchKernelGGL(finish_group_kernel, dim3(group->nftask), dim3(256), 0, s, st, dy,
+    KFAC_LAUNCH(finish_group_kernel, dim3(group->nftask), dim3(256), 0, s, st, dy,
                        tasks + group->ftask0, base);
     KFAC_HIP_CHECK(hipGetLastError());
   }

@@ -112,7 +112,7 @@ extern "C" int kfac_pi_damp_batched_f32(kfac_damp_plan_t plan, float *const *A_p
   tb.dA = plan->d_dA.as<const int>();
   tb.dG = plan->d_dG.as<const int>();
   tb.rW = plan->d_rW.as<const double>();
-  hipLaunchKernelGGL(pi_damp_kernel, dim3(plan->count), dim3(kThreads), 0, s, tb, use_pi,
+  KFAC_LAUNCH(pi_damp_kernel, dim3(plan->count), dim3(kThreads), 0, s, tb, use_pi,
                      pi_out_dev);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;

@@ -89,7 +89,8 @@ const char *const kOptionNames[kOptCount] = {
     "syrk_bm64_max",   "syrk_splits",      "conv_rows",       "rows_wm",          "shift_slices5",
     "shift_slices3",   "conv_shift",       "conv_shift_strict", "group_bm64_max", "group_macro",
     "group_panels",    "group_macro_tasks", "group_graded",   "inverse_group",    "inverse_border",
-    "inverse_lookahead", "inverse_rest_lds", "inverse_align", "precond_tasks",    "bn_stats_loop"};
+    "inverse_lookahead", "inverse_rest_lds", "inverse_align", "precond_tasks",    "bn_stats_loop",
+    "host_only"};
 struct OptionState {
   bool set[kOptCount] = {};
   double value[kOptCount] = {};
@@ -121,6 +122,10 @@ int option_index(const char *name) {
 }
 }  // namespace
 bool option_is_set(Option o) { return option_state().set[o]; }
+bool host_only() {
+  const OptionState &st = option_state();
+  return st.set[kOptHostOnly] && st.value[kOptHostOnly] != 0.0;
+}
 double option_value(Option o, double unset_value) {
   const OptionState &st = option_state();
   return st.set[o] ? st.value[o] : unset_value;
@@ -382,7 +387,7 @@ extern "C" int kfac_axpby_f32(const float *x, float *y, int64_t nelems, float a,
   KFAC_REQUIRE(nelems >= 0, "nelems < 0");
   if (nelems == 0) return KFAC_OK;
   KFAC_REQUIRE(x && y, "null pointer");
-  hipLaunchKernelGGL(axpby_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0,
+  KFAC_LAUNCH(axpby_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0,
                      kfac::as_stream(stream), x, y, (long long)nelems, a, b);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -393,7 +398,7 @@ extern "C" int kfac_add_diag_f32(float *M, int d, int split, double v0, double v
   KFAC_REQUIRE(d >= 0, "d < 0");
   if (d == 0) return KFAC_OK;
   KFAC_REQUIRE(M != nullptr, "M is null");
-  hipLaunchKernelGGL(add_diag_kernel, dim3(kfac::ceil_div(d, kThreads)), dim3(kThreads),
+  KFAC_LAUNCH(add_diag_kernel, dim3(kfac::ceil_div(d, kThreads)), dim3(kThreads),
                      0, kfac::as_stream(stream), M, d, split, v0, v1);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -403,7 +408,7 @@ extern "C" int kfac_keep_diag_f32(float *M, int d, void *stream) {
   KFAC_REQUIRE(d >= 0 && d <= 46340, "bad dimension %d", d);
   if (d == 0) return KFAC_OK;
   KFAC_REQUIRE(M != nullptr, "M is null");
-  hipLaunchKernelGGL(keep_diag_kernel, dim3(grid_for((long long)d * d)), dim3(kThreads), 0,
+  KFAC_LAUNCH(keep_diag_kernel, dim3(grid_for((long long)d * d)), dim3(kThreads), 0,
                      kfac::as_stream(stream), M, d);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -414,7 +419,7 @@ extern "C" int kfac_recip_add_f32(const float *x, int64_t split, double v0, doub
   KFAC_REQUIRE(nelems >= 0, "nelems < 0");
   if (nelems == 0) return KFAC_OK;
   KFAC_REQUIRE(x && out, "null pointer");
-  hipLaunchKernelGGL(recip_add_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0, kfac::as_stream(stream),
+  KFAC_LAUNCH(recip_add_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0, kfac::as_stream(stream),
                      x, (long long)split, v0, v1, out, (long long)nelems);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -456,7 +461,7 @@ extern "C" int kfac_add_diag_batched_f32(kfac_diag_batch_t batch, int count, flo
   hipStream_t s = kfac::as_stream(stream);
   const void *dev = nullptr;
   if (int rc = batch->table.set(batch->host.data(), sizeof(DiagItem) * (size_t)count, s, &dev)) return rc;
-  hipLaunchKernelGGL(add_diag_batched_kernel, dim3(kfac::ceil_div(max_d, kThreads), count), dim3(kThreads),
+  KFAC_LAUNCH(add_diag_batched_kernel, dim3(kfac::ceil_div(max_d, kThreads), count), dim3(kThreads),
                      0, s, static_cast<const DiagItem *>(dev));
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -468,7 +473,7 @@ extern "C" int kfac_momentum_update_f32(float *param, float *v, const float *gra
   KFAC_REQUIRE(nelems >= 0, "nelems < 0");
   if (nelems == 0) return KFAC_OK;
   KFAC_REQUIRE(param && v && grad, "null pointer");
-  hipLaunchKernelGGL(momentum_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0,
+  KFAC_LAUNCH(momentum_kernel, dim3(grid_for(nelems)), dim3(kThreads), 0,
                      kfac::as_stream(stream), param, v, grad, (long long)nelems, lr,
                      momentum);
   KFAC_HIP_CHECK(hipGetLastError());
@@ -544,11 +549,11 @@ extern "C" int kfac_momentum_update_batched_f32(kfac_momentum_batch_t batch, int
   if (int rc = batch->owner_table.set(batch->owner.data(), sizeof(int) * batch->owner.size(), s, &d_owner))
     return rc;
   if (loss_scale != 1.f)
-    hipLaunchKernelGGL(momentum_batched_kernel<true>, dim3((unsigned)units), dim3(kThreads), 0, s,
+    KFAC_LAUNCH(momentum_batched_kernel<true>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const MomentumEntry *>(d_entries), static_cast<const int *>(d_owner), lr,
                        momentum, loss_scale);
   else
-    hipLaunchKernelGGL(momentum_batched_kernel<false>, dim3((unsigned)units), dim3(kThreads), 0, s,
+    KFAC_LAUNCH(momentum_batched_kernel<false>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const MomentumEntry *>(d_entries), static_cast<const int *>(d_owner), lr,
                        momentum, loss_scale);
   KFAC_HIP_CHECK(hipGetLastError());
@@ -609,13 +614,13 @@ int run_axpby_batch(kfac_axpby_batch_t batch, int count, const float *const *xs,
   if (int rc = batch->owner_table.set(batch->owner.data(), sizeof(int) * batch->owner.size(), s, &d_owner))
     return rc;
   if (divide)
-    hipLaunchKernelGGL(axpby_batched_kernel<2>, dim3((unsigned)units), dim3(kThreads), 0, s,
+    KFAC_LAUNCH(axpby_batched_kernel<2>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
   else if (b == 0.f)
-    hipLaunchKernelGGL(axpby_batched_kernel<1>, dim3((unsigned)units), dim3(kThreads), 0, s,
+    KFAC_LAUNCH(axpby_batched_kernel<1>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
   else
-    hipLaunchKernelGGL(axpby_batched_kernel<0>, dim3((unsigned)units), dim3(kThreads), 0, s,
+    KFAC_LAUNCH(axpby_batched_kernel<0>, dim3((unsigned)units), dim3(kThreads), 0, s,
                        static_cast<const AxpbyEntry *>(d_entries), static_cast<const int *>(d_owner), a, b);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;

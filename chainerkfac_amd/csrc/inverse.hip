@@ -861,7 +861,8 @@ struct kfac_inverse_plan {
   std::vector<hipEvent_t> ev_main, ev_side, ev_fork, ev_col;   // per step
   ~kfac_inverse_plan() {
     for (auto *v : {&ev_main, &ev_side, &ev_fork, &ev_col})
-      for (hipEvent_t e : *v) (void)hipEventDestroy(e);
+      for (hipEvent_t e : *v)
+        if (e) (void)hipEventDestroy(e);
     if (side) (void)hipStreamDestroy(side);
     if (col) (void)hipStreamDestroy(col);
   }
@@ -1194,12 +1195,13 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
   up(p->d_tasks, tasks.data(), sizeof(TileTask) * tasks.size());
   if (rc == KFAC_OK && p->lookahead && p->max_t > p->group) {
-    bool ok = hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess &&
-              hipStreamCreateWithFlags(&p->col, hipStreamNonBlocking) == hipSuccess;
+    const bool real = !kfac::host_only();   // host-only mode: null handles that nothing ever uses
+    bool ok = !real || (hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking) == hipSuccess &&
+                        hipStreamCreateWithFlags(&p->col, hipStreamNonBlocking) == hipSuccess);
     for (int g = 0; ok && g < p->max_t; ++g)
       for (auto *v : {&p->ev_main, &p->ev_side, &p->ev_fork, &p->ev_col}) {
         hipEvent_t e = nullptr;
-        ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
+        ok = ok && (!real || hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess);
         if (ok) v->push_back(e);
       }
     if (!ok) rc = kfac::fail(KFAC_EHIP, "cannot create the look-ahead stream or its events");
@@ -1246,7 +1248,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   // captured into a graph that is done only if the caller has declared `s` the
   // capture's origin; otherwise everything stays on `s`, in program order.
   bool lookahead = plan->lookahead;
-  if (lookahead && !plan->capture_origin) {
+  if (lookahead && !plan->capture_origin && !kfac::host_only()) {
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
       (void)hipGetLastError();   // e.g. the null stream beside a global-mode capture
@@ -1298,7 +1300,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.info = info_dev;
 
   kfac::TimedLaunch timed_call(KFAC_TIMED_INV_CALL, s);   // copy-in to the final product (the side streams rejoin `s`)
-  hipLaunchKernelGGL(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
+  KFAC_LAUNCH(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
   KFAC_HIP_CHECK(hipGetLastError());
   // Side stream: after the last column of a group, the rest of its trailing
   // update.  It is queued just after the next step's launch, so that the step's
@@ -1316,7 +1318,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     }
     {
       kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, st);
-      hipLaunchKernelGGL(update_kernel, dim3(r.count), dim3(THREADS), plan->rest_lds, st, tb,
+      KFAC_LAUNCH(update_kernel, dim3(r.count), dim3(THREADS), plan->rest_lds, st, tb,
                          r.task0);
     }
     if (lookahead) {
@@ -1345,11 +1347,11 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
       KFAC_HIP_CHECK(hipStreamWaitEvent(plan->col, plan->ev_fork[k], 0));
       cs = plan->col;
     }
-    hipLaunchKernelGGL(diag_kernel, dim3(na + plan->bdiag_count[k]), dim3(THREADS), kDiagKernelLds, s, tb,
+    KFAC_LAUNCH(diag_kernel, dim3(na + plan->bdiag_count[k]), dim3(THREADS), kDiagKernelLds, s, tb,
                        plan->diag_task0[k], na, plan->bdiag_task0[k]);
     if (w.count > 0) {
       kfac::TimedLaunch timed(KFAC_TIMED_INV_UPDATE, cs);
-      hipLaunchKernelGGL(update_kernel, dim3(w.count), dim3(THREADS), kTileLdsBytes, cs, tb, w.task0);
+      KFAC_LAUNCH(update_kernel, dim3(w.count), dim3(THREADS), kTileLdsBytes, cs, tb, w.task0);
     }
     if (cs != s) {
       KFAC_HIP_CHECK(hipEventRecord(plan->ev_col[k], cs));
@@ -1357,7 +1359,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
     }
     if (int rc2 = queue_rest()) return rc2;
     if (plan->panel_total[k] + plan->bpanel_count[k] > 0)
-      hipLaunchKernelGGL(panel_kernel, dim3(plan->panel_total[k] + plan->bpanel_count[k]), dim3(THREADS),
+      KFAC_LAUNCH(panel_kernel, dim3(plan->panel_total[k] + plan->bpanel_count[k]), dim3(THREADS),
                          kTileLdsBytes, s, tb, plan->panel_task0[k], plan->panel_total[k],
                          plan->bpanel_task0[k]);
     if (plan->rest[k].count == 0) continue;
@@ -1368,12 +1370,12 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   if (pending >= 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_side[pending], 0));
   KFAC_HIP_CHECK(hipGetLastError());
   if (plan->bfinal_count > 0) {
-    hipLaunchKernelGGL(border_kernel, dim3(plan->bfinal_count), dim3(THREADS), 0, s, tb, plan->bfinal_task0);
+    KFAC_LAUNCH(border_kernel, dim3(plan->bfinal_count), dim3(THREADS), 0, s, tb, plan->bfinal_task0);
     KFAC_HIP_CHECK(hipGetLastError());
   }
   {
     kfac::TimedLaunch timed(KFAC_TIMED_INV_LAUUM, s);
-    hipLaunchKernelGGL(lauum_kernel, dim3(plan->lauum_count), dim3(THREADS), kTileLdsBytes, s, tb,
+    KFAC_LAUNCH(lauum_kernel, dim3(plan->lauum_count), dim3(THREADS), kTileLdsBytes, s, tb,
                        plan->lauum_task0);
   }
   KFAC_HIP_CHECK(hipGetLastError());

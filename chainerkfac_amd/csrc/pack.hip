@@ -493,7 +493,7 @@ int run_pack(kfac_pack_plan_t plan, B *buf, int64_t buf_nelems, int target_rank,
   KFAC_REQUIRE(reinterpret_cast<uintptr_t>(buf) % (4 * sizeof(B)) == 0,
                "the buffer must be aligned to four of its elements (%zu bytes)", 4 * sizeof(B));
   kfac::TimedLaunch timed(KFAC_TIMED_PACK, kfac::as_stream(stream));
-  hipLaunchKernelGGL((pack_kernel<B, kPackU>), dim3(plan->pack_units), dim3(kThreads), 0,
+  KFAC_LAUNCH((pack_kernel<B, kPackU>), dim3(plan->pack_units), dim3(kThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -510,7 +510,7 @@ int run_unpack(kfac_pack_plan_t plan, const B *buf, int64_t buf_nelems, int targ
   if (plan->unpack_units == 0) return KFAC_OK;
   KFAC_REQUIRE(buf != nullptr, "buf is null");
   kfac::TimedLaunch timed(KFAC_TIMED_UNPACK, kfac::as_stream(stream));
-  hipLaunchKernelGGL((unpack_kernel<B, kUnpackThreads>), dim3(plan->unpack_blocks), dim3(kUnpackThreads), 0,
+  KFAC_LAUNCH((unpack_kernel<B, kUnpackThreads>), dim3(plan->unpack_blocks), dim3(kUnpackThreads), 0,
                      kfac::as_stream(stream), plan->tables(), buf, target_rank, divisor);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -552,11 +552,11 @@ extern "C" int kfac_stream_copy_f32(float *dst, const float *src, int64_t nelems
   {
     kfac::TimedLaunch timed(KFAC_TIMED_COPY, s);
     if (n4 > 0)
-      hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)kfac::ceil_div<long long>(n4, kThreads)),
+      KFAC_LAUNCH(stream_copy_kernel, dim3((unsigned)kfac::ceil_div<long long>(n4, kThreads)),
                          dim3(kThreads), 0, s, reinterpret_cast<const floatx4a *>(src),
                          reinterpret_cast<floatx4a *>(dst), n4);
     if (n4 * 4 < nelems)
-      hipLaunchKernelGGL(stream_copy_tail_kernel, dim3(1), dim3(kThreads), 0, s, src, dst, n4 * 4,
+      KFAC_LAUNCH(stream_copy_tail_kernel, dim3(1), dim3(kThreads), 0, s, src, dst, n4 * 4,
                          (long long)nelems);
   }
   KFAC_HIP_CHECK(hipGetLastError());

@@ -273,18 +273,18 @@ int launch_gemm(const LA64 &a64, const LB64 &b64, const LA128 &a128, const LB128
   {
     kfac::TimedLaunch timed(KFAC_TIMED_GEMM, stream);
     if (p.w == 2)
-      hipLaunchKernelGGL((gemm_kernel<2, LA128, LB128>), dim3(ntiles * p.nsplit), dim3(THREADS), 0,
+      KFAC_LAUNCH((gemm_kernel<2, LA128, LB128>), dim3(ntiles * p.nsplit), dim3(THREADS), 0,
                          stream, a128, b128, M, N, K, p.klen, p.tn, ntiles, part, C0, ld0, n_main,
                          C1);
     else
-      hipLaunchKernelGGL((gemm_kernel<1, LA64, LB64>), dim3(ntiles * p.nsplit), dim3(THREADS), 0,
+      KFAC_LAUNCH((gemm_kernel<1, LA64, LB64>), dim3(ntiles * p.nsplit), dim3(THREADS), 0,
                          stream, a64, b64, M, N, K, p.klen, p.tn, ntiles, part, C0, ld0, n_main, C1);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   if (part) {
     const long long total = (long long)M * N;
     kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, stream);
-    hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)kfac::ceil_div<long long>(total, 256)),
+    KFAC_LAUNCH(gemm_finish_kernel, dim3((unsigned)kfac::ceil_div<long long>(total, 256)),
                        dim3(256), 0, stream, part, p.nsplit, ntiles, p.tn, 64 * p.w, M, N, C0, ld0,
                        n_main, C1);
     KFAC_HIP_CHECK(hipGetLastError());
@@ -409,9 +409,9 @@ extern "C" int kfac_precond_bn_static_f32(const float *Finv, int d, const float 
   // y[0, d) is written in full by the product before the selection reads it, so
   // nothing of an earlier call's contents is ever seen and nothing needs clearing
   kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
-  hipLaunchKernelGGL(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
+  KFAC_LAUNCH(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
                      n_gamma, g_beta, y);
-  hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
+  KFAC_LAUNCH(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
                      kf_gamma, kf_beta, nan_flag_dev);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -435,9 +435,9 @@ extern "C" int kfac_precond_bn_f32(const float *Finv, int d, const float *g_gamm
   hipStream_t s = kfac::as_stream(stream);
   float *y = static_cast<float *>(ws);
   kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
-  hipLaunchKernelGGL(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
+  KFAC_LAUNCH(gemv_kernel, dim3(kfac::ceil_div(d, 4)), dim3(256), 0, s, Finv, d, g_gamma,
                      n_gamma, g_beta, y);
-  hipLaunchKernelGGL(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
+  KFAC_LAUNCH(bn_select_kernel, dim3(1), dim3(1024), 0, s, y, d, g_gamma, n_gamma, g_beta,
                      kf_gamma, kf_beta, nan_flag_dev);
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -501,10 +501,10 @@ extern "C" int kfac_precond_bn_batched_f32(kfac_precond_bn_batch_t batch, int co
     return rc;
   if (int rc = batch->unit_table.set(batch->units.data(), sizeof(int2) * batch->units.size(), s)) return rc;
   kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
-  hipLaunchKernelGGL(gemv_batched_kernel, dim3((unsigned)batch->units.size()), dim3(256), 0, s,
+  KFAC_LAUNCH(gemv_batched_kernel, dim3((unsigned)batch->units.size()), dim3(256), 0, s,
                      static_cast<const BnPreItem *>(d_items), batch->unit_table.as<const int2>(),
                      static_cast<float *>(ws));
-  hipLaunchKernelGGL(bn_select_batched_kernel, dim3(count), dim3(1024), 0, s,
+  KFAC_LAUNCH(bn_select_batched_kernel, dim3(count), dim3(1024), 0, s,
                      static_cast<const BnPreItem *>(d_items), static_cast<const float *>(ws));
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
@@ -841,17 +841,17 @@ extern "C" int kfac_precond_group_run_f32(kfac_precond_group_t group, const floa
       if (group->ntask[p][k] == 0) continue;
       if (!kerns[p][k]) return kfac::fail(KFAC_EINVAL, "internal: no kernel for kind %d", k);
       kfac::TimedLaunch timed(KFAC_TIMED_GEMM, s);
-      hipLaunchKernelGGL(kerns[p][k], dim3(group->ntask[p][k]), dim3(THREADS), 0, s, st, dy,
+      KFAC_LAUNCH(kerns[p][k], dim3(group->ntask[p][k]), dim3(THREADS), 0, s, st, dy,
                          tasks + group->task0[p][k], base);
     }
     KFAC_HIP_CHECK(hipGetLastError());
     if (group->nftask[p] > 0) {
       kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
       if (p == 0)
-        hipLaunchKernelGGL(gemm_group_finish_kernel<0>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
+        KFAC_LAUNCH(gemm_group_finish_kernel<0>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
                            tasks + group->ftask0[p], base);
       else
-        hipLaunchKernelGGL(gemm_group_finish_kernel<1>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
+        KFAC_LAUNCH(gemm_group_finish_kernel<1>, dim3(group->nftask[p]), dim3(256), 0, s, st, dy,
                            tasks + group->ftask0[p], base);
       KFAC_HIP_CHECK(hipGetLastError());
     }

@@ -49,7 +49,9 @@ const char *kfac_last_error_string(void);
  *   conv_shift, conv_shift_strict, group_bm64_max, group_macro, group_panels,
  *   group_macro_tasks, group_graded, inverse_group, inverse_border,
  *   inverse_lookahead, inverse_rest_lds, inverse_align, precond_tasks,
- *   bn_stats_loop.
+ *   bn_stats_loop, host_only (1: no call reaches the GPU -- plans are built and
+ *   every entry point checks its arguments and walks its launch sites, for runs
+ *   of the host code under a sanitizer on a machine without a GPU).
  * Not thread-safe against concurrent calls into the library. */
 int kfac_option_set(const char *name, double value);
 int kfac_option_unset(const char *name);
