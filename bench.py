@@ -1090,7 +1090,7 @@ def main():
     ap.add_argument('--no-other-configs', action='store_true',
                     help='c3 only: skip the short runs of c1, c2, c4 and c5 and the real-network step that the '
                          'default line carries beside its own figures')
-    ap.add_argument('--lanes', type=int, default=3,
+    ap.add_argument('--lanes', type=int, default=4,
                     help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
     ap.add_argument('--macro-tiles', action='store_true',
                     help='grouped covariance launches use the macro-tile kernel for slabs of several 128-tiles '

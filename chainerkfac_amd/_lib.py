@@ -47,6 +47,7 @@ PROTOTYPES = {
     'kfac_cov_group_create': (c_int, [c_int, c_vp, c_vpp]),
     'kfac_cov_group_workspace_bytes': (c_sz, [c_vp]),
     'kfac_cov_group_destroy': (c_int, [c_vp]),
+    'kfac_cov_group_set_capture_origin': (c_int, [c_vp, c_int]),
     'kfac_cov_group_run_f32': (c_int, [c_vp, c_vpp, c_vpp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     'kfac_bn_workspace_bytes': (c_sz, [c_int, c_int]),
     'kfac_bn_grad_matrix_f32': (c_int, [c_vp, c_vp, c_int, c_int, c_int, c_f, c_f, c_int, c_int,

@@ -244,6 +244,7 @@ enum Option : int {
   kOptGroupPanels,        // grouped launches: panel units per workgroup
   kOptGroupMacroTasks,    // macro-tile launches: workgroups per launch
   kOptGroupGraded,        // grouped covariances: 0 = equal slices, n >= 2: the last n-th is halved
+  kOptGroupSideStream,    // grouped covariances: 0 = every launch on the caller's stream
   kOptInverseGroup,       // inverse: block columns per trailing update
   kOptInverseBorder,      // inverse: 0 = matrices of 128 m + 1 rows are tiled whole
   kOptInverseLookahead,   // inverse: 0 = everything on the caller's stream

@@ -1613,8 +1613,21 @@ struct kfac_cov_group {
   size_t ws_floats = 0;
   int task0[kGroupKinds] = {}, ntask[kGroupKinds] = {};
   int ftask0 = 0, nftask = 0;
+  double kind_work[kGroupKinds] = {};   // matrix work of each launch (panels of a 64-tile)
   kfac::DevTable d_items, d_tasks;
   kfac::DevTableRing d_dyn;
+  // The launches of a group are independent of each other.  Each ends with the GPU
+  // draining (the last round of workgroups of a launch runs on a part of the CUs), so
+  // the longest launch stays on the caller's stream and the others run beside it on a
+  // stream of the group's own, filling each other's tails.
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  bool capture_origin = false;   // see kfac_cov_group_set_capture_origin
+  ~kfac_cov_group() {
+    if (ev_fork) (void)hipEventDestroy(ev_fork);
+    if (ev_join) (void)hipEventDestroy(ev_join);
+    if (side) (void)hipStreamDestroy(side);
+  }
 };
 
 extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac_cov_group_t *out) {
@@ -1792,6 +1805,7 @@ extern "C" int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac
     }
   }
   g->ws_floats = off;
+  for (int k = 0; k < kGroupKinds; ++k) g->kind_work[k] = work[k];
   std::vector<int2> tasks;
   for (int k = 0; k < kGroupKinds; ++k) {
     g->task0[k] = (int)tasks.size();
@@ -1818,6 +1832,12 @@ extern "C" size_t kfac_cov_group_workspace_bytes(kfac_cov_group_t group) {
 
 extern "C" int kfac_cov_group_destroy(kfac_cov_group_t group) {
   delete group;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_cov_group_set_capture_origin(kfac_cov_group_t group, int is_origin) {
+  KFAC_REQUIRE(group != nullptr, "group is null");
+  group->capture_origin = is_origin != 0;
   return KFAC_OK;
 }
 
@@ -1851,10 +1871,47 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
       syrk_group_kernel<1, LoaderKS<64, true>>,   syrk_group_kernel<1, LoaderKS<64, false>>,
       syrk_group_kernel<2, LoaderKC<128, true>>,  syrk_group_kernel<2, LoaderKC<128, false>>,
       syrk_group_kernel<2, LoaderKS<128, true>>,  syrk_group_kernel<2, LoaderKS<128, false>>};
-  for (int k = 0; k < kMacroKind0; ++k) {
+  // The launch with the most work stays on `s`, the others go to the group's side stream
+  // (not while launches are being timed one by one, not in host-only mode, and under stream
+  // capture only when the caller has declared `s` the capture's origin: a fork of a forked
+  // stream has crashed the runtime).
+  int nlaunch = 0, longest = -1;
+  for (int k = 0; k < kGroupKinds; ++k) {
     if (group->ntask[k] == 0) continue;
+    ++nlaunch;
+    if (longest < 0 || group->kind_work[k] > group->kind_work[longest]) longest = k;
+  }
+  bool fork = nlaunch >= 2 && kfac::option_int(kfac::kOptGroupSideStream, 1) != 0 && !kfac::timing_on() &&
+              !kfac::host_only();
+  if (fork && !group->capture_origin) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
+      (void)hipGetLastError();
+      fork = false;
+    } else if (cs != hipStreamCaptureStatusNone) {
+      fork = false;
+    }
+  }
+  if (fork && !group->side) {
+    KFAC_HIP_CHECK(hipStreamCreateWithFlags(&group->side, hipStreamNonBlocking));
+    KFAC_HIP_CHECK(hipEventCreateWithFlags(&group->ev_fork, hipEventDisableTiming));
+    KFAC_HIP_CHECK(hipEventCreateWithFlags(&group->ev_join, hipEventDisableTiming));
+  }
+  if (fork) {
+    KFAC_HIP_CHECK(hipEventRecord(group->ev_fork, s));
+    KFAC_HIP_CHECK(hipStreamWaitEvent(group->side, group->ev_fork, 0));
+  }
+  auto stream_of = [&](int k) { return fork && k != longest ? group->side : s; };
+  // (the longest first: its workgroups are placed before the others fill in)
+  if (longest >= 0 && longest < kMacroKind0) {
     kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
-    KFAC_LAUNCH(kerns[k], dim3(group->ntask[k]), dim3(THREADS), 0, s, st, dy,
+    KFAC_LAUNCH(kerns[longest], dim3(group->ntask[longest]), dim3(THREADS), 0, s, st, dy,
+                tasks + group->task0[longest], base);
+  }
+  for (int k = 0; k < kMacroKind0; ++k) {
+    if (group->ntask[k] == 0 || k == longest) continue;
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream_of(k));
+    KFAC_LAUNCH(kerns[k], dim3(group->ntask[k]), dim3(THREADS), 0, stream_of(k), st, dy,
                        tasks + group->task0[k], base);
   }
   static const Kern macro_kerns[2] = {syrk_macro_kernel<LoaderKC<128, true>>,
@@ -1873,11 +1930,15 @@ extern "C" int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const
   KFAC_HIP_CHECK(macro_attr_rc);
   for (int k = kMacroKind0; k < kGroupKinds; ++k) {
     if (group->ntask[k] == 0) continue;
-    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, s);
+    kfac::TimedLaunch timed(KFAC_TIMED_SYRK, stream_of(k));
     KFAC_LAUNCH(macro_kerns[k - kMacroKind0], dim3(group->ntask[k]), dim3(kMacroThreads),
-                       kMacroLdsBytes, s, st, dy, tasks + group->task0[k], base);
+                       kMacroLdsBytes, stream_of(k), st, dy, tasks + group->task0[k], base);
   }
   KFAC_HIP_CHECK(hipGetLastError());
+  if (fork) {
+    KFAC_HIP_CHECK(hipEventRecord(group->ev_join, group->side));
+    KFAC_HIP_CHECK(hipStreamWaitEvent(s, group->ev_join, 0));
+  }
   if (group->nftask > 0) {
     kfac::TimedLaunch timed(KFAC_TIMED_COV_AUX, s);
     KFAC_LAUNCH(finish_group_kernel, dim3(group->nftask), dim3(256), 0, s, st, dy,

@@ -88,7 +88,7 @@ namespace {
 const char *const kOptionNames[kOptCount] = {
     "syrk_bm64_max",   "syrk_splits",      "conv_rows",       "rows_wm",          "shift_slices5",
     "shift_slices3",   "conv_shift",       "conv_shift_strict", "group_bm64_max", "group_macro",
-    "group_panels",    "group_macro_tasks", "group_graded",   "inverse_group",    "inverse_border",
+    "group_panels",    "group_macro_tasks", "group_graded",   "group_side_stream", "inverse_group",  "inverse_border",
     "inverse_lookahead", "inverse_rest_lds", "inverse_align", "precond_tasks",    "bn_stats_loop",
     "host_only"};
 struct OptionState {

@@ -129,6 +129,9 @@ class CovGroup(object):
             if x.numel() != want or tuple(out.shape) != (d, d):
                 raise ValueError('item {} does not match its tensors'.format(it))
         ws = _dev.workspace('cov_group', self.workspace_bytes, inputs[0].device)
+        # (under HIP-graph capture the group may fork only from the stream the capture began on)
+        origin = stream is None and _dev.current_lane() is None
+        _lib.check(_lib.load().kfac_cov_group_set_capture_origin(self._plan, int(origin)))
         _lib.check(_lib.load().kfac_cov_group_run_f32(
             self._plan, _lib.ptr_array([x.data_ptr() for x in inputs]),
             _lib.ptr_array([o.data_ptr() for o in outputs]),

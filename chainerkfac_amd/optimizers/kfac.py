@@ -241,7 +241,7 @@ class KFAC(object):
     #: are dealt onto (layers are independent of each other and most of their
     #: kernels are too small to fill the GPU alone); 0 keeps everything on the
     #: caller's stream.  Read at ``setup``.
-    lanes = 3
+    lanes = 4
 
     #: apply the momentum rule of all parameters with one launch per set of
     #: hyperparameters (normally one) instead of one launch per parameter

@@ -47,7 +47,7 @@ const char *kfac_last_error_string(void);
  * i < kfac_option_count()):
  *   syrk_bm64_max, syrk_splits, conv_rows, rows_wm, shift_slices5, shift_slices3,
  *   conv_shift, conv_shift_strict, group_bm64_max, group_macro, group_panels,
- *   group_macro_tasks, group_graded, inverse_group, inverse_border,
+ *   group_macro_tasks, group_graded, group_side_stream, inverse_group, inverse_border,
  *   inverse_lookahead, inverse_rest_lds, inverse_align, precond_tasks,
  *   bn_stats_loop, host_only (1: no call reaches the GPU -- plans are built and
  *   every entry point checks its arguments and walks its launch sites, for runs
@@ -194,6 +194,13 @@ typedef struct kfac_cov_group *kfac_cov_group_t;
 int kfac_cov_group_create(int count, const kfac_cov_item *items, kfac_cov_group_t *group_out);
 size_t kfac_cov_group_workspace_bytes(kfac_cov_group_t group);
 int kfac_cov_group_destroy(kfac_cov_group_t group);
+/* A group runs its longest launch on the caller's stream and the others beside it on
+ * a stream of its own, joined again before the call returns.  On a stream that is being
+ * captured into a HIP graph it does so only after kfac_cov_group_set_capture_origin(group,
+ * 1): the caller's statement that the stream is the one the capture began on (a stream
+ * forked from a forked stream has crashed the runtime); otherwise every launch stays on
+ * the given stream. */
+int kfac_cov_group_set_capture_origin(kfac_cov_group_t group, int is_origin);
 int kfac_cov_group_run_f32(kfac_cov_group_t group, const float *const *inputs,
                            float *const *outputs, const float *alpha, const float *beta,
                            void *ws, size_t ws_bytes, void *stream);
