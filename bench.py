@@ -209,11 +209,11 @@ def family_roofline(label, kernels, flop, members, fam, empty, note, reference_f
 
 
 def read_traffic():
+    """The record `bench.py --summarize-traffic` wrote from two counter runs, or None."""
     try:
         with open(TRAFFIC_FILE) as f:
-            t = json.load(f)
-        return float(t['bytes_per_launch'])
-    except (OSError, ValueError, KeyError):
+            return json.load(f)
+    except (OSError, ValueError):
         return None
 
 
@@ -237,23 +237,32 @@ def wire_format(arrays, dev, lib):
     stream = torch.cuda.current_stream().cuda_stream
     copy_ms = timed(lambda: _lib.check(lib.kfac_stream_copy_f32(dst.data_ptr(), src.data_ptr(), n_copy, stream)),
                     reps=11)
-    del src, dst
+    # and a copy with the unpack's mix: n elements read, 2 n written, the same number of bytes
+    n_fan = (nel + full) // 3 // 4 * 4
+    dst2 = torch.empty(n_fan, dtype=torch.float32, device=dev)
+    fan_ms = timed(lambda: _lib.check(lib.kfac_stream_fanout_f32(dst.data_ptr(), dst2.data_ptr(), src.data_ptr(), n_fan,
+                                                                 stream)), reps=11)
+    del src, dst, dst2
     copy_gbps = 8.0 * n_copy / copy_ms / 1e6
+    fan_gbps = 12.0 * n_fan / fan_ms / 1e6
     out = {
         'arrays': len(arrays[0]), 'triangular': sum(1 for _, t in arrays[0] if t),
         'pack': {'ms': round(pack_ms, 4), 'GBps': round(8.0 * nel / pack_ms / 1e6, 1)},
         'unpack': {'ms': round(unpack_ms, 4), 'GBps': round(4.0 * (nel + full) / unpack_ms / 1e6, 1)},
         'stream_copy': {'ms': round(copy_ms, 4), 'GBps': round(copy_gbps, 1), 'bytes': 8 * n_copy},
+        # one read, two writes per element: the traffic mix of the unpack
+        'stream_fanout': {'ms': round(fan_ms, 4), 'GBps': round(fan_gbps, 1), 'bytes': 12 * n_fan},
         'packed_MB': round(4.0 * nel / 1e6, 1), 'full_MB': round(4.0 * full / 1e6, 1),
     }
-    for k in ('pack', 'unpack', 'stream_copy'):
+    for k in ('pack', 'unpack', 'stream_copy', 'stream_fanout'):
         out[k]['frac_of_hbm_peak'] = round(out[k]['GBps'] / HBM_PEAK_GBPS, 3)
     for k in ('pack', 'unpack'):
         out[k]['frac_of_stream_copy'] = round(out[k]['GBps'] / copy_gbps, 3)
+    out['unpack']['frac_of_stream_fanout'] = round(out['unpack']['GBps'] / fan_gbps, 3)
     return out, wire
 
 
-def run_step_config(args, name, cfg):
+def run_step_config(args, name, cfg, host=None):
     """c1, c2, c3, c5: cov (x acc_iters) [+ pack/unpack] + inverse + precondition."""
     import torch
     from chainerkfac_amd import _lib
@@ -329,9 +338,39 @@ def run_step_config(args, name, cfg):
         inv_phase()
         pre_phase()
 
+    if args.host_launch_child:
+        # no lane exists before the brackets have been read (the pool of streams is made on first use)
+        opt._lanes.n = 0
+        _lib.set_option('group_side_stream', 0)
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
+
+    def host_launched():
+        """Every kernel family timed bracket by bracket inside the library, on one stream (with
+        lanes, launches overlap and the time between a launch's events is shared with others);
+        then the step launched kernel by kernel from the host with the lanes back on: what a
+        caller of the drop-in classes gets without capturing a graph of its own."""
+        opt._lanes.n = 0
+        _lib.set_option('group_side_stream', 0)
+        step()
+        torch.cuda.synchronize()
+        _lib.check(lib.kfac_timing_enable(1))
+        step()
+        torch.cuda.synchronize()
+        fam = family_times(lib)
+        _lib.check(lib.kfac_timing_enable(0))
+        empty = bracket_ms()
+        opt._lanes.n = args.lanes
+        _lib.set_option('group_side_stream', None if args.lanes else 0)
+        for _ in range(3):
+            step()
+        eager, _ = timed_steps(step, max(args.steps, 5))
+        return {'eager_ms_per_step': eager, 'lanes': args.lanes, 'fam': fam, 'empty': empty,
+                'info_bad': len(opt.check_numerics())}
+
+    if args.host_launch_child:
+        return host_launched()
     run = step if args.no_graph else capture(step)
     ms_per_step, ms_median = timed_steps(run, args.steps)
 
@@ -401,29 +440,20 @@ def run_step_config(args, name, cfg):
                                'frac_of_hbm_peak': round(12.0 * n_factor_elems / (ema_ms['batched'] * 1e-3) / 1e12 / 8.0, 3),
                                'in_value': False}}
 
-    # the same step launched kernel by kernel from the host (what a caller of the drop-in classes
-    # gets without capturing a graph of its own)
-    eager_ms = None
-    if not args.no_graph and not args.no_extras:
-        step()
-        eager_ms, _ = timed_steps(step, max(args.steps // 2, 5))
-
-    # every kernel family, timed bracket by bracket inside the library (one stream: with lanes,
-    # launches overlap and the time between a launch's events is shared with others)
-    opt._lanes.n = 0
-    _lib.check(lib.kfac_timing_enable(1))
-    step()
-    torch.cuda.synchronize()
-    opt._lanes.n = args.lanes
-    fam = family_times(lib)
-    _lib.check(lib.kfac_timing_enable(0))
-    info_bad = len(opt.check_numerics())
+    # Launches made from the host: the per-family event brackets and the eager step time, measured
+    # here when the caller has not already measured them in a process of their own (see main).
+    if host is None:
+        host = host_launched()
+    real_network = host.pop('real_network', None)
+    eager_ms, eager_lanes = host['eager_ms_per_step'], host['lanes']
+    fam = {k: tuple(v) for k, v in host['fam'].items()}
+    empty = host['empty']
+    info_bad = host['info_bad']
     lowrank = [fb for fb in opt.fblocks if getattr(fb, 'lowrank_inverse_args', lambda: None)() is not None] \
         if opt.bn_lowrank_inverse else []
     # d^3 of the factors that went through the dense Cholesky path (the reference inverts all of them densely)
     dense_inverse_flops = flops['inverse'] - sum(float(fb.cov_emas[0].shape[0]) ** 3 for fb in lowrank)
 
-    empty = bracket_ms()
     # what the matrix cores are actually given: 3x3 stride-1 convolutions compute their A factor from
     # shifted correlations, about a third of the multiply-adds of the patch product
     cov_executed = float(W.cov_flops_executed(layers, batch)) * acc_iters
@@ -450,13 +480,26 @@ def run_step_config(args, name, cfg):
     families['cov_syrk']['main_kernels_only'] = {
         'launches': main_syrk['brackets'], 'kernel_ms_per_step': main_syrk['kernel_ms_per_step'],
         'achieved': main_syrk['achieved'], 'frac': main_syrk['frac']}
-    traffic = read_traffic() if name == 'c3' else None
-    families['cov_syrk']['traffic_main_kernels'] = traffic
-    families['cov_syrk']['traffic_unit'] = 'bytes/launch of the main kernels'
+    # HBM bytes per step of every family, from hardware counters of an earlier profiling run of this
+    # configuration (profiles/), beside the bytes the algorithm has to move
+    record = read_traffic() if name == 'c3' else None
+    factor_bytes = 4.0 * sum(float(c.numel()) for fb in opt.fblocks for c in fb.covs)
+    input_bytes = 4.0 * sum(float(in_data[0].numel()) + float(gy[0].numel()) for _, in_data, gy in work)
+    dense_bytes = 4.0 * sum(float(c.numel()) for fb in opt.fblocks if fb not in lowrank for c in fb.cov_emas)
+    grad_bytes = 4.0 * sum(float(p.data.numel()) for p in model.params())
+    algorithmic = {'cov_syrk': (input_bytes + factor_bytes) * acc_iters,   # inputs read, factors written
+                   'inverse_tiles': 2.0 * dense_bytes,                         # factors read, inverses written
+                   'precond_gemm': factor_bytes + 2.0 * grad_bytes}            # inverses and gradients read, kfgrads written
+    for fam_name, fam_entry in families.items():
+        measured = None if record is None else record.get('families', {}).get(fam_name, {}).get('bytes_per_step')
+        fam_entry['traffic'] = None if measured is None else round(measured / max(fam_entry['brackets'], 1), 1)
+        fam_entry['traffic_unit'] = 'HBM bytes per bracket (the family\'s bytes per step over its brackets per step)'
+        fam_entry['traffic_bytes_per_step'] = measured
+        fam_entry['algorithmic_bytes_per_step'] = algorithmic[fam_name]
+    families['cov_syrk']['traffic_main_kernels_per_launch'] = None if record is None else record.get('bytes_per_launch')
     dominant = max(families, key=lambda k: families[k]['kernel_ms_per_step'])
     roofline = dict(families[dominant])
     roofline['family'] = dominant
-    roofline['traffic'] = traffic if dominant == 'cov_syrk' else None
     roofline['event_bracket_ms'] = round(empty, 4)
     roofline['families'] = families
     result = {
@@ -501,8 +544,10 @@ def run_step_config(args, name, cfg):
         'wire_format': wire_stats,
         'roofline': roofline,
     }
-    if eager_ms is not None:
-        result['eager_ms_per_step'] = round(eager_ms, 4)
+    result['eager_ms_per_step'] = round(eager_ms, 4)
+    result['eager_lanes'] = eager_lanes
+    if real_network is not None:
+        result['real_network'] = real_network
     result.update(extras)
     if name == 'c3' and lowrank and not args.no_dense_field:
         # the reference's algorithm inverts the batch-norm blocks densely as well: the same step with
@@ -539,6 +584,27 @@ def run_step_config(args, name, cfg):
     return result
 
 
+def host_launch_child(args, name, real_network=False):
+    """Runs this script again, in a process of its own, for the measurements of launches made
+    from the host (see run_step_config) and returns what it printed."""
+    import subprocess
+    from chainerkfac_amd.optimizers import KFAC
+    cmd = [sys.executable, os.path.abspath(__file__), '--config', name, '--host-launch-child', '--no-graph',
+           '--no-cpu', '--lanes', str(min(args.lanes, KFAC.lanes)), '--steps', str(max(min(args.steps, 20), 5)),
+           '--warmup', str(max(args.warmup, 1))]
+    if args.dense_bn_inverse:
+        cmd.append('--dense-bn-inverse')
+    if args.macro_tiles:
+        cmd.append('--macro-tiles')
+    if real_network:
+        cmd.append('--real-network')
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+    lines = [l for l in proc.stdout.decode().splitlines() if l.startswith('{')]
+    if proc.returncode != 0 or not lines:
+        raise RuntimeError('the host-launch measurement failed:\n' + proc.stderr.decode()[-3000:])
+    return json.loads(lines[-1])
+
+
 def inverse_dims():
     """The 161 factor sizes of ResNet-50 with the 3x3 no-bias stem of the reference's own model
     file (27 instead of 148): the stated range 27^2 .. 4609^2."""
@@ -571,6 +637,7 @@ def run_inverse_config(args, name, cfg):
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
+
     run = step if args.no_graph else capture(step)
     ms_per_step, ms_median = timed_steps(run, args.steps)
     _lib.check(lib.kfac_timing_enable(1))
@@ -610,7 +677,7 @@ def run_inverse_config(args, name, cfg):
     }, dims
 
 
-def run_real_network(steps=5, warmup=2):
+def run_real_network(steps=10, warmup=5, lanes=None):
     """``KFAC.update(lossfun)`` on the ResNet-50 built from the link classes (batch 32 @ 224): a
     real forward and backward pass under the function hooks, then moving average, damped inverse,
     preconditioning and the momentum rule, launched from the host with no HIP graph.  Gradient and
@@ -642,14 +709,17 @@ def run_real_network(steps=5, warmup=2):
 
     for _ in range(warmup):
         plain()
-    plain_ms = wall(plain, steps)
-    opt = KFAC(lr=1e-3, damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0).setup(model)
+    plain_ms = min(wall(plain, steps) for _ in range(3))
+    opt = KFAC(lr=1e-3, damping=DAMPING, stab_coeff=STAB_COEFF, cov_ema_decay=1.0)
+    if lanes is not None:
+        opt.lanes = lanes
+    opt = opt.setup(model)
     for _ in range(warmup):
         opt.update(lossfun)
-    update_ms = wall(lambda: opt.update(lossfun), steps)
+    update_ms = min(wall(lambda: opt.update(lossfun), steps) for _ in range(3))
     return {'workload': 'KFAC.update(lossfun) on the link-built ResNet-50 v1 (bias), batch 32 @224, 161 factors, '
                         'eager (no HIP graph), torch autograd for the forward / backward pass',
-            'steps': steps, 'ms_per_update': round(update_ms, 3),
+            'steps': steps, 'timed': 'best of 3 runs of {} updates'.format(steps), 'lanes': opt.lanes, 'ms_per_update': round(update_ms, 3),
             'forward_backward_only_ms': round(plain_ms, 3),
             'kfac_part_ms': round(update_ms - plain_ms, 3), 'in_value': False}
 
@@ -666,7 +736,8 @@ def compact(result):
     if result['config'].get('name') == 'c5':
         w = result['wire_format']
         out['wire_format'] = {'arrays': w['arrays'], 'triangular': w['triangular'],
-                              'pack': w['pack'], 'unpack': w['unpack'], 'stream_copy': w['stream_copy']}
+                              'pack': w['pack'], 'unpack': w['unpack'], 'stream_copy': w['stream_copy'],
+                              'stream_fanout': w['stream_fanout']}
     if 'max_residual' in result:
         out['max_residual'] = result['max_residual']
     return out
@@ -1004,12 +1075,23 @@ def summarize_mfma(pmc_dir, out_path, command):
     print('\n'.join(lines[12:40]))
 
 
+TRAFFIC_FAMILIES = (
+    # family, kernels of the family, the kernel whose launches count the steps of the run
+    ('cov_syrk', ('syrk_', 'shift::corr_kernel', 'finish_group_kernel', 'finish_kernel', 'reduce_kernel',
+                  'shift::assemble', 'shift::edge_sums', 'shift::corr_finish'), 'finish_group_kernel'),
+    ('inverse_tiles', ('copy_in_kernel', 'diag_kernel', 'update_kernel', 'panel_kernel', 'border_kernel',
+                       'lauum_kernel'), 'lauum_kernel'),
+    ('precond_gemm', ('gemm_group', 'gemv_', 'bn_select'), 'gemm_group_finish_kernel<1>'),
+)
+
+
 def summarize_traffic(fetch_dir, write_dir, out_path, command):
     """Reads the per-dispatch FETCH_SIZE / WRITE_SIZE counters (KiB) of two
     `rocprofv3 --pmc` runs of this script with --calibrate-copy, scales each by what it
-    reads for the 256 MiB calibration copy (stream_copy_kernel), and writes the average
-    HBM bytes per launch of the covariance SYRK family to ``out_path`` (JSON, read back as
-    roofline.traffic) and a per-kernel table next to it (markdown)."""
+    reads for the 256 MiB calibration copy (stream_copy_kernel), and writes the HBM bytes
+    of every kernel family per step, and per launch of the covariance SYRK main kernels,
+    to ``out_path`` (JSON, read back as roofline.traffic) and a per-kernel table next to
+    it (markdown)."""
     def load(d, counter):
         rows = {}
         for r in _csv_rows(d, 'counter_collection.csv'):
@@ -1018,7 +1100,7 @@ def summarize_traffic(fetch_dir, write_dir, out_path, command):
                 rows[key] = rows.get(key, 0.0) + float(r['Counter_Value'])
         return [(k[1], v) for k, v in sorted(rows.items(), key=lambda kv: int(kv[0][0]))]
 
-    out = {}
+    out = {'families': {}}
     total = 0.0
     per_kernel = {}
     for d, counter, key in ((fetch_dir, 'FETCH_SIZE', 'fetch'), (write_dir, 'WRITE_SIZE', 'write')):
@@ -1034,12 +1116,19 @@ def summarize_traffic(fetch_dir, write_dir, out_path, command):
         out[key + '_bytes_per_launch'] = sum(syrk) / len(syrk) * 1024.0 * scale
         out['launches'] = len(syrk)
         total += out[key + '_bytes_per_launch']
+        for fam, keys, marker in TRAFFIC_FAMILIES:
+            steps = sum(1 for k, _ in rows if marker in k)
+            kib = sum(v for k, v in rows if any(x in k for x in keys))
+            f = out['families'].setdefault(fam, {'steps_in_run': steps})
+            f[key + '_bytes_per_step'] = kib * 1024.0 * scale / max(steps, 1)
         for k, v in rows:
             if _own_kernel(k):
                 a = per_kernel.setdefault(k, {'fetch': [0, 0.0], 'write': [0, 0.0]})[key]
                 a[0] += 1
                 a[1] += v * scale
     out['bytes_per_launch'] = total
+    for f in out['families'].values():
+        f['bytes_per_step'] = f.get('fetch_bytes_per_step', 0.0) + f.get('write_bytes_per_step', 0.0)
     with open(out_path, 'w') as f:
         json.dump(out, f, indent=1)
         f.write('\n')
@@ -1052,11 +1141,19 @@ def summarize_traffic(fetch_dir, write_dir, out_path, command):
              'counters are scaled by {:.3f} and {:.3f} to get KiB.'.format(
                  out['fetch_counter_for_256MiB_copy'], out['write_counter_for_256MiB_copy'],
                  out['fetch_scale'], out['write_scale']), '',
-             'Covariance SYRK family (`syrk_*` and `shift::corr_kernel`, {} launches in the run): **fetch {:.1f} MiB + write {:.1f} MiB = '
-             '{:.1f} MiB per launch** ({:.4g} bytes, the `roofline.traffic` of bench.py).'.format(
+             'Covariance SYRK main kernels (`syrk_*` and `shift::corr_kernel`, {} launches in the run): **fetch {:.1f} MiB + write {:.1f} MiB = '
+             '{:.1f} MiB per launch** ({:.4g} bytes).'.format(
                  out['launches'], out['fetch_bytes_per_launch'] / 2 ** 20, out['write_bytes_per_launch'] / 2 ** 20,
                  total / 2 ** 20, total), '',
-             '| kernel | launches | fetch MiB/launch | write MiB/launch |', '|---|---:|---:|---:|']
+             'Kernel families, all their kernels, per step (the `roofline.traffic` figures of bench.py):', '',
+             '| family | steps in the run | fetch MiB / step | write MiB / step | total MiB / step |', '|---|---:|---:|---:|---:|']
+    for fam, _, _ in TRAFFIC_FAMILIES:
+        f = out['families'][fam]
+        lines.append('| {} | {} | {:.1f} | {:.1f} | {:.1f} |'.format(
+            fam, f['steps_in_run'], f.get('fetch_bytes_per_step', 0) / 2 ** 20, f.get('write_bytes_per_step', 0) / 2 ** 20,
+            f['bytes_per_step'] / 2 ** 20))
+    lines += ['', '| kernel | launches | fetch MiB/launch | write MiB/launch |', '|---|---:|---:|---:|']
+
     def tot(v):
         return v['fetch'][1] + v['write'][1]
     for k, v in sorted(per_kernel.items(), key=lambda kv: -tot(kv[1]))[:24]:
@@ -1087,11 +1184,14 @@ def main():
     ap.add_argument('--no-extras', action='store_true',
                     help='skip the measurements beside the step (momentum rule of all parameters, moving average '
                          'of all factors): profiling runs')
+    ap.add_argument('--host-launch-child', action='store_true', help=argparse.SUPPRESS)
+    ap.add_argument('--real-network', action='store_true', help=argparse.SUPPRESS)
     ap.add_argument('--no-other-configs', action='store_true',
                     help='c3 only: skip the short runs of c1, c2, c4 and c5 and the real-network step that the '
                          'default line carries beside its own figures')
     ap.add_argument('--lanes', type=int, default=4,
-                    help='side streams for the per-layer factor and preconditioning kernels (0 = one stream)')
+                    help='side streams for the per-layer factor and preconditioning kernels (0 = one stream, also for '
+                         'the grouped launches)')
     ap.add_argument('--macro-tiles', action='store_true',
                     help='grouped covariance launches use the macro-tile kernel for slabs of several 128-tiles '
                          '(library option group_macro = 1: less HBM traffic, about 1 %% slower)')
@@ -1124,17 +1224,39 @@ def main():
     if args.summarize_mfma:
         summarize_mfma(args.summarize_mfma[0], args.summarize_mfma[1], args.profiled_command)
         return
+    # Launches made from the host (eager step time, per-family event brackets, the step on a real
+    # network) are measured in processes of their own, with the drop-in's default number of lanes,
+    # when this one replays graphs: a process that has captured the step with four lanes holds more
+    # streams than the GPU gives one process hardware queues, and independent launches from the host
+    # then wait behind each other (the batched inverse took a fifth longer that way).  They run
+    # first, before this process has touched the GPU.
+    with_others = args.config == 'c3' and not args.no_other_configs
+    host = {}
+    if not args.no_graph and not args.host_launch_child:
+        for name in [args.config] + (['c1', 'c2', 'c5'] if with_others else []):
+            if name != 'c4':
+                host[name] = host_launch_child(args, name)
+        if with_others:
+            host[args.config]['real_network'] = host_launch_child(args, args.config, real_network=True)
     if args.macro_tiles:
         from chainerkfac_amd import _lib
         _lib.set_option('group_macro', 1)
+    if args.lanes == 0:
+        # one stream everywhere: the grouped launches keep to the caller's stream as well (profiling
+        # runs, where kernels that run side by side would share their durations)
+        from chainerkfac_amd import _lib
+        _lib.set_option('group_side_stream', 0)
     cfg = configs()[args.config]
+    if args.host_launch_child:
+        print(json.dumps(run_real_network(lanes=args.lanes) if args.real_network else run_step_config(args, args.config, cfg)))
+        return
     if args.config == 'c4':
         result, _ = run_inverse_config(args, args.config, cfg)
     else:
-        result = run_step_config(args, args.config, cfg)
+        result = run_step_config(args, args.config, cfg, host.get(args.config))
         if args.per_layer:
             write_per_layer(args.per_layer, cfg['layers'], args.config)
-    if args.config == 'c3' and not args.no_other_configs:
+    if with_others:
         # the other configurations of the benchmark definition, shorter runs of the same code paths
         # (their full lines: --config c1 | c2 | c4 | c5), and the drop-in step on a real network
         import copy
@@ -1152,12 +1274,9 @@ def main():
             if name == 'c4':
                 line, _ = run_inverse_config(sub, name, sub_cfg)
             else:
-                line = run_step_config(sub, name, sub_cfg)
+                line = run_step_config(sub, name, sub_cfg, host.get(name))
             others[name] = compact(line)
         result['other_configs'] = others
-        gc.collect()
-        torch.cuda.empty_cache()
-        result['real_network'] = run_real_network()
     if not args.no_cpu:
         result['cpu_baseline'] = run_cpu_baseline(args.config, cfg)
     print(json.dumps(result))

@@ -80,6 +80,7 @@ PROTOTYPES = {
     'kfac_precond_group_create': (c_int, [c_int, c_i32p, c_i32p, c_i32p, c_vpp]),
     'kfac_precond_group_workspace_bytes': (c_sz, [c_vp]),
     'kfac_precond_group_destroy': (c_int, [c_vp]),
+    'kfac_precond_group_set_capture_origin': (c_int, [c_vp, c_int]),
     'kfac_precond_group_run_f32': (c_int, [c_vp, c_vpp, c_vpp, c_vpp, c_vpp, c_vpp, c_vpp, c_vp, c_sz, c_vp]),
     'kfac_precond_bn_workspace_bytes': (c_sz, [c_int]),
     'kfac_precond_bn_f32': (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
@@ -95,6 +96,7 @@ PROTOTYPES = {
     'kfac_momentum_update_batched_f32': (c_int, [c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_f, c_f, c_f,
                                                  c_vp]),
     'kfac_stream_copy_f32': (c_int, [c_vp, c_vp, c_i64, c_vp]),
+    'kfac_stream_fanout_f32': (c_int, [c_vp, c_vp, c_vp, c_i64, c_vp]),
     'kfac_timing_enable': (c_int, [c_int]),
     'kfac_timing_read': (c_int, [c_int, c_i64p, c_dp]),
 }

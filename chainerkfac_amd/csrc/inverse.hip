@@ -360,10 +360,11 @@ __device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K,
 // ---------------------------------------------------------------------------
 // copy-in: lower tiles of in -> padded workspace (identity on the padding)
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count) {
-  const int s = find_slot(tb.tile_cs, count, blockIdx.x);
+__global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count, int tile0) {
+  const int t = (int)blockIdx.x + tile0;
+  const int s = find_slot(tb.tile_cs, count, t);
   int I, J;
-  tri_decode(blockIdx.x - tb.tile_cs[s], I, J);
+  tri_decode(t - tb.tile_cs[s], I, J);
   const int d = tb.dim[s], dc = tb.core[s];
   const float *__restrict__ src = tb.in[s];
   float *__restrict__ dst = tile_ptr(tb, s, I, J);
@@ -859,7 +860,13 @@ struct kfac_inverse_plan {
   // on a third stream beside the diagonal kernel.
   hipStream_t col = nullptr;
   std::vector<hipEvent_t> ev_main, ev_side, ev_fork, ev_col;   // per step
+  // The matrices that join the sweep at its first step are copied in on the caller's
+  // stream; the others (they join later) on the side stream, beside the first step.
+  int first_tiles = 0;
+  hipEvent_t ev_copy_fork = nullptr, ev_copy = nullptr;
   ~kfac_inverse_plan() {
+    for (hipEvent_t e : {ev_copy_fork, ev_copy})
+      if (e) (void)hipEventDestroy(e);
     for (auto *v : {&ev_main, &ev_side, &ev_fork, &ev_col})
       for (hipEvent_t e : *v)
         if (e) (void)hipEventDestroy(e);
@@ -952,6 +959,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   p->nborder = (int)border_slots.size();
   p->ws_floats = total;
   p->total_tiles = tile_cs[count];
+  p->first_tiles = tile_cs[count];   // set once the steps are known
   p->max_t = count ? p->nt[0] : 0;
   std::vector<TileTask> tasks;
   std::vector<int2> natural;
@@ -1064,6 +1072,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
     int na = 0;
     while (na < count && shift[na] <= g && g < shift[na] + p->nt[na]) ++na;
     p->nactive.push_back(na);
+    if (g == 0) p->first_tiles = tile_cs[na];
     p->panel_total.push_back(panel_cs[na]);
     const int g0 = g / p->group * p->group;
     const int g1 = std::min(g0 + p->group - 1, p->max_t - 1);
@@ -1204,6 +1213,8 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
         ok = ok && (!real || hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess);
         if (ok) v->push_back(e);
       }
+    for (hipEvent_t *e : {&p->ev_copy_fork, &p->ev_copy})
+      ok = ok && (!real || hipEventCreateWithFlags(e, hipEventDisableTiming) == hipSuccess);
     if (!ok) rc = kfac::fail(KFAC_EHIP, "cannot create the look-ahead stream or its events");
   } else {
     p->lookahead = false;
@@ -1300,7 +1311,16 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.info = info_dev;
 
   kfac::TimedLaunch timed_call(KFAC_TIMED_INV_CALL, s);   // copy-in to the final product (the side streams rejoin `s`)
-  KFAC_LAUNCH(copy_in_kernel, dim3(plan->total_tiles), dim3(256), 0, s, tb, count);
+  // copy-in: what the first step needs on `s`, the rest beside it on the side stream
+  const int late_tiles = lookahead ? plan->total_tiles - plan->first_tiles : 0;
+  if (late_tiles > 0) {
+    KFAC_HIP_CHECK(hipEventRecord(plan->ev_copy_fork, s));
+    KFAC_HIP_CHECK(hipStreamWaitEvent(plan->side, plan->ev_copy_fork, 0));
+    KFAC_LAUNCH(copy_in_kernel, dim3(late_tiles), dim3(256), 0, plan->side, tb, count, plan->first_tiles);
+    KFAC_HIP_CHECK(hipEventRecord(plan->ev_copy, plan->side));
+  }
+  if (plan->total_tiles - late_tiles > 0)
+    KFAC_LAUNCH(copy_in_kernel, dim3(plan->total_tiles - late_tiles), dim3(256), 0, s, tb, count, 0);
   KFAC_HIP_CHECK(hipGetLastError());
   // Side stream: after the last column of a group, the rest of its trailing
   // update.  It is queued just after the next step's launch, so that the step's
@@ -1331,6 +1351,8 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   for (int k = 0; k < plan->max_t; ++k) {
     const int na = plan->nactive[k];
     const UpdateLaunch &w = plan->with_diag[k];
+    // the matrices that join from the second step on have been copied in by then
+    if (k == 1 && late_tiles > 0) KFAC_HIP_CHECK(hipStreamWaitEvent(s, plan->ev_copy, 0));
     // A group's first step applies the previous group to this group's columns,
     // tiles that the rest of the group before that one (two back) also updated.
     // The rest of the previous group itself only touches columns further right

@@ -532,6 +532,18 @@ __global__ __launch_bounds__(kThreads) void stream_copy_kernel(const floatx4a *_
   if (t < n4) __builtin_nontemporal_store(__builtin_nontemporal_load(src + t), dst + t);
 }
 
+// The same with unpack's mix of traffic: every element read once and written twice.
+__global__ __launch_bounds__(kThreads) void stream_fanout_kernel(const floatx4a *__restrict__ src,
+                                                                 floatx4a *__restrict__ dst0,
+                                                                 floatx4a *__restrict__ dst1, long long n4) {
+  const long long t = (long long)blockIdx.x * kThreads + threadIdx.x;
+  if (t < n4) {
+    const floatx4a v = __builtin_nontemporal_load(src + t);
+    __builtin_nontemporal_store(v, dst0 + t);
+    __builtin_nontemporal_store(v, dst1 + t);
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void stream_copy_tail_kernel(const float *__restrict__ src,
                                                                     float *__restrict__ dst,
                                                                     long long from, long long n) {
@@ -558,6 +570,25 @@ extern "C" int kfac_stream_copy_f32(float *dst, const float *src, int64_t nelems
     if (n4 * 4 < nelems)
       KFAC_LAUNCH(stream_copy_tail_kernel, dim3(1), dim3(kThreads), 0, s, src, dst, n4 * 4,
                          (long long)nelems);
+  }
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+extern "C" int kfac_stream_fanout_f32(float *dst0, float *dst1, const float *src, int64_t nelems, void *stream) {
+  KFAC_REQUIRE(nelems >= 0 && nelems % 4 == 0, "nelems must be a non-negative multiple of 4");
+  if (nelems == 0) return KFAC_OK;
+  KFAC_REQUIRE(dst0 && dst1 && src, "null pointer");
+  KFAC_REQUIRE(((reinterpret_cast<uintptr_t>(dst0) | reinterpret_cast<uintptr_t>(dst1) |
+                 reinterpret_cast<uintptr_t>(src)) & 15) == 0,
+               "pointers must be 16-byte aligned");
+  hipStream_t s = kfac::as_stream(stream);
+  const long long n4 = nelems / 4;
+  {
+    kfac::TimedLaunch timed(KFAC_TIMED_COPY, s);
+    KFAC_LAUNCH(stream_fanout_kernel, dim3((unsigned)kfac::ceil_div<long long>(n4, kThreads)), dim3(kThreads), 0, s,
+                reinterpret_cast<const floatx4a *>(src), reinterpret_cast<floatx4a *>(dst0),
+                reinterpret_cast<floatx4a *>(dst1), n4);
   }
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;

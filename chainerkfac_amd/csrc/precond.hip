@@ -674,8 +674,20 @@ struct kfac_precond_group {
   size_t ws_floats = 0;
   int task0[2][kPreKinds] = {}, ntask[2][kPreKinds] = {};
   int ftask0[2] = {0, 0}, nftask[2] = {0, 0};
+  double kind_work[2][kPreKinds] = {};   // matrix work of each launch
   kfac::DevTable d_items, d_tasks;
   kfac::DevTableRing d_dyn;
+  // The launches of a phase are independent of each other: the longest stays on the
+  // caller's stream, the others run beside it on a stream of the group's own (each
+  // launch ends on a partly empty GPU; side by side they fill each other's tails).
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork[2] = {nullptr, nullptr}, ev_join[2] = {nullptr, nullptr};
+  bool capture_origin = false;   // see kfac_precond_group_set_capture_origin
+  ~kfac_precond_group() {
+    for (hipEvent_t e : {ev_fork[0], ev_fork[1], ev_join[0], ev_join[1]})
+      if (e) (void)hipEventDestroy(e);
+    if (side) (void)hipStreamDestroy(side);
+  }
 };
 
 extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int32_t *dA,
@@ -759,6 +771,8 @@ extern "C" int kfac_precond_group_create(int count, const int32_t *dG, const int
       }
     }
   }
+  for (int p = 0; p < 2; ++p)
+    for (int k = 0; k < kPreKinds; ++k) g->kind_work[p][k] = work[p][k];
   // partial tiles: one area per item, shared by the two phases
   for (int i = 0; i < count; ++i) {
     PreStatic &s = g->items[i];
@@ -800,6 +814,12 @@ extern "C" int kfac_precond_group_destroy(kfac_precond_group_t group) {
   return KFAC_OK;
 }
 
+extern "C" int kfac_precond_group_set_capture_origin(kfac_precond_group_t group, int is_origin) {
+  KFAC_REQUIRE(group != nullptr, "group is null");
+  group->capture_origin = is_origin != 0;
+  return KFAC_OK;
+}
+
 extern "C" int kfac_precond_group_run_f32(kfac_precond_group_t group, const float *const *Ginv,
                                           const float *const *Ainv, const float *const *gradW,
                                           const float *const *gradb, float *const *kfW,
@@ -836,15 +856,50 @@ extern "C" int kfac_precond_group_run_f32(kfac_precond_group_t group, const floa
        gemm_group_kernel<2, 0, true, true>, nullptr, gemm_group_kernel<2, 0, false, false>},
       {gemm_group_kernel<1, 1, true, true>, gemm_group_kernel<1, 1, true, false>, nullptr,
        gemm_group_kernel<2, 1, true, true>, gemm_group_kernel<2, 1, true, false>, nullptr}};
+  // side stream: not while launches are timed one by one, not in host-only mode, and under
+  // stream capture only from the stream the capture began on (the caller says so)
+  bool may_fork = kfac::option_int(kfac::kOptGroupSideStream, 1) != 0 && !kfac::timing_on() && !kfac::host_only();
+  if (may_fork && !group->capture_origin) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
+      (void)hipGetLastError();
+      may_fork = false;
+    } else if (cs != hipStreamCaptureStatusNone) {
+      may_fork = false;
+    }
+  }
   for (int p = 0; p < 2; ++p) {
+    int nlaunch = 0, longest = -1;
     for (int k = 0; k < kPreKinds; ++k) {
       if (group->ntask[p][k] == 0) continue;
       if (!kerns[p][k]) return kfac::fail(KFAC_EINVAL, "internal: no kernel for kind %d", k);
-      kfac::TimedLaunch timed(KFAC_TIMED_GEMM, s);
-      KFAC_LAUNCH(kerns[p][k], dim3(group->ntask[p][k]), dim3(THREADS), 0, s, st, dy,
-                         tasks + group->task0[p][k], base);
+      ++nlaunch;
+      if (longest < 0 || group->kind_work[p][k] > group->kind_work[p][longest]) longest = k;
     }
+    const bool fork = may_fork && nlaunch >= 2;
+    if (fork) {
+      if (!group->side) KFAC_HIP_CHECK(hipStreamCreateWithFlags(&group->side, hipStreamNonBlocking));
+      if (!group->ev_fork[p]) {
+        KFAC_HIP_CHECK(hipEventCreateWithFlags(&group->ev_fork[p], hipEventDisableTiming));
+        KFAC_HIP_CHECK(hipEventCreateWithFlags(&group->ev_join[p], hipEventDisableTiming));
+      }
+      KFAC_HIP_CHECK(hipEventRecord(group->ev_fork[p], s));
+      KFAC_HIP_CHECK(hipStreamWaitEvent(group->side, group->ev_fork[p], 0));
+    }
+    // (the longest first: its workgroups are placed before the others fill in)
+    for (int pass = 0; pass < 2; ++pass)
+      for (int k = 0; k < kPreKinds; ++k) {
+        if (group->ntask[p][k] == 0 || (pass == 0) != (k == longest)) continue;
+        hipStream_t st_k = fork && k != longest ? group->side : s;
+        kfac::TimedLaunch timed(KFAC_TIMED_GEMM, st_k);
+        KFAC_LAUNCH(kerns[p][k], dim3(group->ntask[p][k]), dim3(THREADS), 0, st_k, st, dy,
+                    tasks + group->task0[p][k], base);
+      }
     KFAC_HIP_CHECK(hipGetLastError());
+    if (fork) {
+      KFAC_HIP_CHECK(hipEventRecord(group->ev_join[p], group->side));
+      KFAC_HIP_CHECK(hipStreamWaitEvent(s, group->ev_join[p], 0));
+    }
     if (group->nftask[p] > 0) {
       kfac::TimedLaunch timed(KFAC_TIMED_GEMM_AUX, s);
       if (p == 0)

@@ -635,6 +635,8 @@ class PrecondGroup(object):
                 _dev.require_gpu_tensor(gb, 'gradb')
                 _dev.require_gpu_tensor(kb, 'kfb')
         ws = _dev.workspace('precond_group', self.workspace_bytes, Ginvs[0].device)
+        origin = stream is None and _dev.current_lane() is None
+        _lib.check(_lib.load().kfac_precond_group_set_capture_origin(self._plan, int(origin)))
         _lib.check(_lib.load().kfac_precond_group_run_f32(
             self._plan, _lib.ptr_array([t.data_ptr() for t in Ginvs]),
             _lib.ptr_array([t.data_ptr() for t in Ainvs]), _lib.ptr_array([t.data_ptr() for t in gradWs]),

@@ -240,8 +240,13 @@ class KFAC(object):
     #: number of side streams the per-layer factor and preconditioning kernels
     #: are dealt onto (layers are independent of each other and most of their
     #: kernels are too small to fill the GPU alone); 0 keeps everything on the
-    #: caller's stream.  Read at ``setup``.
-    lanes = 4
+    #: caller's stream.  Read at ``setup``.  Three is the best count for launches
+    #: made from the host: a process has four hardware queues, and with more
+    #: streams than queues (the caller's stream, the lanes, the library's own side
+    #: streams) independent launches wait behind each other (measured on the
+    #: ResNet-50 step: 13.4 ms with three lanes, 14.7 with four).  A step replayed
+    #: from a captured HIP graph is fastest with four (12.7 against 13.0 ms).
+    lanes = 3
 
     #: apply the momentum rule of all parameters with one launch per set of
     #: hyperparameters (normally one) instead of one launch per parameter

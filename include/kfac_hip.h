@@ -388,6 +388,10 @@ int kfac_precond_group_create(int count, const int32_t *dG, const int32_t *dA,
                               const int32_t *has_bias, kfac_precond_group_t *group_out);
 size_t kfac_precond_group_workspace_bytes(kfac_precond_group_t group);
 int kfac_precond_group_destroy(kfac_precond_group_t group);
+/* Like a covariance group, a preconditioning group runs the longest launch of each
+ * phase on the caller's stream and the others on a stream of its own; under stream
+ * capture only after the caller has declared the stream the capture's origin. */
+int kfac_precond_group_set_capture_origin(kfac_precond_group_t group, int is_origin);
 int kfac_precond_group_run_f32(kfac_precond_group_t group, const float *const *Ginv,
                                const float *const *Ainv, const float *const *gradW,
                                const float *const *gradb, float *const *kfW,
@@ -507,6 +511,13 @@ int kfac_momentum_update_batched_f32(kfac_momentum_batch_t batch, int count,
  * puts beside the pack / unpack bandwidth (what a copy kernel reaches on the
  * same GPU in the same run).  No counterpart in the reference. */
 int kfac_stream_copy_f32(float *dst, const float *src, int64_t nelems, void *stream);
+
+/* dst0[i] = dst1[i] = src[i]: the same streaming kernel with the traffic mix of the
+ * unpack kernel (every packed element is read once and, but for the diagonal,
+ * written twice: 12 bytes per element), as a second yardstick.  nelems a multiple
+ * of 4, 16-byte aligned pointers.  No counterpart in the reference. */
+int kfac_stream_fanout_f32(float *dst0, float *dst1, const float *src, int64_t nelems,
+                           void *stream);
 
 int kfac_timing_enable(int on);
 int kfac_timing_read(int family, int64_t *launches, double *total_ms);
