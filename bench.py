@@ -1185,6 +1185,9 @@ def main():
                     help='skip the measurements beside the step (momentum rule of all parameters, moving average '
                          'of all factors): profiling runs')
     ap.add_argument('--host-launch-child', action='store_true', help=argparse.SUPPRESS)
+    ap.add_argument('--in-process', action='store_true',
+                    help='measure the eager step and the per-family brackets in this process instead of '
+                         'a fresh one (needed under rocprofv3: a profiled process must not start others)')
     ap.add_argument('--real-network', action='store_true', help=argparse.SUPPRESS)
     ap.add_argument('--no-other-configs', action='store_true',
                     help='c3 only: skip the short runs of c1, c2, c4 and c5 and the real-network step that the '
@@ -1232,7 +1235,7 @@ def main():
     # first, before this process has touched the GPU.
     with_others = args.config == 'c3' and not args.no_other_configs
     host = {}
-    if not args.no_graph and not args.host_launch_child:
+    if not args.no_graph and not args.host_launch_child and not args.in_process:
         for name in [args.config] + (['c1', 'c2', 'c5'] if with_others else []):
             if name != 'c4':
                 host[name] = host_launch_child(args, name)
