@@ -366,13 +366,34 @@ def run_step_config(args, name, cfg, host=None):
         for _ in range(3):
             step()
         eager, _ = timed_steps(step, max(args.steps, 5))
-        return {'eager_ms_per_step': eager, 'lanes': args.lanes, 'fam': fam, 'empty': empty,
-                'info_bad': len(opt.check_numerics())}
+        # how long the host takes to queue a step (no synchronisation until the last one is queued)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            step()
+        queued = (time.perf_counter() - t0) * 1e3 / 5
+        torch.cuda.synchronize()
+        return {'eager_ms_per_step': eager, 'host_ms_to_queue_a_step': queued, 'lanes': args.lanes, 'fam': fam,
+                'empty': empty, 'info_bad': len(opt.check_numerics())}
 
     if args.host_launch_child:
         return host_launched()
     run = step if args.no_graph else capture(step)
     ms_per_step, ms_median = timed_steps(run, args.steps)
+    replay_equals_eager = None
+    if not args.no_graph:
+        # the timed replays must have computed what the eager step computes: every factor inverse
+        # and every preconditioned gradient, bit for bit (a step of these configurations has no
+        # history, so the eager step afterwards starts from the same inputs)
+        def results():
+            return [t.clone() for fb in opt.fblocks for t in fb.invs] + \
+                   [p.kfgrad.clone() for _, p in sorted(model.namedparams()) if getattr(p, 'kfgrad', None) is not None]
+        replayed = results()
+        step()
+        torch.cuda.synchronize()
+        eager = results()
+        replay_equals_eager = len(eager) == len(replayed) and all(torch.equal(a, b) for a, b in zip(replayed, eager))
+        del replayed, eager
 
     # per-phase split: each phase launched the same way as the step (its own graph), timed with events
     phases = {'cov': cov_phase, 'inverse': inv_phase, 'precondition': pre_phase}
@@ -544,8 +565,11 @@ def run_step_config(args, name, cfg, host=None):
         'wire_format': wire_stats,
         'roofline': roofline,
     }
+    if replay_equals_eager is not None:
+        result['graph_replay_equals_eager_step'] = replay_equals_eager
     result['eager_ms_per_step'] = round(eager_ms, 4)
     result['eager_lanes'] = eager_lanes
+    result['eager_host_ms_to_queue_a_step'] = round(host['host_ms_to_queue_a_step'], 3)
     if real_network is not None:
         result['real_network'] = real_network
     result.update(extras)

@@ -530,6 +530,81 @@ def test_side_streams_do_not_change_results(monkeypatch):
             assert np.array_equal(a0, a1), (n0, k0)
 
 
+@pytest.mark.parametrize('decay', [1.0, 0.9])
+def test_step_replayed_from_a_hip_graph_matches_the_eager_step(monkeypatch, decay):
+    """The benchmark times the step as a HIP-graph replay with four lanes (and the
+    library's own side streams forked inside the capture).  Every replay must leave
+    exactly what the eager step leaves: two optimizers built from the same seed run
+    in lockstep, one eagerly and one replaying its captured step, with unrelated
+    eager work and synchronisations between the replays.  decay 1: every step is a
+    first step (factors aliased, rank-n batch-norm inverses); decay 0.9: the moving
+    average carries history from replay to replay."""
+    import bench
+    from chainerkfac_amd.optimizers import KFAC
+    layers = [
+        dict(kind='conv', name='c0', c_in=3, c_out=64, k=3, s=1, p=1, bias=True, h=14, w=14),
+        dict(kind='bn', name='b0', c=64, h=14, w=14),
+        dict(kind='conv', name='c1', c_in=64, c_out=64, k=3, s=1, p=1, bias=True, h=14, w=14),   # shifted correlations, d = 577
+        dict(kind='bn', name='b1', c=64, h=14, w=14),
+        dict(kind='conv', name='c2', c_in=64, c_out=136, k=1, s=1, p=0, bias=True, h=14, w=14),
+        dict(kind='conv', name='c3', c_in=136, c_out=40, k=3, s=2, p=1, bias=False, h=14, w=14),
+        dict(kind='conv', name='c4', c_in=40, c_out=256, k=1, s=1, p=0, bias=True, h=7, w=7),   # d = 257: bordered inverse
+        dict(kind='linear', name='fc', d_in=640, d_out=10, bias=True),
+    ]
+    monkeypatch.setattr(KFAC, 'lanes', 4)
+    dev = torch.device('cuda:0')
+
+    def make():
+        gen = torch.Generator(device='cuda').manual_seed(23)
+        model, calls = bench.build_model(layers, dev, gen, 8)
+        opt = KFAC(damping=1e-2, cov_ema_decay=decay).setup(model)
+        assert opt._lanes.n == 4
+
+        def step():
+            for _, func, in_data, gy in calls:
+                opt.kfhook.forward_postprocess(func, in_data)
+                opt.kfhook.backward_preprocess(func, in_data, (gy,))
+            opt.finish_covs()
+            opt.update_cov_emas(opt.fblocks)
+            opt.update_invs_batched(opt.fblocks)
+            opt.precondition(opt.fblocks)
+        opt.reallocate_cleared_grads()
+        return model, opt, step
+
+    def state(model, opt):
+        torch.cuda.synchronize()
+        got = []
+        for fb in opt.fblocks:
+            got += [(fb.linkname, 'cov', c.cpu().numpy()) for c in fb.cov_emas]
+            got += [(fb.linkname, 'inv', c.cpu().numpy()) for c in fb.invs]
+        got += [(n, 'kfgrad', p.kfgrad.cpu().numpy()) for n, p in sorted(model.namedparams())]
+        return got
+
+    eager_model, eager_opt, eager_step = make()
+    graph_model, graph_opt, graph_step = make()
+    for _ in range(2):   # plans, device tables and lane workspaces exist before the capture
+        eager_step()
+        graph_step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        graph_step()
+    scratch = torch.randn(512, 512, device=dev)
+    for replay in range(3):
+        eager_step()
+        graph.replay()
+        a, b = state(eager_model, eager_opt), state(graph_model, graph_opt)
+        assert len(a) == len(b) and len(a) > 30
+        for (n0, k0, x0), (n1, k1, x1) in zip(a, b):
+            assert (n0, k0) == (n1, k1)
+            assert np.isfinite(x0).all(), (replay, n0, k0)
+            assert np.array_equal(x0, x1), (replay, n0, k0)
+        # the program's own eager work between the replays
+        scratch = torch.tanh(scratch @ scratch)
+        assert not eager_opt.check_numerics() and not graph_opt.check_numerics()
+        torch.cuda.synchronize()
+
+
 def test_constructor_defaults_and_plugin_seam():
     from chainerkfac_amd import links as L
     from chainerkfac_amd.optimizers import KFAC, fblock_constructor
