@@ -52,6 +52,11 @@ PROTOTYPES = {
     'kfac_bn_workspace_bytes': (c_sz, [c_int, c_int]),
     'kfac_bn_grad_matrix_f32': (c_int, [c_vp, c_vp, c_int, c_int, c_int, c_f, c_f, c_int, c_int,
                                         c_vp, c_vp, c_sz, c_vp]),
+    'kfac_bn_stats_f32': (c_int, [c_vp, c_vp, c_int, c_int, c_int, c_vp, c_sz, c_vp]),
+    'kfac_bn_finish_batch_create': (c_int, [c_vp]),
+    'kfac_bn_finish_batch_destroy': (c_int, [c_vp]),
+    'kfac_bn_finish_batched_f32': (c_int, [c_vp, c_int, c_vpp, c_vpp, c_i32p, c_i32p, c_i32p, c_vp, c_vp,
+                                           c_i32p, c_i32p, c_vp]),
     'kfac_axpby_f32': (c_int, [c_vp, c_vp, c_i64, c_f, c_f, c_vp]),
     'kfac_axpby_batch_create': (c_int, [c_vp]),
     'kfac_axpby_batch_destroy': (c_int, [c_vp]),

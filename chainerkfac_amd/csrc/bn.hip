@@ -7,6 +7,8 @@
 // Replaces chainerkfac/optimizers/fisher_blocks/normalizations/
 // batch_normalization.py:86-119.
 #include <cstdlib>
+#include <new>
+#include <vector>
 
 #include "common.h"
 
@@ -139,13 +141,13 @@ __global__ __launch_bounds__(kThreads) void bn_stats_reg_kernel(
 // coalesced), the samples dealt to the 4 waves: batch mean and variance of the
 // channel from the slab statistics, then the channel's column(s) of U.
 //   sum_hw gy (x - mean_c) = sgx_s + (mean_s - mean_c) sg_s
-__global__ __launch_bounds__(256) void bn_finish_kernel(
-    int n, int c, int hw, float eps, float gy_scale, int has_gamma, int has_beta,
+__device__ __forceinline__ void bn_finish_block(
+    int block, int n, int c, int hw, float eps, float gy_scale, int has_gamma, int has_beta,
     const float *__restrict__ smean, const float *__restrict__ sm2, const float *__restrict__ sg,
     const float *__restrict__ sgx, float *__restrict__ U) {
   __shared__ float part[2][4][64];
   const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
-  const int ch = blockIdx.x * 64 + lane;
+  const int ch = block * 64 + lane;
   const bool live = ch < c;
   const int width = c * (has_gamma + has_beta);
   float mean = 0.f, rstd = 0.f;
@@ -186,6 +188,50 @@ __global__ __launch_bounds__(256) void bn_finish_kernel(
   }
 }
 
+__global__ __launch_bounds__(256) void bn_finish_kernel(
+    int n, int c, int hw, float eps, float gy_scale, int has_gamma, int has_beta,
+    const float *__restrict__ smean, const float *__restrict__ sm2, const float *__restrict__ sg,
+    const float *__restrict__ sgx, float *__restrict__ U) {
+  bn_finish_block(blockIdx.x, n, c, hw, eps, gy_scale, has_gamma, has_beta, smean, sm2, sg, sgx, U);
+}
+
+// The finish step of many layers in one launch: a unit is 64 channels of one layer.
+struct BnFinishItem {
+  const float *stats;   // [4][n][c]: slab mean, centred second moment, sum gy, sum gy (x - slab mean)
+  float *U;
+  int n, c, hw, has_gamma, has_beta;
+  float eps, gy_scale;
+};
+
+__global__ __launch_bounds__(256) void bn_finish_batched_kernel(const BnFinishItem *__restrict__ items,
+                                                                const int2 *__restrict__ units) {
+  const int2 u = units[blockIdx.x];
+  const BnFinishItem it = items[u.x];
+  const long long nslab = (long long)it.n * it.c;
+  bn_finish_block(u.y, it.n, it.c, it.hw, it.eps, it.gy_scale, it.has_gamma, it.has_beta, it.stats,
+                  it.stats + nslab, it.stats + 2 * nslab, it.stats + 3 * nslab, it.U);
+}
+
+// The slab statistics of one layer (the kernel is chosen from the slab size and alignment).
+void launch_stats(const float *x, const float *gy, int nslab, int hw, float *smean, float *sm2, float *sg,
+                  float *sgx, hipStream_t s) {
+  const bool vec =
+      (hw & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gy)) & 15) == 0;
+  const bool stats_loop = kfac::option_int(kfac::kOptBnStatsLoop, 0) != 0;   // tuning override
+  if (vec && hw <= 4 * 16 * 4 && !stats_loop)
+    KFAC_LAUNCH((bn_stats_reg_kernel<16, 4>), dim3(kfac::ceil_div(nslab, kThreads / 16)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  else if (vec && hw > 256 && hw <= 4 * 64 * 13 && !stats_loop)
+    KFAC_LAUNCH((bn_stats_reg_kernel<64, 13>), dim3(kfac::ceil_div(nslab, kThreads / 64)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  else if (hw <= 256)
+    KFAC_LAUNCH(bn_stats_kernel<16>, dim3(kfac::ceil_div(nslab, kThreads / 16)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  else
+    KFAC_LAUNCH(bn_stats_kernel<64>, dim3(kfac::ceil_div(nslab, kThreads / 64)),
+                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+}
+
 }  // namespace
 
 extern "C" size_t kfac_bn_workspace_bytes(int n, int c) {
@@ -207,24 +253,75 @@ extern "C" int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, i
   const int nslab = n * c;
   float *smean = static_cast<float *>(ws);
   float *sm2 = smean + nslab, *sg = sm2 + nslab, *sgx = sg + nslab;
-  const bool vec =
-      (hw & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gy)) & 15) == 0;
   kfac::TimedLaunch timed(KFAC_TIMED_BN, s);
-  const bool stats_loop = kfac::option_int(kfac::kOptBnStatsLoop, 0) != 0;   // tuning override
-  if (vec && hw <= 4 * 16 * 4 && !stats_loop)
-    KFAC_LAUNCH((bn_stats_reg_kernel<16, 4>), dim3(kfac::ceil_div(nslab, kThreads / 16)),
-                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
-  else if (vec && hw > 256 && hw <= 4 * 64 * 13 && !stats_loop)
-    KFAC_LAUNCH((bn_stats_reg_kernel<64, 13>), dim3(kfac::ceil_div(nslab, kThreads / 64)),
-                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
-  else if (hw <= 256)
-    KFAC_LAUNCH(bn_stats_kernel<16>, dim3(kfac::ceil_div(nslab, kThreads / 16)),
-                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
-  else
-    KFAC_LAUNCH(bn_stats_kernel<64>, dim3(kfac::ceil_div(nslab, kThreads / 64)),
-                       dim3(kThreads), 0, s, x, gy, nslab, hw, smean, sm2, sg, sgx);
+  launch_stats(x, gy, nslab, hw, smean, sm2, sg, sgx, s);
   KFAC_LAUNCH(bn_finish_kernel, dim3(kfac::ceil_div(c, 64)), dim3(256), 0, s, n, c, hw, eps,
                      gy_scale, has_gamma ? 1 : 0, has_beta ? 1 : 0, smean, sm2, sg, sgx, U);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+extern "C" int kfac_bn_stats_f32(const float *x, const float *gy, int n, int c, int hw, float *stats,
+                                 size_t stats_bytes, void *stream) {
+  KFAC_REQUIRE(n > 0 && c > 0 && hw > 0, "bad shape n=%d c=%d hw=%d", n, c, hw);
+  KFAC_REQUIRE((long long)n * c < 0x7fffffffLL, "too many (sample, channel) slabs");
+  KFAC_REQUIRE(x && gy, "null pointer");
+  if (stats == nullptr || stats_bytes < kfac_bn_workspace_bytes(n, c))
+    return kfac::fail(KFAC_ENOMEM, "batch-norm statistics buffer too small: %zu < %zu bytes", stats_bytes,
+                      kfac_bn_workspace_bytes(n, c));
+  hipStream_t s = kfac::as_stream(stream);
+  const int nslab = n * c;
+  kfac::TimedLaunch timed(KFAC_TIMED_BN, s);
+  launch_stats(x, gy, nslab, hw, stats, stats + nslab, stats + 2 * (size_t)nslab, stats + 3 * (size_t)nslab, s);
+  KFAC_HIP_CHECK(hipGetLastError());
+  return KFAC_OK;
+}
+
+struct kfac_bn_finish_batch {
+  std::vector<BnFinishItem> items;
+  std::vector<int2> units;
+  kfac::DevTableRing item_table;
+  kfac::DevTable unit_table;
+};
+
+extern "C" int kfac_bn_finish_batch_create(kfac_bn_finish_batch_t *batch_out) {
+  KFAC_REQUIRE(batch_out != nullptr, "batch_out is null");
+  *batch_out = new (std::nothrow) kfac_bn_finish_batch;
+  return *batch_out ? KFAC_OK : kfac::fail(KFAC_ENOMEM, "out of host memory");
+}
+
+extern "C" int kfac_bn_finish_batch_destroy(kfac_bn_finish_batch_t batch) {
+  delete batch;
+  return KFAC_OK;
+}
+
+extern "C" int kfac_bn_finish_batched_f32(kfac_bn_finish_batch_t batch, int count, const float *const *stats,
+                                          float *const *U, const int32_t *n, const int32_t *c,
+                                          const int32_t *hw, const float *eps, const float *gy_scale,
+                                          const int32_t *has_gamma, const int32_t *has_beta, void *stream) {
+  KFAC_REQUIRE(batch != nullptr, "batch is null");
+  KFAC_REQUIRE(count >= 0, "count < 0");
+  if (count == 0) return KFAC_OK;
+  KFAC_REQUIRE(stats && U && n && c && hw && eps && gy_scale && has_gamma && has_beta, "null table");
+  batch->items.resize(count);
+  batch->units.clear();
+  for (int i = 0; i < count; ++i) {
+    KFAC_REQUIRE(n[i] > 0 && c[i] > 0 && hw[i] > 0, "layer %d: bad shape n=%d c=%d hw=%d", i, n[i], c[i], hw[i]);
+    KFAC_REQUIRE((long long)n[i] * c[i] < 0x7fffffffLL, "layer %d: too many (sample, channel) slabs", i);
+    KFAC_REQUIRE(has_gamma[i] || has_beta[i], "layer %d: gamma and beta are both absent", i);
+    KFAC_REQUIRE(stats[i] && U[i], "layer %d: null pointer", i);
+    batch->items[i] = BnFinishItem{stats[i], U[i],           n[i],         c[i], hw[i], has_gamma[i] ? 1 : 0,
+                                   has_beta[i] ? 1 : 0, eps[i], gy_scale[i]};
+    for (int b = 0; b < kfac::ceil_div(c[i], 64); ++b) batch->units.push_back(make_int2(i, b));
+  }
+  hipStream_t s = kfac::as_stream(stream);
+  const void *d_items = nullptr;
+  if (int rc = batch->item_table.set(batch->items.data(), sizeof(BnFinishItem) * (size_t)count, s, &d_items))
+    return rc;
+  if (int rc = batch->unit_table.set(batch->units.data(), sizeof(int2) * batch->units.size(), s)) return rc;
+  kfac::TimedLaunch timed(KFAC_TIMED_BN, s);
+  KFAC_LAUNCH(bn_finish_batched_kernel, dim3((unsigned)batch->units.size()), dim3(256), 0, s,
+                     static_cast<const BnFinishItem *>(d_items), batch->unit_table.as<const int2>());
   KFAC_HIP_CHECK(hipGetLastError());
   return KFAC_OK;
 }

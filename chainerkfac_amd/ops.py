@@ -164,6 +164,7 @@ class PendingCovs(object):
 
     def __init__(self):
         self.items, self.inputs, self.outputs, self.alphas, self.betas = [], [], [], [], []
+        self.bn_finishes = []
 
     def accepts(self, rows, d):
         return float(rows) * d * (d + 1) <= self.max_flops
@@ -180,11 +181,19 @@ class PendingCovs(object):
         self.alphas.append(alpha)
         self.betas.append(beta)
 
+    def add_bn_finish(self, stats, U, n, c, hw, eps, gy_scale, has_gamma, has_beta):
+        """The second part of a batch-norm layer's gradient matrix (``bn_stats`` has been
+        queued): all layers' finishes run as one launch at ``flush``, before the factors."""
+        self.bn_finishes.append((stats, U, n, c, hw, eps, gy_scale, has_gamma, has_beta))
+
     def flush(self, stream=None):
-        if not self.items:
+        if not self.items and not self.bn_finishes:
             return
         try:
-            cov_group(self.items).run(self.inputs, self.outputs, self.alphas, self.betas, stream)
+            if self.bn_finishes:
+                bn_finish_batched(self.bn_finishes, stream)
+            if self.items:
+                cov_group(self.items).run(self.inputs, self.outputs, self.alphas, self.betas, stream)
         finally:
             self.__init__()
 
@@ -210,6 +219,76 @@ def bn_grad_matrix(x, gy, eps, gy_scale, has_gamma=True, has_beta=True, out=None
         x.data_ptr(), gy.data_ptr(), n, c, hw, eps, gy_scale, int(bool(has_gamma)),
         int(bool(has_beta)), out.data_ptr(), ws.data_ptr(), ws.numel(), _dev.stream_handle(stream)))
     return out
+
+
+def bn_stats(x, gy, out=None, stream=None):
+    """First part of ``bn_grad_matrix``: the per (sample, channel) statistics of one layer,
+    a (4, n, C) array that ``bn_finish_batched`` turns into the gradient matrix."""
+    _dev.require_gpu_tensor(x, 'x')
+    _dev.require_gpu_tensor(gy, 'gy')
+    if x.ndim not in (2, 4):
+        raise RuntimeError('len(x.shape) must be 2 or 4, not {}.'.format(x.ndim))
+    if x.shape != gy.shape:
+        raise ValueError('x and gy shapes differ')
+    n, c = x.shape[0], x.shape[1]
+    hw = 1 if x.ndim == 2 else x.shape[2] * x.shape[3]
+    out = _out(out, (4, n, c), x)
+    _lib.check(_lib.load().kfac_bn_stats_f32(x.data_ptr(), gy.data_ptr(), n, c, hw, out.data_ptr(),
+                                             out.numel() * 4, _dev.stream_handle(stream)))
+    return out
+
+
+class _BnFinishBatch(object):
+    def __init__(self):
+        h = ctypes.c_void_p()
+        _lib.check(_lib.load().kfac_bn_finish_batch_create(ctypes.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        try:
+            h, self._h = self._h, None
+            if h is not None:
+                _lib._lib.kfac_bn_finish_batch_destroy(h)
+        except Exception:   # interpreter shutdown: the library may be gone
+            pass
+
+
+_bn_finish_batches = None
+
+
+def bn_finish_batched(layers, stream=None):
+    """Second part of ``bn_grad_matrix`` for a list of layers in one launch.  Every entry is
+    ``(stats, U, n, c, hw, eps, gy_scale, has_gamma, has_beta)`` with ``stats`` from
+    ``bn_stats`` and ``U`` the (n, width) output."""
+    global _bn_finish_batches
+    if not layers:
+        return
+    if _bn_finish_batches is None:
+        _bn_finish_batches = _PlanCache(16)
+    # one batch object per list of buffers (persistent per layer), so that its tables are written once
+    key = tuple(l[0].data_ptr() for l in layers) + tuple(l[1].data_ptr() for l in layers)
+    batch = _bn_finish_batches.get(key, _BnFinishBatch)
+    described = tuple(l[2:] for l in layers)
+    if getattr(batch, 'described', None) != described:
+        for stats, U, n, c, hw, eps, gy_scale, has_gamma, has_beta in layers:
+            _dev.require_gpu_tensor(stats, 'stats')
+            _dev.require_gpu_tensor(U, 'U')
+            width = c * (int(bool(has_gamma)) + int(bool(has_beta)))
+            if width == 0:
+                raise RuntimeError('gamma and beta must not be None as the same time')
+            if stats.numel() != 4 * n * c or U.numel() != n * width:
+                raise ValueError('stats {} / U {} do not match n={} c={}'.format(
+                    tuple(stats.shape), tuple(U.shape), n, c))
+        # the argument arrays of a list that comes back every step are built once
+        batch.arrays = (
+            _lib.ptr_array([l[0].data_ptr() for l in layers]), _lib.ptr_array([l[1].data_ptr() for l in layers]),
+            _lib.i32_array([l[2] for l in layers]), _lib.i32_array([l[3] for l in layers]),
+            _lib.i32_array([l[4] for l in layers]), _lib.f32_array([l[5] for l in layers]),
+            _lib.f32_array([l[6] for l in layers]), _lib.i32_array([int(bool(l[7])) for l in layers]),
+            _lib.i32_array([int(bool(l[8])) for l in layers]))
+        batch.described = described
+    _lib.check(_lib.load().kfac_bn_finish_batched_f32(batch._h, len(layers), *batch.arrays,
+                                                      _dev.stream_handle(stream)))
 
 
 def axpby(x, y, a, b, stream=None):

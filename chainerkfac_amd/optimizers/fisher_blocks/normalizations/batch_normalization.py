@@ -113,7 +113,12 @@ class FisherBlockBatchNormalization(FisherBlock):
             self._on_lane(diagonal_factor, (x, gy))
             return out
         if self.pending_covs is not None and self.pending_covs.accepts(n, width):
-            self._on_lane(stats, (x, gy))
+            # the pass over x and gy now, on a lane; U from the statistics with all other layers'
+            # in one launch, right before the grouped launch that reads it
+            slabs = self._buffer('bn_stats', (4, n, x.shape[1]), x.device)
+            self._on_lane(lambda: ops.bn_stats(x, gy, out=slabs), (x, gy))
+            hw = 1 if x.ndim == 2 else x.shape[2] * x.shape[3]
+            self.pending_covs.add_bn_finish(slabs, U, n, x.shape[1], hw, eps, gy_scale, has_gamma, has_beta)
             self._defer_cov(ops.COV_LINEAR, U, False, n, out, alpha, beta)
             return out
 

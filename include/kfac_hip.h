@@ -218,6 +218,27 @@ int kfac_bn_grad_matrix_f32(const float *x, const float *gy, int n, int c,
                             int has_beta, float *U, void *ws, size_t ws_bytes,
                             void *stream);
 
+/* The same in two parts, so that the second part of every batch-norm layer of
+ * a network is one launch.  kfac_bn_stats_f32: the pass over x and gy of one
+ * layer, which leaves per (sample, channel) statistics in `stats`
+ * (kfac_bn_workspace_bytes(n, c) bytes, kept by the caller until the finish).
+ * kfac_bn_finish_batched_f32: U of `count` layers from their statistics; the
+ * arithmetic of kfac_bn_grad_matrix_f32, bit-identical results.  Replaces the
+ * loop over normalizations/batch_normalization.py:86-119 that the function
+ * hook drives (optimizers/kfac.py:33-48).  The batch object keeps device
+ * tables of the layers and rewrites them when the arguments change. */
+int kfac_bn_stats_f32(const float *x, const float *gy, int n, int c, int hw,
+                      float *stats, size_t stats_bytes, void *stream);
+typedef struct kfac_bn_finish_batch *kfac_bn_finish_batch_t;
+int kfac_bn_finish_batch_create(kfac_bn_finish_batch_t *batch_out);
+int kfac_bn_finish_batch_destroy(kfac_bn_finish_batch_t batch);
+int kfac_bn_finish_batched_f32(kfac_bn_finish_batch_t batch, int count,
+                               const float *const *stats, float *const *U,
+                               const int32_t *n, const int32_t *c,
+                               const int32_t *hw, const float *eps,
+                               const float *gy_scale, const int32_t *has_gamma,
+                               const int32_t *has_beta, void *stream);
+
 /* y = a*x + b*y over one pair of arrays of `nelems` floats; with b == 0, y is
  * overwritten without being read.
  * Moving average of optimizers/fisher_block.py:162-163 (a = decay on the new

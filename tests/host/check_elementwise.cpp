@@ -12,6 +12,42 @@ int check_elementwise(const std::vector<Workload> &workloads) {
                                        fake_ptr(4), kfac_bn_workspace_bytes(b.n, b.c), nullptr);
       EXPECT(rc == KFAC_OK, "%s: batch-norm statistics %d ch @%d: %s", what, b.c, b.h, kfac_last_error_string());
     }
+    {
+      // the same in two parts: statistics per layer, one finish launch for all layers
+      const int nb = (int)w.bns.size();
+      std::vector<const float *> stats(nb);
+      std::vector<float *> U(nb);
+      std::vector<int32_t> bn_n(nb), bn_c(nb), bn_hw(nb), yes(nb, 1), no(nb, 0);
+      std::vector<float> eps(nb, 2e-5f), scale(nb);
+      for (int i = 0; i < nb; ++i) {
+        const BnShape &b = w.bns[i];
+        stats[i] = fake_ptr(10 + 2 * i);
+        U[i] = fake_ptr(11 + 2 * i);
+        bn_n[i] = b.n, bn_c[i] = b.c, bn_hw[i] = b.h * b.w, scale[i] = (float)b.n;
+        int rc = kfac_bn_stats_f32(fake_ptr(1), fake_ptr(2), b.n, b.c, b.h * b.w, fake_ptr(10 + 2 * i),
+                                   kfac_bn_workspace_bytes(b.n, b.c), nullptr);
+        EXPECT(rc == KFAC_OK, "%s: batch-norm statistics alone %d ch @%d: %s", what, b.c, b.h, kfac_last_error_string());
+        rc = kfac_bn_stats_f32(fake_ptr(1), fake_ptr(2), b.n, b.c, b.h * b.w, fake_ptr(10 + 2 * i),
+                               kfac_bn_workspace_bytes(b.n, b.c) - 1, nullptr);
+        EXPECT(rc == KFAC_ENOMEM, "%s: a statistics buffer one byte short was accepted", what);
+      }
+      kfac_bn_finish_batch_t fb = nullptr;
+      EXPECT(kfac_bn_finish_batch_create(&fb) == KFAC_OK && fb, "%s: bn finish batch", what);
+      for (int rep = 0; rep < 2; ++rep)
+        EXPECT(kfac_bn_finish_batched_f32(fb, nb, stats.data(), U.data(), bn_n.data(), bn_c.data(), bn_hw.data(), eps.data(),
+                                          scale.data(), yes.data(), yes.data(), nullptr) == KFAC_OK,
+               "%s: batched finish: %s", what, kfac_last_error_string());
+      if (nb) {
+        EXPECT(kfac_bn_finish_batched_f32(fb, nb, stats.data(), U.data(), bn_n.data(), bn_c.data(), bn_hw.data(), eps.data(),
+                                          scale.data(), no.data(), no.data(), nullptr) == KFAC_EINVAL,
+               "%s: layers with neither gamma nor beta accepted", what);
+        U[nb - 1] = nullptr;
+        EXPECT(kfac_bn_finish_batched_f32(fb, nb, stats.data(), U.data(), bn_n.data(), bn_c.data(), bn_hw.data(), eps.data(),
+                                          scale.data(), yes.data(), no.data(), nullptr) == KFAC_EINVAL,
+               "%s: a null output accepted", what);
+      }
+      kfac_bn_finish_batch_destroy(fb);
+    }
     const int n = (int)w.factor_dims.size();
     std::vector<float *> mats(n);
     std::vector<const float *> xs(n);

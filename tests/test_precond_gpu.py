@@ -94,6 +94,39 @@ def test_bn_factor(shape):
     assert rel(Ub.cpu().numpy(), O.bn_grad_matrix(x, gy, eps, has_gamma=False)) < 1e-4
 
 
+def test_bn_factor_in_two_parts_for_many_layers():
+    """The statistics pass per layer and the finish of all layers in one launch give,
+    bit for bit, what the one-layer entry point gives (the same arithmetic), against
+    the oracle, for every combination of gamma / beta, channel counts that are not
+    multiples of the 64-channel unit, 2-D inputs and different scales per layer."""
+    from chainerkfac_amd import ops
+    cases = [((6, 4, 5, 3), True, True, 6.0), ((8, 5), True, True, 8.0), ((32, 64, 8, 8), True, False, 1.0),
+             ((4, 130, 7, 7), False, True, 4.0), ((16, 1000), True, True, 0.25), ((3, 65, 16, 16), True, True, 3.0)]
+    r = np.random.default_rng(41)
+    layers, singles, refs = [], [], []
+    for shape, has_gamma, has_beta, scale in cases:
+        x = (r.standard_normal(shape) * 2 + 0.7).astype(np.float32)
+        gy = (r.standard_normal(shape) / shape[0]).astype(np.float32)
+        eps = 2e-5
+        n, c = shape[0], shape[1]
+        hw = int(np.prod(shape[2:])) if len(shape) == 4 else 1
+        xd, gd = torch.from_numpy(x).cuda(), torch.from_numpy(gy).cuda()
+        singles.append(ops.bn_grad_matrix(xd, gd, eps, scale, has_gamma, has_beta))
+        refs.append(O.bn_grad_matrix(x, gy, eps, has_gamma=has_gamma, has_beta=has_beta) * (scale / n))
+        stats = ops.bn_stats(xd, gd)
+        assert tuple(stats.shape) == (4, n, c)
+        U = torch.full((n, c * (int(has_gamma) + int(has_beta))), float('nan'), device='cuda')
+        layers.append((stats, U, n, c, hw, eps, scale, has_gamma, has_beta))
+    for _ in range(2):   # the second call finds its tables in place
+        ops.bn_finish_batched(layers)
+    for layer, single, ref in zip(layers, singles, refs):
+        assert torch.equal(layer[1], single), layer[2:]
+        assert rel(single.cpu().numpy(), ref) < 1e-4
+    ops.bn_finish_batched([])
+    with pytest.raises(ValueError):
+        ops.bn_finish_batched([(layers[0][0], layers[1][1]) + layers[0][2:]])
+
+
 def test_bn_rejects_other_ranks():
     from chainerkfac_amd import ops
     x = torch.zeros(2, 3, 4, device='cuda')
