@@ -86,6 +86,15 @@ class DevTable {
     const bool capturing = cs != hipStreamCaptureStatusNone;
     if (matches(host, bytes)) {
       if (capturing) pinned_ = true;
+      // the contents may still be on their way, queued on another stream: this one waits for them
+      // (a capture starts after the device has been synchronised, so nothing is pending then)
+      if (copy_pending_ && !capturing) {
+        if (hipEventQuery(copied_) == hipSuccess)
+          copy_pending_ = false;
+        else if (stream != upload_stream_)
+          KFAC_HIP_CHECK(hipStreamWaitEvent(stream, copied_, 0));
+        (void)hipGetLastError();   // hipErrorNotReady of the query is not an error
+      }
       return KFAC_OK;
     }
     // an upload cannot be part of a capture (its source is gone by the time of a replay)
@@ -122,6 +131,7 @@ class DevTable {
       KFAC_HIP_CHECK(hipMemcpyAsync(dev_, staging_, bytes, hipMemcpyHostToDevice, stream));
       KFAC_HIP_CHECK(hipEventRecord(copied_, stream));
       copy_pending_ = true;
+      upload_stream_ = stream;
     }
     shadow_.assign(static_cast<const char *>(host),
                    static_cast<const char *>(host) + bytes);
@@ -165,6 +175,7 @@ class DevTable {
   size_t capacity_ = 0;
   std::vector<char> shadow_;
   hipEvent_t copied_ = nullptr;
+  hipStream_t upload_stream_ = nullptr;
   bool copy_pending_ = false, pinned_ = false;
   char host_only_address_ = 0;   // what as<T>() returns in host-only mode (never dereferenced)
   // the contents last set, for checks of the tables on the host
