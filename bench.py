@@ -1020,12 +1020,32 @@ def summarize_kernel_trace(trace_dir, out_path, command):
     if not agg:
         raise SystemExit('no kernel_trace.csv under ' + trace_dir)
     total = float(sum(a[1] for a in agg.values()))
+    # elapsed time of every batched inverse: first copy_in after the previous call's lauum .. end of lauum
+    # (only calls with the whole sweep in between: the three-matrix inverses of other runs are left out)
+    spans, begin, inside = [], None, 0
+    ordered = sorted((int(r['Start_Timestamp']), int(r['End_Timestamp']), r['Kernel_Name'])
+                     for r in _csv_rows(trace_dir, 'kernel_trace.csv'))
+    for t0, t1, name in ordered:
+        if 'copy_in_kernel' in name and begin is None:
+            begin, inside = t0, 0
+        elif begin is not None and ('diag_kernel' in name or 'update_kernel' in name):
+            inside += 1
+        elif 'lauum_kernel' in name and begin is not None:
+            spans.append((t1 - begin, inside))
+            begin = None
+    most = max((n for _, n in spans), default=0)
+    spans = sorted(d for d, n in spans if n == most)
     lines = ['# Kernel time by kernel: ' + os.path.basename(out_path)[:-3].replace('_', ' '), '',
              'Command (one MI355X, repository root; raw output stays outside the repository):', '', '```',
              command, '```', '',
              'All launches of the run are counted (warm-up, timed steps, the phase split and the pass that times '
-             'every launch with HIP events), so "launches" is a multiple of the per-step count.', '',
-             '| family | launches | total ms | avg us / launch | share of GPU time |', '|---|---:|---:|---:|---:|']
+             'every launch with HIP events), so "launches" is a multiple of the per-step count. Durations are '
+             'summed per kernel: the kernels of the batched inverse run side by side on three streams (diagonal '
+             'tiles and panels, column updates, trailing updates), so their sum is about 1.7 times the time the '
+             'inverse takes (what `roofline.families.inverse_tiles` of the bench line divides by is the time '
+             'between the first and the last launch of the call), and "share" is a share of summed kernel time, '
+             'not of elapsed time.', '',
+             '| family | launches | total ms | avg us / launch | share of summed kernel time |', '|---|---:|---:|---:|---:|']
     fam = {}
     for name, a in agg.items():
         f = _family_of(name)
@@ -1037,6 +1057,10 @@ def summarize_kernel_trace(trace_dir, out_path, command):
         if f in fam:
             n, t = fam[f]
             lines.append('| {} | {} | {:.3f} | {:.1f} | {:.1f} % |'.format(f, n, t / 1e6, t / n / 1e3, 100 * t / total))
+    if spans:
+        lines += ['', 'Elapsed time of a batched inverse (start of its first `copy_in_kernel` to the end of its '
+                  '`lauum_kernel`, {} calls with the full sweep): median {:.3f} ms, min {:.3f}, max {:.3f}.'.format(
+                      len(spans), spans[len(spans) // 2] / 1e6, spans[0] / 1e6, spans[-1] / 1e6)]
     lines += ['', '| kernel | launches | total ms | avg us | min us | max us | share |', '|---|---:|---:|---:|---:|---:|---:|']
     for name, a in sorted(agg.items(), key=lambda kv: -kv[1][1])[:40]:
         if a[1] / total < 0.001:
@@ -1045,7 +1069,7 @@ def summarize_kernel_trace(trace_dir, out_path, command):
             name, a[0], a[1] / 1e6, a[1] / a[0] / 1e3, a[2] / 1e3, a[3] / 1e3, 100 * a[1] / total))
     with open(out_path, 'w') as f:
         f.write('\n'.join(lines) + '\n')
-    print('\n'.join(lines[:22]))
+    print('\n'.join(lines[:24]))
 
 
 def summarize_mfma(pmc_dir, out_path, command):
