@@ -983,14 +983,19 @@ def _csv_rows(directory, suffix):
                 yield r
 
 
+# (first match wins: the finish kernels of the GEMMs and of the batch-norm statistics carry their
+# own family's prefix and must not fall to the covariances' 'finish_')
 KERNEL_FAMILIES = (
     ('covariance SYRK family', ('syrk_', 'shift::corr_kernel')),
-    ('split-K finish of the covariances', ('finish_', 'reduce_kernel', 'shift::assemble', 'shift::edge_sums')),
+    ('preconditioning GEMMs (with their split-K finish and the batch-norm GEMV)', ('gemm_', 'gemv_', 'bn_select')),
+    ('batch-norm statistics and finish', ('bn_',)),
+    ('batch-norm rank-n inverses', ('lr_',)),
+    ('split-K finish, edge sums and assembly of the covariances', ('finish_', 'reduce_kernel', 'shift::assemble',
+                                                                  'shift::edge_sums')),
     ('inverse tile kernels', ('diag_kernel', 'update_kernel', 'lauum_kernel', 'panel_kernel', 'copy_in', 'copy_out',
-                              'trtri', 'potrf', 'small_inverse')),
-    ('preconditioning GEMMs', ('gemm_',)),
-    ('batch-norm statistics', ('bn_',)),
-    ('pack / unpack / copy', ('pack_kernel', 'unpack_kernel', 'stream_copy')),
+                              'border_kernel', 'trtri', 'potrf', 'small_inverse')),
+    ('damping', ('pi_damp', 'add_diag')),
+    ('pack / unpack / copy', ('pack_kernel', 'unpack_kernel', 'stream_copy', 'stream_fanout')),
 )
 
 
@@ -1166,7 +1171,9 @@ def summarize_traffic(fetch_dir, write_dir, out_path, command):
         total += out[key + '_bytes_per_launch']
         for fam, keys, marker in TRAFFIC_FAMILIES:
             steps = sum(1 for k, _ in rows if marker in k)
-            kib = sum(v for k, v in rows if any(x in k for x in keys))
+            # (the finish kernels of the GEMMs and of the batch-norm statistics are not the covariances')
+            kib = sum(v for k, v in rows if any(x in k for x in keys)
+                      and (fam != 'cov_syrk' or not any(x in k for x in ('gemm_', 'bn_'))))
             f = out['families'].setdefault(fam, {'steps_in_run': steps})
             f[key + '_bytes_per_step'] = kib * 1024.0 * scale / max(steps, 1)
         for k, v in rows:
