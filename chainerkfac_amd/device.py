@@ -47,6 +47,10 @@ class Workspace(object):
         if self._buf is None or self._buf.numel() < nbytes or self._buf.device != device:
             # wait for work that may still use the old buffer before dropping it
             if self._buf is not None:
+                if torch.cuda.is_current_stream_capturing():
+                    raise _lib.KfacHipError(
+                        'a scratch buffer would have to grow ({} -> {} bytes) while a HIP graph is being '
+                        'captured: run the same calls once before the capture'.format(self._buf.numel(), nbytes))
                 torch.cuda.synchronize(self._buf.device)
             self._buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
         return self._buf
@@ -129,6 +133,13 @@ class Lanes(object):
         if lane not in self._busy:
             self._busy.append(lane)
         return out
+
+    def skip(self):
+        """Passes the turn on without queueing anything: for a piece of work that the caller
+        keeps on its own stream this time, so that the pieces after it go to the lanes they go
+        to when it does take one (a lane's scratch buffers keep the sizes its pieces need)."""
+        if self.n > 0:
+            self._turn += 1
 
     def join(self):
         # every phase deals its work the same way each time it runs (the scratch
