@@ -87,6 +87,7 @@ struct InvTables {
   const int *nt;             // [count] tiles per side
   const long long *ws_off;   // [count] float offset of the padded matrix
   const int *tile_cs;        // [count+1] cumulative lower-tile counts (copy-in)
+  const int2 *tile_owner;    // [tiles] copy-in: (slot, I | J << 16) of every lower tile, one load instead of a search
   const TileTask *tasks;     // the tile tasks of all launches
   const BorderTask *btasks;  // the vector tasks of the bordered matrices
   float *ws;                 // padded matrices
@@ -361,10 +362,8 @@ __device__ __forceinline__ void tile_mainloop(const LA &la, const LB &lb, int K,
 // copy-in: lower tiles of in -> padded workspace (identity on the padding)
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void copy_in_kernel(InvTables tb, int count, int tile0) {
-  const int t = (int)blockIdx.x + tile0;
-  const int s = find_slot(tb.tile_cs, count, t);
-  int I, J;
-  tri_decode(t - tb.tile_cs[s], I, J);
+  const int2 owner = tb.tile_owner[(int)blockIdx.x + tile0];
+  const int s = owner.x, I = owner.y & 0xffff, J = owner.y >> 16;
   const int d = tb.dim[s], dc = tb.core[s];
   const float *__restrict__ src = tb.in[s];
   float *__restrict__ dst = tile_ptr(tb, s, I, J);
@@ -883,7 +882,7 @@ struct kfac_inverse_plan {
   kfac::DevTable d_core, d_orig, d_vec, d_btasks;
   size_t ws_floats = 0;            // padded matrices
   std::vector<const void *> in_sorted, out_sorted;
-  kfac::DevTable d_in, d_out, d_dim, d_nt, d_off, d_tile, d_tasks;
+  kfac::DevTable d_in, d_out, d_dim, d_nt, d_off, d_tile, d_tile_owner, d_tasks;
   bool attr_set = false;
 };
 
@@ -960,6 +959,12 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   p->ws_floats = total;
   p->total_tiles = tile_cs[count];
   p->first_tiles = tile_cs[count];   // set once the steps are known
+  // copy-in: the lower tiles of every matrix in row-major order, slot by slot
+  std::vector<int2> tile_owner;
+  tile_owner.reserve((size_t)p->total_tiles);
+  for (int s = 0; s < count; ++s)
+    for (int I = 0; I < p->nt[s]; ++I)
+      for (int J = 0; J <= I; ++J) tile_owner.push_back(make_int2(s, I | (J << 16)));
   p->max_t = count ? p->nt[0] : 0;
   std::vector<TileTask> tasks;
   std::vector<int2> natural;
@@ -1202,6 +1207,7 @@ extern "C" int kfac_inverse_plan_create(int count, const int32_t *dims,
   up(p->d_nt, p->nt.data(), sizeof(int) * count);
   up(p->d_off, off.data(), sizeof(long long) * count);
   up(p->d_tile, tile_cs.data(), sizeof(int) * (count + 1));
+  up(p->d_tile_owner, tile_owner.data(), sizeof(int2) * tile_owner.size());
   up(p->d_tasks, tasks.data(), sizeof(TileTask) * tasks.size());
   if (rc == KFAC_OK && p->lookahead && p->max_t > p->group) {
     const bool real = !kfac::host_only();   // host-only mode: null handles that nothing ever uses
@@ -1304,6 +1310,7 @@ extern "C" int kfac_spd_inverse_batched_f32(kfac_inverse_plan_t plan,
   tb.nt = plan->d_nt.as<const int>();
   tb.ws_off = plan->d_off.as<const long long>();
   tb.tile_cs = plan->d_tile.as<const int>();
+  tb.tile_owner = plan->d_tile_owner.as<const int2>();
   tb.tasks = plan->d_tasks.as<const TileTask>();
   tb.btasks = plan->d_btasks.as<const BorderTask>();
   uintptr_t base = (reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255;

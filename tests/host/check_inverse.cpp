@@ -57,6 +57,21 @@ void check_dims(const std::vector<int> &dims, const char *what) {
              "%s: slot %d vectors outside the workspace", what, s);
   }
   EXPECT((size_t)tiles_end * sizeof(float) <= ws_bytes, "%s: tiles outside the workspace", what);
+  {
+    // copy-in: one workgroup per lower tile, told its matrix and tile by the owner table
+    const auto &own_raw = plan->d_tile_owner.shadow();
+    const int2 *own = reinterpret_cast<const int2 *>(own_raw.data());
+    const long long nown = (long long)(own_raw.size() / sizeof(int2));
+    EXPECT(nown == plan->total_tiles, "%s: owner table has %lld entries for %d tiles", what, nown, plan->total_tiles);
+    long long at = 0;
+    for (int s = 0; s < count && at <= nown; ++s)
+      for (int I = 0; I < plan->nt[s]; ++I)
+        for (int J = 0; J <= I; ++J, ++at)
+          if (at < nown)
+            EXPECT(own[at].x == s && (own[at].y & 0xffff) == I && (own[at].y >> 16) == J, "%s: owner of tile %lld", what, at);
+    EXPECT(at == nown, "%s: owner table does not cover every lower tile once", what);
+    EXPECT(plan->first_tiles >= 0 && plan->first_tiles <= plan->total_tiles, "%s: first_tiles", what);
+  }
 
   // applied[s][(a, b)][j] = how often column j's product reached tile (a, b)
   std::vector<std::map<std::pair<int, int>, std::vector<int>>> applied(count);
