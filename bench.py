@@ -1242,7 +1242,7 @@ def main():
     ap.add_argument('--host-launch-child', action='store_true', help=argparse.SUPPRESS)
     ap.add_argument('--in-process', action='store_true',
                     help='measure the eager step and the per-family brackets in this process instead of '
-                         'a fresh one (needed under rocprofv3: a profiled process must not start others)')
+                         'a fresh one (chosen by itself under rocprofv3: a profiled process must not start others)')
     ap.add_argument('--real-network', action='store_true', help=argparse.SUPPRESS)
     ap.add_argument('--no-other-configs', action='store_true',
                     help='c3 only: skip the short runs of c1, c2, c4 and c5 and the real-network step that the '
@@ -1290,7 +1290,11 @@ def main():
     # first, before this process has touched the GPU.
     with_others = args.config == 'c3' and not args.no_other_configs
     host = {}
-    if not args.no_graph and not args.host_launch_child and not args.in_process:
+    # (a process started under rocprofv3 must not start others: the profiler's library has touched
+    # the GPU before main() runs; such a run measures everything in this process, like --in-process)
+    profiled = any(k.startswith(('ROCPROF', 'ROCP_')) for k in os.environ) or \
+        'rocprof' in os.environ.get('LD_PRELOAD', '')
+    if not args.no_graph and not args.host_launch_child and not args.in_process and not profiled:
         for name in [args.config] + (['c1', 'c2', 'c5'] if with_others else []):
             if name != 'c4':
                 host[name] = host_launch_child(args, name)
