@@ -55,7 +55,7 @@ def plan_check():
 def test_planners_under_sanitizers(plan_check, part, tmp_path):
     shapes = tmp_path / 'workloads.txt'
     _write_workloads(str(shapes))
-    env = dict(os.environ, ASAN_OPTIONS='detect_leaks=0:abort_on_error=0', UBSAN_OPTIONS='print_stacktrace=1')
+    env = dict(os.environ, ASAN_OPTIONS='detect_leaks=0:abort_on_error=0:verify_asan_link_order=0', UBSAN_OPTIONS='print_stacktrace=1')
     proc = subprocess.run([plan_check, str(shapes), part], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
                           timeout=600, env=env)
     out = proc.stdout.decode() + proc.stderr.decode()
